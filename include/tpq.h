@@ -1,0 +1,136 @@
+/*
+ * tpq.h - C ABI of the gfx950 (MI355X) quantized-linear kernel library.
+ *
+ * Conventions shared by every entry point:
+ *   - all tensor arguments are raw DEVICE pointers owned by the caller; the
+ *     library never allocates, frees or keeps them;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     work is enqueued on it and the call returns without synchronising;
+ *   - the return value is 0 on success and a TPQ_ERR_* code otherwise; the
+ *     text of the last failure on the calling thread is tpq_last_error();
+ *   - zero-sized problems succeed without launching anything;
+ *   - floating tensors carry a TPQ_DTYPE_* tag; 16-bit floats are raw bits.
+ *
+ * Each entry point names the operator of the TensorPlay reference it stands
+ * behind (paths relative to the reference root).
+ */
+#ifndef TPQ_H
+#define TPQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPQ_DTYPE_F32 0
+#define TPQ_DTYPE_F16 1
+#define TPQ_DTYPE_BF16 2
+
+#define TPQ_OK 0
+#define TPQ_ERR_INVALID_VALUE 1 /* reference raises ValueError  */
+#define TPQ_ERR_INVALID_TYPE 2  /* reference raises TypeError   */
+#define TPQ_ERR_RUNTIME 3       /* HIP launch / runtime failure */
+#define TPQ_ERR_UNSUPPORTED 4   /* valid in the reference, not built here */
+
+/* Library ABI version (bumped on any signature change). */
+int tpq_abi_version(void);
+
+/* Message of the most recent non-zero return on this thread ("" if none). */
+const char* tpq_last_error(void);
+
+/*
+ * Fused row-wise signed quantizer.
+ *   absmax = max_k |x[m,k]|; scale = max(absmax, eps) / divisor;
+ *   code = clamp(rint(x / scale), qmin, qmax)   (sign_mode: x >= 0 ? qmax : qmin)
+ * Replaces _quantize_int8_rowwise (divisor 127, [-127,127]),
+ * _quantize_int4_rowwise (7, [-8,7]), _quantize_int2_rowwise (2, [-2,1]) and
+ * _quantize_binary_rowwise (1, sign mode):
+ *   config/native_functions.yaml:5338-5347,
+ *   p10/src/backend/cuda/QuantGemmKernels.cu:1421-1609,
+ *   p10/src/backend/cuda/LowBitGemmKernels.cu:27-76.
+ * x [M,K] contiguous of x_dtype; codes int8 [M,K]; scales f32 [M].
+ */
+int tpq_quantize_rowwise(const void* x, int x_dtype, int64_t M, int64_t K, float eps,
+                         float divisor, int qmin, int qmax, int sign_mode, int8_t* codes,
+                         float* scales, void* stream);
+
+/*
+ * Integer matrix product C[M,N] (int32) = A[M,K] (int8, or uint8 when
+ * a_unsigned) x B[K,N] (int8).  B is addressed as b[k*b_stride_k + n*b_stride_n]
+ * so both a contiguous [K,N] operand (N,1) and the transposed view of a
+ * contiguous [N,K] weight (1,K) are accepted without a copy.
+ * Replaces _int_mm / _int_mm.out: config/native_functions.yaml:7987-7989,
+ * p10/src/backend/cuda/IntMM.cu:383-454.
+ */
+int tpq_int_mm(const void* a, int a_unsigned, const int8_t* b, int64_t b_stride_k,
+               int64_t b_stride_n, int32_t* c, int64_t M, int64_t K, int64_t N, void* stream);
+
+/*
+ * out[m,n] (f32) = (float(acc[m,n]) * row_scale[m]) * col_scale[n].
+ * Replaces _int8_mm_rescale: config/native_functions.yaml:5350,
+ * p10/src/backend/cuda/QuantGemmKernels.cu:1611-1650.
+ */
+int tpq_int8_mm_rescale(const int32_t* acc, const float* row_scale, const float* col_scale,
+                        float* out, int64_t M, int64_t N, void* stream);
+
+/*
+ * Fused int8 GEMM + dequant epilogue: out[m,n] = cast_out(
+ *   (float(sum_k a[m,k]*w[n,k]) * row_scale[m]) * col_scale[n] (+ bias[n])).
+ * a int8 [M,K], w int8 [N,K] (both K-contiguous), bias f32 [N] or NULL,
+ * out [M,N] of out_dtype.  One launch for the pair _int_mm + _int8_mm_rescale
+ * that _int8_mm issues (tensorplay/ao/quantization/int8_mixed_precision.py:60-77)
+ * and, with bias, the add at :242.
+ */
+int tpq_int8_mm_dequant(const int8_t* a, const int8_t* w, const float* row_scale,
+                        const float* col_scale, const float* bias, void* out, int out_dtype,
+                        int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
+ * int32 codes [N,K] in 0..15 -> int32 [ceil(N/8)][ceil(K/(16 I))][32][I/2],
+ * the packed layout of the reference's device op (I = inner_k_tiles in {2,4,8}).
+ * Replaces _convert_weight_to_int4pack: config/native_functions.yaml:7991,
+ * p10/src/backend/cuda/QuantGemmKernels.cu:322-330, 838-877, 1349-1408.
+ */
+int tpq_int4_pack(const int32_t* codes, int64_t N, int64_t K, int inner_k_tiles, int32_t* out,
+                  void* stream);
+
+/*
+ * y[m,n] = sum_k x[m,k] * ((code[n,k] - 8) * scale[k/g,n] + zero[k/g,n]).
+ * x [M,K] and y [M,N] of `dtype`; packed as written by tpq_int4_pack with
+ * inner_k_tiles = 2 and N = 8 * (first packed dimension); scales_and_zeros
+ * [ceil(K/g), N, 2] of `dtype`; g in {32,64,128}.
+ * Replaces _weight_int4pack_mm: config/native_functions.yaml:7993,
+ * p10/src/backend/cuda/QuantGemmKernels.cu:1210-1341.
+ */
+int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
+                int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
+                void* out, void* stream);
+
+/*
+ * int8 ternary codes [rows, cols] <-> uint8 [rows, ceil(cols/4)], four 2-bit
+ * fields per byte, first code in the two most significant bits.
+ * Replace pack_ternary / unpack_ternary:
+ * tensorplay/ao/quantization/bitnet.py:72-107.
+ */
+int tpq_ternary_pack(const int8_t* codes, int64_t rows, int64_t cols, uint8_t* out, void* stream);
+int tpq_ternary_unpack(const uint8_t* packed, int64_t rows, int64_t cols, int8_t* out,
+                       void* stream);
+
+/*
+ * BitNet packed linear after the activation quantizer:
+ *   acc[m,n] = sum_k x[m,k] * code[n,k]               (int32, exact)
+ *   out[m,n] = cast((float(acc) * row_scale[m]) * w_scale (+ bias[n]))
+ * x int8 [M,K]; packed uint8 [N, ceil(K/4)]; bias f32 [N] or NULL; acc_out
+ * int32 [M,N] or NULL (for parity checks); out [M,N] of out_dtype or NULL.
+ * Replaces the unpack + PackedWeight.run + rescale sequence of
+ * bitnet_linear_packed: tensorplay/ao/quantization/bitnet.py:215-241.
+ */
+int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packed, float w_scale,
+                   const float* bias, int64_t M, int64_t N, int64_t K, void* out, int out_dtype,
+                   int32_t* acc_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPQ_H */

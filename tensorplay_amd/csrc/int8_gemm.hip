@@ -1,0 +1,98 @@
+// Entry points of the integer matrix product (_int_mm) and of the fused
+// int8 GEMM + dequant; the matrix-core kernel itself lives in
+// int8_gemm_kernel.h, shared with the ternary matmul.
+#include "int8_gemm_kernel.h"
+
+namespace tpq {
+namespace {
+
+// Any strides, any K, signed or unsigned left operand: 16x16 outputs per
+// workgroup, operands staged through LDS 16 k at a time.
+template <typename LhsT, class Epilogue>
+__global__ __launch_bounds__(256) void int_mm_generic_kernel(const LhsT* __restrict__ a,
+                                                             const int8_t* __restrict__ b,
+                                                             int64_t sbk, int64_t sbn, int64_t M,
+                                                             int64_t K, int64_t N, Epilogue ep) {
+    __shared__ int sa[16][17], sb[16][17];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int64_t m = blockIdx.y * 16ll + ty, n = blockIdx.x * 16ll + tx;
+    int acc = 0;
+    for (int64_t k0 = 0; k0 < K; k0 += 16) {
+        const int64_t ka = k0 + tx, kb = k0 + ty;
+        sa[ty][tx] = (m < M && ka < K) ? static_cast<int>(a[m * K + ka]) : 0;
+        sb[ty][tx] = (n < N && kb < K) ? static_cast<int>(b[kb * sbk + n * sbn]) : 0;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; ++k) acc += sa[ty][k] * sb[k][tx];
+        __syncthreads();
+    }
+    if (m < M && n < N) ep.store(m * N + n, static_cast<int>(m), static_cast<int>(n), acc);
+}
+
+__global__ __launch_bounds__(256) void fill_zero_i32(int32_t* p, int64_t n) {
+    for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll) p[i] = 0;
+}
+
+template <class Epilogue>
+int launch_generic(const void* a, int a_unsigned, const int8_t* b, int64_t sbk, int64_t sbn,
+                   int64_t M, int64_t K, int64_t N, Epilogue ep, hipStream_t s) {
+    const int64_t gx = (N + 15) / 16, gy = (M + 15) / 16;
+    TPQ_REQUIRE(gx <= 0x7FFFFFFF && gy <= 65535, TPQ_ERR_INVALID_VALUE, "_int_mm: shape too large for the generic path");
+    const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
+    if (a_unsigned)
+        int_mm_generic_kernel<uint8_t, Epilogue><<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(a), b, sbk, sbn, M, K, N, ep);
+    else
+        int_mm_generic_kernel<int8_t, Epilogue><<<grid, 256, 0, s>>>(static_cast<const int8_t*>(a), b, sbk, sbn, M, K, N, ep);
+    return check_launch("_int_mm generic");
+}
+
+}  // namespace
+}  // namespace tpq
+
+using namespace tpq;
+
+TPQ_EXPORT int tpq_int_mm(const void* a, int a_unsigned, const int8_t* b, int64_t b_stride_k,
+                          int64_t b_stride_n, int32_t* c, int64_t M, int64_t K, int64_t N,
+                          void* stream) {
+    TPQ_REQUIRE(M >= 0 && N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "_int_mm: negative shape");
+    if (M == 0 || N == 0) return TPQ_OK;
+    TPQ_REQUIRE(c, TPQ_ERR_INVALID_VALUE, "_int_mm: null destination");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (K == 0) {  // empty reduction: zeros (p10/src/backend/cuda/IntMM.cu:388-394)
+        const int64_t total = M * N;
+        const int64_t blocks = (total + 255) / 256;
+        fill_zero_i32<<<static_cast<unsigned>(blocks > 8192 ? 8192 : blocks), 256, 0, s>>>(c, total);
+        return check_launch("_int_mm zero fill");
+    }
+    TPQ_REQUIRE(a && b, TPQ_ERR_INVALID_VALUE, "_int_mm: null operand");
+    const EpilogueInt32 ep{c};
+    if (!a_unsigned && b_stride_k == 1 && b_stride_n == K && mfma_path_ok(a, b, M, N, K))
+        return launch_mfma(static_cast<const int8_t*>(a), b, M, N, K, ep, s);
+    return launch_generic(a, a_unsigned, b, b_stride_k, b_stride_n, M, K, N, ep, s);
+}
+
+TPQ_EXPORT int tpq_int8_mm_dequant(const int8_t* a, const int8_t* w, const float* row_scale,
+                                   const float* col_scale, const float* bias, void* out,
+                                   int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+    TPQ_REQUIRE(M >= 0 && N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "int8_mm_dequant: negative shape");
+    TPQ_REQUIRE(out_dtype == TPQ_DTYPE_F32 || out_dtype == TPQ_DTYPE_F16 || out_dtype == TPQ_DTYPE_BF16,
+                TPQ_ERR_INVALID_TYPE, "int8_mm_dequant: unsupported output dtype");
+    if (M == 0 || N == 0) return TPQ_OK;
+    TPQ_REQUIRE(out && row_scale && col_scale && (K == 0 || (a && w)), TPQ_ERR_INVALID_VALUE,
+                "int8_mm_dequant: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool fast = K > 0 && mfma_path_ok(a, w, M, N, K);
+#define TPQ_DISPATCH(DT)                                                                            \
+    {                                                                                               \
+        const EpilogueDequant<DT> ep{static_cast<typename Elem<DT>::storage*>(out), row_scale,      \
+                                     col_scale, bias};                                              \
+        if (fast) return launch_mfma(a, w, M, N, K, ep, s);                                         \
+        return launch_generic(a, 0, w, 1, K, M, K, N, ep, s);                                       \
+    }
+    switch (out_dtype) {
+        case TPQ_DTYPE_F32: TPQ_DISPATCH(TPQ_DTYPE_F32)
+        case TPQ_DTYPE_F16: TPQ_DISPATCH(TPQ_DTYPE_F16)
+        default: TPQ_DISPATCH(TPQ_DTYPE_BF16)
+    }
+#undef TPQ_DISPATCH
+}

@@ -1,0 +1,167 @@
+// Fused row-wise signed quantizer for gfx950.
+//
+// One 256-thread workgroup per row.  The row is read from HBM once, kept in
+// registers (8 elements per 16/32-byte vector load, up to 8 such chunks per
+// lane), reduced to its absolute maximum with a 64-lane butterfly and one LDS
+// exchange between the four wavefronts, and written back as int8 codes with
+// 8-byte stores.  Rows longer than the register budget (K > 16384) or rows
+// that cannot be vector-loaded (K % 8 != 0) take the streaming kernel, which
+// reads the row a second time (the second read comes from L2).
+//
+// Arithmetic (bit-exact with the reference's CPU kernel,
+// p10/include/QuantNativeImpl.h:1162-1187 and
+// p10/src/backend/cpu/LowBitGemmKernels.cpp:19-52):
+//   absmax = max |float(x)|;  scale = fmaxf(absmax, eps) / divisor  (IEEE divide)
+//   code   = clamp(rintf(float(x) / scale), qmin, qmax)              (IEEE divide, RNE)
+#include "tpq_common.h"
+
+namespace tpq {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kVec = 8;  // elements per lane per chunk
+
+struct QParams {
+    float eps, divisor;
+    int qmin, qmax, sign_mode;
+};
+
+__device__ __forceinline__ int quantize_one(float v, float scale, const QParams& p) {
+    if (p.sign_mode) return v >= 0.0f ? p.qmax : p.qmin;
+    // __fdiv_rn: correctly rounded division regardless of compiler flags
+    float q = rintf(__fdiv_rn(v, scale));
+    q = fminf(fmaxf(q, static_cast<float>(p.qmin)), static_cast<float>(p.qmax));
+    return static_cast<int>(q);
+}
+
+// Block-wide max over 256 threads; every thread gets the result.
+__device__ __forceinline__ float block_max(float v, float* smem) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float r = smem[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / kWave; ++w) r = fmaxf(r, smem[w]);
+    return r;
+}
+
+template <int DT>
+__device__ __forceinline__ void load_chunk(const typename Elem<DT>::storage* p, float (&v)[kVec]) {
+    if constexpr (DT == TPQ_DTYPE_F32) {
+        const float4 a = reinterpret_cast<const float4*>(p)[0];
+        const float4 b = reinterpret_cast<const float4*>(p)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = Elem<DT>::load(static_cast<uint16_t>(w[i] & 0xFFFFu));
+            v[2 * i + 1] = Elem<DT>::load(static_cast<uint16_t>(w[i] >> 16));
+        }
+    }
+}
+
+// Row cached in registers: CHUNKS * 256 * 8 >= K, K % 8 == 0.
+template <int DT, int CHUNKS>
+__global__ __launch_bounds__(kThreads) void quantize_rows_cached(
+    const typename Elem<DT>::storage* __restrict__ x, int8_t* __restrict__ codes,
+    float* __restrict__ scales, int K, QParams p) {
+    __shared__ float smem[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const auto* xr = x + row * K;
+    int8_t* cr = codes + row * K;
+
+    float v[CHUNKS][kVec];
+    float absmax = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k0 = (c * kThreads + threadIdx.x) * kVec;
+        if (k0 < K) {
+            load_chunk<DT>(xr + k0, v[c]);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
+        }
+    }
+    absmax = block_max(absmax, smem);
+    const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
+    if (threadIdx.x == 0) scales[row] = scale;
+
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k0 = (c * kThreads + threadIdx.x) * kVec;
+        if (k0 < K) {
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                lo |= (static_cast<uint32_t>(quantize_one(v[c][i], scale, p)) & 0xFFu) << (8 * i);
+                hi |= (static_cast<uint32_t>(quantize_one(v[c][i + 4], scale, p)) & 0xFFu) << (8 * i);
+            }
+            *reinterpret_cast<uint2*>(cr + k0) = make_uint2(lo, hi);
+        }
+    }
+}
+
+// Any K: two passes over the row with scalar accesses.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quantize_rows_streaming(
+    const typename Elem<DT>::storage* __restrict__ x, int8_t* __restrict__ codes,
+    float* __restrict__ scales, int64_t K, QParams p) {
+    __shared__ float smem[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const auto* xr = x + row * K;
+    int8_t* cr = codes + row * K;
+    float absmax = 0.0f;
+    for (int64_t k = threadIdx.x; k < K; k += kThreads) absmax = fmaxf(absmax, fabsf(Elem<DT>::load(xr[k])));
+    absmax = block_max(absmax, smem);
+    const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
+    if (threadIdx.x == 0) scales[row] = scale;
+    for (int64_t k = threadIdx.x; k < K; k += kThreads)
+        cr[k] = static_cast<int8_t>(quantize_one(Elem<DT>::load(xr[k]), scale, p));
+}
+
+template <int DT>
+int launch(const void* x, int64_t M, int64_t K, const QParams& p, int8_t* codes, float* scales,
+           hipStream_t stream) {
+    using S = typename Elem<DT>::storage;
+    const S* xp = static_cast<const S*>(x);
+    const dim3 grid(static_cast<unsigned>(M)), block(kThreads);
+    const bool vec_ok = (K % kVec == 0) && aligned(x, 16) && aligned(codes, 8) && K <= 8 * kThreads * kVec;
+    if (vec_ok) {
+        const int chunks = static_cast<int>((K + kThreads * kVec - 1) / (kThreads * kVec));
+        const int k = static_cast<int>(K);
+        if (chunks <= 1) quantize_rows_cached<DT, 1><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
+        else if (chunks <= 2) quantize_rows_cached<DT, 2><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
+        else if (chunks <= 4) quantize_rows_cached<DT, 4><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
+        else quantize_rows_cached<DT, 8><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
+    } else {
+        quantize_rows_streaming<DT><<<grid, block, 0, stream>>>(xp, codes, scales, K, p);
+    }
+    return check_launch("tpq_quantize_rowwise");
+}
+
+}  // namespace
+}  // namespace tpq
+
+TPQ_EXPORT int tpq_quantize_rowwise(const void* x, int x_dtype, int64_t M, int64_t K, float eps,
+                                    float divisor, int qmin, int qmax, int sign_mode,
+                                    int8_t* codes, float* scales, void* stream) {
+    using namespace tpq;
+    TPQ_REQUIRE(M >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "quantize_rowwise: negative shape");
+    TPQ_REQUIRE(x_dtype == TPQ_DTYPE_F32 || x_dtype == TPQ_DTYPE_F16 || x_dtype == TPQ_DTYPE_BF16,
+                TPQ_ERR_INVALID_TYPE, "rowwise quantize: unsupported input dtype");
+    TPQ_REQUIRE(qmin >= -128 && qmax <= 127 && qmin <= qmax && divisor > 0.0f, TPQ_ERR_INVALID_VALUE,
+                "quantize_rowwise: code range must fit int8 and divisor must be positive");
+    if (M == 0 || K == 0) return TPQ_OK;
+    TPQ_REQUIRE(x && codes && scales, TPQ_ERR_INVALID_VALUE, "quantize_rowwise: null pointer");
+    TPQ_REQUIRE(M <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "quantize_rowwise: more than 2^31-1 rows");
+    const QParams p{eps, divisor, qmin, qmax, sign_mode ? 1 : 0};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (x_dtype) {
+        case TPQ_DTYPE_F32: return launch<TPQ_DTYPE_F32>(x, M, K, p, codes, scales, s);
+        case TPQ_DTYPE_F16: return launch<TPQ_DTYPE_F16>(x, M, K, p, codes, scales, s);
+        default: return launch<TPQ_DTYPE_BF16>(x, M, K, p, codes, scales, s);
+    }
+}

@@ -1,0 +1,98 @@
+// Internal helpers shared by the gfx950 kernels: error reporting, dtype
+// conversion on the device, wavefront (64-lane) reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/tpq.h"
+
+#define TPQ_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace tpq {
+
+constexpr int kWave = 64;
+
+char* error_buffer();
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+inline int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TPQ_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+    return TPQ_OK;
+}
+
+#define TPQ_REQUIRE(cond, code, ...)                    \
+    do {                                                \
+        if (!(cond)) return ::tpq::fail(code, __VA_ARGS__); \
+    } while (0)
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- 16-bit float conversions (bit patterns) ------------------------------
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(b) << 16);
+}
+
+// Round to nearest even; NaN becomes the quiet pattern 0x7FC0.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu) != 0) return 0x7FC0u;
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));  // v_cvt_f16_f32: RNE
+}
+
+template <int DT>
+struct Elem;
+template <>
+struct Elem<TPQ_DTYPE_F32> {
+    using storage = float;
+    static __device__ __forceinline__ float load(float v) { return v; }
+    static __device__ __forceinline__ float store(float v) { return v; }
+};
+template <>
+struct Elem<TPQ_DTYPE_F16> {
+    using storage = uint16_t;
+    static __device__ __forceinline__ float load(uint16_t v) { return f16_bits_to_f32(v); }
+    static __device__ __forceinline__ uint16_t store(float v) { return f32_to_f16_bits(v); }
+};
+template <>
+struct Elem<TPQ_DTYPE_BF16> {
+    using storage = uint16_t;
+    static __device__ __forceinline__ float load(uint16_t v) { return bf16_bits_to_f32(v); }
+    static __device__ __forceinline__ uint16_t store(float v) { return f32_to_bf16_bits(v); }
+};
+
+// ---- 64-lane reductions -----------------------------------------------------
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+}  // namespace tpq

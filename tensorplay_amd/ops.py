@@ -1,0 +1,288 @@
+"""The quantized-linear native operators, under the names and argument orders the
+reference's Python calls them with (``tp._C.<op>`` / ``tp.ops.tp.<op>``), over
+PyTorch-ROCm tensors.  Every function validates like the reference's device op,
+allocates the result like it, and enqueues the gfx950 kernel on the current
+stream through the C ABI of ``include/tpq.h``; none of them synchronises.
+
+Signatures: ``config/native_functions.yaml:5338-5350, 7987-7993`` of the reference.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+_ERRORS = {
+    _lib.TPQ_ERR_INVALID_VALUE: ValueError,
+    _lib.TPQ_ERR_INVALID_TYPE: TypeError,
+    _lib.TPQ_ERR_RUNTIME: RuntimeError,
+    _lib.TPQ_ERR_UNSUPPORTED: NotImplementedError,
+}
+
+
+def _check(status: int) -> None:
+    if status != _lib.TPQ_OK:
+        raise _ERRORS.get(status, RuntimeError)(_lib.last_error())
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def _require_device(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: expected a tensor on the GPU; this build has no CPU kernels")
+
+
+def _quantize_rowwise(self, eps, divisor, qmin, qmax, sign_mode, name):
+    if self.dim() != 2:
+        raise ValueError(f"{name}(): expected a 2-D tensor")
+    if self.dtype not in _DT:
+        raise TypeError("rowwise quantize: unsupported input dtype")
+    _require_device(self, name)
+    x = self.contiguous()
+    M, K = x.shape
+    codes = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scales = torch.empty((M,), dtype=torch.float32, device=x.device)
+    if M == 0 or K == 0:
+        return codes, scales
+    with torch.cuda.device(x.device):
+        _check(_lib.load().tpq_quantize_rowwise(_ptr(x), _DT[x.dtype], M, K, float(eps), divisor, qmin,
+                                                qmax, int(sign_mode), _ptr(codes), _ptr(scales), _stream(x)))
+    return codes, scales
+
+
+def _quantize_int8_rowwise(self: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """codes int8 [M,K] in [-127,127], scales f32 [M] = max(absmax, eps) / 127."""
+    return _quantize_rowwise(self, eps, 127.0, -127, 127, False, "_quantize_int8_rowwise")
+
+
+def _quantize_int4_rowwise(self: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """codes int8 in [-8,7], scales = max(absmax, eps) / 7."""
+    return _quantize_rowwise(self, eps, 7.0, -8, 7, False, "_quantize_int4_rowwise")
+
+
+def _quantize_int2_rowwise(self: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """codes int8 in {-2,-1,0,1}, scales = max(absmax, eps) / 2."""
+    return _quantize_rowwise(self, eps, 2.0, -2, 1, False, "_quantize_int2_rowwise")
+
+
+def _quantize_binary_rowwise(self: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """codes int8 in {-1,+1} (x >= 0 -> +1), scales = max(absmax, eps)."""
+    return _quantize_rowwise(self, eps, 1.0, -1, 1, True, "_quantize_binary_rowwise")
+
+
+def _check_int_mm_operands(self, mat2):
+    if self.dim() != 2 or mat2.dim() != 2:
+        raise RuntimeError(f"_int_mm: expected two matrices but got {self.dim()}-D and {mat2.dim()}-D tensors")
+    if self.size(1) != mat2.size(0):
+        raise RuntimeError(f"_int_mm: cannot multiply a {self.size(0)} by {self.size(1)} matrix with a "
+                           f"{mat2.size(0)} by {mat2.size(1)} matrix")
+    if self.dtype not in (torch.int8, torch.uint8):
+        raise RuntimeError("_int_mm: expected the left operand to be int8 or uint8")
+    if mat2.dtype != torch.int8:
+        raise RuntimeError("_int_mm: expected the right operand to be int8")
+
+
+def _int_mm(self: torch.Tensor, mat2: torch.Tensor, *, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C[M,N] int32 = self[M,K] (int8/uint8) @ mat2[K,N] (int8).
+
+    The transposed view of a contiguous [N,K] weight (strides (1,K)) is consumed in place;
+    any other layout of mat2 is made contiguous first.
+    """
+    _check_int_mm_operands(self, mat2)
+    _require_device(self, "_int_mm")
+    M, K = self.shape
+    N = mat2.size(1)
+    if out is not None:
+        if out.dtype != torch.int32:
+            raise RuntimeError("_int_mm: expected an int32 destination")
+        if tuple(out.shape) != (M, N):
+            out.resize_((M, N))
+    dst = out if (out is not None and out.is_contiguous()) else torch.empty((M, N), dtype=torch.int32, device=self.device)
+    if M and N:
+        a = self.contiguous()
+        if K and mat2.stride(0) == 1 and mat2.stride(1) == K:
+            b, sbk, sbn = mat2, 1, K
+        else:
+            b = mat2.contiguous()
+            sbk, sbn = N, 1
+        with torch.cuda.device(self.device):
+            _check(_lib.load().tpq_int_mm(_ptr(a), int(a.dtype == torch.uint8), _ptr(b), sbk, sbn, _ptr(dst),
+                                          M, K, N, _stream(self)))
+    if out is not None and dst is not out:
+        out.copy_(dst)
+    return out if out is not None else dst
+
+
+def _int8_mm_rescale(out: torch.Tensor, row_scale: torch.Tensor, col_scale: torch.Tensor) -> torch.Tensor:
+    """float32 result[m,n] = (float(out[m,n]) * row_scale[m]) * col_scale[n]."""
+    if out.dim() != 2 or out.dtype != torch.int32:
+        raise ValueError("_int8_mm_rescale(): expected a 2-D int32 output")
+    _require_device(out, "_int8_mm_rescale")
+    M, N = out.shape
+    result = torch.empty((M, N), dtype=torch.float32, device=out.device)
+    if M == 0 or N == 0:
+        return result
+    acc = out.contiguous()
+    rs = row_scale.contiguous().to(torch.float32)
+    cs = col_scale.contiguous().to(torch.float32)
+    if rs.numel() != M or cs.numel() != N:
+        raise ValueError("_int8_mm_rescale(): scale sizes do not match the output")
+    with torch.cuda.device(out.device):
+        _check(_lib.load().tpq_int8_mm_rescale(_ptr(acc), _ptr(rs), _ptr(cs), _ptr(result), M, N, _stream(out)))
+    return result
+
+
+def int8_mm_dequant(A_i8: torch.Tensor, B_t_i8: torch.Tensor, row_scale: torch.Tensor, col_scale: torch.Tensor,
+                    bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``_int_mm`` + ``_int8_mm_rescale`` (+ bias) in one launch.
+
+    ``A_i8`` [M,K] int8, ``B_t_i8`` [N,K] int8, both contiguous; the result is
+    ``cast((float(acc) * row_scale[m]) * col_scale[n] (+ bias[n]))``: the fp32 value the two
+    reference ops produce, rounded once when ``out_dtype`` is a 16-bit float.
+    """
+    if A_i8.dim() != 2 or B_t_i8.dim() != 2 or A_i8.size(1) != B_t_i8.size(1):
+        raise ValueError("int8_mm_dequant: expected A [M,K] and B_t [N,K]")
+    if A_i8.dtype != torch.int8 or B_t_i8.dtype != torch.int8:
+        raise TypeError("int8_mm_dequant: operands must be int8")
+    if out_dtype not in _DT:
+        raise TypeError("int8_mm_dequant: unsupported output dtype")
+    _require_device(A_i8, "int8_mm_dequant")
+    M, K = A_i8.shape
+    N = B_t_i8.size(0)
+    out = torch.empty((M, N), dtype=out_dtype, device=A_i8.device)
+    if M == 0 or N == 0:
+        return out
+    a, w = A_i8.contiguous(), B_t_i8.contiguous()
+    rs = row_scale.contiguous().to(torch.float32)
+    cs = col_scale.contiguous().to(torch.float32)
+    if rs.numel() != M or cs.numel() != N:
+        raise ValueError("int8_mm_dequant: scale sizes do not match the output")
+    b = None if bias is None else bias.contiguous().to(torch.float32)
+    if b is not None and b.numel() != N:
+        raise ValueError("int8_mm_dequant: bias must have one value per output channel")
+    with torch.cuda.device(a.device):
+        _check(_lib.load().tpq_int8_mm_dequant(_ptr(a), _ptr(w), _ptr(rs), _ptr(cs), _ptr(b), _ptr(out),
+                                               _DT[out_dtype], M, N, K, _stream(a)))
+    return out
+
+
+def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.Tensor:
+    """int32 codes [N,K] (0..15) -> int32 [ceil(N/8), ceil(K/(16*innerKTiles)), 32, innerKTiles/2]."""
+    if self.dim() != 2:
+        raise ValueError("_convert_weight_to_int4pack(): expected 2-D codes [N,K]")
+    if innerKTiles not in (2, 4, 8):
+        raise ValueError("_convert_weight_to_int4pack(): innerKTiles must be 2, 4 or 8")
+    N, K = self.shape
+    if K % 2 != 0:
+        raise ValueError("_convert_weight_to_int4pack(): K must be even")
+    _require_device(self, "_convert_weight_to_int4pack")
+    n_tiles = (N + 7) // 8
+    k_super = (K + innerKTiles * 16 - 1) // (innerKTiles * 16)
+    out = torch.empty((n_tiles, k_super, 32, innerKTiles // 2), dtype=torch.int32, device=self.device)
+    if N == 0 or K == 0:
+        return out
+    codes = self.to(torch.int32).contiguous()
+    with torch.cuda.device(self.device):
+        _check(_lib.load().tpq_int4_pack(_ptr(codes), N, K, innerKTiles, _ptr(out), _stream(self)))
+    return out
+
+
+def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
+                        qScaleAndZeros: torch.Tensor) -> torch.Tensor:
+    """``self @ W.T`` with W dequantised per group: (code - 8) * scale + zero; result in self.dtype."""
+    if mat2.dtype != torch.int32 or mat2.dim() != 4:
+        raise TypeError("_weight_int4pack_mm(): packed weight must be 4-D int32 in the tensor-core B layout")
+    if self.dim() != 2:
+        raise ValueError("_weight_int4pack_mm(): expected 2-D activations [m,k]")
+    if not self.is_floating_point():
+        raise TypeError("_weight_int4pack_mm(): activations must be floating point")
+    if qGroupSize not in (32, 64, 128):
+        raise ValueError("_weight_int4pack_mm(): qGroupSize must be 32, 64 or 128")
+    m, k = self.shape
+    n_tiles, k_super, inner = mat2.size(0), mat2.size(1), mat2.size(3) * 2
+    n = n_tiles * 8
+    if mat2.size(2) != 32 or inner not in (2, 4, 8):
+        raise ValueError("_weight_int4pack_mm(): packed weight layout is invalid")
+    if k_super != (k + inner * 16 - 1) // (inner * 16):
+        raise ValueError("_weight_int4pack_mm(): K dimension does not match packed B")
+    groups = (k + qGroupSize - 1) // qGroupSize
+    if qScaleAndZeros.dim() != 3 or tuple(qScaleAndZeros.shape) != (groups, n, 2):
+        raise ValueError("_weight_int4pack_mm(): qScaleAndZeros must be [K/group, N, 2]")
+    if self.dtype not in _DT:
+        raise TypeError("_weight_int4pack_mm(): unsupported activation dtype")
+    _require_device(self, "_weight_int4pack_mm")
+    out = torch.empty((m, n), dtype=self.dtype, device=self.device)
+    if m == 0 or n == 0 or k == 0:
+        return out
+    x = self.contiguous()
+    w = mat2.contiguous()
+    sz = qScaleAndZeros.to(self.dtype).contiguous()
+    with torch.cuda.device(self.device):
+        _check(_lib.load().tpq_int4_mm(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz),
+                                       _ptr(out), _stream(self)))
+    return out
+
+
+def pack_ternary(codes: torch.Tensor) -> torch.Tensor:
+    """int8 codes {-1,0,1} -> uint8, four per byte along the last dim (first code in bits 7..6)."""
+    _require_device(codes, "pack_ternary")
+    x = codes.to(torch.int8).contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    out = torch.empty((*x.shape[:-1], (cols + 3) // 4), dtype=torch.uint8, device=x.device)
+    if rows and cols:
+        with torch.cuda.device(x.device):
+            _check(_lib.load().tpq_ternary_pack(_ptr(x), rows, cols, _ptr(out), _stream(x)))
+    return out
+
+
+def unpack_ternary(packed: torch.Tensor, columns: int) -> torch.Tensor:
+    """uint8 packed -> int8 codes, sign-extending every 2-bit field; keeps the first `columns`."""
+    _require_device(packed, "unpack_ternary")
+    p = packed.contiguous()
+    bytes_per_row = p.shape[-1]
+    cols = min(int(columns), bytes_per_row * 4)
+    rows = p.numel() // bytes_per_row if bytes_per_row else 0
+    out = torch.empty((*p.shape[:-1], cols), dtype=torch.int8, device=p.device)
+    if rows and cols:
+        if (cols + 3) // 4 != bytes_per_row:
+            p = p[..., : (cols + 3) // 4].contiguous()
+        with torch.cuda.device(p.device):
+            _check(_lib.load().tpq_ternary_unpack(_ptr(p), rows, cols, _ptr(out), _stream(p)))
+    return out
+
+
+def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor, w_scale: float,
+               in_features: int, bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32,
+               return_acc: bool = False):
+    """``(float(x_i8 @ codes.T) * row_scale) * w_scale (+ bias)`` straight from the packed weight."""
+    if x_i8.dim() != 2 or x_i8.dtype != torch.int8 or x_i8.size(1) != in_features:
+        raise ValueError("ternary_mm: expected int8 activations [M, in_features]")
+    if packed.dim() != 2 or packed.dtype != torch.uint8 or packed.size(1) != (in_features + 3) // 4:
+        raise ValueError("ternary_mm: packed weight must be uint8 [N, ceil(in_features/4)]")
+    if out_dtype not in _DT:
+        raise TypeError("ternary_mm: unsupported output dtype")
+    _require_device(x_i8, "ternary_mm")
+    M, K = x_i8.shape
+    N = packed.size(0)
+    out = torch.empty((M, N), dtype=out_dtype, device=x_i8.device)
+    acc = torch.empty((M, N), dtype=torch.int32, device=x_i8.device) if return_acc else None
+    if M and N:
+        x, p = x_i8.contiguous(), packed.contiguous()
+        rs = row_scale.contiguous().to(torch.float32)
+        if rs.numel() != M:
+            raise ValueError("ternary_mm: one row scale per activation row expected")
+        b = None if bias is None else bias.contiguous().to(torch.float32)
+        with torch.cuda.device(x.device):
+            _check(_lib.load().tpq_ternary_mm(_ptr(x), _ptr(rs), _ptr(p), float(w_scale), _ptr(b), M, N, K,
+                                              _ptr(out), _DT[out_dtype], _ptr(acc), _stream(x)))
+    return (out, acc) if return_acc else out

@@ -1,0 +1,51 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/tpq.h declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "tpq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tpq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared()
+    for must in ("tpq_quantize_rowwise", "tpq_int_mm", "tpq_int8_mm_rescale", "tpq_int8_mm_dequant", "tpq_int4_pack",
+                 "tpq_int4_mm", "tpq_ternary_pack", "tpq_ternary_unpack", "tpq_ternary_mm", "tpq_last_error"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from tensorplay_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} not built: run `python -m tensorplay_amd.build`")
+    lib = _lib.load()
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} declared in include/tpq.h but not exported"
+    assert set(_lib.SIGNATURES) | {"tpq_last_error"} == set(_declared())
+    assert lib.tpq_abi_version() == 1
+    assert isinstance(_lib.last_error(), str)
+
+
+def test_argument_validation_needs_no_gpu():
+    """Shape/type checks run on the host before any launch."""
+    from tensorplay_amd import _lib
+
+    lib = _lib.load()
+    assert lib.tpq_int4_pack(None, 8, 33, 2, None, None) == _lib.TPQ_ERR_INVALID_VALUE
+    assert "K must be even" in _lib.last_error()
+    assert lib.tpq_int4_pack(None, 8, 32, 3, None, None) == _lib.TPQ_ERR_INVALID_VALUE
+    assert lib.tpq_quantize_rowwise(None, 7, 1, 1, 1e-5, 127.0, -127, 127, 0, None, None, None) == _lib.TPQ_ERR_INVALID_TYPE
+    assert lib.tpq_int4_mm(None, 1, 1, 64, None, 2, 8, 48, None, None, None) == _lib.TPQ_ERR_INVALID_VALUE
+    assert lib.tpq_int4_mm(None, 1, 1, 64, None, 4, 8, 32, None, None, None) == _lib.TPQ_ERR_UNSUPPORTED
+    # zero-sized problems succeed without touching the device
+    assert lib.tpq_quantize_rowwise(None, 0, 0, 16, 1e-5, 127.0, -127, 127, 0, None, None, None) == _lib.TPQ_OK
+    assert lib.tpq_int_mm(None, 0, None, 1, 1, None, 0, 4, 4, None) == _lib.TPQ_OK
+    assert lib.tpq_ternary_mm(None, None, None, 1.0, None, 0, 4, 4, None, 0, None, None) == _lib.TPQ_OK

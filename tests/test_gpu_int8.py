@@ -1,0 +1,140 @@
+"""GPU parity: _int_mm (exact int32), _int8_mm_rescale and the fused dequant GEMM."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import DEV, cast_bits, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tensorplay_amd import ops as _ops
+
+    return _ops
+
+
+def _rand_i8(rng, shape, lo=-128, hi=128):
+    return rng.integers(lo, hi, size=shape).astype(np.int8)
+
+
+# (M, K, N): generic path (odd sizes), small-M path, matrix-core path with ragged edges
+SHAPES = [(5, 7, 3), (1, 1, 1), (64, 12, 32), (16, 1024, 1024), (64, 128, 32), (33, 257, 65),
+          (129, 64, 65), (256, 4096, 128), (300, 208, 200), (128, 2560, 6912 // 8), (513, 80, 257)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("layout", ["weight_view", "contiguous"])
+def test_int_mm_exact(ops, shape, layout):
+    M, K, N = shape
+    rng = np.random.default_rng(M * 31 + K * 7 + N)
+    a = _rand_i8(rng, (M, K))
+    w = _rand_i8(rng, (N, K))
+    want = a.astype(np.int32) @ w.astype(np.int32).T
+    np.testing.assert_array_equal(oracle.int_mm(a, w.T), want)
+    wd = dev(w)
+    b = wd.t() if layout == "weight_view" else wd.t().contiguous()
+    got = ops._int_mm(dev(a), b)
+    assert got.dtype == torch.int32 and got.shape == (M, N)
+    np.testing.assert_array_equal(host(got), want)
+
+
+def test_int_mm_unsigned_lhs_out_and_empty(ops):
+    rng = np.random.default_rng(1)
+    a = rng.integers(0, 256, size=(40, 100)).astype(np.uint8)
+    b = _rand_i8(rng, (100, 24))
+    want = a.astype(np.int32) @ b.astype(np.int32)
+    np.testing.assert_array_equal(host(ops._int_mm(dev(a), dev(b))), want)
+    out = torch.zeros(40, 24, dtype=torch.int32, device=DEV)
+    assert ops._int_mm(dev(a), dev(b), out=out) is out
+    np.testing.assert_array_equal(host(out), want)
+    z = ops._int_mm(torch.empty(3, 0, dtype=torch.int8, device=DEV), torch.empty(0, 4, dtype=torch.int8, device=DEV))
+    assert z.shape == (3, 4) and not z.any()
+    assert ops._int_mm(torch.empty(0, 5, dtype=torch.int8, device=DEV), torch.empty(5, 4, dtype=torch.int8, device=DEV)).shape == (0, 4)
+    with pytest.raises(Exception):
+        ops._int_mm(torch.zeros(2, 2, device=DEV), torch.zeros(2, 2, dtype=torch.int8, device=DEV))
+    with pytest.raises(Exception):
+        ops._int_mm(torch.zeros(2, 3, dtype=torch.int8, device=DEV), torch.zeros(2, 2, dtype=torch.int8, device=DEV))
+
+
+def test_int_mm_extreme_values(ops):
+    K = 6912
+    a = np.full((130, K), -128, np.int8)
+    w = np.full((70, K), -128, np.int8)
+    got = host(ops._int_mm(dev(a), dev(w).t()))
+    assert (got == 128 * 128 * K).all()
+
+
+def test_rescale_bit_exact(ops):
+    rng = np.random.default_rng(9)
+    for M, N in [(37, 53), (16, 1024), (5, 7), (64, 4096)]:
+        acc = rng.integers(-2**22, 2**22, size=(M, N)).astype(np.int32)
+        rs = rng.uniform(1e-3, 1e-1, M).astype(np.float32)
+        cs = rng.uniform(1e-4, 1e-2, N).astype(np.float32)
+        got = ops._int8_mm_rescale(dev(acc), dev(rs).unsqueeze(-1), dev(cs).unsqueeze(-1))
+        assert got.dtype == torch.float32
+        np.testing.assert_array_equal(host(got), oracle.int8_mm_rescale(acc, rs, cs))
+    with pytest.raises(ValueError):
+        ops._int8_mm_rescale(torch.zeros(2, 2, device=DEV), torch.ones(2, device=DEV), torch.ones(2, device=DEV))
+
+
+@pytest.mark.parametrize("out_dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape", [(16, 1024, 1024), (300, 208, 200), (5, 7, 3), (256, 512, 384)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_fused_dequant_bit_exact(ops, out_dtype, shape, with_bias):
+    from gpu_util import TORCH_DT
+
+    M, K, N = shape
+    rng = np.random.default_rng(M + K + N)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    w = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    bias = rng.normal(0, 0.01, N).astype(np.float32) if with_bias else None
+    xq, xs = oracle.quantize_int8_rowwise(x)
+    wq, ws = oracle.quantize_int8_rowwise(w)
+    acc = oracle.int_mm(xq, wq.T)
+    want = oracle.int8_mm_rescale(acc, xs, ws, bias=bias, out_dtype=out_dtype)
+    got = ops.int8_mm_dequant(dev(xq), dev(wq), dev(xs), dev(ws), None if bias is None else dev(bias), TORCH_DT[out_dtype])
+    np.testing.assert_array_equal(host(got), want)
+
+
+def test_dynamic_int8_linear_config1_end_to_end(ops):
+    """CPU-plumbing configuration: M=16, K=1024, N=1024 fp32 with bias, quantize -> mm -> rescale."""
+    rng = np.random.default_rng(2026)
+    x = rng.normal(0, 1, (16, 1024)).astype(np.float32)
+    w = rng.normal(0, 0.02, (1024, 1024)).astype(np.float32)
+    b = rng.normal(0, 0.01, 1024).astype(np.float32)
+    xq, xs = oracle.quantize_int8_rowwise(x)
+    wq, ws = oracle.quantize_int8_rowwise(w)
+    want = oracle.int8_mm_rescale(oracle.int_mm(xq, wq.T), xs, ws) + b
+    a_q, a_s = ops._quantize_int8_rowwise(dev(x), 1e-5)
+    w_q, w_s = ops._quantize_int8_rowwise(dev(w), 1e-5)
+    out = ops._int8_mm_rescale(ops._int_mm(a_q, w_q.t()), a_s, w_s) + dev(b)
+    np.testing.assert_array_equal(host(out), want)
+
+
+def test_prefill_config3_full_size(ops):
+    """M=2048, K=4096, N=4096 bf16 activations with outlier columns: int32 accumulators exact
+    against an fp64 product on the device (exact for |acc| < 2^53) and against the oracle on a
+    sample of rows; bf16 output equal to the oracle's rounding of the same accumulators."""
+    M, K, N = 2048, 4096, 4096
+    rng = np.random.default_rng(3)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    x[:, rng.choice(K, 41, replace=False)] *= 20.0
+    w = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    xb = cast_bits(x, "bf16")
+    wb = cast_bits(w, "bf16")   # the reference casts the weight to the activation dtype first
+    a_q, a_s = ops._quantize_int8_rowwise(dev(xb, "bf16"), 1e-5)
+    w_q, w_s = ops._quantize_int8_rowwise(dev(wb, "bf16"), 1e-5)
+    acc = ops._int_mm(a_q, w_q.t())
+    ref = (a_q.double() @ w_q.double().t())
+    assert torch.equal(acc.double(), ref)
+    rows = np.arange(0, M, 171)
+    aq_h, wq_h = host(a_q), host(w_q)
+    np.testing.assert_array_equal(host(acc)[rows], oracle.int_mm_nk(aq_h[rows], wq_h))
+    fused = ops.int8_mm_dequant(a_q, w_q, a_s, w_s, None, torch.bfloat16)
+    want = oracle.int8_mm_rescale(host(acc)[rows], host(a_s)[rows], host(w_s), out_dtype="bf16")
+    np.testing.assert_array_equal(host(fused)[rows], want)
+    two_step = ops._int8_mm_rescale(acc, a_s, w_s).to(torch.bfloat16)
+    assert torch.equal(fused, two_step)

@@ -1,0 +1,83 @@
+"""GPU parity: ternary pack/unpack (bit-exact) and the BitNet packed matmul (exact int32 sums,
+fp32 outputs equal to the oracle's evaluation of the reference formula)."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import DEV, TORCH_DT, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tensorplay_amd import ops as _ops
+
+    return _ops
+
+
+def _ternary(rng, shape):
+    return rng.choice(np.int8([-1, 0, 1]), size=shape, p=[0.325, 0.35, 0.325])
+
+
+@pytest.mark.parametrize("shape", [(2, 9), (1, 1), (7, 4), (6912, 2560), (33, 1023), (3, 5, 10)])
+def test_pack_unpack_bit_exact(ops, shape):
+    rng = np.random.default_rng(sum(shape))
+    codes = _ternary(rng, shape)
+    want = oracle.pack_ternary(codes)
+    got = ops.pack_ternary(dev(codes))
+    assert got.dtype == torch.uint8 and tuple(got.shape) == want.shape
+    np.testing.assert_array_equal(host(got), want)
+    back = ops.unpack_ternary(got, shape[-1])
+    np.testing.assert_array_equal(host(back), codes)
+
+
+def test_unpack_every_byte_value(ops):
+    every = np.arange(256, dtype=np.uint8).reshape(256, 1)
+    np.testing.assert_array_equal(host(ops.unpack_ternary(dev(every), 4)), oracle.unpack_ternary(every, 4))
+    table = np.int8(list(itertools.product([-1, 0, 1], repeat=4)))
+    np.testing.assert_array_equal(host(ops.pack_ternary(dev(table))), oracle.pack_ternary(table))
+
+
+# (M, K, N): decode kernel, matrix-core kernel, generic kernel
+CASES = [(1, 2560, 6912), (1, 6912, 2560), (4, 2560, 256), (8, 128, 67), (5, 64, 9), (128, 2560, 6912),
+         (128, 6912, 2560), (16, 256, 100), (33, 48, 70), (3, 9, 5), (2, 10, 4), (9, 2560, 130)]
+
+
+@pytest.mark.parametrize("M,K,N", CASES)
+def test_ternary_mm_exact(ops, M, K, N):
+    rng = np.random.default_rng(M + K + N)
+    codes = _ternary(rng, (N, K))
+    packed = oracle.pack_ternary(codes)
+    x = rng.normal(size=(M, K)).astype(np.float32)
+    xq, rs = oracle.quantize_int8_rowwise(x, "f32", 1e-5)
+    w_scale = float(np.float16(0.0173))   # an fp16-representable absmean scale, applied in fp32
+    bias = rng.normal(0, 0.01, N).astype(np.float32)
+    want, want_acc = oracle.ternary_mm(xq, rs, packed, w_scale, K, bias=bias)
+    got, acc = ops.ternary_mm(dev(xq), dev(rs), dev(packed), w_scale, K, bias=dev(bias), return_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    np.testing.assert_array_equal(want_acc, xq.astype(np.int32) @ codes.astype(np.int32).T)
+    np.testing.assert_array_equal(host(got), want)
+    for dt in ("f16", "bf16"):
+        w16, _ = oracle.ternary_mm(xq, rs, packed, w_scale, K, out_dtype=dt)
+        g16 = ops.ternary_mm(dev(xq), dev(rs), dev(packed), w_scale, K, out_dtype=TORCH_DT[dt])
+        np.testing.assert_array_equal(host(g16), w16)
+
+
+def test_ternary_mm_arbitrary_bytes_and_extremes(ops):
+    """Any byte is a legal packed value (0b10 decodes to -2); activations at the int8 extremes."""
+    rng = np.random.default_rng(8)
+    K, N = 6912, 64
+    packed = rng.integers(0, 256, size=(N, K // 4)).astype(np.uint8)
+    x = np.where(rng.random((3, K)) < 0.5, -127, 127).astype(np.int8)
+    rs = np.ones(3, np.float32)
+    want, want_acc = oracle.ternary_mm(x, rs, packed, 1.0, K)
+    got, acc = ops.ternary_mm(dev(x), dev(rs), dev(packed), 1.0, K, return_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    x128 = np.repeat(x, 43, axis=0)[:128]
+    _, want_acc = oracle.ternary_mm(x128, np.ones(128, np.float32), packed, 1.0, K)
+    _, acc = ops.ternary_mm(dev(x128), dev(np.ones(128, np.float32)), dev(packed), 1.0, K, return_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
