@@ -1,0 +1,329 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): int4 weight-only decode GEMV, M=1, K=4096,
+N=11008, group 128, fp16 activations / scales / zeros, weights in the reference's packed device
+layout.  One "step" = one call of the GEMV on weights that are NOT cache resident: the calls walk
+round-robin through enough distinct copies of the packed weight (> 512 MiB) that every call
+streams its 24 MB from HBM.  The K timed steps are recorded into one HIP graph and replayed once,
+so launch gaps do not dilute the kernel time; the region is bracketed by HIP events on the launch
+stream and by device synchronisation.
+
+Prints ONE JSON line (see the keys at the bottom).  `value` is GB/s of algorithmic bytes
+(packed nibbles + scales/zeros + activations + outputs = 23,983,616 B per call).  `extras` carries
+the other kernels of the path (int8 GEMM TOPS at 2048x4096x4096 with the fused dequant epilogue,
+activation quantizer, ternary matmul, batched int4).  `cpu_baseline` times the CPU oracle's port of
+the reference's CPU int4 kernel on the host cores, on the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "int4 GEMV GB/s (% HBM peak) at M=1; int8 GEMM TOPS (% MFMA peak) at M=2048"
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
+M, K, N, GROUP = 1, 4096, 11008, 128
+GEMV_BYTES = N * K // 2 + (K // GROUP) * N * 4 + 2 * M * K + 2 * M * N   # 23,983,616
+# HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled
+# by a copy kernel of known size); None until measured.  Summary: profiles/int4_decode_gemv_pmc.md
+MEASURED_TRAFFIC_BYTES = None
+
+
+def asym_quant_int4(w, group):
+    """Asymmetric uint4 group quantizer of the benchmark configuration: s = (max-min)/15,
+    q = clamp(round((w-min)/s), 0, 15), zero = min + 8 s, so (q-8)*s + zero = min + q*s."""
+    import numpy as np
+
+    n, k = w.shape
+    wg = w.reshape(n, k // group, group)
+    lo, hi = wg.min(-1), wg.max(-1)
+    s = np.maximum((hi - lo) / 15.0, 1e-8).astype(np.float32)
+    q = np.clip(np.rint((wg - lo[..., None]) / s[..., None]), 0, 15).astype(np.int32).reshape(n, k)
+    z = (lo + 8 * s).astype(np.float32)
+    return q, np.ascontiguousarray(np.stack([s.T, z.T], axis=-1))  # [K/g, N, 2]
+
+
+def time_region(fn, stream_sync, reps):
+    """Run fn() `reps` times between two HIP events on the current stream; returns ms per call."""
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream_sync()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    stream_sync()
+    return start.elapsed_time(stop) / reps
+
+
+def graph_of(fn):
+    """Record fn() (which only enqueues kernels on the current stream) into a HIP graph."""
+    import torch
+
+    g = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):  # switches the current stream to a capturing side stream
+        fn()
+    return g
+
+
+def cpu_baseline(x16, codes, sz16, want, budget_s=12.0):
+    """The CPU oracle's port of the reference's CPU int4 kernel (AVX-512 layout, 4-row x 64-column
+    tasks spread over threads), timed on the host on the full M=1 workload."""
+    import numpy as np
+
+    import oracle
+
+    threads = max(1, min(16, os.cpu_count() or 1))
+    packed = oracle.int4_pack_cpu(codes, 64, True)
+    out = np.zeros((M, N), np.uint16)
+    blocks = N // 64
+    per = (blocks + threads - 1) // threads
+    spans = [(b, min(b + per, blocks)) for b in range(0, blocks, per)]
+    pool = ThreadPoolExecutor(max_workers=threads)
+
+    def call():
+        list(pool.map(lambda sp: oracle.int4_mm_cpu_blocked(x16, "f16", packed, sz16, GROUP, sp, out), spans))
+
+    call()
+    err = float(np.abs(oracle.to_f32(out, "f16") - want).max() / np.abs(want).max())
+    t0 = time.perf_counter()
+    calls = 0
+    while True:
+        call()
+        calls += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or calls >= 2000:
+            break
+    pool.shutdown()
+    per_call = dt / calls
+    return {
+        "value": round(GEMV_BYTES / per_call / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{calls} calls of the full M=1 K=4096 N=11008 GEMV ({per_call * 1e6:.0f} us/call), "
+                  f"oracle port of the reference CPU int4 kernel; max rel diff vs GPU {err:.2e}",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="time the headline GEMV only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from tensorplay_amd import _lib, ops
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    sync = torch.cuda.synchronize
+
+    def cur():  # the stream to launch on: the capturing stream while a graph is being recorded
+        return torch.cuda.current_stream().cuda_stream
+
+    # ---- synthetic workload (seeded) -------------------------------------------------------
+    rng = np.random.default_rng(20260101)
+    w = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    codes, sz = asym_quant_int4(w, GROUP)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    x_d = torch.from_numpy(x).to(dev).half()
+    sz_d = torch.from_numpy(sz).to(dev).half().contiguous()
+    packed0 = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(dev), 2)
+    copies = 26  # 26 x (22.5 + 1.4) MB = 622 MB: far beyond L2 + the 256 MB last-level cache
+    packs = [packed0] + [packed0.clone() for _ in range(copies - 1)]
+    szs = [sz_d] + [sz_d.clone() for _ in range(copies - 1)]
+    y_d = torch.empty((M, N), dtype=torch.float16, device=dev)
+
+    def gemv(i):
+        rc = lib.tpq_int4_mm(x_d.data_ptr(), _lib.F16, M, K, packs[i % copies].data_ptr(), 2, N, GROUP,
+                             szs[i % copies].data_ptr(), y_d.data_ptr(), cur())
+        if rc:
+            raise RuntimeError(_lib.last_error())
+
+    # correctness of what is being timed (fp64 evaluation of the same quantized weights)
+    gemv(0)
+    sync()
+    sz16 = sz_d.cpu().view(torch.int16).numpy().view(np.uint16)
+    x16 = x_d.cpu().view(torch.int16).numpy().view(np.uint16)
+    sz32 = sz_d.float().cpu().numpy().astype(np.float64)
+    wq = (codes - 8) * np.repeat(sz32[:, :, 0].T, GROUP, axis=1) + np.repeat(sz32[:, :, 1].T, GROUP, axis=1)
+    want = x_d.float().cpu().numpy().astype(np.float64) @ wq.T
+    got = y_d.float().cpu().numpy()
+    gpu_err = float(np.abs(got - want).max() / np.abs(want).max())
+    if not gpu_err < 1e-3:
+        raise RuntimeError(f"int4 GEMV output is off by {gpu_err:.3e} (limit 1e-3)")
+
+    # ---- headline: W warmup steps, then exactly K timed steps ------------------------------------
+    steps, warmup = max(1, args.steps), max(0, args.warmup)
+    for i in range(warmup):
+        gemv(i)
+    sync()
+    g = graph_of(lambda: [gemv(i) for i in range(steps)])
+    g.replay()  # untimed: first replay uploads the graph
+    sync()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    sync()
+    t0 = time.perf_counter()
+    start.record()
+    g.replay()
+    stop.record()
+    sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = start.elapsed_time(stop) / steps
+    gbs = GEMV_BYTES / (ms_per_step * 1e-3) / 1e9
+
+    extras = {"gemv_max_rel_err_vs_fp64": gpu_err, "graph_wall_ms_per_step": wall_ms / steps}
+    if not args.no_extras:
+        # same kernel, launched eagerly through the C ABI (python + launch overhead included)
+        sync()
+        t = time.perf_counter()
+        for i in range(500):
+            gemv(i)
+        sync()
+        extras["int4_gemv_eager_us"] = (time.perf_counter() - t) / 500 * 1e6
+        # cache-resident variant: one copy, weights stay in the last-level cache
+        gc = graph_of(lambda: [gemv(0) for _ in range(500)])
+        gc.replay(); sync()
+        ms = time_region(gc.replay, sync, 1) / 500
+        extras["int4_gemv_cache_resident_us"] = ms * 1e3
+        extras["int4_gemv_cache_resident_GBs"] = GEMV_BYTES / (ms * 1e-3) / 1e9
+        # batched decode M = 4, 16 (rotating weights)
+        for mb in (4, 16):
+            xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
+            yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
+
+            def gemv_b(i, xb=xb, yb=yb, mb=mb):
+                lib.tpq_int4_mm(xb.data_ptr(), _lib.F16, mb, K, packs[i % copies].data_ptr(), 2, N, GROUP,
+                                szs[i % copies].data_ptr(), yb.data_ptr(), cur())
+
+            gb = graph_of(lambda: [gemv_b(i) for i in range(260)])
+            gb.replay(); sync()
+            ms = time_region(gb.replay, sync, 1) / 260
+            bytes_b = N * K // 2 + (K // GROUP) * N * 4 + 2 * mb * K + 2 * mb * N
+            extras[f"int4_gemv_M{mb}_us"] = ms * 1e3
+            extras[f"int4_gemv_M{mb}_GBs"] = bytes_b / (ms * 1e-3) / 1e9
+        del packs[1:], szs[1:]
+        torch.cuda.empty_cache()
+
+        # int8 prefill GEMM with fused dequant: M=2048, K=4096, N=4096, bf16 in/out
+        M8, K8, N8 = 2048, 4096, 4096
+        xa = rng.normal(0, 1, (M8, K8)).astype(np.float32)
+        xa[:, rng.choice(K8, 41, replace=False)] *= 20.0
+        xa_d = torch.from_numpy(xa).to(dev).bfloat16()
+        w8_d = torch.from_numpy(rng.normal(0, 0.02, (N8, K8)).astype(np.float32)).to(dev).bfloat16()
+        a_q, a_s = ops._quantize_int8_rowwise(xa_d, 1e-5)
+        w_q, w_s = ops._quantize_int8_rowwise(w8_d, 1e-5)
+        out8 = torch.empty((M8, N8), dtype=torch.bfloat16, device=dev)
+
+        def gemm8():
+            lib.tpq_int8_mm_dequant(a_q.data_ptr(), w_q.data_ptr(), a_s.data_ptr(), w_s.data_ptr(), None,
+                                    out8.data_ptr(), _lib.BF16, M8, N8, K8, cur())
+
+        for _ in range(5):
+            gemm8()
+        ms = time_region(gemm8, sync, 50)
+        tops = 2.0 * M8 * N8 * K8 / (ms * 1e-3) / 1e12
+        extras["int8_gemm_2048x4096x4096_us"] = ms * 1e3
+        extras["int8_gemm_TOPS"] = tops
+        extras["int8_gemm_frac_of_mfma_peak"] = tops / INT8_PEAK_TOPS
+        acc_chk = (a_q[:64].double() @ w_q.double().t())
+        fused_chk = ((acc_chk.float() * a_s[:64, None]) * w_s[None, :]).bfloat16()
+        extras["int8_gemm_rows_checked_equal"] = bool(torch.equal(fused_chk, out8[:64]))
+
+        # activation quantizer on the same activations: 2*M*K + M*K + 4*M bytes
+        cq = torch.empty((M8, K8), dtype=torch.int8, device=dev)
+        sq = torch.empty((M8,), dtype=torch.float32, device=dev)
+
+        def quant():
+            lib.tpq_quantize_rowwise(xa_d.data_ptr(), _lib.BF16, M8, K8, 1e-5, 127.0, -127, 127, 0, cq.data_ptr(),
+                                     sq.data_ptr(), cur())
+
+        for _ in range(5):
+            quant()
+        ms = time_region(quant, sync, 100)
+        extras["quantize_2048x4096_bf16_us"] = ms * 1e3
+        extras["quantize_GBs"] = (3 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
+
+        # BitNet ternary: M in {1,128}, 2560 -> 6912 and 6912 -> 2560 (weights cache resident at this size)
+        for (mt, kt, nt) in ((1, 2560, 6912), (1, 6912, 2560), (128, 2560, 6912), (128, 6912, 2560)):
+            tern = rng.choice(np.int8([-1, 0, 1]), size=(nt, kt), p=[0.325, 0.35, 0.325])
+            pk = ops.pack_ternary(torch.from_numpy(tern).to(dev))
+            xt = torch.from_numpy(rng.normal(0, 1, (mt, kt)).astype(np.float32)).to(dev)
+            xq_t, rs_t = ops._quantize_int8_rowwise(xt, 1e-5)
+            yt = torch.empty((mt, nt), dtype=torch.float16, device=dev)
+
+            def tmm(xq_t=xq_t, rs_t=rs_t, pk=pk, yt=yt, mt=mt, kt=kt, nt=nt):
+                lib.tpq_ternary_mm(xq_t.data_ptr(), rs_t.data_ptr(), pk.data_ptr(), 0.0173, None, mt, nt, kt,
+                                   yt.data_ptr(), _lib.F16, None, cur())
+
+            gt = graph_of(lambda: [tmm() for _ in range(200)])
+            gt.replay(); sync()
+            ms = time_region(gt.replay, sync, 1) / 200
+            key = f"ternary_M{mt}_{kt}x{nt}"
+            extras[key + "_us"] = ms * 1e3
+            if mt == 1:
+                extras[key + "_GBs_cache_resident"] = (nt * kt // 4 + mt * kt + 4 * mt + 2 * mt * nt) / (ms * 1e-3) / 1e9
+            else:
+                extras[key + "_TOPS"] = 2.0 * mt * nt * kt / (ms * 1e-3) / 1e12
+
+    line = {
+        "metric": METRIC,
+        "value": round(gbs, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "int4 weight-only decode GEMV M=1 K=4096 N=11008 group=128 fp16 (BASELINE configs[1])",
+            "weights": f"reference device int4 layout, {copies} rotating copies (HBM resident, not cache resident)",
+            "launch": "K steps in one HIP graph replay",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbs, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES,
+            "kernel": "int4_decode_kernel<f16, M=1, g=128>",
+            "algorithmic_bytes_per_launch": GEMV_BYTES,
+            "avg_launch_us": ms_per_step * 1e3,
+        },
+        "cpu_baseline": None,
+        "extras": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in extras.items()},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(x16, codes, sz16, want)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

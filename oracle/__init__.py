@@ -165,6 +165,24 @@ def int4_mm_cpu(x, dtype, packed, params, group, columns=64, half_split=True, ro
     return out
 
 
+def int4_mm_cpu_blocked(x, dtype, packed, params, group, blocks=None, out=None):
+    """Vectorisable twin of int4_mm_cpu (64-column AVX-512 layout); `blocks` = (begin, end)
+    column blocks to compute, so that threads can split the work."""
+    x = _c(x, storage(dtype))
+    packed = _c(packed, np.uint8)
+    params = _c(params, storage(dtype))
+    m, k = x.shape
+    n = packed.shape[0]
+    assert n % 64 == 0
+    b0, b1 = (0, n // 64) if blocks is None else blocks
+    if out is None:
+        out = np.zeros((m, n), storage(dtype))
+    lib().orc_int4_mm_cpu_blocked(_p(x), _DT[dtype], _p(packed), _p(params), _p(out), ctypes.c_int64(m),
+                                  ctypes.c_int64(n), ctypes.c_int64(k), ctypes.c_int64(group),
+                                  ctypes.c_int64(b0), ctypes.c_int64(b1))
+    return out
+
+
 def int4_pack_tc(codes, inner_k_tiles=2):
     codes = _c(codes, np.int32)
     N, K = codes.shape

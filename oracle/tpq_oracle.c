@@ -325,6 +325,59 @@ ORC_API void orc_int4_mm_cpu(const void* x, int dtype, const uint8_t* packed, co
     }
 }
 
+/*
+ * The same kernel as orc_int4_mm_cpu, organised like the reference's task
+ * split (4 rows x one block of 64 columns per task, k outermost inside a
+ * task; QuantizedElementwiseKernels.cpp:402-479) so that the compiler can
+ * vectorise across the 64 columns.  Used as the timed CPU baseline; callers
+ * spread column blocks over threads the way parallel_for spreads tasks.
+ * AVX-512 layout only (columns = 64, half split), n % 64 == 0.  Every output
+ * sees the identical fmaf sequence, so results equal orc_int4_mm_cpu bit for
+ * bit (asserted in tests/test_oracle_int4.py).
+ */
+ORC_API void orc_int4_mm_cpu_blocked(const void* x, int dtype, const uint8_t* packed,
+                                     const void* params, void* out, int64_t m, int64_t n,
+                                     int64_t k, int64_t group, int64_t block_begin,
+                                     int64_t block_end) {
+    enum { C = 64, H = 32 };
+    float* xf = (float*)malloc(sizeof(float) * (size_t)(m * k > 0 ? m * k : 1));
+    for (int64_t i = 0; i < m * k; ++i) xf[i] = load_as_f32(x, dtype, i);
+    for (int64_t block = block_begin; block < block_end; ++block) {
+        const int64_t first = block * C;
+        const uint8_t* wp = packed + first * k / 2;
+        for (int64_t row = 0; row < m; row += 4) {
+            const int rows = (int)(m - row < 4 ? m - row : 4);
+            float acc[4][C];
+            float scale[C], zero[C];
+            for (int r = 0; r < 4; ++r)
+                for (int c = 0; c < C; ++c) acc[r][c] = 0.0f;
+            for (int64_t f = 0; f < k; ++f) {
+                if (f % group == 0) {
+                    const int64_t g = f / group;
+                    for (int c = 0; c < C; ++c) {
+                        scale[c] = load_as_f32(params, dtype, (g * n + first + c) * 2);
+                        zero[c] = load_as_f32(params, dtype, (g * n + first + c) * 2 + 1);
+                    }
+                }
+                const uint8_t* bytes = wp + f * H;
+                float w[C];
+                for (int lane = 0; lane < H; ++lane) {
+                    const int b = bytes[lane];
+                    w[lane] = fmaf((float)((b & 15) - 8), scale[lane], zero[lane]);
+                    w[lane + H] = fmaf((float)((b >> 4) - 8), scale[lane + H], zero[lane + H]);
+                }
+                for (int r = 0; r < rows; ++r) {
+                    const float a = xf[(row + r) * k + f];
+                    for (int c = 0; c < C; ++c) acc[r][c] = fmaf(a, w[c], acc[r][c]);
+                }
+            }
+            for (int r = 0; r < rows; ++r)
+                for (int c = 0; c < C; ++c) store_from_f32(out, dtype, (row + r) * n + first + c, acc[r][c]);
+        }
+    }
+    free(xf);
+}
+
 /* ------------------------------------------------------------------------ */
 /* A6: device int4 packed layout                                             */
 /* ------------------------------------------------------------------------ */

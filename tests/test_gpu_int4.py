@@ -30,7 +30,7 @@ def asym_quant(w, group):
     s = np.maximum((hi - lo) / 15.0, 1e-8).astype(np.float32)
     q = np.clip(np.rint((wg - lo[..., None]) / s[..., None]), 0, 15).astype(np.int32).reshape(N, K)
     z = (lo + 8 * s).astype(np.float32)
-    return q, np.stack([s.T, z.T], axis=-1)
+    return q, np.ascontiguousarray(np.stack([s.T, z.T], axis=-1))  # [K/g, N, 2]
 
 
 @pytest.mark.parametrize("inner", [2, 4, 8])

@@ -172,3 +172,16 @@ def test_dequantize_rounds_through_activation_dtype():
     s, z = torch.tensor(sz[0, 0, 0]).half(), torch.tensor(sz[0, 0, 1]).half()
     want = ((torch.tensor(3.0).half() * s).half() + z).half()  # each op rounded to half
     assert (from_bits(W, "f16") == want).all()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_blocked_baseline_kernel_equals_scalar_kernel(dtype):
+    rng = np.random.default_rng(77)
+    N, K, g, M = 128, 256, 64, 5
+    codes = rng.integers(0, 16, size=(N, K), dtype="int32")
+    packed = oracle.int4_pack_cpu(codes)
+    x = cast_bits(rng.normal(size=(M, K)).astype(np.float32), dtype)
+    sz = cast_bits(rng.uniform(-0.05, 0.05, size=(K // g, N, 2)).astype(np.float32), dtype)
+    np.testing.assert_array_equal(oracle.int4_mm_cpu_blocked(x, dtype, packed, sz, g), oracle.int4_mm_cpu(x, dtype, packed, sz, g))
+    half = oracle.int4_mm_cpu_blocked(x, dtype, packed, sz, g, blocks=(1, 2))
+    np.testing.assert_array_equal(half[:, 64:], oracle.int4_mm_cpu(x, dtype, packed, sz, g)[:, 64:])
