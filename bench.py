@@ -124,6 +124,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="time the headline GEMV only")
+    ap.add_argument("--gemv-only", action="store_true", help="extras of the int4 GEMV only (no int8 / quantizer / ternary)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -155,9 +156,11 @@ def main() -> int:
     szs = [sz_d] + [sz_d.clone() for _ in range(copies - 1)]
     y_d = torch.empty((M, N), dtype=torch.float16, device=dev)
 
+    ws = torch.zeros(lib.tpq_int4_mm_workspace_bytes(N), dtype=torch.uint8, device=dev)
+
     def gemv(i):
-        rc = lib.tpq_int4_mm(x_d.data_ptr(), _lib.F16, M, K, packs[i % copies].data_ptr(), 2, N, GROUP,
-                             szs[i % copies].data_ptr(), y_d.data_ptr(), cur())
+        rc = lib.tpq_int4_mm_ws(x_d.data_ptr(), _lib.F16, M, K, packs[i % copies].data_ptr(), 2, N, GROUP,
+                                szs[i % copies].data_ptr(), y_d.data_ptr(), ws.data_ptr(), ws.numel(), cur())
         if rc:
             raise RuntimeError(_lib.last_error())
 
@@ -214,8 +217,8 @@ def main() -> int:
             yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
 
             def gemv_b(i, xb=xb, yb=yb, mb=mb):
-                lib.tpq_int4_mm(xb.data_ptr(), _lib.F16, mb, K, packs[i % copies].data_ptr(), 2, N, GROUP,
-                                szs[i % copies].data_ptr(), yb.data_ptr(), cur())
+                lib.tpq_int4_mm_ws(xb.data_ptr(), _lib.F16, mb, K, packs[i % copies].data_ptr(), 2, N, GROUP,
+                                   szs[i % copies].data_ptr(), yb.data_ptr(), ws.data_ptr(), ws.numel(), cur())
 
             gb = graph_of(lambda: [gemv_b(i) for i in range(260)])
             gb.replay(); sync()
@@ -226,6 +229,7 @@ def main() -> int:
         del packs[1:], szs[1:]
         torch.cuda.empty_cache()
 
+    if not args.no_extras and not args.gemv_only:
         # int8 prefill GEMM with fused dequant: M=2048, K=4096, N=4096, bf16 in/out
         M8, K8, N8 = 2048, 4096, 4096
         xa = rng.normal(0, 1, (M8, K8)).astype(np.float32)

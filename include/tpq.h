@@ -17,6 +17,7 @@
 #ifndef TPQ_H
 #define TPQ_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -106,6 +107,25 @@ int tpq_int4_pack(const int32_t* codes, int64_t N, int64_t K, int inner_k_tiles,
 int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
                 int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
                 void* out, void* stream);
+
+/*
+ * Same operator with a caller-provided scratch buffer, which lets the decode
+ * kernel slice the k range of a column group across several workgroups (all
+ * compute units busy when N/64 is small against their number).
+ *   workspace: device memory, 16-byte aligned, at least
+ *              tpq_int4_mm_workspace_bytes(N) bytes, ZERO-FILLED once after
+ *              allocation; every call leaves its first 16 KiB (the arrival
+ *              counters) zero again, so the buffer can be reused call after
+ *              call.  Calls that share a workspace must not overlap in time
+ *              (one workspace per stream).  NULL or too small = the
+ *              single-workgroup path of tpq_int4_mm.
+ * Results do not depend on the slicing order (partials are added in slice
+ * order), so repeated calls are bit-identical.
+ */
+size_t tpq_int4_mm_workspace_bytes(int64_t N);
+int tpq_int4_mm_ws(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
+                   int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
+                   void* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * int8 ternary codes [rows, cols] <-> uint8 [rows, ceil(cols/4)], four 2-bit

@@ -25,6 +25,8 @@ SIGNATURES = {
     "tpq_int8_mm_dequant": [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _ptr],
     "tpq_int4_pack": [_ptr, _i64, _i64, _int, _ptr, _ptr],
     "tpq_int4_mm": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr],
+    "tpq_int4_mm_ws": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, ctypes.c_size_t, _ptr],
+    "tpq_int4_mm_workspace_bytes": [_i64],
     "tpq_ternary_pack": [_ptr, _i64, _i64, _ptr, _ptr],
     "tpq_ternary_unpack": [_ptr, _i64, _i64, _ptr, _ptr],
     "tpq_ternary_mm": [_ptr, _ptr, _ptr, _f32, _ptr, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],
@@ -51,7 +53,7 @@ def load() -> ctypes.CDLL:
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.argtypes = args
-        fn.restype = _int
+        fn.restype = ctypes.c_size_t if name.endswith("_bytes") else _int
     lib.tpq_last_error.argtypes = []
     lib.tpq_last_error.restype = ctypes.c_char_p
     _lib = lib

@@ -19,7 +19,7 @@
 //     loads straight into SGPRs, which feed v_dot2_f32_f16 / v_dot2_f32_bf16
 //     as the scalar operand - no LDS traffic and no cross-lane traffic for x;
 //   * nibbles become 16-bit floats in place with the "magic exponent" trick:
-//     ((w << 4) & 0x00F000F0) | 0x54005400 is the fp16 pair (64+c_even, 64+c_odd)
+//     (w & 0x000F000F) | 0x64006400 is the fp16 pair (1024+c, 1024+c), (w & 0x00F000F0) | 0x54005400 is (64+c, 64+c)
 //     (bf16: (w & 0x000F000F) | 0x43004300 = 128 + c), one shift and one
 //     v_and_or_b32 per pair;
 //   * the offset is removed per group, not per element: with
@@ -34,57 +34,12 @@
 // through a plain fp32 kernel that evaluates w = fma(code-8, scale, zero),
 // y = fma(x, w, y) like the reference's CPU kernel
 // (p10/src/backend/cpu/QuantizedElementwiseKernels.cpp:470-479).
-#include "tpq_common.h"
+#include <cstdlib>
+
+#include "int4_lane.h"
 
 namespace tpq {
 namespace {
-
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef short short2_t __attribute__((ext_vector_type(2)));
-
-constexpr int kDecodeWaves = 16;  // 1024 threads: the whole K range of 64 columns in one workgroup
-constexpr int kChunkKT = 4;       // k-tiles (of 32) per chunk
-constexpr int kRing = 2;          // chunks in flight per wavefront
-
-// (a & mask) | magic in one VALU op; magic lives in a VGPR, mask in an SGPR
-// (one constant-bus operand per instruction on this target).
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) {
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(magic));
-    return r;
-}
-
-template <int DT>
-struct Lane16;
-
-template <>
-struct Lane16<TPQ_DTYPE_F16> {
-    static constexpr float kOffset = 72.0f;  // 64 (magic) + 8 (code bias)
-    static constexpr uint32_t kMask = 0x00F000F0u, kMagic = 0x54005400u, kOnes = 0x3C003C00u;
-    static __device__ __forceinline__ float dot(uint32_t x, uint32_t w, float acc) {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, x), __builtin_bit_cast(half2_t, w), acc, false);
-    }
-    // pair j of word w (codes at k0 + 8j, k0 + 8j + 1) moved to bits 4..7 / 20..23
-    static __device__ __forceinline__ uint32_t align(uint32_t w, int j) {
-        return j == 0 ? (w << 4) : (j == 1 ? w : (w >> (4 * j - 4)));
-    }
-    static __device__ __forceinline__ float lo(uint32_t p) { return f16_bits_to_f32(p & 0xFFFFu); }
-    static __device__ __forceinline__ float hi(uint32_t p) { return f16_bits_to_f32(p >> 16); }
-    static __device__ __forceinline__ uint16_t out(float v) { return f32_to_f16_bits(v); }
-};
-
-template <>
-struct Lane16<TPQ_DTYPE_BF16> {
-    static constexpr float kOffset = 136.0f;  // 128 (magic) + 8
-    static constexpr uint32_t kMask = 0x000F000Fu, kMagic = 0x43004300u, kOnes = 0x3F803F80u;
-    static __device__ __forceinline__ float dot(uint32_t x, uint32_t w, float acc) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(short2_t, x), __builtin_bit_cast(short2_t, w), acc, false);
-    }
-    static __device__ __forceinline__ uint32_t align(uint32_t w, int j) { return j == 0 ? w : (w >> (4 * j)); }
-    static __device__ __forceinline__ float lo(uint32_t p) { return bf16_bits_to_f32(p & 0xFFFFu); }
-    static __device__ __forceinline__ float hi(uint32_t p) { return bf16_bits_to_f32(p >> 16); }
-    static __device__ __forceinline__ uint16_t out(float v) { return f32_to_bf16_bits(v); }
-};
 
 // One chunk in flight: 4 k-tiles x 16 bytes of weights, the (scale, zero)
 // words of its groups, and this lane's word of the chunk's activations.
@@ -97,17 +52,24 @@ struct Chunk {
 
 // x: [M][K/2] 32-bit words (pairs of 16-bit floats); sz: [G][N] words (scale, zero);
 // GROUP_KT = group / 32 in {1, 2, 4}; k_super % 4 == 0.
-template <int DT, int MROWS, int GROUP_KT>
-__global__ __launch_bounds__(kDecodeWaves* kWave) void int4_decode_kernel(
+//
+// WPB wavefronts per workgroup; gridDim.y = KS workgroups share one column group, each taking
+// every (WPB*KS)-th chunk.  With KS > 1 the workgroups leave their partial columns in
+// ws_part[KS][MROWS][N] and bump ws_count[column group]; the one that arrives last adds the KS
+// partials in slice order (so the result does not depend on arrival order), stores y and puts
+// the counter back to zero.  Partials and counter move with agent-scope atomic accesses, which
+// are coherent across the chip's L2 slices.
+template <int DT, int MROWS, int GROUP_KT, int WPB>
+__global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
     const uint32_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
-    uint16_t* __restrict__ y, int N, int K, int k_super) {
+    uint16_t* __restrict__ y, int N, int K, int k_super, float* ws_part, unsigned* ws_count) {
     using L = Lane16<DT>;
     constexpr int kGroups = kChunkKT / GROUP_KT;
-    __shared__ float red[kDecodeWaves * MROWS * kWave];
+    __shared__ float red[WPB * MROWS * kWave];
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = WPB == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = blockIdx.x * kWave + lane;
     const int n_ld = n < N ? n : N - 1;  // lanes past the edge read a valid column and drop the result
     const uint4* wp = packed + (static_cast<size_t>(n_ld >> 3) * k_super) * 8 + (n_ld & 7);
@@ -115,8 +77,9 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void int4_decode_kernel(
     const int words_per_row = K >> 1;
     const int n_chunks = k_super / kChunkKT;
 
-    uint32_t magic;
-    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(L::kMagic));
+    uint32_t magic_even, magic_odd;  // kept in VGPRs: v_and_or_b32 takes one scalar operand only
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic_even) : "s"(L::kMagicEven));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic_odd) : "s"(L::kMagicOdd));
 
     auto issue = [&](Chunk<MROWS, kGroups>& ch, int chunk) {
         chunk = chunk < n_chunks ? chunk : n_chunks - 1;  // past the end: harmless re-read, never used
@@ -133,13 +96,16 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void int4_decode_kernel(
     for (int m = 0; m < MROWS; ++m) yacc[m] = 0.0f;
 
     auto consume = [&](const Chunk<MROWS, kGroups>& ch, int chunk) {
-        // per k-tile sums of the activations: lanes 16i..16i+15 reduce k-tile i
+        // Sums of the activations per k-tile and pair parity.  Lane l holds word l%16 of k-tile
+        // l/16, i.e. pair j = (l%16)/4: adding across lane bits 0, 1 and 3 leaves the sum over
+        // even pairs in lanes with bit 2 clear and the sum over odd pairs in those with it set.
         float xs[MROWS];
 #pragma unroll
         for (int m = 0; m < MROWS; ++m) {
             float s = L::dot(ch.xw[m], L::kOnes, 0.0f);
-#pragma unroll
-            for (int off = 1; off < 16; off <<= 1) s += __shfl_xor(s, off, kWave);
+            s += __shfl_xor(s, 1, kWave);
+            s += __shfl_xor(s, 2, kWave);
+            s += __shfl_xor(s, 8, kWave);
             xs[m] = s;
         }
         float part[MROWS];
@@ -151,9 +117,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void int4_decode_kernel(
             const uint32_t wq[4] = {ch.q[i].x, ch.q[i].y, ch.q[i].z, ch.q[i].w};
             uint32_t v[4][4];
 #pragma unroll
-            for (int t4 = 0; t4 < 4; ++t4)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[t4][j] = and_or(L::align(wq[t4], j), L::kMask, magic);
+            for (int t4 = 0; t4 < 4; ++t4) L::template unpack<false>(wq[t4], v[t4], magic_even, magic_odd);
 #pragma unroll
             for (int m = 0; m < MROWS; ++m) {
                 // wave-uniform address: scalar loads into SGPRs
@@ -169,13 +133,17 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void int4_decode_kernel(
                 const float scale = L::lo(pw), zero = L::hi(pw);
 #pragma unroll
                 for (int m = 0; m < MROWS; ++m) {
-                    float sx = 0.0f;
+                    float sx_even = 0.0f, sx_odd = 0.0f;
 #pragma unroll
-                    for (int g = 0; g < GROUP_KT; ++g)
-                        sx += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xs[m]), 16 * (i + 1 - GROUP_KT + g)));
-                    const float dotp = __builtin_fmaf(-L::kOffset, sx, part[m]);
+                    for (int g = 0; g < GROUP_KT; ++g) {
+                        const int l0 = 16 * (i + 1 - GROUP_KT + g);
+                        sx_even += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xs[m]), l0));
+                        sx_odd += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xs[m]), l0 + 4));
+                    }
+                    float dotp = __builtin_fmaf(-L::kOffsetEven, sx_even, part[m]);
+                    dotp = __builtin_fmaf(-L::kOffsetOdd, sx_odd, dotp);
                     yacc[m] = __builtin_fmaf(scale, dotp, yacc[m]);
-                    yacc[m] = __builtin_fmaf(zero, sx, yacc[m]);
+                    yacc[m] = __builtin_fmaf(zero, sx_even + sx_odd, yacc[m]);
                     part[m] = 0.0f;
                 }
             }
@@ -185,31 +153,82 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void int4_decode_kernel(
         }
     };
 
+    const int slices = gridDim.y;
+    const int stride = WPB * slices;                 // chunks between two turns of this wavefront
+    const int first = blockIdx.y * WPB + wave;
     Chunk<MROWS, kGroups> ring[kRing];
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) issue(ring[u], wave + u * kDecodeWaves);
-    for (int c = wave; c < n_chunks; c += kRing * kDecodeWaves) {
+    for (int u = 0; u < kRing; ++u) issue(ring[u], first + u * stride);
+    for (int c = first; c < n_chunks; c += kRing * stride) {
 #pragma unroll
         for (int u = 0; u < kRing; ++u) {
-            const int cu = c + u * kDecodeWaves;
+            const int cu = c + u * stride;
             if (cu < n_chunks) {
                 consume(ring[u], cu);
-                if (cu + kRing * kDecodeWaves < n_chunks) issue(ring[u], cu + kRing * kDecodeWaves);
+                if (cu + kRing * stride < n_chunks) issue(ring[u], cu + kRing * stride);
             }
         }
     }
 
+    // wavefronts of the workgroup meet in LDS
+    if (WPB > 1) {
 #pragma unroll
-    for (int m = 0; m < MROWS; ++m) red[(wave * MROWS + m) * kWave + lane] = yacc[m];
-    __syncthreads();
-    if (tid < MROWS * kWave) {
-        const int m = tid >> 6;
-        float s = 0.0f;
+        for (int m = 0; m < MROWS; ++m) red[(wave * MROWS + m) * kWave + lane] = yacc[m];
+        __syncthreads();
+        if (wave == 0) {
 #pragma unroll
-        for (int w = 0; w < kDecodeWaves; ++w) s += red[(w * MROWS + m) * kWave + lane];
-        if (n < N) y[static_cast<size_t>(m) * N + n] = L::out(s);
+            for (int m = 0; m < MROWS; ++m) {
+                float s = 0.0f;
+#pragma unroll
+                for (int w = 0; w < WPB; ++w) s += red[(w * MROWS + m) * kWave + lane];
+                yacc[m] = s;
+            }
+        }
+    }
+    if (slices == 1) {
+        if (wave == 0 && n < N) {
+#pragma unroll
+            for (int m = 0; m < MROWS; ++m) y[static_cast<size_t>(m) * N + n] = L::out(yacc[m]);
+        }
+        return;
+    }
+    // several workgroups per column group: leave the partial, count arrivals
+    if (wave == 0) {
+        if (n < N) {
+#pragma unroll
+            for (int m = 0; m < MROWS; ++m)
+                __hip_atomic_store(ws_part + (static_cast<size_t>(blockIdx.y) * MROWS + m) * N + n, yacc[m],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // every lane's partial has reached the coherent level before lane 0 announces the arrival
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned seen = 0;
+        if (lane == 0)
+            seen = __hip_atomic_fetch_add(ws_count + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        seen = __builtin_amdgcn_readfirstlane(seen);
+        if (seen == static_cast<unsigned>(slices - 1)) {  // last to arrive: fold in slice order
+            if (n < N) {
+#pragma unroll
+                for (int m = 0; m < MROWS; ++m) {
+                    float s = 0.0f;
+                    for (int ks = 0; ks < slices; ++ks)
+                        s += __hip_atomic_load(ws_part + (static_cast<size_t>(ks) * MROWS + m) * N + n,
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    y[static_cast<size_t>(m) * N + n] = L::out(s);
+                }
+            }
+            if (lane == 0) __hip_atomic_store(ws_count + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
+
+}  // namespace
+}  // namespace tpq
+
+#include "int4_stream_kernel.h"
+
+namespace tpq {
+namespace {
 
 // Plain fp32 evaluation for every case the decode kernel does not take.
 // Workgroup = one tile of 8 columns x one activation row; thread t: row t%8,
@@ -254,26 +273,123 @@ __global__ __launch_bounds__(256) void int4_generic_kernel(
     }
 }
 
-template <int DT, int MROWS>
+// Workspace handed in by the caller: kCounterSlots arrival counters (zero between calls),
+// then the partial columns [KS][MROWS][N].
+constexpr int kCounterSlots = 4096;
+constexpr size_t kCounterBytes = kCounterSlots * sizeof(unsigned);
+
+inline int compute_units() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+        return n;
+    }();
+    return cus;
+}
+
+struct DecodePlan {
+    int wpb;     // wavefronts per workgroup
+    int slices;  // workgroups per column group (1 = no workspace needed)
+};
+
+// Each wavefront should own about two chunks (256 k of 64 columns); beyond one workgroup of 16
+// wavefronts per column group the k range is sliced across workgroups, which lets all compute
+// units share the columns evenly when there are few column groups.
+inline DecodePlan plan_decode(int N, int K, int mrows, size_t workspace_bytes) {
+    const int n_chunks = K / 128;
+    const int col_groups = (N + kWave - 1) / kWave;
+    DecodePlan plan{kDecodeWaves, 1};
+    const char* env_wpb = std::getenv("TPQ_INT4_WPB");
+    const char* env_ks = std::getenv("TPQ_INT4_KS");
+    int wpb = 0, ks = 0;
+    if (workspace_bytes > kCounterBytes && col_groups <= kCounterSlots) {
+        const size_t per_slice = static_cast<size_t>(mrows) * N * sizeof(float);
+        const int max_slices = static_cast<int>((workspace_bytes - kCounterBytes) / per_slice);
+        // Slicing costs a trip through memory per workgroup (partials out, counter, partials in:
+        // about 1.5 us measured), so it only pays when one workgroup per column group would
+        // leave most of the chip idle.  TPQ_INT4_WPB / TPQ_INT4_KS override for experiments.
+        if (env_wpb || env_ks) {
+            wpb = env_wpb ? std::atoi(env_wpb) : 4;
+            ks = env_ks ? std::atoi(env_ks) : (n_chunks + 2 * wpb - 1) / (2 * wpb);
+        } else if (col_groups * 4 <= compute_units() && n_chunks >= 16) {
+            wpb = 8;
+            ks = 2;
+        }
+        if (ks > max_slices) ks = max_slices;
+        if (ks > 64) ks = 64;
+    }
+    if (ks >= 2 && (wpb == 1 || wpb == 2 || wpb == 4 || wpb == 8 || wpb == 16)) plan = DecodePlan{wpb, ks};
+    return plan;
+}
+
+template <int DT, int MROWS, int WPB>
 int launch_decode_rows(const void* x, const int32_t* packed, const void* sz, void* y, int N, int K,
-                       int group, hipStream_t s) {
+                       int group, int slices, void* workspace, hipStream_t s) {
     const int k_super = K / 32;
-    const dim3 grid((N + kWave - 1) / kWave), block(kDecodeWaves * kWave);
+    const dim3 grid((N + kWave - 1) / kWave, slices), block(WPB * kWave);
     const auto* xp = static_cast<const uint32_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
     const auto* sp = static_cast<const uint32_t*>(sz);
     auto* yp = static_cast<uint16_t*>(y);
+    auto* counters = static_cast<unsigned*>(workspace);
+    auto* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kCounterBytes);
     switch (group) {
-        case 32: int4_decode_kernel<DT, MROWS, 1><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super); break;
-        case 64: int4_decode_kernel<DT, MROWS, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super); break;
-        default: int4_decode_kernel<DT, MROWS, 4><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super); break;
+        case 32: int4_decode_kernel<DT, MROWS, 1, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); break;
+        case 64: int4_decode_kernel<DT, MROWS, 2, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); break;
+        default: int4_decode_kernel<DT, MROWS, 4, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); break;
     }
     return check_launch("tpq_int4_mm (decode)");
 }
 
+template <int DT, int MROWS>
+int launch_decode_plan(const void* x, const int32_t* packed, const void* sz, void* y, int N, int K,
+                       int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
+    const DecodePlan plan = plan_decode(N, K, MROWS, workspace ? workspace_bytes : 0);
+    switch (plan.wpb) {
+        case 1: return launch_decode_rows<DT, MROWS, 1>(x, packed, sz, y, N, K, group, plan.slices, workspace, s);
+        case 2: return launch_decode_rows<DT, MROWS, 2>(x, packed, sz, y, N, K, group, plan.slices, workspace, s);
+        case 4: return launch_decode_rows<DT, MROWS, 4>(x, packed, sz, y, N, K, group, plan.slices, workspace, s);
+        case 8: return launch_decode_rows<DT, MROWS, 8>(x, packed, sz, y, N, K, group, plan.slices, workspace, s);
+        default: return launch_decode_rows<DT, MROWS, 16>(x, packed, sz, y, N, K, group, plan.slices, workspace, s);
+    }
+}
+
+// One activation row through the streaming kernel; false if the shape does not fit it.
+template <int DT>
+bool launch_stream(const void* x, const int32_t* packed, const void* sz, void* y, int N, int K, int group,
+                   hipStream_t s, int* rc) {
+    // Measured on MI355X at M=1, K=4096, N=11008 the column-per-lane kernel is the faster of the
+    // two (7.1 us against 8.3 us); the streaming kernel is kept selectable for comparison runs.
+    const char* force = std::getenv("TPQ_INT4_KERNEL");
+    if (!(force && force[0] == 's')) return false;  // TPQ_INT4_KERNEL=stream opts in
+    const int k_super = K / 32, n_tiles = N / 8;
+    int tiles_per_block = (n_tiles + compute_units() - 1) / compute_units();
+    if (tiles_per_block > 8) tiles_per_block = 8;   // 16 wavefronts per workgroup at most
+    const int waves = 2 * tiles_per_block;
+    const size_t smem = sizeof(uint32_t) * (static_cast<size_t>(k_super) * (kXStride + 2) + waves * 8);
+    if (smem > 64 * 1024) return false;
+    const dim3 grid((n_tiles + tiles_per_block - 1) / tiles_per_block), block(waves * kWave);
+    const auto* xp = static_cast<const uint32_t*>(x);
+    const auto* pp = reinterpret_cast<const uint4*>(packed);
+    const auto* sp = static_cast<const uint32_t*>(sz);
+    auto* yp = static_cast<uint16_t*>(y);
+#define TPQ_STREAM(GKT, EX) \
+    int4_stream_kernel<DT, GKT, EX><<<grid, block, smem, s>>>(xp, pp, sp, yp, N, k_super, n_tiles, tiles_per_block)
+    const bool exact = k_super % 16 == 0;
+    switch (group) {
+        case 32: if (exact) TPQ_STREAM(1, true); else TPQ_STREAM(1, false); break;
+        case 64: if (exact) TPQ_STREAM(2, true); else TPQ_STREAM(2, false); break;
+        default: if (exact) TPQ_STREAM(4, true); else TPQ_STREAM(4, false); break;
+    }
+#undef TPQ_STREAM
+    *rc = check_launch("tpq_int4_mm (stream)");
+    return true;
+}
+
 template <int DT>
 int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* sz, void* y, int N,
-                  int K, int group, hipStream_t s) {
+                  int K, int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
     // rows go through in slabs of at most four; each slab streams the weight once
     const size_t row_bytes_x = static_cast<size_t>(K) * 2, row_bytes_y = static_cast<size_t>(N) * 2;
     for (int64_t m0 = 0; m0 < M; m0 += 4) {
@@ -281,11 +397,15 @@ int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* s
         const void* xs = static_cast<const char*>(x) + m0 * row_bytes_x;
         void* ys = static_cast<char*>(y) + m0 * row_bytes_y;
         int rc;
+        if (rows == 1 && launch_stream<DT>(xs, packed, sz, ys, N, K, group, s, &rc)) {
+            if (rc != TPQ_OK) return rc;
+            continue;
+        }
         switch (rows) {
-            case 1: rc = launch_decode_rows<DT, 1>(xs, packed, sz, ys, N, K, group, s); break;
-            case 2: rc = launch_decode_rows<DT, 2>(xs, packed, sz, ys, N, K, group, s); break;
-            case 3: rc = launch_decode_rows<DT, 3>(xs, packed, sz, ys, N, K, group, s); break;
-            default: rc = launch_decode_rows<DT, 4>(xs, packed, sz, ys, N, K, group, s); break;
+            case 1: rc = launch_decode_plan<DT, 1>(xs, packed, sz, ys, N, K, group, workspace, workspace_bytes, s); break;
+            case 2: rc = launch_decode_plan<DT, 2>(xs, packed, sz, ys, N, K, group, workspace, workspace_bytes, s); break;
+            case 3: rc = launch_decode_plan<DT, 3>(xs, packed, sz, ys, N, K, group, workspace, workspace_bytes, s); break;
+            default: rc = launch_decode_plan<DT, 4>(xs, packed, sz, ys, N, K, group, workspace, workspace_bytes, s); break;
         }
         if (rc != TPQ_OK) return rc;
     }
@@ -313,9 +433,14 @@ int launch_generic(const void* x, int64_t M, const int32_t* packed, const void* 
 
 using namespace tpq;
 
-TPQ_EXPORT int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
-                           int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
-                           void* out, void* stream) {
+TPQ_EXPORT size_t tpq_int4_mm_workspace_bytes(int64_t N) {
+    // counters + up to 16 slices of 4 rows of fp32 partial columns
+    return N <= 0 ? 0 : kCounterBytes + static_cast<size_t>(16) * 4 * static_cast<size_t>(N) * sizeof(float);
+}
+
+TPQ_EXPORT int tpq_int4_mm_ws(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
+                              int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
+                              void* out, void* workspace, size_t workspace_bytes, void* stream) {
     TPQ_REQUIRE(dtype == TPQ_DTYPE_F32 || dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16,
                 TPQ_ERR_INVALID_TYPE, "_weight_int4pack_mm(): activations must be floating point");
     TPQ_REQUIRE(group == 32 || group == 64 || group == 128, TPQ_ERR_INVALID_VALUE,
@@ -338,13 +463,20 @@ TPQ_EXPORT int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const
     const bool fast = dtype != TPQ_DTYPE_F32 && K % 128 == 0 && aligned(x, 16) &&
                       aligned(packed, 16) && aligned(scales_and_zeros, 4) && aligned(out, 2);
     if (fast) {
+        if (workspace && !aligned(workspace, 16)) workspace = nullptr;
         if (dtype == TPQ_DTYPE_F16)
-            return launch_decode<TPQ_DTYPE_F16>(x, M, packed, scales_and_zeros, out, (int)N, (int)K, (int)group, s);
-        return launch_decode<TPQ_DTYPE_BF16>(x, M, packed, scales_and_zeros, out, (int)N, (int)K, (int)group, s);
+            return launch_decode<TPQ_DTYPE_F16>(x, M, packed, scales_and_zeros, out, (int)N, (int)K, (int)group, workspace, workspace_bytes, s);
+        return launch_decode<TPQ_DTYPE_BF16>(x, M, packed, scales_and_zeros, out, (int)N, (int)K, (int)group, workspace, workspace_bytes, s);
     }
     switch (dtype) {
         case TPQ_DTYPE_F32: return launch_generic<TPQ_DTYPE_F32>(x, M, packed, scales_and_zeros, out, N, K, group, s);
         case TPQ_DTYPE_F16: return launch_generic<TPQ_DTYPE_F16>(x, M, packed, scales_and_zeros, out, N, K, group, s);
         default: return launch_generic<TPQ_DTYPE_BF16>(x, M, packed, scales_and_zeros, out, N, K, group, s);
     }
+}
+
+TPQ_EXPORT int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
+                           int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
+                           void* out, void* stream) {
+    return tpq_int4_mm_ws(x, dtype, M, K, packed, inner_k_tiles, N, group, scales_and_zeros, out, nullptr, 0, stream);
 }

@@ -175,6 +175,21 @@ def int8_mm_dequant(A_i8: torch.Tensor, B_t_i8: torch.Tensor, row_scale: torch.T
     return out
 
 
+_int4_workspaces = {}
+
+
+def _int4_workspace(device: torch.device, n: int) -> torch.Tensor:
+    """Zero-filled scratch buffer of the int4 decode kernel, one per (device, stream), grown on demand.
+    The kernel leaves the counters at the front of it zero again after every call."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    need = _lib.load().tpq_int4_mm_workspace_bytes(n)
+    ws = _int4_workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        _int4_workspaces[key] = ws
+    return ws
+
+
 def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.Tensor:
     """int32 codes [N,K] (0..15) -> int32 [ceil(N/8), ceil(K/(16*innerKTiles)), 32, innerKTiles/2]."""
     if self.dim() != 2:
@@ -227,8 +242,9 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     w = mat2.contiguous()
     sz = qScaleAndZeros.to(self.dtype).contiguous()
     with torch.cuda.device(self.device):
-        _check(_lib.load().tpq_int4_mm(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz),
-                                       _ptr(out), _stream(self)))
+        ws = _int4_workspace(self.device, n)
+        _check(_lib.load().tpq_int4_mm_ws(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz),
+                                          _ptr(out), _ptr(ws), ws.numel(), _stream(self)))
     return out
 
 
