@@ -1,10 +1,26 @@
 // Entry points of the integer matrix product (_int_mm) and of the fused
 // int8 GEMM + dequant; the matrix-core kernel itself lives in
 // int8_gemm_kernel.h, shared with the ternary matmul.
-#include "int8_gemm_kernel.h"
+#include <cstdlib>
+
+#include "int8_gemm_dma.h"
 
 namespace tpq {
 namespace {
+
+// Large problems with K a multiple of the 64-byte k-step take the ring-buffered kernel.
+inline TileInt32 to_tile(const EpilogueInt32& ep) { return TileInt32{ep.c, nullptr, nullptr, nullptr}; }
+template <int DT>
+TileDequant<DT> to_tile(const EpilogueDequant<DT>& ep) {
+    return TileDequant<DT>{ep.out, ep.rs, ep.cs, ep.bias};
+}
+
+template <class Epilogue>
+int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
+    const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
+    if (M > 128 && K % kBK == 0 && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
+    return launch_mfma(a, w, M, N, K, ep, s);
+}
 
 // Any strides, any K, signed or unsigned left operand: 16x16 outputs per
 // workgroup, operands staged through LDS 16 k at a time.
@@ -67,7 +83,7 @@ TPQ_EXPORT int tpq_int_mm(const void* a, int a_unsigned, const int8_t* b, int64_
     TPQ_REQUIRE(a && b, TPQ_ERR_INVALID_VALUE, "_int_mm: null operand");
     const EpilogueInt32 ep{c};
     if (!a_unsigned && b_stride_k == 1 && b_stride_n == K && mfma_path_ok(a, b, M, N, K))
-        return launch_mfma(static_cast<const int8_t*>(a), b, M, N, K, ep, s);
+        return launch_best(static_cast<const int8_t*>(a), b, M, N, K, ep, s);
     return launch_generic(a, a_unsigned, b, b_stride_k, b_stride_n, M, K, N, ep, s);
 }
 
@@ -86,7 +102,7 @@ TPQ_EXPORT int tpq_int8_mm_dequant(const int8_t* a, const int8_t* w, const float
     {                                                                                               \
         const EpilogueDequant<DT> ep{static_cast<typename Elem<DT>::storage*>(out), row_scale,      \
                                      col_scale, bias};                                              \
-        if (fast) return launch_mfma(a, w, M, N, K, ep, s);                                         \
+        if (fast) return launch_best(a, w, M, N, K, ep, s);                                         \
         return launch_generic(a, 0, w, 1, K, M, K, N, ep, s);                                       \
     }
     switch (out_dtype) {
