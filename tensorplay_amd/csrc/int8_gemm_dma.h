@@ -33,6 +33,8 @@
 // handled by clamping source rows and masking the stores.
 #pragma once
 
+#include <cstdlib>
+
 #include "int8_gemm_kernel.h"
 
 namespace tpq {
@@ -71,19 +73,23 @@ struct TileDequant {
     }
 };
 
-template <int STAGES, class Tile>
-__global__ __launch_bounds__(256) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
+template <int STAGES, int KSPLIT, class Tile>
+__global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
                                                             const int8_t* __restrict__ W, int M, int N,
                                                             int K, Tile tile, int vector_stores) {
     using out_t = typename Tile::out_t;
     constexpr int BM = 256, BN = 128, WM = 128, WN = 64, TM = 4, TN = 2;
     constexpr int kStageChunks = (BM + BN) * kChunksPerRow;  // 1536 x 16 B = 24 KB
-    constexpr int kLoadsPerWave = kStageChunks / kWave / 4;  // 6
+    constexpr int kThreads = 256 * KSPLIT, kWaves = 4 * KSPLIT;
+    constexpr int kLoadsPerWave = kStageChunks / kWave / kWaves;  // wave-level loads per stage: 6 or 3
+    constexpr int kUnitsPerStage = 2 / KSPLIT;               // 32-byte k-substeps a wavefront multiplies per stage
     constexpr int kPerChunk = 16 / sizeof(out_t);            // outputs per 16 bytes
     constexpr int kPitch = BN * sizeof(out_t) + 16;          // bytes per row of the output image
     constexpr int kRingBytes = STAGES * kStageChunks * 16;
     constexpr int kImageBytes = BM * kPitch;
-    constexpr int kScaleOffset = kRingBytes > kImageBytes ? kRingBytes : kImageBytes;
+    constexpr int kPartialBytes = KSPLIT > 1 ? 4 * 128 * kWave * 4 : 0;  // accumulators of the second k-half
+    constexpr int kScaleOffset = (kRingBytes > kImageBytes ? kRingBytes : kImageBytes) > kPartialBytes
+                                     ? (kRingBytes > kImageBytes ? kRingBytes : kImageBytes) : kPartialBytes;
     extern __shared__ uint4 ring[];                          // [STAGES][kStageChunks], later the image
     char* lds_bytes = reinterpret_cast<char*>(ring);
     float* cs_lds = reinterpret_cast<float*>(lds_bytes + kScaleOffset);  // [BN] column scales, [BN] bias
@@ -91,7 +97,8 @@ __global__ __launch_bounds__(256) void int8_gemm_dma_kernel(const int8_t* __rest
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int kh = wave >> 2;               // which k-substep of every stage this wavefront multiplies (KSPLIT = 2)
+    const int wm = (wave >> 1) & 1, wn = wave & 1;
 
     // Workgroups are dealt to the 8 XCDs round-robin (workgroup id mod 8), each with its own L2:
     // give every XCD a compact patch of tiles, as close to square in bytes as the grid allows,
@@ -199,21 +206,69 @@ __global__ __launch_bounds__(256) void int8_gemm_dma_kernel(const int8_t* __rest
     v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
     landed(0, std::integral_constant<int, STAGES - 2>{});
     asm volatile("s_barrier" ::: "memory");
-    read_frags(0, 0, fa0, fb0);
-    for (int kt = 0; kt < nk; ++kt) {
-        read_frags(kt, 1, fa1, fb1);  // second half of this stage, in flight during the first MFMAs
-        multiply(fa0, fb0);
-        if (kt + 1 < nk) {
-            landed(kt + 1, std::integral_constant<int, STAGES - 3>{});
-            asm volatile("s_barrier" ::: "memory");
-            if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1);
-            read_frags(kt + 1, 0, fa0, fb0);  // first half of the next stage, in flight during the second MFMAs
+    // moving on to stage kt: wait for it, meet, refill the buffer stage kt-2 was read from
+    auto advance = [&](int kt) {
+        landed(kt, std::integral_constant<int, STAGES - 3>{});
+        asm volatile("s_barrier" ::: "memory");
+        if (kt + STAGES - 2 < nk) issue(kt + STAGES - 2);
+    };
+    if constexpr (KSPLIT == 1) {
+        read_frags(0, 0, fa0, fb0);
+        for (int kt = 0; kt < nk; ++kt) {
+            read_frags(kt, 1, fa1, fb1);  // second half of this stage, in flight during the first MFMAs
+            multiply(fa0, fb0);
+            if (kt + 1 < nk) {
+                advance(kt + 1);
+                read_frags(kt + 1, 0, fa0, fb0);  // first half of the next stage, in flight during the second MFMAs
+            }
+            multiply(fa1, fb1);
         }
-        multiply(fa1, fb1);
+    } else {  // one substep (kh) per stage and wavefront; fragments of the next stage in flight during the MFMAs
+        read_frags(0, kh, fa0, fb0);
+        for (int kt = 0; kt < nk; kt += 2) {
+            if (kt + 1 < nk) {
+                advance(kt + 1);
+                read_frags(kt + 1, kh, fa1, fb1);
+            }
+            multiply(fa0, fb0);
+            if (kt + 1 < nk) {
+                if (kt + 2 < nk) {
+                    advance(kt + 2);
+                    read_frags(kt + 2, kh, fa0, fb0);
+                }
+                multiply(fa1, fb1);
+            }
+        }
     }
 
     // ---- epilogue: scale, convert, image in LDS, row-contiguous stores -----------------------------
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring no longer needed
+    if constexpr (KSPLIT > 1) {  // fold the second k-half into the first through LDS
+        int4* part = reinterpret_cast<int4*>(lds_bytes) + (wave & 3) * (TM * TN * 4) * kWave + lane;
+        if (kh == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        part[((i * TN + j) * 4 + q) * kWave] = make_int4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        }
+        __syncthreads();
+        if (kh == 0) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int4 o = part[((i * TN + j) * 4 + q) * kWave];
+                        acc[i][j][4 * q] += o.x; acc[i][j][4 * q + 1] += o.y; acc[i][j][4 * q + 2] += o.z; acc[i][j][4 * q + 3] += o.w;
+                    }
+        }
+        __syncthreads();  // partials consumed before the image overwrites them
+    }
+    if (kh == 0) {
     float rs_r[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -249,9 +304,10 @@ __global__ __launch_bounds__(256) void int8_gemm_dma_kernel(const int8_t* __rest
                 }
             }
         }
+    }  // kh == 0
     __syncthreads();
     constexpr int kChunksPerOutRow = BN / kPerChunk;  // 16-byte chunks per image row
-    for (int c = tid; c < BM * kChunksPerOutRow; c += 256) {
+    for (int c = tid; c < BM * kChunksPerOutRow; c += kThreads) {
         const int row = c / kChunksPerOutRow, col = (c % kChunksPerOutRow) * kPerChunk;
         const int m = m0 + row, n = n0 + col;
         if (m >= M || n >= N) continue;
@@ -265,20 +321,22 @@ __global__ __launch_bounds__(256) void int8_gemm_dma_kernel(const int8_t* __rest
     }
 }
 
-template <int STAGES, class Tile>
+template <int STAGES, int KSPLIT, class Tile>
 constexpr size_t dma_lds_bytes() {
     constexpr size_t ring = static_cast<size_t>(STAGES) * (256 + 128) * kBK;
     constexpr size_t image = 256 * (128 * sizeof(typename Tile::out_t) + 16);
-    return (ring > image ? ring : image) + 2 * 128 * sizeof(float);
+    constexpr size_t partial = KSPLIT > 1 ? 4 * 128 * kWave * 4 : 0;
+    constexpr size_t body = ring > image ? (ring > partial ? ring : partial) : (image > partial ? image : partial);
+    return body + 2 * 128 * sizeof(float);
 }
 
-template <class Tile>
-int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+template <int KSPLIT, class Tile>
+int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
     constexpr int kStages = 5;
-    constexpr size_t smem = dma_lds_bytes<kStages, Tile>();
+    constexpr size_t smem = dma_lds_bytes<kStages, KSPLIT, Tile>();
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
-    auto kernel = int8_gemm_dma_kernel<kStages, Tile>;
+    auto kernel = int8_gemm_dma_kernel<kStages, KSPLIT, Tile>;
     static bool configured = false;  // per instantiation: raise the dynamic LDS limit once
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -287,9 +345,19 @@ int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K
         configured = true;
     }
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
-    kernel<<<dim3(static_cast<unsigned>(tiles)), 256, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
-                                                               static_cast<int>(K), tile, vector_stores);
+    kernel<<<dim3(static_cast<unsigned>(tiles)), 256 * KSPLIT, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
+                                                                        static_cast<int>(K), tile, vector_stores);
     return check_launch("int8 mfma gemm (dma)");
+}
+
+// KSPLIT = 2: eight wavefronts per workgroup, the two k-substeps of every stage go to different
+// wavefronts (two per SIMD keep LDS and the matrix cores busier than one).  TPQ_INT8_KSPLIT=1
+// selects the four-wavefront variant for comparison runs.
+template <class Tile>
+int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+    const char* env = std::getenv("TPQ_INT8_KSPLIT");
+    if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s);
+    return launch_dma_split<2>(a, w, M, N, K, tile, s);
 }
 
 }  // namespace
