@@ -8,7 +8,7 @@
 namespace tpq {
 namespace {
 
-// Large problems with K a multiple of the 64-byte k-step take the ring-buffered kernel.
+// Large problems with K a multiple of the 128-byte stage take the ring-buffered kernel.
 inline TileInt32 to_tile(const EpilogueInt32& ep) { return TileInt32{ep.c, nullptr, nullptr, nullptr}; }
 template <int DT>
 TileDequant<DT> to_tile(const EpilogueDequant<DT>& ep) {
@@ -18,7 +18,7 @@ TileDequant<DT> to_tile(const EpilogueDequant<DT>& ep) {
 template <class Epilogue>
 int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
     const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
-    if (M > 128 && K % kBK == 0 && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
+    if (dma_path_ok(M, K) && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
     return launch_mfma(a, w, M, N, K, ep, s);
 }
 

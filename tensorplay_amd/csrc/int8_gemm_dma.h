@@ -1,39 +1,62 @@
-// int8 GEMM for large problems: 256 x 128 tile per workgroup, multi-stage LDS
-// ring filled by direct global -> LDS loads, fragment reads one k-substep
-// ahead of the matrix cores, and an epilogue that goes back through LDS so
-// that the result leaves in 16-byte row-contiguous stores.
+// int8 GEMM for large problems: 256 x 128 tile per workgroup, three-stage LDS
+// ring filled by direct global -> LDS loads of whole 128-byte cache lines,
+// fragment reads one k-substep ahead of the matrix cores, and an epilogue
+// that goes back through LDS so that the result leaves in 16-byte
+// row-contiguous stores.
 //
-// Main loop.  k-step 64 bytes, 4 wavefronts of 128 (m) x 64 (n) = 4 x 2 blocks
-// of v_mfma_i32_32x32x32_i8.  LDS layout of a stage: row r holds its four
-// 16-byte chunks at position chunk ^ swz(r) (conflict-free for the fragment
-// reads).  A direct load (global_load_lds_dwordx4) writes lane l's 16 bytes to
-// slot l of a 1 KB LDS region whose base is wave-uniform, so the swizzle is
-// applied on the global side: lane l fetches the chunk that belongs in slot l.
-// A stage is 24 wave-level loads, six per wavefront, and STAGES-1 stages are
-// in flight while one is being multiplied.
+// What bounds it (measured on MI355X, M = 2048, N = K = 4096).  Every
+// workgroup pulls (256 + 128) x K bytes through its compute unit's vector
+// memory path, 403 MB over the chip.  Filling LDS with nothing else going on
+// takes 27.5 us when a row contributes 64 bytes per request and 17.4 us when
+// it contributes a whole 128-byte line (8 consecutive lanes of a
+// global_load_lds_dwordx4), which is about what the matrix cores need for the
+// arithmetic (16 - 20 us depending on clock).  So a stage is 128 bytes of k,
+// and the loop is arranged so that fills, fragment reads and MFMAs overlap.
 //
-// Measured on MI355X: LDS serves about 98 bytes/clock/CU to four wavefronts
-// issuing ds_read_b128, and this tiling reads 96 bytes per clock of MFMA work,
-// so the fragment reads have to overlap the MFMAs completely: the reads of
-// substep s+1 are issued before the MFMAs of substep s.
+// Main loop.  Eight wavefronts: four positions of 128 (m) x 64 (n) = 4 x 2
+// blocks of v_mfma_i32_32x32x32_i8, times two k-halves: of the four 32-byte
+// k-substeps of a stage a wavefront multiplies two (kh*2, kh*2+1); the two
+// partial sums meet in the epilogue.  LDS layout of a stage: row r holds its
+// eight 16-byte chunks at position chunk ^ ((r >> 1) & 7), which makes the
+// fragment reads conflict-free.  A direct load writes lane l's 16 bytes to slot
+// l of a 1 KB region whose base is wave-uniform, so the swizzle is applied on
+// the global side: lane l fetches the chunk that belongs in slot l.  A stage is
+// 48 wave-level loads, six per wavefront.
 //
-// Ordering.  Vector loads of a wavefront complete in order: once at most
-// (STAGES-2)*6 are outstanding, this wavefront's share of the oldest stage has
-// landed.  The workgroup barrier that follows makes every wavefront's share
-// visible and proves that everybody is done with the buffer the next direct
-// load overwrites.  The barrier is the bare instruction: __syncthreads() would
-// also drain all outstanding direct loads, i.e. the prefetched stages.
+// Ordering.  Per stage kt a wavefront does
+//     request fragments (kt, second substep)
+//     multiply (kt, first substep)
+//     wait for its own reads of stage kt, first half of multiply (kt, second)
+//     wait for its share of stage kt+1, BARRIER, refill kt's buffer with kt+3,
+//     request fragments (kt+1, first substep)
+//     second half of multiply (kt, second)
+// Passing the barrier proves that every wavefront has finished reading stage kt
+// (its buffer may be overwritten) and that every wavefront's share of stage kt+1
+// has landed.  Vector loads of a wavefront complete in order, so "my share of
+// kt+1 has landed" is "at most the six loads of kt+2 are outstanding".  The
+// barrier is the bare instruction: __syncthreads() would also drain all
+// outstanding direct loads, i.e. the prefetched stages.  Stages kt+1 .. kt+3
+// are in flight or landed while kt is multiplied, 2.5 stage times of lookahead.
 //
-// Epilogue.  The MFMA is issued with the W fragment as its first operand, so a
-// lane ends up with 4 consecutive n for one m in each accumulator quad; those
-// are scaled, converted and written to an LDS image of the output tile, which
-// the workgroup then stores row by row, 16 bytes per lane.
+// Fragment reads and the waits for them are spelled out.  While a direct load
+// is in flight the compiler treats the LDS counter as unordered and waits for
+// it to reach zero before the first use of ANY fragment, including the reads
+// issued a moment ago for the next substep, whose latency the MFMAs are there to
+// cover; the steady-state loop is also free of branches for the same reason.
 //
-// Requires K % 64 == 0 and 16-byte aligned operands.  Edges in M and N are
+// Epilogue.  The two k-halves swap half of their accumulators through LDS, so
+// each finishes 64 of the 128 rows of its position.  The MFMA is issued with the
+// W fragment as its first operand, so a lane ends up with 4 consecutive n for
+// one m in each accumulator quad; those are scaled, converted and written to an
+// LDS image of the output tile, which the workgroup then stores row by row, 16
+// bytes per lane.
+//
+// Requires K % 128 == 0 and 16-byte aligned operands.  Edges in M and N are
 // handled by clamping source rows and masking the stores.
 #pragma once
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "int8_gemm_kernel.h"
 
@@ -73,31 +96,30 @@ struct TileDequant {
     }
 };
 
-template <int STAGES, int KSPLIT, class Tile>
-__global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
+constexpr int kDmaRowBytes = 128;  // bytes of k per stage: one cache line per row
+constexpr int kDmaStages = 3;
+
+template <class Tile>
+__global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
                                                             const int8_t* __restrict__ W, int M, int N,
                                                             int K, Tile tile, int vector_stores) {
     using out_t = typename Tile::out_t;
     constexpr int BM = 256, BN = 128, WM = 128, WN = 64, TM = 4, TN = 2;
-    constexpr int kStageChunks = (BM + BN) * kChunksPerRow;  // 1536 x 16 B = 24 KB
-    constexpr int kThreads = 256 * KSPLIT, kWaves = 4 * KSPLIT;
-    constexpr int kLoadsPerWave = kStageChunks / kWave / kWaves;  // wave-level loads per stage: 6 or 3
-    constexpr int kUnitsPerStage = 2 / KSPLIT;               // 32-byte k-substeps a wavefront multiplies per stage
+    constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;    // 48 KB
+    constexpr int kThreads = 512, kWaves = 8;
+    constexpr int kLoads = kStageBytes / 1024 / kWaves;      // wave-level loads per stage and wavefront: 6
     constexpr int kPerChunk = 16 / sizeof(out_t);            // outputs per 16 bytes
     constexpr int kPitch = BN * sizeof(out_t) + 16;          // bytes per row of the output image
-    constexpr int kRingBytes = STAGES * kStageChunks * 16;
-    constexpr int kImageBytes = BM * kPitch;
-    constexpr int kPartialBytes = KSPLIT > 1 ? 4 * 128 * kWave * 4 : 0;  // accumulators of the second k-half
-    constexpr int kScaleOffset = (kRingBytes > kImageBytes ? kRingBytes : kImageBytes) > kPartialBytes
-                                     ? (kRingBytes > kImageBytes ? kRingBytes : kImageBytes) : kPartialBytes;
-    extern __shared__ uint4 ring[];                          // [STAGES][kStageChunks], later the image
+    constexpr int kRingBytes = kDmaStages * kStageBytes;     // 144 KB, covers the image and the exchange area
+    static_assert(BM * kPitch <= kRingBytes && kWaves * 16 * kWave * 16 <= kRingBytes, "epilogue areas live in the ring");
+    extern __shared__ uint4 ring[];                          // [stage][row][128 B], later exchange area and image
     char* lds_bytes = reinterpret_cast<char*>(ring);
-    float* cs_lds = reinterpret_cast<float*>(lds_bytes + kScaleOffset);  // [BN] column scales, [BN] bias
+    float* cs_lds = reinterpret_cast<float*>(lds_bytes + kRingBytes);  // [BN] column scales, [BN] bias
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kh = wave >> 2;               // which k-substep of every stage this wavefront multiplies (KSPLIT = 2)
+    const int kh = wave >> 2;               // k-half: substeps 2*kh and 2*kh+1 of every stage
     const int wm = (wave >> 1) & 1, wn = wave & 1;
 
     // Workgroups are dealt to the 8 XCDs round-robin (workgroup id mod 8), each with its own L2:
@@ -118,7 +140,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         }
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int nk = K / kBK;
+    const int nk = K / kDmaRowBytes;
 
     if (Tile::kScaled && tid < BN) {  // column scales and bias of this tile: read once, used in the epilogue
         const int n = n0 + tid < N ? n0 + tid : N - 1;
@@ -126,12 +148,13 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         cs_lds[BN + tid] = tile.bias ? tile.bias[n] : 0.0f;
     }
 
-    // what lane l of wave-level load i fetches: slot (wave*6 + i)*64 + l of the stage
-    const int8_t* src[kLoadsPerWave];
+    // wave-level load i of this wavefront fills rows (wave*6 + i)*8 .. +7 of the stage; lane l
+    // fetches what belongs in slot l%8 of row l/8
+    const int8_t* src[kLoads];
 #pragma unroll
-    for (int i = 0; i < kLoadsPerWave; ++i) {
-        const int row = (wave * kLoadsPerWave + i) * 16 + (lane >> 2);   // stage row 0..383
-        const int chunk = (lane & 3) ^ swz(row);
+    for (int i = 0; i < kLoads; ++i) {
+        const int row = (wave * kLoads + i) * 8 + (lane >> 3);            // stage row 0..383
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
         if (row < BM) {
             int gr = m0 + row;
             gr = gr < M ? gr : M - 1;
@@ -142,19 +165,12 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
             src[i] = W + static_cast<size_t>(gr) * K + chunk * 16;
         }
     }
-    auto issue = [&](int kt) {
-        uint4* stage = ring + (kt % STAGES) * kStageChunks;
+    auto issue = [&](int kt, int slot) {
+        char* dst = lds_bytes + slot * kStageBytes + wave * (kLoads * 1024);
 #pragma unroll
-        for (int i = 0; i < kLoadsPerWave; ++i)
-            __builtin_amdgcn_global_load_lds((global_void_ptr)(src[i] + static_cast<size_t>(kt) * kBK),
-                                             (lds_void_ptr)(stage + (wave * kLoadsPerWave + i) * kWave), 16, 0, 0);
-    };
-    // this wavefront's loads of stage kt are complete: at the points where it is called the
-    // stages up to kt + YOUNGER have been issued, so that many may still be outstanding
-    auto landed = [&](int kt, auto younger) {
-        constexpr int kYounger = decltype(younger)::value;
-        if (nk - 1 - kt >= kYounger) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kYounger * kLoadsPerWave));
-        else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        for (int i = 0; i < kLoads; ++i)
+            __builtin_amdgcn_global_load_lds((global_void_ptr)(src[i] + static_cast<size_t>(kt) * kDmaRowBytes),
+                                             (lds_void_ptr)(dst + i * 1024), 16, 0, 0);
     };
 
     v16i acc[TM][TN];
@@ -165,146 +181,176 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
+    // Fragment addresses.  Lane (row = lane % 32, half = lane / 32) of block i reads 16 bytes of
+    // row base + 32 i, chunk 2 * substep + half.  All rows a lane touches differ by multiples of
+    // 16, so they share one swizzle value, and the blocks are 32 rows = 4 KB apart: one address
+    // register per operand and substep, the block picked by the instruction's offset field.
     const int frag_row = lane & 31, frag_half = lane >> 5;
-    int a_off[TM], b_off[TN], a_swz[TM], b_swz[TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int r = wm * WM + i * 32 + frag_row;
-        a_off[i] = r * kChunksPerRow;
-        a_swz[i] = swz(r);
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int r = BM + wn * WN + j * 32 + frag_row;
-        b_off[j] = r * kChunksPerRow;
-        b_swz[j] = swz(r);
-    }
-    auto read_frags = [&](int kt, int ks, v4i (&fa)[TM], v4i (&fb)[TN]) {
-        const uint4* stage = ring + (kt % STAGES) * kStageChunks;
-        const int chunk = ks * 2 + frag_half;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = __builtin_bit_cast(v4i, stage[a_off[i] + (chunk ^ a_swz[i])]);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = __builtin_bit_cast(v4i, stage[b_off[j] + (chunk ^ b_swz[j])]);
+    const uint32_t ring_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)ring));
+    const uint32_t sw16 = ((frag_row >> 1) & 7) * 16;
+    const uint32_t chunk_first = ((kh * 4 + frag_half) * 16) ^ sw16, chunk_second = ((kh * 4 + 2 + frag_half) * 16) ^ sw16;
+    const uint32_t a_row = ring_addr + (wm * WM + frag_row) * kDmaRowBytes;
+    const uint32_t b_row = ring_addr + (BM + wn * WN + frag_row) * kDmaRowBytes;
+    auto read_frags = [&](int slot, uint32_t chunk_off, v4i (&fa)[TM], v4i (&fb)[TN]) {
+        static_assert(TM == 4 && TN == 2, "offsets below");
+        const uint32_t a = a_row + slot * kStageBytes + chunk_off, b = b_row + slot * kStageBytes + chunk_off;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(fa[0]) : "v"(a) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[1]) : "v"(a) : "memory");
+        asm volatile("ds_read_b128 %0, %1" : "=v"(fb[0]) : "v"(b) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fb[1]) : "v"(b) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[2]) : "v"(a) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa[3]) : "v"(a) : "memory");
+        // keep the reads ahead of the MFMAs that follow in program order: left alone, the
+        // scheduler sinks them below those MFMAs to shorten the fragments' live ranges
+        __builtin_amdgcn_sched_barrier(0);
     };
-    auto multiply = [&](const v4i (&fa)[TM], const v4i (&fb)[TN]) {
+    // LDS reads of a wavefront return in order: once at most NEWER remain outstanding, every
+    // read before the newest NEWER has delivered.  The fragments pass through the statement so
+    // that the MFMAs consuming them cannot be moved above the wait.
+    auto frags_ready = [&](auto newer, v4i (&fa)[TM], v4i (&fb)[TN]) {
+        constexpr int kNewer = decltype(newer)::value;
+        asm volatile("s_waitcnt lgkmcnt(%6)"
+                     : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1])
+                     : "n"(kNewer));
+    };
+    constexpr std::integral_constant<int, TM + TN> kOneBatch{};  // the reads of one substep
+    constexpr std::integral_constant<int, 0> kNone{};
+    // blocks i in [I0, I0 + 2); W fragment first: accumulator rows run along n
+    auto multiply = [&](auto i0, const v4i (&fa)[TM], const v4i (&fb)[TN]) {
+        constexpr int I0 = decltype(i0)::value;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = I0; i < I0 + 2; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)  // W fragment first: accumulator rows run along n
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
     };
+    constexpr std::integral_constant<int, 0> kLow{};
+    constexpr std::integral_constant<int, 2> kHigh{};
 
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s)
-        if (s < nk) issue(s);
+    for (int s = 0; s < kDmaStages; ++s)
+        if (s < nk) issue(s, s);
+    {  // this wavefront's share of stage 0: everything issued after it may still be outstanding
+        const int younger = nk - 1 < kDmaStages - 1 ? nk - 1 : kDmaStages - 1;
+        if (younger == 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * kLoads));
+        else if (younger == 1) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads));
+        else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    // The LDS counter is shared with scalar loads (kernel arguments, which return out of order)
+    // and the column-scale writes above: drain it, so that only fragment reads are counted.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-    // Buffers in use while stage kt is multiplied: kt (being read), kt+1 .. kt+STAGES-2 (landed
-    // or in flight).  The barrier sits in the middle of a stage; when a wavefront passes it,
-    // all wavefronts have consumed their reads of stage kt-1, whose buffer takes stage
-    // kt+STAGES-1.
     v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-    landed(0, std::integral_constant<int, STAGES - 2>{});
-    asm volatile("s_barrier" ::: "memory");
-    // moving on to stage kt: wait for it, meet, refill the buffer stage kt-2 was read from
-    auto advance = [&](int kt) {
-        landed(kt, std::integral_constant<int, STAGES - 3>{});
+    int kt = 0, slot = 0;  // slot: kt % kDmaStages
+    read_frags(0, chunk_first, fa0, fb0);
+    for (; kt + kDmaStages < nk; ++kt) {  // steady state: stages kt+1 .. kt+3 all exist
+        const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
+        read_frags(slot, chunk_second, fa1, fb1);
+        frags_ready(kOneBatch, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        multiply(kHigh, fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);  // the waits below stay behind the MFMAs that cover them
+        frags_ready(kNone, fa1, fb1);  // this wavefront is done reading stage kt
+        multiply(kLow, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads));  // own share of kt+1 landed (kt+2 may be in flight)
         asm volatile("s_barrier" ::: "memory");
-        if (kt + STAGES - 2 < nk) issue(kt + STAGES - 2);
-    };
-    if constexpr (KSPLIT == 1) {
-        read_frags(0, 0, fa0, fb0);
-        for (int kt = 0; kt < nk; ++kt) {
-            read_frags(kt, 1, fa1, fb1);  // second half of this stage, in flight during the first MFMAs
-            multiply(fa0, fb0);
-            if (kt + 1 < nk) {
-                advance(kt + 1);
-                read_frags(kt + 1, 0, fa0, fb0);  // first half of the next stage, in flight during the second MFMAs
-            }
-            multiply(fa1, fb1);
+        issue(kt + kDmaStages, slot);
+        read_frags(next, chunk_first, fa0, fb0);
+        multiply(kHigh, fa1, fb1);
+        slot = next;
+    }
+    for (; kt < nk; ++kt) {  // last stages: nothing left to issue
+        const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
+        read_frags(slot, chunk_second, fa1, fb1);
+        frags_ready(kOneBatch, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        multiply(kHigh, fa0, fb0);
+        frags_ready(kNone, fa1, fb1);
+        if (kt + 1 < nk) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            asm volatile("s_barrier" ::: "memory");
+            read_frags(next, chunk_first, fa0, fb0);
         }
-    } else {  // one substep (kh) per stage and wavefront; fragments of the next stage in flight during the MFMAs
-        read_frags(0, kh, fa0, fb0);
-        for (int kt = 0; kt < nk; kt += 2) {
-            if (kt + 1 < nk) {
-                advance(kt + 1);
-                read_frags(kt + 1, kh, fa1, fb1);
-            }
-            multiply(fa0, fb0);
-            if (kt + 1 < nk) {
-                if (kt + 2 < nk) {
-                    advance(kt + 2);
-                    read_frags(kt + 2, kh, fa0, fb0);
-                }
-                multiply(fa1, fb1);
-            }
-        }
+        multiply(kLow, fa1, fb1);
+        multiply(kHigh, fa1, fb1);
+        slot = next;
     }
 
-    // ---- epilogue: scale, convert, image in LDS, row-contiguous stores -----------------------------
+    // ---- epilogue ------------------------------------------------------------------------------------
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring no longer needed
-    if constexpr (KSPLIT > 1) {  // fold the second k-half into the first through LDS
-        int4* part = reinterpret_cast<int4*>(lds_bytes) + (wave & 3) * (TM * TN * 4) * kWave + lane;
-        if (kh == 1) {
+    // Exchange: a wavefront keeps blocks i in [KEEP, KEEP+2) and hands the other two to its
+    // partner (same position, other k-half), 16 KB per wavefront.
+    int4* mine = reinterpret_cast<int4*>(lds_bytes) + wave * (16 * kWave) + lane;
+    const int4* theirs = reinterpret_cast<const int4*>(lds_bytes) + (wave ^ 4) * (16 * kWave) + lane;
+    auto hand_over = [&](auto give) {
+        constexpr int G = decltype(give)::value;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        part[((i * TN + j) * 4 + q) * kWave] = make_int4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-        }
-        __syncthreads();
-        if (kh == 0) {
+                for (int q = 0; q < 4; ++q)
+                    mine[((i * TN + j) * 4 + q) * kWave] = make_int4(acc[G + i][j][4 * q], acc[G + i][j][4 * q + 1],
+                                                                     acc[G + i][j][4 * q + 2], acc[G + i][j][4 * q + 3]);
+    };
+    auto take_over = [&](auto keep) {
+        constexpr int KEEP = decltype(keep)::value;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int4 o = part[((i * TN + j) * 4 + q) * kWave];
-                        acc[i][j][4 * q] += o.x; acc[i][j][4 * q + 1] += o.y; acc[i][j][4 * q + 2] += o.z; acc[i][j][4 * q + 3] += o.w;
-                    }
-        }
-        __syncthreads();  // partials consumed before the image overwrites them
-    }
-    if (kh == 0) {
-    float rs_r[TM];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wm * WM + i * 32 + frag_row;
-        rs_r[i] = Tile::kScaled ? tile.rs[m < M ? m : M - 1] : 0.0f;
-    }
+                for (int q = 0; q < 4; ++q) {
+                    const int4 o = theirs[((i * TN + j) * 4 + q) * kWave];
+                    acc[KEEP + i][j][4 * q] += o.x; acc[KEEP + i][j][4 * q + 1] += o.y;
+                    acc[KEEP + i][j][4 * q + 2] += o.z; acc[KEEP + i][j][4 * q + 3] += o.w;
+                }
+    };
+    // scale, convert and place blocks [KEEP, KEEP+2) in the image
     const bool has_bias = tile.bias != nullptr;
+    auto to_image = [&](auto keep) {
+        constexpr int KEEP = decltype(keep)::value;
+        float rs_r[2];
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < 2; ++i) {
+            const int m = m0 + wm * WM + (KEEP + i) * 32 + frag_row;
+            rs_r[i] = Tile::kScaled ? tile.rs[m < M ? m : M - 1] : 0.0f;
+        }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int n_local = wn * WN + j * 32 + 8 * q + 4 * frag_half;  // 4 consecutive columns
-            float c4[4] = {0, 0, 0, 0}, b4[4] = {0, 0, 0, 0};
-            if (Tile::kScaled) {
-                const float4 c = *reinterpret_cast<const float4*>(cs_lds + n_local);
-                const float4 b = *reinterpret_cast<const float4*>(cs_lds + BN + n_local);
-                c4[0] = c.x; c4[1] = c.y; c4[2] = c.z; c4[3] = c.w;
-                b4[0] = b.x; b4[1] = b.y; b4[2] = b.z; b4[3] = b.w;
-            }
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int m_local = wm * WM + i * 32 + frag_row;
-                out_t vals[4];
+            for (int q = 0; q < 4; ++q) {
+                const int n_local = wn * WN + j * 32 + 8 * q + 4 * frag_half;  // 4 consecutive columns
+                float c4[4] = {0, 0, 0, 0}, b4[4] = {0, 0, 0, 0};
+                if (Tile::kScaled) {
+                    const float4 c = *reinterpret_cast<const float4*>(cs_lds + n_local);
+                    const float4 b = *reinterpret_cast<const float4*>(cs_lds + BN + n_local);
+                    c4[0] = c.x; c4[1] = c.y; c4[2] = c.z; c4[3] = c.w;
+                    b4[0] = b.x; b4[1] = b.y; b4[2] = b.z; b4[3] = b.w;
+                }
 #pragma unroll
-                for (int t = 0; t < 4; ++t) vals[t] = Tile::convert(acc[i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
-                char* dst = lds_bytes + m_local * kPitch + n_local * sizeof(out_t);
-                if constexpr (sizeof(out_t) == 2) {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(vals[0] | (static_cast<uint32_t>(vals[1]) << 16),
-                                                                vals[2] | (static_cast<uint32_t>(vals[3]) << 16));
-                } else {
-                    *reinterpret_cast<uint4*>(dst) = make_uint4(__builtin_bit_cast(uint32_t, vals[0]), __builtin_bit_cast(uint32_t, vals[1]),
-                                                                __builtin_bit_cast(uint32_t, vals[2]), __builtin_bit_cast(uint32_t, vals[3]));
+                for (int i = 0; i < 2; ++i) {
+                    const int m_local = wm * WM + (KEEP + i) * 32 + frag_row;
+                    out_t vals[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) vals[t] = Tile::convert(acc[KEEP + i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
+                    char* dst = lds_bytes + m_local * kPitch + n_local * sizeof(out_t);
+                    if constexpr (sizeof(out_t) == 2) {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(vals[0] | (static_cast<uint32_t>(vals[1]) << 16),
+                                                                    vals[2] | (static_cast<uint32_t>(vals[3]) << 16));
+                    } else {
+                        *reinterpret_cast<uint4*>(dst) = make_uint4(__builtin_bit_cast(uint32_t, vals[0]), __builtin_bit_cast(uint32_t, vals[1]),
+                                                                    __builtin_bit_cast(uint32_t, vals[2]), __builtin_bit_cast(uint32_t, vals[3]));
+                    }
                 }
             }
-        }
-    }  // kh == 0
+    };
+    if (kh == 0) hand_over(kHigh); else hand_over(kLow);
+    __syncthreads();
+    if (kh == 0) take_over(kLow); else take_over(kHigh);
+    __syncthreads();  // exchange area consumed before the image overwrites it
+    if (kh == 0) to_image(kLow); else to_image(kHigh);
     __syncthreads();
     constexpr int kChunksPerOutRow = BN / kPerChunk;  // 16-byte chunks per image row
     for (int c = tid; c < BM * kChunksPerOutRow; c += kThreads) {
@@ -321,22 +367,15 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     }
 }
 
-template <int STAGES, int KSPLIT, class Tile>
-constexpr size_t dma_lds_bytes() {
-    constexpr size_t ring = static_cast<size_t>(STAGES) * (256 + 128) * kBK;
-    constexpr size_t image = 256 * (128 * sizeof(typename Tile::out_t) + 16);
-    constexpr size_t partial = KSPLIT > 1 ? 4 * 128 * kWave * 4 : 0;
-    constexpr size_t body = ring > image ? (ring > partial ? ring : partial) : (image > partial ? image : partial);
-    return body + 2 * 128 * sizeof(float);
-}
+// K must be a multiple of the 128-byte stage.
+inline bool dma_path_ok(int64_t M, int64_t K) { return M > 128 && K % kDmaRowBytes == 0; }
 
-template <int KSPLIT, class Tile>
-int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
-    constexpr int kStages = 5;
-    constexpr size_t smem = dma_lds_bytes<kStages, KSPLIT, Tile>();
+template <class Tile>
+int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+    constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + 2 * 128 * sizeof(float);
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
-    auto kernel = int8_gemm_dma_kernel<kStages, KSPLIT, Tile>;
+    auto kernel = int8_gemm_dma_kernel<Tile>;
     static bool configured = false;  // per instantiation: raise the dynamic LDS limit once
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -345,19 +384,9 @@ int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int
         configured = true;
     }
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
-    kernel<<<dim3(static_cast<unsigned>(tiles)), 256 * KSPLIT, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
-                                                                        static_cast<int>(K), tile, vector_stores);
+    kernel<<<dim3(static_cast<unsigned>(tiles)), 512, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
+                                                                 static_cast<int>(K), tile, vector_stores);
     return check_launch("int8 mfma gemm (dma)");
-}
-
-// KSPLIT = 2: eight wavefronts per workgroup, the two k-substeps of every stage go to different
-// wavefronts (two per SIMD keep LDS and the matrix cores busier than one).  TPQ_INT8_KSPLIT=1
-// selects the four-wavefront variant for comparison runs.
-template <class Tile>
-int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
-    const char* env = std::getenv("TPQ_INT8_KSPLIT");
-    if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s);
-    return launch_dma_split<2>(a, w, M, N, K, tile, s);
 }
 
 }  // namespace
