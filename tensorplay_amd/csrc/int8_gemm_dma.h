@@ -26,10 +26,9 @@
 // Ordering.  Per stage kt a wavefront does
 //     request fragments (kt, second substep)
 //     multiply (kt, first substep)
-//     wait for its own reads of stage kt, first half of multiply (kt, second)
-//     wait for its share of stage kt+1, BARRIER, refill kt's buffer with kt+3,
-//     request fragments (kt+1, first substep)
-//     second half of multiply (kt, second)
+//     wait for its own reads of stage kt and for its share of stage kt+1, BARRIER
+//     multiply (kt, second substep), and between its MFMAs: request fragments
+//     (kt+1, first substep), refill kt's buffer with kt+3
 // Passing the barrier proves that every wavefront has finished reading stage kt
 // (its buffer may be overwritten) and that every wavefront's share of stage kt+1
 // has landed.  Vector loads of a wavefront complete in order, so "my share of
@@ -165,12 +164,19 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
             src[i] = W + static_cast<size_t>(gr) * K + chunk * 16;
         }
     }
-    auto issue = [&](int kt, int slot) {
+    // loads FIRST, FIRST+1 of this wavefront's six
+    auto issue_pair = [&](auto first, int kt, int slot) {
+        constexpr int FIRST = decltype(first)::value;
         char* dst = lds_bytes + slot * kStageBytes + wave * (kLoads * 1024);
 #pragma unroll
-        for (int i = 0; i < kLoads; ++i)
+        for (int i = FIRST; i < FIRST + 2; ++i)
             __builtin_amdgcn_global_load_lds((global_void_ptr)(src[i] + static_cast<size_t>(kt) * kDmaRowBytes),
                                              (lds_void_ptr)(dst + i * 1024), 16, 0, 0);
+    };
+    auto issue = [&](int kt, int slot) {
+        issue_pair(std::integral_constant<int, 0>{}, kt, slot);
+        issue_pair(std::integral_constant<int, 2>{}, kt, slot);
+        issue_pair(std::integral_constant<int, 4>{}, kt, slot);
     };
 
     v16i acc[TM][TN];
@@ -191,15 +197,23 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
     const uint32_t chunk_first = ((kh * 4 + frag_half) * 16) ^ sw16, chunk_second = ((kh * 4 + 2 + frag_half) * 16) ^ sw16;
     const uint32_t a_row = ring_addr + (wm * WM + frag_row) * kDmaRowBytes;
     const uint32_t b_row = ring_addr + (BM + wn * WN + frag_row) * kDmaRowBytes;
-    auto read_frags = [&](int slot, uint32_t chunk_off, v4i (&fa)[TM], v4i (&fb)[TN]) {
+    // the six reads of a substep, in two groups of three: (A0, A1, W0), then (W1, A2, A3)
+    auto read_group = [&](auto group, int slot, uint32_t chunk_off, v4i (&fa)[TM], v4i (&fb)[TN]) {
         static_assert(TM == 4 && TN == 2, "offsets below");
         const uint32_t a = a_row + slot * kStageBytes + chunk_off, b = b_row + slot * kStageBytes + chunk_off;
-        asm volatile("ds_read_b128 %0, %1" : "=v"(fa[0]) : "v"(a) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[1]) : "v"(a) : "memory");
-        asm volatile("ds_read_b128 %0, %1" : "=v"(fb[0]) : "v"(b) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fb[1]) : "v"(b) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[2]) : "v"(a) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa[3]) : "v"(a) : "memory");
+        if constexpr (decltype(group)::value == 0) {
+            asm volatile("ds_read_b128 %0, %1" : "=v"(fa[0]) : "v"(a) : "memory");
+            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[1]) : "v"(a) : "memory");
+            asm volatile("ds_read_b128 %0, %1" : "=v"(fb[0]) : "v"(b) : "memory");
+        } else {
+            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fb[1]) : "v"(b) : "memory");
+            asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[2]) : "v"(a) : "memory");
+            asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa[3]) : "v"(a) : "memory");
+        }
+    };
+    auto read_frags = [&](int slot, uint32_t chunk_off, v4i (&fa)[TM], v4i (&fb)[TN]) {
+        read_group(std::integral_constant<int, 0>{}, slot, chunk_off, fa, fb);
+        read_group(std::integral_constant<int, 1>{}, slot, chunk_off, fa, fb);
         // keep the reads ahead of the MFMAs that follow in program order: left alone, the
         // scheduler sinks them below those MFMAs to shorten the fragments' live ranges
         __builtin_amdgcn_sched_barrier(0);
@@ -226,6 +240,18 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
     };
     constexpr std::integral_constant<int, 0> kLow{};
     constexpr std::integral_constant<int, 2> kHigh{};
+    // one MFMA, block (I, J), fenced: nothing is scheduled across it
+    auto multiply_one = [&](auto ic, auto jc, const v4i (&fa)[TM], const v4i (&fb)[TN]) {
+        constexpr int I = decltype(ic)::value, J = decltype(jc)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        acc[I][J] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[J], fa[I], acc[I][J], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    constexpr std::integral_constant<int, 0> k0{};
+    constexpr std::integral_constant<int, 1> k1{};
+    constexpr std::integral_constant<int, 2> k2{};
+    constexpr std::integral_constant<int, 3> k3{};
+    constexpr std::integral_constant<int, 4> k4{};
 
 #pragma unroll
     for (int s = 0; s < kDmaStages; ++s)
@@ -251,13 +277,24 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
         multiply(kHigh, fa0, fb0);
         __builtin_amdgcn_sched_barrier(0);  // the waits below stay behind the MFMAs that cover them
         frags_ready(kNone, fa1, fb1);  // this wavefront is done reading stage kt
-        multiply(kLow, fa1, fb1);
-        __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads));  // own share of kt+1 landed (kt+2 may be in flight)
         asm volatile("s_barrier" ::: "memory");
-        issue(kt + kDmaStages, slot);
-        read_frags(next, chunk_first, fa0, fb0);
-        multiply(kHigh, fa1, fb1);
+        // Second substep.  An MFMA occupies the matrix core for 32 clocks but the wavefront's
+        // issue slot only briefly, so the fragment requests for stage kt+1 and the refill (address
+        // arithmetic and all) go between the MFMAs instead of in front of them.
+        multiply_one(k0, k0, fa1, fb1);
+        read_group(k0, next, chunk_first, fa0, fb0);
+        multiply_one(k0, k1, fa1, fb1);
+        read_group(k1, next, chunk_first, fa0, fb0);
+        multiply_one(k1, k0, fa1, fb1);
+        issue_pair(k0, kt + kDmaStages, slot);
+        multiply_one(k1, k1, fa1, fb1);
+        issue_pair(k2, kt + kDmaStages, slot);
+        multiply_one(k2, k0, fa1, fb1);
+        issue_pair(k4, kt + kDmaStages, slot);
+        multiply_one(k2, k1, fa1, fb1);
+        multiply_one(k3, k0, fa1, fb1);
+        multiply_one(k3, k1, fa1, fb1);
         slot = next;
     }
     for (; kt < nk; ++kt) {  // last stages: nothing left to issue
