@@ -125,6 +125,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="time the headline GEMV only")
     ap.add_argument("--gemv-only", action="store_true", help="extras of the int4 GEMV only (no int8 / quantizer / ternary)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain 256 MiB device copy a few times: the known-size kernel that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -197,6 +200,14 @@ def main() -> int:
     gbs = GEMV_BYTES / (ms_per_step * 1e-3) / 1e9
 
     extras = {"gemv_max_rel_err_vs_fp64": gpu_err, "graph_wall_ms_per_step": wall_ms / steps}
+    if args.calibrate_copy:
+        src_c = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst_c = torch.empty_like(src_c)
+        for _ in range(5):
+            dst_c.copy_(src_c)  # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        sync()
+        extras["calibration_copy_bytes_each_way"] = 256 << 20
+        del src_c, dst_c
     if not args.no_extras:
         # same kernel, launched eagerly through the C ABI (python + launch overhead included)
         sync()
