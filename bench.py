@@ -33,9 +33,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 M, K, N, GROUP = 1, 4096, 11008, 128
 GEMV_BYTES = N * K // 2 + (K // GROUP) * N * 4 + 2 * M * K + 2 * M * N   # 23,983,616
-# HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled
-# by a copy kernel of known size); None until measured.  Summary: profiles/int4_decode_gemv_pmc.md
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
+# by what the same counter reads for a 256 MiB device copy (--calibrate-copy): 11770.35 KiB x 1.99981
+# fetched + 21.50 KiB x 1.0 written.  Summary: profiles/int4_decode_gemv_M1_K4096_N11008.md
+MEASURED_TRAFFIC_BYTES = 24_125_400
 
 
 def asym_quant_int4(w, group):
