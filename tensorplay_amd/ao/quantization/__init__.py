@@ -1,0 +1,30 @@
+"""Quantized-linear host code: the reference's function and module names over PyTorch-ROCm tensors.
+
+Every forward runs through the HIP library (``tensorplay_amd.ops``); there is no CPU path here.
+"""
+from .bitnet import (  # noqa: F401
+    BitNetPacked2bitLinear,
+    bitnet_linear_packed,
+    get_bitnet_scale,
+    pack_ternary,
+    quantize_bitnet_weight,
+    quantize_int8_rowwise,
+    unpack_ternary,
+)
+from .int4_weight_only import (  # noqa: F401
+    Int4WeightOnlyConfig,
+    WeightOnlyInt4Linear,
+    _int4_mm,
+    _pack_int4_weight,
+    _quantize_int4_groupwise,
+    int4_weight_only,
+)
+from .int8_mixed_precision import (  # noqa: F401
+    Int8DynamicLinear,
+    Int8DynamicLinearConfig,
+    _dynamic_int8_mm,
+    _int8_mm,
+    int8_dynamic_linear,
+    scaled_int8_mm,
+)
+from .quantize_api import quantize_, register_quantize_module_handler  # noqa: F401

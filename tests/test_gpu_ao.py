@@ -1,0 +1,143 @@
+"""The ao modules on the GPU against the CPU oracle and the reference tests' closed forms
+(test/quantization/test_int4_modules.py:26-82, test_awq.py:75-99, test_int8_mixed_precision.py:26-34,
+219-229, test_native_1bit.py:200-210)."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import oracle
+from gpu_util import DEV, assert_close_norm, dev, host
+from helpers import bits_of, cast_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _ao():
+    import tensorplay_amd.ao.quantization as q
+    return q
+
+
+@pytest.mark.parametrize("dtype,tag", [(torch.float16, "f16"), (torch.bfloat16, "bf16"), (torch.float32, "f32")])
+@pytest.mark.parametrize("rows", [1, 8, 33])
+def test_weight_only_int4_linear(dtype, tag, rows):
+    q = _ao()
+    rng = np.random.default_rng(31)
+    N, K, g = 264, 512, 128
+    lin = nn.Linear(K, N, bias=True)
+    with torch.no_grad():
+        lin.weight.copy_(torch.from_numpy(rng.normal(0, 0.02, (N, K)).astype(np.float32)))
+        lin.bias.copy_(torch.from_numpy(rng.normal(0, 0.01, (N,)).astype(np.float32)))
+    lin = lin.to(DEV, dtype)
+    mod = q.WeightOnlyInt4Linear.from_float(lin, g)
+    assert mod.weight.shape == (N // 8, K // 32, 32, 1) and mod.scales_and_zeros.shape == (K // g, N, 2)
+    # quantizer parity: same closed form evaluated by torch on the CPU in the weight's dtype
+    codes_cpu, scale_cpu, _ = q._quantize_int4_groupwise(lin.weight.detach().cpu(), g)
+    np.testing.assert_array_equal(host(mod.weight), oracle.int4_pack_tc(codes_cpu.numpy(), 2))
+    np.testing.assert_array_equal(host(mod.scales_and_zeros[..., 0]), bits_of(scale_cpu.t().contiguous()))
+    x = torch.from_numpy(rng.normal(0, 1, (2, rows, K)).astype(np.float32)).to(DEV, dtype)
+    y = mod(x)
+    assert y.shape == (2, rows, N) and y.dtype == dtype
+    xb = bits_of(x.reshape(-1, K).cpu())
+    szb = bits_of(mod.scales_and_zeros.cpu())
+    ref, y64 = oracle.int4_mm_tc(xb, tag, host(mod.weight), szb, g, want_f64=True)
+    want = y64 + lin.bias.detach().double().cpu().numpy()[None, :]
+    got = y.reshape(-1, N).float().cpu().numpy()
+    assert_close_norm(got, want, 1e-2 if tag != "f32" else 1e-3, f"int4 linear {tag}")
+    # the reference module test: close to the float linear
+    dense = (x.reshape(-1, K).float() @ lin.weight.detach().float().t() + lin.bias.detach().float()).cpu().numpy()
+    assert np.abs(got - dense).max() < 1.0
+
+
+def test_act_pre_scale_is_applied():
+    q = _ao()
+    rng = np.random.default_rng(32)
+    lin = nn.Linear(256, 64, bias=False).to(DEV, torch.float16)
+    mod = q.WeightOnlyInt4Linear.from_float(lin, 64)
+    x = torch.from_numpy(rng.normal(0, 1, (4, 256)).astype(np.float32)).to(DEV, torch.float16)
+    pre = torch.from_numpy(rng.uniform(0.5, 2.0, (256,)).astype(np.float32)).to(DEV, torch.float16)
+    plain = mod(x * pre)
+    mod.act_pre_scale = pre
+    assert torch.equal(mod(x), plain)
+
+
+@pytest.mark.parametrize("dtype,tag", [(torch.float32, "f32"), (torch.bfloat16, "bf16"), (torch.float16, "f16")])
+def test_dynamic_int8_linear_matches_oracle_chain(dtype, tag):
+    q = _ao()
+    rng = np.random.default_rng(33)
+    M, K, N = 48, 320, 200
+    x32 = rng.normal(0, 1, (3, M // 3, K)).astype(np.float32)
+    w32 = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    b32 = rng.normal(0, 0.01, (N,)).astype(np.float32)
+    x = torch.from_numpy(x32).to(DEV, dtype)
+    w = torch.from_numpy(w32).to(DEV)  # float32 master weight: cast to the activation dtype inside
+    y = q.int8_dynamic_linear(x, w, torch.from_numpy(b32).to(DEV))
+    assert y.shape == (3, M // 3, N) and y.dtype == torch.float32
+    xq, xs = oracle.quantize_int8_rowwise(cast_bits(x32.reshape(M, K), tag), tag, 1e-5)
+    wq, ws = oracle.quantize_int8_rowwise(cast_bits(w32, tag), tag, 1e-5)
+    want = oracle.int8_mm_rescale(oracle.int_mm_nk(xq, wq), xs, ws) + b32[None, :]
+    np.testing.assert_array_equal(host(y).reshape(M, N), want.astype(np.float32))
+    # manual_int8mp_linear of the reference's test: float closed form, atol/rtol 1e-3 on small values
+    ref = ((xq.astype(np.float64) * xs[:, None]) @ (wq.astype(np.float64) * ws[:, None]).T) + b32
+    np.testing.assert_allclose(host(y).reshape(M, N), ref, rtol=1e-3, atol=1e-3)
+
+
+def test_scaled_int8_mm_and_module():
+    q = _ao()
+    rng = np.random.default_rng(34)
+    A = rng.integers(-127, 128, (40, 96), dtype=np.int8)
+    B = rng.integers(-127, 128, (96, 24), dtype=np.int8)
+    rs = rng.uniform(0.001, 0.01, 40).astype(np.float32)
+    cs = rng.uniform(0.001, 0.01, 24).astype(np.float32)
+    got = q.scaled_int8_mm(dev(A), dev(B), dev(rs), dev(cs))
+    want = oracle.int8_mm_rescale(oracle.int_mm(A, B), rs, cs)
+    np.testing.assert_array_equal(host(got), want)
+    lin = nn.Linear(96, 24).to(DEV)
+    mod = q.Int8DynamicLinear.from_float(lin, out_dtype=torch.bfloat16)
+    x = torch.from_numpy(rng.normal(0, 1, (5, 96)).astype(np.float32)).to(DEV)
+    y = mod(x)
+    want = q.int8_dynamic_linear(x, lin.weight.detach(), lin.bias.detach())
+    # same fp32 value rounded once to bf16 (bias inside the rounding here, outside in the reference chain)
+    assert_close_norm(y.float().cpu().numpy(), want.cpu().numpy(), 1e-2, "int8 module bf16")
+    model = nn.Sequential(nn.Linear(96, 64), nn.ReLU(), nn.Linear(64, 24)).to(DEV)
+    dense = model(x)
+    q.quantize_(model, q.Int8DynamicLinearConfig())
+    assert isinstance(model[0], q.Int8DynamicLinear)
+    assert_close_norm(model(x).cpu().detach().numpy(), dense.cpu().detach().numpy(), 5e-2, "int8 swapped model")
+
+
+@pytest.mark.parametrize("shape", [(1, 256, 96), (7, 132, 40), (128, 512, 64)])
+def test_bitnet_linear_packed(shape):
+    q = _ao()
+    M, K, N = shape
+    rng = np.random.default_rng(612)
+    w = rng.normal(0, 0.05, (N, K)).astype(np.float32)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    b = rng.normal(0, 0.1, (N,)).astype(np.float32)
+    codes, scale = q.quantize_bitnet_weight(dev(w))
+    ocodes, oscale = oracle.quantize_bitnet_weight(w)
+    np.testing.assert_array_equal(host(codes), ocodes)
+    np.testing.assert_allclose(scale.item(), oscale, rtol=1e-6)
+    packed = q.pack_ternary(codes)
+    y = q.bitnet_linear_packed(dev(x), packed, scale, K, bias=dev(b))
+    xq, xs = oracle.quantize_int8_rowwise(x, "f32", 1e-5)
+    want, _ = oracle.ternary_mm(xq, xs, oracle.pack_ternary(ocodes), float(scale.item()), K, bias=b)
+    np.testing.assert_array_equal(host(y), want)
+    # manual_bitnet_linear of the reference test, rtol/atol 1e-5
+    ref = (xq.astype(np.int32) @ ocodes.astype(np.int32).T) * xs[:, None] * np.float32(scale.item()) + b
+    np.testing.assert_allclose(host(y), ref, rtol=1e-5, atol=1e-5)
+    lin = nn.Linear(K, N).to(DEV)
+    mod = q.BitNetPacked2bitLinear.from_float(lin)
+    assert mod(dev(x)).shape == (M, N)
+
+
+def test_quantize_swaps_int4_modules():
+    q = _ao()
+    model = nn.Sequential(nn.Linear(256, 128, bias=False), nn.SiLU(), nn.Linear(128, 64, bias=False)).to(DEV, torch.float16)
+    x = torch.randn(3, 256, device=DEV, dtype=torch.float16)
+    dense = model(x)
+    q.quantize_(model, q.Int4WeightOnlyConfig(groupsize=64))
+    assert isinstance(model[0], q.WeightOnlyInt4Linear) and isinstance(model[2], q.WeightOnlyInt4Linear)
+    y = model(x)
+    assert y.shape == dense.shape
+    assert (y.float() - dense.float()).abs().max().item() < 0.25 * dense.float().abs().max().item() + 0.05
