@@ -1,0 +1,195 @@
+// int4 decode kernel for 1..16 activation rows on the matrix cores (fp16 / bf16,
+// group a multiple of 128, K % 128 == 0): every packed byte is read once for
+// all rows, and the multiply-accumulate work leaves the vector ALU.
+//
+// v_mfma_f32_16x16x16 computes D[i][j] += sum_k A[i][k] B[k][j] with lane
+// l = (i or j) + 16 q holding the four k-slots 4q..4q+3 of its row / column.
+// Which actual k sits in a slot is free as long as A and B agree, and that is
+// what makes the packed layout usable without any shuffle:
+//   * A = weights.  Lane (i, q) owns row n0 + i and, in a step of four k-tiles
+//     (128 k), the k-tile 4 s + q: one 16-byte load = the row's four words =
+//     all 32 k of that tile.  A word unpacks in place into four 16-bit pairs
+//     (magic + code, see int4_lane.h); pair j of words r and r + 1 is k = 2r + 8j
+//     .. + 3, the A operand of one MFMA, eight MFMAs per step and 16 rows.
+//   * B = activations.  Lane (m, q) loads the 64 bytes x[m][32 (4s+q) .. +32)
+//     and the operand of MFMA u is simply dwords 2u and 2u + 1 of them, the same
+//     four k as the weight pairs.  Columns m >= M repeat row M-1 and are dropped.
+//   * One more MFMA per four k with a constant A (row 0: the magic offsets + 8,
+//     row 1: ones) yields, per activation row, corr = sum x (offset + 8) and
+//     sx = sum x over the step; they come out in lanes 0..15 and are broadcast
+//     with two cross-lane reads.
+//   * D is lane (m, q) x rows n0 + 4q + v.  A step lies inside one quantization
+//     group, so after its MFMAs  y += scale (D - corr) + zero sx  in fp32 with
+//     this lane's four (scale, zero) pairs, one 16-byte load.
+// A workgroup owns 16 NB consecutive output channels; its wavefronts take the
+// steps round-robin and meet in LDS at the end.
+#pragma once
+
+#include "int4_lane.h"
+
+namespace tpq {
+namespace {
+
+
+// dword r of a 16-byte vector; r is a constant once the loops around the call are unrolled
+__device__ __forceinline__ uint32_t dword_of(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
+
+template <int DT>
+struct MfmaLane;
+template <>
+struct MfmaLane<TPQ_DTYPE_F16> {
+    static constexpr uint32_t kOffEven = 0x64086408u, kOffOdd = 0x54805480u, kOnes = 0x3C003C00u;  // 1032, 72, 1
+    static __device__ __forceinline__ float4_t mfma(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+        const word2_t a = {a0, a1}, b = {b0, b1};
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
+    }
+};
+template <>
+struct MfmaLane<TPQ_DTYPE_BF16> {
+    static constexpr uint32_t kOffEven = 0x43084308u, kOffOdd = 0x43084308u, kOnes = 0x3F803F80u;  // 136, 136, 1
+    static __device__ __forceinline__ float4_t mfma(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+        const word2_t a = {a0, a1}, b = {b0, b1};
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+    }
+};
+
+// x: [M][K] 16-bit; packed: [N/8][K/32][8] x 16 bytes; sz: [K/group][N] words (scale, zero);
+// steps = K / 128; a group is 128 << group_shift k.
+//
+template <int DT, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
+    uint16_t* __restrict__ y, int M, int N, int K, int group_shift) {
+    using L = Lane16<DT>;
+    using ML = MfmaLane<DT>;
+    __shared__ float red[WAVES][NB][4][kWave];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, q = lane >> 4;
+    const int k_super = K / 32, steps = K / 128, n_tiles = N / 8;
+    const int n0 = blockIdx.x * (16 * NB);
+
+    // per-lane bases
+    const uint4* w_base[NB];
+    const uint32_t* sz_base[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        int tile = (n0 + 16 * b + i) >> 3;                 // tile of row n0 + 16 b + i
+        tile = tile < n_tiles ? tile : n_tiles - 1;        // rows past N: any valid tile, result dropped
+        w_base[b] = packed + (static_cast<size_t>(tile) * k_super + q) * 8 + (i & 7);
+        int n4 = n0 + 16 * b + 4 * q;                      // this lane's four output channels
+        n4 = n4 + 4 <= N ? n4 : N - 4;
+        sz_base[b] = sz + n4;
+    }
+    const bool row_live = i < M;
+    // columns m >= M repeat the last row: their products are computed and never stored
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : M - 1) * K) + q * 4;
+
+    // constant A of the correction MFMA: row 0 = offset + 8 of the pair parity, row 1 = ones
+    uint32_t a_corr_even = 0, a_corr_odd = 0;
+    if (i == 0) { a_corr_even = ML::kOffEven; a_corr_odd = ML::kOffOdd; }
+    if (i == 1) { a_corr_even = ML::kOnes; a_corr_odd = ML::kOnes; }
+    uint32_t magic_even, magic_odd;  // kept in VGPRs behind an opaque move: v_and_or_b32 takes one literal only
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic_even) : "s"(L::kMagicEven));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic_odd) : "s"(L::kMagicOdd));
+
+    struct Step {
+        uint4 w[NB];
+        uint4 p[NB];
+        uint4 xv[4];
+    };
+    auto load = [&](int s, Step& st) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            st.w[b] = w_base[b][static_cast<size_t>(s) * 32];                       // four k-tiles further per step
+            st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
+    };
+
+    float yacc[NB][4];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) yacc[b][v] = 0.0f;
+
+    auto compute = [&](const Step& st) {
+        auto xd = [&](int k) { return dword_of(st.xv[k >> 2], k & 3); };  // dword k of the lane's 64 activation bytes
+        // the correction product and the weight products alternate, so that no MFMA waits for
+        // the one issued just before it
+        float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t d[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) d[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        uint32_t v[NB][4][4];  // [block][word r][pair j] = codes at k = 2 r + 8 j, + 1 of the lane's k-tile
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) L::template unpack<true>(dword_of(st.w[b], r), v[b][r], magic_even, magic_odd);
+        // MFMA u covers k = 4u .. 4u+3 of the k-tile: B is dwords 2u, 2u+1 of the activations (adjacent
+        // registers of one load), A is pair j = u/2 of words r0 = 2 (u%2) and r0 + 1.
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int r0 = 2 * (u & 1), j = u >> 1;
+            const bool odd = j & 1;
+            aux = ML::mfma(odd ? a_corr_odd : a_corr_even, odd ? a_corr_odd : a_corr_even, xd(2 * u), xd(2 * u + 1), aux);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) d[b] = ML::mfma(v[b][r0][j], v[b][r0 + 1][j], xd(2 * u), xd(2 * u + 1), d[b]);
+        }
+        // rows 0 and 1 of the correction product sit in lanes 0..15, registers 0 and 1
+        const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t pw = dword_of(st.p[b], v);  // (scale, zero) of channel n0 + 16 b + 4 q + v
+                yacc[b][v] = __builtin_fmaf(L::lo(pw), d[b][v] - corr, __builtin_fmaf(L::hi(pw), sx, yacc[b][v]));
+            }
+        }
+    };
+
+    // this wavefront's steps: wave, wave + WAVES, ...; two in flight
+    Step s0, s1;
+    int s = wave;
+    if (s < steps) load(s, s0);
+    if (s + WAVES < steps) load(s + WAVES, s1);
+    for (; s + 3 * WAVES < steps; s += 2 * WAVES) {  // steady state: no branches in the body
+        compute(s0);
+        load(s + 2 * WAVES, s0);
+        compute(s1);
+        load(s + 3 * WAVES, s1);
+    }
+    if (s < steps) {
+        compute(s0);
+        if (s + 2 * WAVES < steps) load(s + 2 * WAVES, s0);
+        if (s + WAVES < steps) compute(s1);
+        if (s + 2 * WAVES < steps) compute(s0);
+    }
+
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = yacc[b][v];
+    __syncthreads();
+    // wavefront w finishes block b = w, w + W, ...: lane (m, q) stores channels n0 + 16 b + 4 q + v
+    for (int b = wave; b < NB; b += WAVES) {
+        float sum[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            sum[v] = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) sum[v] += red[w][b][v][lane];
+        }
+        const int n = n0 + 16 * b + 4 * q;
+        if (row_live && n < N) {  // N % 8 == 0 and n % 4 == 0: all four channels exist
+            const uint32_t lo = L::out(sum[0]) | (static_cast<uint32_t>(L::out(sum[1])) << 16);
+            const uint32_t hi = L::out(sum[2]) | (static_cast<uint32_t>(L::out(sum[3])) << 16);
+            *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
+        }
+    }
+}
+
+}  // namespace
+}  // namespace tpq

@@ -37,6 +37,7 @@
 #include <cstdlib>
 
 #include "int4_lane.h"
+#include "int4_mfma_kernel.h"
 
 namespace tpq {
 namespace {
@@ -387,9 +388,55 @@ bool launch_stream(const void* x, const int32_t* packed, const void* sz, void* y
     return true;
 }
 
+// Up to 16 rows per launch on the matrix cores; false if the shape does not fit that kernel.
+template <int DT>
+bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void* sz, void* y, int N, int K,
+                      int group, hipStream_t s, int* rc) {
+    if ((group != 128 && group != 256) || !aligned(sz, 16) || !aligned(y, 8)) return false;
+    const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
+    if (force && force[0] == 'd') return false;
+    if (rows == 1 && !(force && force[0] == 'm')) return false;
+    // Measured at K = 4096, N = 11008 (us, rotating weights): 4 rows 9.7 with 16 channels per
+    // workgroup and 8 wavefronts; 16 rows 11.9 with 64 channels and 4 wavefronts (14.6 with 32).
+    int nb = rows <= 4 ? 1 : 4;
+    if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
+    const auto* xp = static_cast<const uint16_t*>(x);
+    const auto* pp = reinterpret_cast<const uint4*>(packed);
+    const auto* sp = static_cast<const uint32_t*>(sz);
+    auto* yp = static_cast<uint16_t*>(y);
+    const int shift = group == 128 ? 0 : 1;  // a group is 128 << shift k (128 or 256)
+    int waves = nb == 1 ? 8 : 4;
+    if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
+#define TPQ_MFMA(NBV, WV) \
+    int4_mfma_kernel<DT, NBV, WV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>(xp, pp, sp, yp, rows, N, K, shift)
+    if (waves == 8) {
+        if (nb == 1) TPQ_MFMA(1, 8); else TPQ_MFMA(2, 8);
+    } else {
+        if (nb == 1) TPQ_MFMA(1, 4); else if (nb == 2) TPQ_MFMA(2, 4); else TPQ_MFMA(4, 4);
+    }
+#undef TPQ_MFMA
+    *rc = check_launch("tpq_int4_mm (mfma)");
+    return true;
+}
+
 template <int DT>
 int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* sz, void* y, int N,
                   int K, int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
+    {   // slabs of 16 rows on the matrix cores where the shape allows
+        const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;
+        int64_t m0 = 0;
+        for (; m0 < M; m0 += 16) {
+            const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+            int rc;
+            if (!launch_mfma_rows<DT>(static_cast<const char*>(x) + m0 * row_x, rows, packed, sz,
+                                      static_cast<char*>(y) + m0 * row_y, N, K, group, s, &rc)) break;
+            if (rc != TPQ_OK) return rc;
+        }
+        if (m0 >= M) return TPQ_OK;
+        x = static_cast<const char*>(x) + m0 * row_x;  // what is left (a single last row, or everything) takes the paths below
+        y = static_cast<char*>(y) + m0 * row_y;
+        M -= m0;
+    }
     // rows go through in slabs of at most four; each slab streams the weight once
     const size_t row_bytes_x = static_cast<size_t>(K) * 2, row_bytes_y = static_cast<size_t>(N) * 2;
     for (int64_t m0 = 0; m0 < M; m0 += 4) {
