@@ -118,6 +118,84 @@ def cpu_baseline(x16, codes, sz16, want, budget_s=12.0):
     }
 
 
+def decoder_layer_share(dev, rng_seed=5):
+    """BASELINE configs[4]: one Llama-style decoder layer (d=4096, 32 heads x 128, MLP 11008, SwiGLU,
+    RMSNorm eps 1e-5, interleaved RoPE, no biases, as in the reference's benchmark/bench_llama_e2e.py:37-92),
+    all seven projections int4 group-128 weight-only, decode step at batch 8 against a 2048-token fp16
+    KV cache.  Attention, norms, RoPE and the elementwise glue are PyTorch-ROCm fp16 ops; the seven
+    linears are this library's.  Three copies of the layer's weights rotate so that they are read from
+    HBM, as they would be in a 32-layer model.  Returns layer us, linears-only us and the share."""
+    import torch
+    import torch.nn.functional as F
+
+    from tensorplay_amd.ao.quantization import WeightOnlyInt4Linear
+
+    d, H, D, inter, B, T = 4096, 32, 128, 11008, 8, 2048
+    gen = torch.Generator(device=dev).manual_seed(rng_seed)
+    shapes = {"q": (d, d), "k": (d, d), "v": (d, d), "o": (d, d), "gate": (inter, d), "up": (inter, d), "down": (d, inter)}
+    copies = 3
+    layers = []
+    for _ in range(copies):
+        mods = {}
+        for name, (n, k) in shapes.items():
+            lin = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.float16)
+            with torch.no_grad():
+                lin.weight.copy_((torch.randn(n, k, device=dev, generator=gen) * 0.02).half())
+            mods[name] = WeightOnlyInt4Linear.from_float(lin, 128)
+            del lin
+        layers.append(mods)
+    torch.cuda.empty_cache()
+    n1 = torch.ones(d, device=dev, dtype=torch.float16)
+    n2 = torch.ones(d, device=dev, dtype=torch.float16)
+    kc = (torch.randn(B, H, T + 1, D, device=dev, generator=gen) * 0.5).half()
+    vc = (torch.randn(B, H, T + 1, D, device=dev, generator=gen) * 0.5).half()
+    x0 = torch.randn(B, 1, d, device=dev, generator=gen).half()
+    inv = 1.0 / (10000.0 ** (torch.arange(D // 2, device=dev, dtype=torch.float32) * 2.0 / D))
+    ang = float(T) * inv
+    cos, sin = ang.cos().half().view(1, 1, 1, D // 2), ang.sin().half().view(1, 1, 1, D // 2)
+
+    def rope(t):
+        e, o = t[..., 0::2], t[..., 1::2]
+        return torch.stack((e * cos - o * sin, e * sin + o * cos), dim=-1).reshape_as(t)
+
+    def layer(L, x):
+        r = x
+        xn = F.rms_norm(x, (d,), n1, 1e-5)
+        q = L["q"](xn).view(B, 1, H, D).transpose(1, 2)
+        k = L["k"](xn).view(B, 1, H, D).transpose(1, 2)
+        v = L["v"](xn).view(B, 1, H, D).transpose(1, 2)
+        q, k = rope(q), rope(k)
+        kc[:, :, T:T + 1] = k
+        vc[:, :, T:T + 1] = v
+        a = F.scaled_dot_product_attention(q, kc, vc)
+        x = r + L["o"](a.transpose(1, 2).reshape(B, 1, H * D))
+        r = x
+        xn = F.rms_norm(x, (d,), n2, 1e-5)
+        return r + L["down"](F.silu(L["gate"](xn)) * L["up"](xn))
+
+    xin = {n: torch.randn(B, 1, k, device=dev, generator=gen).half() for n, (_, k) in shapes.items()}
+
+    def linears(L):
+        for name in shapes:
+            L[name](xin[name])
+
+    reps = 12
+    out = layer(layers[0], x0)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    g_layer = graph_of(lambda: [layer(layers[i % copies], x0) for i in range(reps)])
+    g_lin = graph_of(lambda: [linears(layers[i % copies]) for i in range(reps)])
+    res = {}
+    for key, g in (("layer_decode_b8_kv2048_us", g_layer), ("layer_int4_linears_us", g_lin)):
+        g.replay(); torch.cuda.synchronize()
+        ts = [time_region(g.replay, torch.cuda.synchronize, 1) / reps for _ in range(5)]
+        res[key] = sorted(ts)[2] * 1e3
+    res["layer_int4_linear_share"] = res["layer_int4_linears_us"] / res["layer_decode_b8_kv2048_us"]
+    lin_bytes = sum(n * k // 2 + (k // 128) * n * 4 + 2 * B * k + 2 * B * n for n, k in shapes.values())
+    res["layer_int4_linears_GBs"] = lin_bytes / (res["layer_int4_linears_us"] * 1e-6) / 1e9
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -126,6 +204,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="time the headline GEMV only")
     ap.add_argument("--gemv-only", action="store_true", help="extras of the int4 GEMV only (no int8 / quantizer / ternary)")
+    ap.add_argument("--no-layer", action="store_true", help="skip the decoder-layer share measurement (config 5)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB device copy a few times: the known-size kernel that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -302,6 +381,11 @@ def main() -> int:
                 extras[key + "_GBs_cache_resident"] = (nt * kt // 4 + mt * kt + 4 * mt + 2 * mt * nt) / (ms * 1e-3) / 1e9
             else:
                 extras[key + "_TOPS"] = 2.0 * mt * nt * kt / (ms * 1e-3) / 1e12
+
+    if not args.no_extras and not args.gemv_only and not args.no_layer:
+        del packs, szs
+        torch.cuda.empty_cache()
+        extras.update(decoder_layer_share(dev))
 
     line = {
         "metric": METRIC,

@@ -396,20 +396,24 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
     if (force && force[0] == 'd') return false;
     if (rows == 1 && !(force && force[0] == 'm')) return false;
-    // Measured at K = 4096, N = 11008 (us, rotating weights): 4 rows 9.7 with 16 channels per
-    // workgroup and 8 wavefronts; 16 rows 11.9 with 64 channels and 4 wavefronts (14.6 with 32).
-    int nb = rows <= 4 ? 1 : 4;
+    // Every workgroup reads all of x from cache, so many rows want wide workgroups (64 channels),
+    // but only when N still yields enough of them to fill the chip.  Measured (us, weights from
+    // HBM): N=11008 K=4096: 4 rows 9.6 (16 ch, 8 waves); 8 rows 10.9 (64 ch) vs 11.3 (16 ch);
+    // 16 rows 11.8 (64 ch) vs 16.7 (16 ch).  N=4096 K=4096: 8 rows 5.7 (16 ch) vs 9.9 (64 ch).
+    int nb = (rows > 4 && N >= 8192) ? 4 : 1;
     if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
+    int waves = nb == 1 && rows <= 8 ? 8 : 4;
+    if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
     const auto* sp = static_cast<const uint32_t*>(sz);
     auto* yp = static_cast<uint16_t*>(y);
     const int shift = group == 128 ? 0 : 1;  // a group is 128 << shift k (128 or 256)
-    int waves = nb == 1 ? 8 : 4;
-    if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
 #define TPQ_MFMA(NBV, WV) \
     int4_mfma_kernel<DT, NBV, WV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>(xp, pp, sp, yp, rows, N, K, shift)
-    if (waves == 8) {
+    if (waves == 16 && nb == 1) {
+        TPQ_MFMA(1, 16);
+    } else if (waves == 8) {
         if (nb == 1) TPQ_MFMA(1, 8); else TPQ_MFMA(2, 8);
     } else {
         if (nb == 1) TPQ_MFMA(1, 4); else if (nb == 2) TPQ_MFMA(2, 4); else TPQ_MFMA(4, 4);

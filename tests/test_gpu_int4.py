@@ -66,6 +66,8 @@ def test_pack_errors(ops):
 CASES = [  # M, N, K, group
     (1, 64, 256, 128), (1, 72, 128, 128), (4, 40, 128, 32), (16, 128, 512, 64), (3, 200, 384, 128),
     (2, 64, 4096, 128), (5, 24, 96, 32), (1, 16, 70, 32), (7, 136, 1024, 64),
+    # matrix-core decode kernel: 5..16 rows (64-channel workgroups, partial last one), slabs of 16 plus a last row
+    (16, 72, 256, 128), (9, 136, 1024, 128), (17, 64, 256, 128), (33, 40, 384, 128), (8, 200, 2048, 128),
 ]
 
 
