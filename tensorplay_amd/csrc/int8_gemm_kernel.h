@@ -85,7 +85,10 @@ __device__ __forceinline__ uint4 ternary_word_to_i8x16(uint32_t w) {
 }
 
 // TERNARY_W: W is the 2-bit packed matrix [N, K/4]; a 16-code chunk is one 32-bit word.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool TERNARY_W, class Epilogue>
+// DEPTH: k-stages held in registers ahead of the one being multiplied.  With small tiles a stage
+// is little arithmetic, and one stage of lookahead leaves the global-load latency exposed in
+// every iteration.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool TERNARY_W, class Epilogue, int DEPTH = 1>
 __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void int8_gemm_nk_kernel(
     const int8_t* __restrict__ A, const int8_t* __restrict__ W, int M, int N, int K, Epilogue ep) {
     constexpr int kThreads = WAVES_M * WAVES_N * kWave;
@@ -129,17 +132,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void int8_gemm_nk_kernel(
         r = r < N ? r : N - 1;
         b_src[i] = reinterpret_cast<const BChunk*>(W + static_cast<size_t>(r) * (TERNARY_W ? K / 4 : K)) + ld_chunk;
     }
-    uint4 ra[kLoadsA];
-    BChunk rb[kLoadsB];
-    auto fetch = [&](int stage) {
+    uint4 ra_ring[DEPTH][kLoadsA];
+    BChunk rb_ring[DEPTH][kLoadsB];
+    auto fetch = [&](int stage, uint4 (&ra)[kLoadsA], BChunk (&rb)[kLoadsB]) {
         const int kc = stage * kChunksPerRow + ld_chunk;
-        const bool in = kc < k_chunks;
+        const bool in = kc < k_chunks;  // also false for stages past the end
 #pragma unroll
         for (int i = 0; i < kLoadsA; ++i) ra[i] = in ? a_src[i][stage * kChunksPerRow] : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < kLoadsB; ++i) rb[i] = in ? b_src[i][stage * kChunksPerRow] : BChunk{};
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, const uint4 (&ra)[kLoadsA], const BChunk (&rb)[kLoadsB]) {
 #pragma unroll
         for (int i = 0; i < kLoadsA; ++i) {
             const int r = ld_row + i * (kThreads / 4);
@@ -163,14 +166,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void int8_gemm_nk_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-    fetch(0);
-    stash(0);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) fetch(d, ra_ring[d], rb_ring[d]);
+    stash(0, ra_ring[0], rb_ring[0]);
+    fetch(DEPTH, ra_ring[0], rb_ring[0]);
     __syncthreads();
 
+    // stage t waits in ring slot t % DEPTH
     const int frag_row = lane & 31, frag_half = lane >> 5;
-    for (int s = 0; s < stages; ++s) {
+    for (int s0 = 0; s0 < stages; s0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int s = s0 + d;
+        if (s >= stages) break;
         const int buf = s & 1;
-        if (s + 1 < stages) fetch(s + 1);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int chunk = ks * 2 + frag_half;
@@ -192,9 +201,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N* kWave) void int8_gemm_nk_kernel(
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
         if (s + 1 < stages) {
-            stash(buf ^ 1);
+            stash(buf ^ 1, ra_ring[(d + 1) % DEPTH], rb_ring[(d + 1) % DEPTH]);
+            fetch(s + 1 + DEPTH, ra_ring[(d + 1) % DEPTH], rb_ring[(d + 1) % DEPTH]);
             __syncthreads();
         }
+      }
     }
 
     // C fragment of a 32x32 block: lane holds column lane%32, rows 8*(v/4) + 4*(lane/32) + v%4
@@ -227,12 +238,17 @@ int launch_mfma(const int8_t* a, const void* w, int64_t M, int64_t N, int64_t K,
         TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
         int8_gemm_nk_kernel<BM, BN, 2, 2, TERNARY_W, Epilogue>
             <<<dim3(static_cast<unsigned>(tiles)), 256, 0, s>>>(a, wp, m, n, k, ep);
-    } else {  // short activations: narrower tiles, more of them
+    } else if (((M + 127) / 128) * ((N + 63) / 64) >= 512) {  // short activations: narrower tiles, more of them
         constexpr int BM = 128, BN = 64;
         const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
         TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
-        int8_gemm_nk_kernel<BM, BN, 4, 1, TERNARY_W, Epilogue>
+        int8_gemm_nk_kernel<BM, BN, 4, 1, TERNARY_W, Epilogue, 2>
             <<<dim3(static_cast<unsigned>(tiles)), 256, 0, s>>>(a, wp, m, n, k, ep);
+    } else {  // too few of those to fill the chip: 64 x 32 tiles, two wavefronts each
+        constexpr int BM = 64, BN = 32;
+        const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+        int8_gemm_nk_kernel<BM, BN, 2, 1, TERNARY_W, Epilogue, 4>
+            <<<dim3(static_cast<unsigned>(tiles)), 128, 0, s>>>(a, wp, m, n, k, ep);
     }
     return check_launch("int8 mfma gemm");
 }

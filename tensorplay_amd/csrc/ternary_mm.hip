@@ -21,6 +21,7 @@
 //
 // Anything else: one thread per output.
 #include "int8_gemm_kernel.h"
+#include "ternary_gemm_kernel.h"
 
 namespace tpq {
 namespace {
@@ -128,6 +129,8 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
         }
         return check_launch("tpq_ternary_mm (decode)");
     }
+    if (sizes_ok && M <= 256 && ternary_gemm_m128_ok(M, K) && aligned(x, 16) && aligned(packed, 4))
+        return launch_ternary_gemm_m128(x, packed, M, N, K, ep, s);
     if (sizes_ok && K % 16 == 0 && aligned(x, 16) && aligned(packed, 4))
         return launch_mfma<true>(x, packed, M, N, K, ep, s);
     const int64_t blocks = (M * N + 255) / 256;

@@ -44,7 +44,8 @@ def test_unpack_every_byte_value(ops):
 
 # (M, K, N): decode kernel, matrix-core kernel, generic kernel
 CASES = [(1, 2560, 6912), (1, 6912, 2560), (4, 2560, 256), (8, 128, 67), (5, 64, 9), (128, 2560, 6912),
-         (128, 6912, 2560), (16, 256, 100), (33, 48, 70), (3, 9, 5), (2, 10, 4), (9, 2560, 130)]
+         (128, 6912, 2560), (16, 256, 100), (33, 48, 70), (3, 9, 5), (2, 10, 4), (9, 2560, 130),
+         (200, 512, 70), (97, 256, 33), (300, 256, 64)]
 
 
 @pytest.mark.parametrize("M,K,N", CASES)
