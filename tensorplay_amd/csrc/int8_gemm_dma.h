@@ -78,6 +78,8 @@ struct TileInt32 {
     const float* cs;
     const float* bias;
     static __device__ __forceinline__ int32_t convert(int acc, float, float, float, bool) { return acc; }
+    static __device__ __forceinline__ float value(int, float, float, float, bool) { return 0.0f; }
+    static __device__ __forceinline__ uint32_t pack2(float, float) { return 0; }
 };
 
 template <int DT>
@@ -88,10 +90,25 @@ struct TileDequant {
     const float* rs;
     const float* cs;
     const float* bias;
-    static __device__ __forceinline__ out_t convert(int acc, float r, float c, float b, bool has_bias) {
+    static __device__ __forceinline__ float value(int acc, float r, float c, float b, bool has_bias) {
         float f = __fmul_rn(__fmul_rn(static_cast<float>(acc), r), c);
         if (has_bias) f = __fadd_rn(f, b);
-        return Elem<DT>::store(f);
+        return f;
+    }
+    static __device__ __forceinline__ out_t convert(int acc, float r, float c, float b, bool has_bias) {
+        return Elem<DT>::store(value(acc, r, c, b, has_bias));
+    }
+    // two results rounded to nearest even and packed, with the hardware's packed conversion
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        typedef float f2_t __attribute__((ext_vector_type(2)));
+        const f2_t v = {lo, hi};
+        if constexpr (DT == TPQ_DTYPE_BF16) {
+            typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+            return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2_t));
+        } else {
+            typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+            return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2_t));
+        }
     }
 };
 
@@ -369,14 +386,16 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
                     const int m_local = wm * WM + (KEEP + i) * 32 + frag_row;
-                    out_t vals[4];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) vals[t] = Tile::convert(acc[KEEP + i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
                     char* dst = lds_bytes + m_local * kPitch + n_local * sizeof(out_t);
                     if constexpr (sizeof(out_t) == 2) {
-                        *reinterpret_cast<uint2*>(dst) = make_uint2(vals[0] | (static_cast<uint32_t>(vals[1]) << 16),
-                                                                    vals[2] | (static_cast<uint32_t>(vals[3]) << 16));
+                        float f[4];
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) f[t] = Tile::value(acc[KEEP + i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(Tile::pack2(f[0], f[1]), Tile::pack2(f[2], f[3]));
                     } else {
+                        out_t vals[4];
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) vals[t] = Tile::convert(acc[KEEP + i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
                         *reinterpret_cast<uint4*>(dst) = make_uint4(__builtin_bit_cast(uint32_t, vals[0]), __builtin_bit_cast(uint32_t, vals[1]),
                                                                     __builtin_bit_cast(uint32_t, vals[2]), __builtin_bit_cast(uint32_t, vals[3]));
                     }
