@@ -319,6 +319,24 @@ def main() -> int:
             extras[f"int4_gemv_M{mb}_GBs"] = bytes_b / (ms * 1e-3) / 1e9
         del packs[1:], szs[1:]
         torch.cuda.empty_cache()
+        # int8 weight-only decode (next-row op _weight_int8pack_mm): same shape, one byte per weight
+        w8s = [torch.randint(-128, 128, (N, K), dtype=torch.int8, device=dev) for _ in range(14)]  # 631 MB
+        s8 = torch.rand(N, device=dev) * 0.01
+        for mb in (1, 8):
+            xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
+            yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
+
+            def i8mm(i, xb=xb, yb=yb, mb=mb):
+                lib.tpq_weight_int8pack_mm(xb.data_ptr(), _lib.F16, mb, K, w8s[i % 14].data_ptr(), s8.data_ptr(), N,
+                                           yb.data_ptr(), cur())
+
+            g8 = graph_of(lambda: [i8mm(i) for i in range(140)])
+            g8.replay(); sync()
+            ms = time_region(g8.replay, sync, 1) / 140
+            extras[f"int8pack_M{mb}_us"] = ms * 1e3
+            extras[f"int8pack_M{mb}_GBs"] = (N * K + 4 * N + 2 * mb * K + 2 * mb * N) / (ms * 1e-3) / 1e9
+        del w8s
+        torch.cuda.empty_cache()
 
     if not args.no_extras and not args.gemv_only:
         # int8 prefill GEMM with fused dequant: M=2048, K=4096, N=4096, bf16 in/out

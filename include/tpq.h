@@ -150,6 +150,15 @@ int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packe
                    const float* bias, int64_t M, int64_t N, int64_t K, void* out, int out_dtype,
                    int32_t* acc_out, void* stream);
 
+/*
+ * int8 weight-only matmul: out[m,n] = cast((sum_k float(x[m,k]) * w[n,k]) * scales[n]), fp32
+ * accumulation, out dtype = x dtype.  x [M,K] f32/f16/bf16; w int8 [N,K] row-major; scales f32 [N].
+ * Replaces _weight_int8pack_mm: config/native_functions.yaml:8005,
+ * p10/src/backend/cuda/QuantGemmKernels.cu:86-180, 339-405.
+ */
+int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64_t K, const int8_t* w,
+                           const float* scales, int64_t N, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -298,3 +298,16 @@ def ternary_mm(x_i8, row_scale, packed, w_scale, K, bias=None, out_dtype="f32"):
                          ctypes.c_int64(M), ctypes.c_int64(N), ctypes.c_int64(K), _p(out),
                          _DT[out_dtype], _p(acc))
     return out, acc
+
+
+def weight_int8pack_mm(x, dtype, w, scales, want_f64=False):
+    x = _c(x, storage(dtype))
+    w = _c(w, np.int8)
+    scales = _c(scales, np.float32)
+    M, K = x.shape
+    N = w.shape[0]
+    out = np.zeros((M, N), storage(dtype))
+    y64 = np.zeros((M, N), np.float64) if want_f64 else None
+    lib().orc_weight_int8pack_mm(_p(x), _DT[dtype], _p(w), _p(scales), ctypes.c_int64(M), ctypes.c_int64(N),
+                                 ctypes.c_int64(K), _p(out), _p(y64))
+    return (out, y64) if want_f64 else out

@@ -662,3 +662,27 @@ ORC_API void orc_ternary_mm(const int8_t* x, const float* row_scale, const uint8
         }
     free(codes);
 }
+
+/* ---- _weight_int8pack_mm ------------------------------------------------------------------------
+ * out[m,n] = cast((sum_k float(x[m,k]) * float(w[n,k])) * scale[n]); x is converted to fp32 first and
+ * the sum is an fp32 fma chain (p10/src/backend/cuda/QuantGemmKernels.cu:86-130, 339-405; the device
+ * kernel strides k over lanes, so its summation order differs - tolerance, not bit parity).
+ * y64 (optional) receives the same sums evaluated in double precision.
+ * Pinned by: the literal 2x4 / 3x4 example and closed form (x @ w.T) * s of
+ * test/test_mps.py:1052-1061, and the float64 product.
+ */
+ORC_API void orc_weight_int8pack_mm(const void* x, int dtype, const int8_t* w, const float* scale,
+                                    int64_t M, int64_t N, int64_t K, void* out, double* y64) {
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            float acc = 0.0f;
+            double acc64 = 0.0;
+            for (int64_t k = 0; k < K; ++k) {
+                const float xv = load_as_f32(x, dtype, m * K + k);
+                acc = fmaf((float)w[n * K + k], xv, acc);
+                acc64 += (double)w[n * K + k] * (double)xv;
+            }
+            store_from_f32(out, dtype, m * N + n, acc * scale[n]);
+            if (y64) y64[m * N + n] = acc64 * (double)scale[n];
+        }
+}

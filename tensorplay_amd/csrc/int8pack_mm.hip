@@ -1,0 +1,179 @@
+// int8 weight-only matmul: out[m,n] = (sum_k x[m,k] * w[n,k]) * scale[n], out dtype = x dtype
+// (reference: _weight_int8pack_mm, p10/src/backend/cuda/QuantGemmKernels.cu:86-180, 339-405:
+// activations converted to fp32, fp32 accumulation, per-row scale applied to the sum).
+//
+// Decode kernel (fp16 activations, K % 128 == 0, 1..16 rows per launch), bandwidth bound at one byte
+// per weight: v_mfma_f32_16x16x16_f16 with the weights as A and the activations as B, as in the int4
+// decode kernel for several rows.  Lane (i, q) owns weight row n0 + i and, in a step of 128 k, the 32
+// bytes at k = 128 s + 32 q: two 16-byte loads, whole 128-byte lines per row and step.  Every dword
+// (four int8) becomes two fp16 pairs: xor 0x80808080 turns the bytes into b + 128, v_perm_b32 drops
+// each next to the exponent byte 0x64 (fp16 1024 + 128 + b), and one packed fp16 subtract of 1152
+// leaves b exactly.  The products are exact and accumulate in fp32 over the whole K range, two
+// accumulators taking turns; the per-row scale multiplies the final sum.
+//
+// Everything else (bf16 / fp32 activations, other K, unaligned pointers) takes a plain kernel: one
+// workgroup per output channel and slab of up to 8 rows, fp32 fma over k, block reduction.
+#include "int4_lane.h"
+
+namespace tpq {
+namespace {
+
+constexpr int kI8Waves = 8;
+
+__device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
+
+// x: [M][K] fp16; w: [N][K] int8; scale: [N] fp32; steps = K / 128
+__global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
+    const uint16_t* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
+    uint16_t* __restrict__ y, int M, int N, int K) {
+    __shared__ float red[kI8Waves][4][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, q = lane >> 4;
+    const int steps = K / 128;
+    const int n0 = blockIdx.x * 16;
+    const int n_row = n0 + i < N ? n0 + i : N - 1;  // rows past N: a valid row, result dropped
+    const uint4* w_base = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n_row) * K) + q * 2;
+    // columns m >= M repeat the last row: their products are computed and never stored
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(i < M ? i : M - 1) * K) + q * 4;
+
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+    uint32_t magic;  // exponent bytes, kept in a VGPR behind an opaque move
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(0x64646464u));
+
+    struct Step {
+        uint4 w[2];
+        uint4 xv[4];
+    };
+    auto load = [&](int s, Step& st) {
+        st.w[0] = w_base[s * 8];
+        st.w[1] = w_base[s * 8 + 1];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
+    };
+    float4_t d0 = {0.0f, 0.0f, 0.0f, 0.0f}, d1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto compute = [&](const Step& st) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {  // MFMA u: k = 4u .. 4u+3 of the lane's 32
+            const uint32_t t = dword_at(st.w[u >> 2], u & 3) ^ 0x80808080u;
+            const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
+            const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
+            const uint32_t a0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
+            const uint32_t a1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
+            const uint32_t b0 = dword_at(st.xv[u >> 1], (2 * u) & 3), b1 = dword_at(st.xv[u >> 1], (2 * u + 1) & 3);
+            const word2_t a = {a0, a1}, b = {b0, b1};
+            if (u & 1) d1 = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), d1, 0, 0, 0);
+            else d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), d0, 0, 0, 0);
+        }
+    };
+
+    Step s0, s1;
+    int s = wave;
+    if (s < steps) load(s, s0);
+    if (s + kI8Waves < steps) load(s + kI8Waves, s1);
+    for (; s + 3 * kI8Waves < steps; s += 2 * kI8Waves) {
+        compute(s0);
+        load(s + 2 * kI8Waves, s0);
+        compute(s1);
+        load(s + 3 * kI8Waves, s1);
+    }
+    if (s < steps) {
+        compute(s0);
+        if (s + 2 * kI8Waves < steps) load(s + 2 * kI8Waves, s0);
+        if (s + kI8Waves < steps) compute(s1);
+        if (s + 2 * kI8Waves < steps) compute(s0);
+    }
+
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][v][lane] = d0[v] + d1[v];
+    __syncthreads();
+    if (wave == 0) {  // lane (m, q): channels n0 + 4 q + v
+        const int n = n0 + 4 * q;
+        float sum[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            sum[v] = 0.0f;
+#pragma unroll
+            for (int ww = 0; ww < kI8Waves; ++ww) sum[v] += red[ww][v][lane];
+        }
+        if (i < M) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = f32_to_f16_bits(__fmul_rn(sum[v], scale[n + v]));
+        }
+    }
+}
+
+// One workgroup per output channel n and slab of up to 8 activation rows.
+template <int DT>
+__global__ __launch_bounds__(256) void int8pack_generic_kernel(
+    const typename Elem<DT>::storage* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
+    typename Elem<DT>::storage* __restrict__ y, int64_t M, int64_t N, int64_t K) {
+    __shared__ float red[8][256 / kWave];
+    const int64_t n = blockIdx.x, m0 = static_cast<int64_t>(blockIdx.y) * 8;
+    const int rows = static_cast<int>(M - m0 < 8 ? M - m0 : 8);
+    const int8_t* wr = w + n * K;
+    float acc[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) acc[b] = 0.0f;
+    for (int64_t k = threadIdx.x; k < K; k += 256) {
+        const float wv = static_cast<float>(wr[k]);
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+            if (b < rows) acc[b] = __builtin_fmaf(wv, Elem<DT>::load(x[(m0 + b) * K + k]), acc[b]);
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        float v = acc[b];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+        if (lane == 0) red[b][wave] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < rows) {
+        const int b = threadIdx.x;
+        const float total = (red[b][0] + red[b][1]) + (red[b][2] + red[b][3]);
+        y[(m0 + b) * N + n] = Elem<DT>::store(__fmul_rn(total, scale[n]));
+    }
+}
+
+template <int DT>
+int launch_generic(const void* x, const int8_t* w, const float* scale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+    using S = typename Elem<DT>::storage;
+    const int64_t slabs = (M + 7) / 8;
+    TPQ_REQUIRE(N <= 0x7FFFFFFF && slabs <= 65535, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): shape too large");
+    int8pack_generic_kernel<DT><<<dim3(static_cast<unsigned>(N), static_cast<unsigned>(slabs)), 256, 0, s>>>(
+        static_cast<const S*>(x), w, scale, static_cast<S*>(y), M, N, K);
+    return check_launch("_weight_int8pack_mm (generic)");
+}
+
+}  // namespace
+}  // namespace tpq
+
+using namespace tpq;
+
+TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64_t K, const int8_t* w,
+                                      const float* scales, int64_t N, void* out, void* stream) {
+    TPQ_REQUIRE(dtype == TPQ_DTYPE_F32 || dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16, TPQ_ERR_INVALID_TYPE,
+                "_weight_int8pack_mm(): activations must be floating point");
+    TPQ_REQUIRE(M >= 0 && N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): negative shape");
+    if (M == 0 || N == 0 || K == 0) return TPQ_OK;  // the reference returns an uninitialised [B, N] here
+    TPQ_REQUIRE(x && w && scales && out, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == TPQ_DTYPE_F16 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+            const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+            int8pack_mfma_kernel<<<dim3(static_cast<unsigned>((N + 15) / 16)), kI8Waves * kWave, 0, s>>>(
+                static_cast<const uint16_t*>(x) + m0 * K, w, scales, static_cast<uint16_t*>(out) + m0 * N, rows,
+                static_cast<int>(N), static_cast<int>(K));
+        }
+        return check_launch("_weight_int8pack_mm (mfma)");
+    }
+    switch (dtype) {
+        case TPQ_DTYPE_F32: return launch_generic<TPQ_DTYPE_F32>(x, w, scales, out, M, N, K, s);
+        case TPQ_DTYPE_F16: return launch_generic<TPQ_DTYPE_F16>(x, w, scales, out, M, N, K, s);
+        default: return launch_generic<TPQ_DTYPE_BF16>(x, w, scales, out, M, N, K, s);
+    }
+}

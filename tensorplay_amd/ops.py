@@ -302,3 +302,29 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
             _check(_lib.load().tpq_ternary_mm(_ptr(x), _ptr(rs), _ptr(p), float(w_scale), _ptr(b), M, N, K,
                                               _ptr(out), _DT[out_dtype], _ptr(acc), _stream(x)))
     return (out, acc) if return_acc else out
+
+
+def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """``(self @ mat2.T) * scales``: activations [B,K] float, int8 weight [N,K], per-row scales [N];
+    fp32 accumulation, result in the activation dtype (reference: QuantGemmKernels.cu:345-405)."""
+    if mat2.dtype != torch.int8:
+        raise TypeError("_weight_int8pack_mm(): weight must be QInt8")
+    if self.dim() != 2 or mat2.dim() != 2 or scales.dim() != 1:
+        raise ValueError("_weight_int8pack_mm(): expected 2-D activations [B,K], 2-D weight [N,K] and 1-D scales [N]")
+    if self.dtype not in _DT:
+        raise TypeError("_weight_int8pack_mm(): activations must be floating point")
+    B, K = self.shape
+    N = mat2.size(0)
+    if mat2.size(1) != K:
+        raise ValueError("_weight_int8pack_mm(): K dimension mismatch")
+    if scales.size(0) != N:
+        raise ValueError("_weight_int8pack_mm(): scales length mismatch")
+    _require_device(self, "_weight_int8pack_mm")
+    out = torch.empty((B, N), dtype=self.dtype, device=self.device)
+    if B == 0 or N == 0 or K == 0:
+        return out
+    x, w = self.contiguous(), mat2.contiguous()
+    sc = scales.to(torch.float32).contiguous()
+    with torch.cuda.device(x.device):
+        _check(_lib.load().tpq_weight_int8pack_mm(_ptr(x), _DT[x.dtype], B, K, _ptr(w), _ptr(sc), N, _ptr(out), _stream(x)))
+    return out
