@@ -34,6 +34,27 @@ __device__ __forceinline__ int quantize_one(float v, float scale, const QParams&
     return static_cast<int>(q);
 }
 
+// Eight codes with one reciprocal instead of eight divisions, same bits as quantize_one.
+// q = v * (1/scale) is within 2^-21 relative of the true quotient, |quotient| <= 128 here, so its
+// absolute error is below 2^-14.  If q lies at least 2^-13 inside (c - 1/2, c + 1/2), so does the
+// correctly rounded quotient, and both round to c.  Otherwise (about one element in a few thousand;
+// also NaN and infinities) the element is redone with the IEEE division.
+__device__ __forceinline__ void quantize_eight(const float (&v)[kVec], float scale, float inv_scale, const QParams& p,
+                                               int (&code)[kVec]) {
+    bool redo = false;
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+        const float q = v[i] * inv_scale;
+        const float c = rintf(q);
+        redo |= !(fabsf(q - c) <= 0.5f - 0x1p-13f);
+        code[i] = static_cast<int>(fminf(fmaxf(c, static_cast<float>(p.qmin)), static_cast<float>(p.qmax)));
+    }
+    if (redo) {
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) code[i] = quantize_one(v[i], scale, p);
+    }
+}
+
 // Block-wide max over 256 threads; every thread gets the result.
 __device__ __forceinline__ float block_max(float v, float* smem) {
     v = wave_max(v);
@@ -88,16 +109,27 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_cached(
     absmax = block_max(absmax, smem);
     const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
     if (threadIdx.x == 0) scales[row] = scale;
+    // the shortcut needs |quotient| <= 128 and a finite reciprocal: true for every scale the formula
+    // above produces from finite inputs with divisor <= 128; anything else takes the divisions
+    const float inv_scale = __fdiv_rn(1.0f, scale);
+    const bool shortcut = !p.sign_mode && p.divisor <= 128.0f && inv_scale < 3.0e38f && absmax <= 3.0e38f;
 
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * kThreads + threadIdx.x) * kVec;
         if (k0 < K) {
+            int code[kVec];
+            if (shortcut) {
+                quantize_eight(v[c], scale, inv_scale, p, code);
+            } else {
+#pragma unroll
+                for (int i = 0; i < kVec; ++i) code[i] = quantize_one(v[c][i], scale, p);
+            }
             uint32_t lo = 0, hi = 0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                lo |= (static_cast<uint32_t>(quantize_one(v[c][i], scale, p)) & 0xFFu) << (8 * i);
-                hi |= (static_cast<uint32_t>(quantize_one(v[c][i + 4], scale, p)) & 0xFFu) << (8 * i);
+                lo |= (static_cast<uint32_t>(code[i]) & 0xFFu) << (8 * i);
+                hi |= (static_cast<uint32_t>(code[i + 4]) & 0xFFu) << (8 * i);
             }
             *reinterpret_cast<uint2*>(cr + k0) = make_uint2(lo, hi);
         }
