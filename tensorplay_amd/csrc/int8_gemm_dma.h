@@ -115,19 +115,21 @@ struct TileDequant {
 constexpr int kDmaRowBytes = 128;  // bytes of k per stage: one cache line per row
 constexpr int kDmaStages = 3;
 
-template <class Tile>
-__global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
+// KSPLIT = 2: eight wavefronts as described above.  KSPLIT = 1: four wavefronts, each multiplying
+// all four substeps of a stage (no k-half exchange in the epilogue, one wavefront per SIMD).
+template <class Tile, int KSPLIT>
+__global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
                                                             const int8_t* __restrict__ W, int M, int N,
                                                             int K, Tile tile, int vector_stores) {
     using out_t = typename Tile::out_t;
     constexpr int BM = 256, BN = 128, WM = 128, WN = 64, TM = 4, TN = 2;
     constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;    // 48 KB
-    constexpr int kThreads = 512, kWaves = 8;
-    constexpr int kLoads = kStageBytes / 1024 / kWaves;      // wave-level loads per stage and wavefront: 6
+    constexpr int kThreads = 256 * KSPLIT, kWaves = 4 * KSPLIT;
+    constexpr int kLoads = kStageBytes / 1024 / kWaves;      // wave-level loads per stage and wavefront: 6 or 12
     constexpr int kPerChunk = 16 / sizeof(out_t);            // outputs per 16 bytes
     constexpr int kPitch = BN * sizeof(out_t) + 16;          // bytes per row of the output image
     constexpr int kRingBytes = kDmaStages * kStageBytes;     // 144 KB, covers the image and the exchange area
-    static_assert(BM * kPitch <= kRingBytes && kWaves * 16 * kWave * 16 <= kRingBytes, "epilogue areas live in the ring");
+    static_assert(BM * kPitch <= kRingBytes && 8 * 16 * kWave * 16 <= kRingBytes, "epilogue areas live in the ring");
     extern __shared__ uint4 ring[];                          // [stage][row][128 B], later exchange area and image
     char* lds_bytes = reinterpret_cast<char*>(ring);
     float* cs_lds = reinterpret_cast<float*>(lds_bytes + kRingBytes);  // [BN] column scales, [BN] bias
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kh = wave >> 2;               // k-half: substeps 2*kh and 2*kh+1 of every stage
+    const int kh = KSPLIT == 2 ? wave >> 2 : 0;  // k-half: substeps 2*kh and 2*kh+1 of every stage
     const int wm = (wave >> 1) & 1, wn = wave & 1;
 
     // Workgroups are dealt to the 8 XCDs round-robin (workgroup id mod 8), each with its own L2:
@@ -194,6 +196,11 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
         issue_pair(std::integral_constant<int, 0>{}, kt, slot);
         issue_pair(std::integral_constant<int, 2>{}, kt, slot);
         issue_pair(std::integral_constant<int, 4>{}, kt, slot);
+        if constexpr (kLoads == 12) {
+            issue_pair(std::integral_constant<int, 6>{}, kt, slot);
+            issue_pair(std::integral_constant<int, 8>{}, kt, slot);
+            issue_pair(std::integral_constant<int, 10>{}, kt, slot);
+        }
     };
 
     v16i acc[TM][TN];
@@ -212,6 +219,7 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
     const uint32_t ring_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)ring));
     const uint32_t sw16 = ((frag_row >> 1) & 7) * 16;
     const uint32_t chunk_first = ((kh * 4 + frag_half) * 16) ^ sw16, chunk_second = ((kh * 4 + 2 + frag_half) * 16) ^ sw16;
+    const uint32_t chunk_third = ((4 + frag_half) * 16) ^ sw16, chunk_fourth = ((6 + frag_half) * 16) ^ sw16;  // KSPLIT = 1
     const uint32_t a_row = ring_addr + (wm * WM + frag_row) * kDmaRowBytes;
     const uint32_t b_row = ring_addr + (BM + wn * WN + frag_row) * kDmaRowBytes;
     // the six reads of a substep, in two groups of three: (A0, A1, W0), then (W1, A2, A3)
@@ -269,6 +277,9 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
     constexpr std::integral_constant<int, 2> k2{};
     constexpr std::integral_constant<int, 3> k3{};
     constexpr std::integral_constant<int, 4> k4{};
+    constexpr std::integral_constant<int, 6> k6{};
+    constexpr std::integral_constant<int, 8> k8{};
+    constexpr std::integral_constant<int, 10> k10{};
 
 #pragma unroll
     for (int s = 0; s < kDmaStages; ++s)
@@ -286,6 +297,73 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
     v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
     int kt = 0, slot = 0;  // slot: kt % kDmaStages
     read_frags(0, chunk_first, fa0, fb0);
+    if constexpr (KSPLIT == 1) {
+    for (; kt + kDmaStages < nk; ++kt) {  // steady state: stages kt+1 .. kt+3 all exist
+        const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
+        read_frags(slot, chunk_second, fa1, fb1);
+        frags_ready(kOneBatch, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        multiply(kHigh, fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot, chunk_third, fa0, fb0);
+        frags_ready(kOneBatch, fa1, fb1);
+        multiply(kLow, fa1, fb1);
+        multiply(kHigh, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot, chunk_fourth, fa1, fb1);
+        frags_ready(kOneBatch, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        multiply(kHigh, fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        frags_ready(kNone, fa1, fb1);  // this wavefront is done reading stage kt
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads));
+        asm volatile("s_barrier" ::: "memory");
+        multiply_one(k0, k0, fa1, fb1);
+        read_group(k0, next, chunk_first, fa0, fb0);
+        multiply_one(k0, k1, fa1, fb1);
+        read_group(k1, next, chunk_first, fa0, fb0);
+        multiply_one(k1, k0, fa1, fb1);
+        issue_pair(k0, kt + kDmaStages, slot);
+        multiply_one(k1, k1, fa1, fb1);
+        issue_pair(k2, kt + kDmaStages, slot);
+        multiply_one(k2, k0, fa1, fb1);
+        issue_pair(k4, kt + kDmaStages, slot);
+        multiply_one(k2, k1, fa1, fb1);
+        if constexpr (kLoads == 12) issue_pair(k6, kt + kDmaStages, slot);
+        multiply_one(k3, k0, fa1, fb1);
+        if constexpr (kLoads == 12) issue_pair(k8, kt + kDmaStages, slot);
+        multiply_one(k3, k1, fa1, fb1);
+        if constexpr (kLoads == 12) issue_pair(k10, kt + kDmaStages, slot);
+        slot = next;
+    }
+    for (; kt < nk; ++kt) {  // last stages: nothing left to issue
+        const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
+        read_frags(slot, chunk_second, fa1, fb1);
+        frags_ready(kOneBatch, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        multiply(kHigh, fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot, chunk_third, fa0, fb0);
+        frags_ready(kOneBatch, fa1, fb1);
+        multiply(kLow, fa1, fb1);
+        multiply(kHigh, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot, chunk_fourth, fa1, fb1);
+        frags_ready(kOneBatch, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        multiply(kHigh, fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        frags_ready(kNone, fa1, fb1);
+        if (kt + 1 < nk) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            asm volatile("s_barrier" ::: "memory");
+            read_frags(next, chunk_first, fa0, fb0);
+        }
+        multiply(kLow, fa1, fb1);
+        multiply(kHigh, fa1, fb1);
+        slot = next;
+    }
+    } else {
     for (; kt + kDmaStages < nk; ++kt) {  // steady state: stages kt+1 .. kt+3 all exist
         const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
         read_frags(slot, chunk_second, fa1, fb1);
@@ -329,6 +407,8 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
         multiply(kLow, fa1, fb1);
         multiply(kHigh, fa1, fb1);
         slot = next;
+    }
+
     }
 
     // ---- epilogue ------------------------------------------------------------------------------------
@@ -402,11 +482,16 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
                 }
             }
     };
-    if (kh == 0) hand_over(kHigh); else hand_over(kLow);
-    __syncthreads();
-    if (kh == 0) take_over(kLow); else take_over(kHigh);
-    __syncthreads();  // exchange area consumed before the image overwrites it
-    if (kh == 0) to_image(kLow); else to_image(kHigh);
+    if constexpr (KSPLIT == 2) {
+        if (kh == 0) hand_over(kHigh); else hand_over(kLow);
+        __syncthreads();
+        if (kh == 0) take_over(kLow); else take_over(kHigh);
+        __syncthreads();  // exchange area consumed before the image overwrites it
+        if (kh == 0) to_image(kLow); else to_image(kHigh);
+    } else {
+        to_image(kLow);
+        to_image(kHigh);
+    }
     __syncthreads();
     constexpr int kChunksPerOutRow = BN / kPerChunk;  // 16-byte chunks per image row
     for (int c = tid; c < BM * kChunksPerOutRow; c += kThreads) {
@@ -426,12 +511,12 @@ __global__ __launch_bounds__(512) void int8_gemm_dma_kernel(const int8_t* __rest
 // K must be a multiple of the 128-byte stage.
 inline bool dma_path_ok(int64_t M, int64_t K) { return M > 128 && K % kDmaRowBytes == 0; }
 
-template <class Tile>
-int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+template <int KSPLIT, class Tile>
+int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
     constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + 2 * 128 * sizeof(float);
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
-    auto kernel = int8_gemm_dma_kernel<Tile>;
+    auto kernel = int8_gemm_dma_kernel<Tile, KSPLIT>;
     static bool configured = false;  // per instantiation: raise the dynamic LDS limit once
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -440,9 +525,17 @@ int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K
         configured = true;
     }
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
-    kernel<<<dim3(static_cast<unsigned>(tiles)), 512, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
+    kernel<<<dim3(static_cast<unsigned>(tiles)), 256 * KSPLIT, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
                                                                  static_cast<int>(K), tile, vector_stores);
     return check_launch("int8 mfma gemm (dma)");
+}
+
+// TPQ_INT8_KSPLIT=1 selects the four-wavefront variant for comparison runs.
+template <class Tile>
+int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+    const char* env = std::getenv("TPQ_INT8_KSPLIT");
+    if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s);
+    return launch_dma_split<2>(a, w, M, N, K, tile, s);
 }
 
 }  // namespace
