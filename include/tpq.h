@@ -151,6 +151,25 @@ int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packe
                    int32_t* acc_out, void* stream);
 
 /*
+ * int4 CPU layout written on the device: uint8 [N, K/2] as produced by the reference's CPU pack
+ * (block_cols = 64 with half_split = 1 is the AVX-512 tier, 32/1 AVX2, 32/0 the plain tier).
+ * Replaces _convert_weight_to_int4pack_for_cpu: config/native_functions.yaml:7997,
+ * p10/src/backend/cpu/QuantizedElementwiseKernels.cpp:19, 370-390.
+ */
+int tpq_int4_pack_cpu_layout(const int32_t* codes, int64_t N, int64_t K, int block_cols,
+                             int half_split, uint8_t* out, void* stream);
+
+/*
+ * CPU layout -> device layout (int32 [N/8][ceil(K/32)][32][1], innerKTiles = 2), so that a weight
+ * packed by a CPU model (buffer `weight` of WeightOnlyInt4Linear,
+ * tensorplay/ao/quantization/int4_weight_only.py:150-154) can be used by tpq_int4_mm.  The reference
+ * has no such converter: its device op rejects the 2-D uint8 layout
+ * (p10/src/backend/cuda/QuantGemmKernels.cu:1216-1254).
+ */
+int tpq_int4_cpu_layout_to_device(const uint8_t* packed_cpu, int64_t N, int64_t K, int block_cols,
+                                  int half_split, int32_t* out, void* stream);
+
+/*
  * int8 weight-only matmul: out[m,n] = cast((sum_k float(x[m,k]) * w[n,k]) * scales[n]), fp32
  * accumulation, out dtype = x dtype.  x [M,K] f32/f16/bf16; w int8 [N,K] row-major; scales f32 [N].
  * Replaces _weight_int8pack_mm: config/native_functions.yaml:8005,

@@ -143,6 +143,73 @@ inline unsigned grid_for(int64_t items, int per_block = 256, unsigned cap = 256u
     return static_cast<unsigned>(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
 }
 
+
+// ---------------------------------------------------------------------------
+// int4 CPU layout (p10/src/backend/cpu/QuantizedElementwiseKernels.cpp:370-390): uint8 [N, K/2];
+// N in blocks of `columns`; inside a block, for each k, width/2 bytes; byte `lane` of a full block
+// on a vector tier pairs column lane (low nibble) with lane + width/2 (high nibble), tail blocks and
+// the plain tier pair 2*lane with 2*lane + 1.
+// ---------------------------------------------------------------------------
+struct CpuLayout {
+    int64_t N, K;
+    int columns, half_split;
+    // where code (col, feature) lives: byte index and shift
+    __device__ __forceinline__ void locate(int64_t col, int64_t feature, int64_t* byte, int* shift) const {
+        const int64_t first = col / columns * columns;
+        const int64_t width = N - first < columns ? N - first : columns;
+        const int64_t c = col - first;
+        const bool full = half_split && width == columns;
+        const int64_t lane = full ? c % (width / 2) : c / 2;
+        *shift = full ? (c >= width / 2 ? 4 : 0) : static_cast<int>(c & 1) * 4;
+        *byte = first * K / 2 + feature * (width / 2) + lane;
+    }
+};
+
+__global__ __launch_bounds__(256) void int4_pack_cpu_bytes(const int32_t* __restrict__ codes, uint8_t* __restrict__ out,
+                                                           CpuLayout lay, int64_t total_bytes) {
+    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total_bytes; idx += gridDim.x * 256ll) {
+        // invert locate(): idx -> (block, feature, lane)
+        const int64_t per_block = static_cast<int64_t>(lay.columns) * lay.K / 2;
+        const int64_t block = idx / per_block, first = block * lay.columns;
+        const int64_t width = lay.N - first < lay.columns ? lay.N - first : lay.columns;
+        const int64_t off = idx - first * lay.K / 2;
+        const int64_t feature = off / (width / 2), lane = off % (width / 2);
+        const bool full = lay.half_split && width == lay.columns;
+        const int64_t lo = full ? lane : 2 * lane, hi = full ? lane + width / 2 : 2 * lane + 1;
+        const uint32_t a = static_cast<uint32_t>(codes[(first + lo) * lay.K + feature]) & 0xFFu;
+        const uint32_t b = static_cast<uint32_t>(codes[(first + hi) * lay.K + feature]) & 0xFFu;
+        out[idx] = static_cast<uint8_t>(a | (b << 4));
+    }
+}
+
+// CPU layout -> device layout (innerKTiles = 2): same word indexing as int4_pack_words.
+__global__ __launch_bounds__(256) void int4_cpu_to_device_words(const uint8_t* __restrict__ packed, int32_t* __restrict__ out,
+                                                                CpuLayout lay, int64_t k_super, int64_t total_words) {
+    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total_words; idx += gridDim.x * 256ll) {
+        const int t = static_cast<int>(idx & 31);
+        const int64_t tile = idx >> 5;
+        const int64_t kT = tile % k_super, nT = tile / k_super;
+        const int64_t n = nT * 8 + (t >> 2);
+        const int64_t k0 = kT * 32 + 2 * (t & 3);
+        uint32_t word = 0;
+        if (n < lay.N) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int odd = 0; odd < 2; ++odd) {
+                    const int64_t k = k0 + 8 * j + odd;
+                    if (k < lay.K) {
+                        int64_t byte;
+                        int shift;
+                        lay.locate(n, k, &byte, &shift);
+                        word |= ((static_cast<uint32_t>(packed[byte]) >> shift) & 15u) << (4 * j + 16 * odd);
+                    }
+                }
+        }
+        out[idx] = static_cast<int32_t>(word);
+    }
+}
+
 }  // namespace
 }  // namespace tpq
 
@@ -209,4 +276,34 @@ TPQ_EXPORT int tpq_ternary_unpack(const uint8_t* packed, int64_t rows, int64_t c
     ternary_unpack_bytes<<<grid_for(rows * bpr), 256, 0, static_cast<hipStream_t>(stream)>>>(
         packed, out, rows, cols, bpr);
     return check_launch("tpq_ternary_unpack");
+}
+
+TPQ_EXPORT int tpq_int4_pack_cpu_layout(const int32_t* codes, int64_t N, int64_t K, int block_cols,
+                                        int half_split, uint8_t* out, void* stream) {
+    TPQ_REQUIRE(N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "_convert_weight_to_int4pack_for_cpu(): negative shape");
+    TPQ_REQUIRE(N % 16 == 0 && K % 2 == 0, TPQ_ERR_INVALID_VALUE,
+                "_convert_weight_to_int4pack_for_cpu(): N must be a multiple of 16 and K even");
+    TPQ_REQUIRE(block_cols == 32 || block_cols == 64, TPQ_ERR_INVALID_VALUE,
+                "_convert_weight_to_int4pack_for_cpu(): block width must be 32 or 64");
+    if (N == 0 || K == 0) return TPQ_OK;
+    TPQ_REQUIRE(codes && out, TPQ_ERR_INVALID_VALUE, "_convert_weight_to_int4pack_for_cpu(): null pointer");
+    const CpuLayout lay{N, K, block_cols, half_split ? 1 : 0};
+    const int64_t total = N * K / 2;
+    int4_pack_cpu_bytes<<<grid_for(total), 256, 0, static_cast<hipStream_t>(stream)>>>(codes, out, lay, total);
+    return check_launch("tpq_int4_pack_cpu_layout");
+}
+
+TPQ_EXPORT int tpq_int4_cpu_layout_to_device(const uint8_t* packed_cpu, int64_t N, int64_t K, int block_cols,
+                                             int half_split, int32_t* out, void* stream) {
+    TPQ_REQUIRE(N >= 0 && K >= 0 && N % 16 == 0 && K % 2 == 0, TPQ_ERR_INVALID_VALUE,
+                "int4 layout conversion: N must be a multiple of 16 and K even");
+    TPQ_REQUIRE(block_cols == 32 || block_cols == 64, TPQ_ERR_INVALID_VALUE,
+                "int4 layout conversion: block width must be 32 or 64");
+    if (N == 0 || K == 0) return TPQ_OK;
+    TPQ_REQUIRE(packed_cpu && out, TPQ_ERR_INVALID_VALUE, "int4 layout conversion: null pointer");
+    const CpuLayout lay{N, K, block_cols, half_split ? 1 : 0};
+    const int64_t k_super = (K + 31) / 32;
+    const int64_t total = (N / 8) * k_super * 32;
+    int4_cpu_to_device_words<<<grid_for(total), 256, 0, static_cast<hipStream_t>(stream)>>>(packed_cpu, out, lay, k_super, total);
+    return check_launch("tpq_int4_cpu_layout_to_device");
 }

@@ -328,3 +328,31 @@ def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Te
     with torch.cuda.device(x.device):
         _check(_lib.load().tpq_weight_int8pack_mm(_ptr(x), _DT[x.dtype], B, K, _ptr(w), _ptr(sc), N, _ptr(out), _stream(x)))
     return out
+
+
+def _convert_weight_to_int4pack_for_cpu(self: torch.Tensor, innerKTiles: int, *, block_cols: int = 64,
+                                        half_split: bool = True) -> torch.Tensor:
+    """int32 codes [N,K] -> the reference's CPU layout, uint8 [N, K/2] (default: the AVX-512 tier, whose bytes
+    equal PyTorch's CPU pack), written by the GPU."""
+    if self.dim() != 2 or self.dtype != torch.int32:
+        raise ValueError("_convert_weight_to_int4pack_for_cpu(): expected 2-D int32 codes")
+    _require_device(self, "_convert_weight_to_int4pack_for_cpu")
+    N, K = self.shape
+    out = torch.empty((N, K // 2), dtype=torch.uint8, device=self.device)
+    codes = self.contiguous()
+    with torch.cuda.device(self.device):
+        _check(_lib.load().tpq_int4_pack_cpu_layout(_ptr(codes), N, K, int(block_cols), int(bool(half_split)), _ptr(out), _stream(self)))
+    return out
+
+
+def int4pack_cpu_to_device(packed_cpu: torch.Tensor, *, block_cols: int = 64, half_split: bool = True) -> torch.Tensor:
+    """CPU-layout packed weight uint8 [N, K/2] -> device layout int32 [N/8, ceil(K/32), 32, 1]."""
+    if packed_cpu.dim() != 2 or packed_cpu.dtype != torch.uint8:
+        raise ValueError("int4pack_cpu_to_device(): expected a 2-D uint8 packed weight")
+    _require_device(packed_cpu, "int4pack_cpu_to_device")
+    N, K = packed_cpu.size(0), packed_cpu.size(1) * 2
+    out = torch.empty((N // 8, (K + 31) // 32, 32, 1), dtype=torch.int32, device=packed_cpu.device)
+    p = packed_cpu.contiguous()
+    with torch.cuda.device(p.device):
+        _check(_lib.load().tpq_int4_cpu_layout_to_device(_ptr(p), N, K, int(block_cols), int(bool(half_split)), _ptr(out), _stream(p)))
+    return out

@@ -130,3 +130,26 @@ def test_mm_errors(ops):
     with pytest.raises(ValueError):
         ops._weight_int4pack_mm(x[:, :32], packed, 32, sz)
     assert ops._weight_int4pack_mm(x[:0], packed, 32, sz).shape == (0, 16)
+
+
+@pytest.mark.parametrize("columns,half_split", [(64, True), (32, True), (32, False)])
+@pytest.mark.parametrize("shape", [(16, 64), (80, 128), (128, 256), (48, 70), (256, 4096)])
+def test_cpu_layout_pack_and_conversion(ops, columns, half_split, shape):
+    """The CPU layout written on the GPU equals the oracle's (itself byte-equal to PyTorch's CPU pack), and
+    converting it to the device layout gives what the device pack writes from the codes."""
+    N, K = shape
+    rng = np.random.default_rng(N * 31 + K)
+    codes = rng.integers(0, 16, size=(N, K), dtype=np.int32)
+    cpu_layout = ops._convert_weight_to_int4pack_for_cpu(dev(codes), 2, block_cols=columns, half_split=half_split)
+    np.testing.assert_array_equal(host(cpu_layout), oracle.int4_pack_cpu(codes, columns, half_split))
+    converted = ops.int4pack_cpu_to_device(cpu_layout, block_cols=columns, half_split=half_split)
+    np.testing.assert_array_equal(host(converted), oracle.int4_pack_tc(codes, 2))
+
+
+def test_cpu_layout_equals_torch_cpu_pack(ops):
+    rng = np.random.default_rng(124)
+    codes = rng.integers(0, 16, size=(64, 256), dtype="int32")
+    want = torch._convert_weight_to_int4pack_for_cpu(torch.tensor(codes), 2).numpy()
+    np.testing.assert_array_equal(host(ops._convert_weight_to_int4pack_for_cpu(dev(codes), 2)), want)
+    with pytest.raises(ValueError):
+        ops._convert_weight_to_int4pack_for_cpu(torch.zeros(8, 32, dtype=torch.int32, device=DEV), 2)
