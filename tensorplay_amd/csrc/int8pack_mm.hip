@@ -18,7 +18,8 @@
 namespace tpq {
 namespace {
 
-constexpr int kI8Waves = 8;
+constexpr int kI8Waves = 2;
+constexpr int kI8Ring = 2;  // steps in flight per wavefront
 
 __device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
 
@@ -68,21 +69,20 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
         }
     };
 
-    Step s0, s1;
-    int s = wave;
-    if (s < steps) load(s, s0);
-    if (s + kI8Waves < steps) load(s + kI8Waves, s1);
-    for (; s + 3 * kI8Waves < steps; s += 2 * kI8Waves) {
-        compute(s0);
-        load(s + 2 * kI8Waves, s0);
-        compute(s1);
-        load(s + 3 * kI8Waves, s1);
-    }
-    if (s < steps) {
-        compute(s0);
-        if (s + 2 * kI8Waves < steps) load(s + 2 * kI8Waves, s0);
-        if (s + kI8Waves < steps) compute(s1);
-        if (s + 2 * kI8Waves < steps) compute(s0);
+    // this wavefront's steps: wave, wave + W, ...; kI8Ring of them in flight
+    Step ring[kI8Ring];
+#pragma unroll
+    for (int r = 0; r < kI8Ring; ++r)
+        if (wave + r * kI8Waves < steps) load(wave + r * kI8Waves, ring[r]);
+    for (int base = wave; base < steps; base += kI8Ring * kI8Waves) {
+#pragma unroll
+        for (int r = 0; r < kI8Ring; ++r) {
+            const int s = base + r * kI8Waves;
+            if (s < steps) {
+                compute(ring[r]);
+                if (s + kI8Ring * kI8Waves < steps) load(s + kI8Ring * kI8Waves, ring[r]);
+            }
+        }
     }
 
 #pragma unroll
