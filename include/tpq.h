@@ -151,6 +151,15 @@ int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packe
                    int32_t* acc_out, void* stream);
 
 /*
+ * Dense weight [N, K] of `dtype` from the packed device layout: W = T(code - 8) * scale + zero, the
+ * product and the sum each rounded to T.  The reference runs this before its library GEMM
+ * (int4_tc_dequantize_kernel, p10/src/backend/cuda/QuantGemmKernels.cu:1170-1202, 1296-1341); the
+ * host op uses it the same way for many activation rows.
+ */
+int tpq_int4_dequantize(const int32_t* packed, int inner_k_tiles, int64_t N, int64_t K, int64_t group,
+                        const void* scales_and_zeros, int dtype, void* out, void* stream);
+
+/*
  * int4 CPU layout written on the device: uint8 [N, K/2] as produced by the reference's CPU pack
  * (block_cols = 64 with half_split = 1 is the AVX-512 tier, 32/1 AVX2, 32/0 the plain tier).
  * Replaces _convert_weight_to_int4pack_for_cpu: config/native_functions.yaml:7997,

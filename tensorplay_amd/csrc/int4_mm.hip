@@ -479,6 +479,49 @@ int launch_generic(const void* x, int64_t M, const int32_t* packed, const void* 
     return check_launch("tpq_int4_mm (generic)");
 }
 
+// Dense [N, K] weight from the packed layout, W = T(code - 8) * scale + zero with the product and the
+// sum each rounded to T (reference: int4_tc_dequantize_kernel, QuantGemmKernels.cu:1170-1202).
+// Thread = (row, k-tile): one 16-byte load, 32 consecutive outputs.
+template <int DT>
+__global__ __launch_bounds__(256) void int4_dequantize_kernel(const uint4* __restrict__ packed,
+                                                              const typename Elem<DT>::storage* __restrict__ sz,
+                                                              typename Elem<DT>::storage* __restrict__ W, int64_t N,
+                                                              int64_t K, int64_t k_super, int64_t group, int64_t total, int vector_stores) {
+    using S = typename Elem<DT>::storage;
+    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += gridDim.x * 256ll) {
+        const int r = static_cast<int>(idx & 7);
+        const int64_t tile = idx >> 3, kT = tile % k_super, nT = tile / k_super;
+        const int64_t n = nT * 8 + r;
+        const uint4 q = packed[idx];
+        const int64_t g = (kT * 32) / group;
+        const float scale = Elem<DT>::load(sz[(g * N + n) * 2]), zero = Elem<DT>::load(sz[(g * N + n) * 2 + 1]);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        __attribute__((aligned(16))) S out[32];
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int odd = 0; odd < 2; ++odd) {
+                    const int code = static_cast<int>((w[t4] >> (4 * j + 16 * odd)) & 15u);
+                    const float prod = Elem<DT>::load(Elem<DT>::store(__fmul_rn(static_cast<float>(code - 8), scale)));
+                    out[2 * t4 + 8 * j + odd] = Elem<DT>::store(__fadd_rn(prod, zero));
+                }
+        S* dst = W + n * K + kT * 32;
+        if (vector_stores && kT * 32 + 32 <= K) {  // 64 or 128 contiguous, 16-byte aligned bytes
+            uint4* dst16 = reinterpret_cast<uint4*>(dst);
+            const uint4* src16 = reinterpret_cast<const uint4*>(out);
+#pragma unroll
+            for (int e = 0; e < static_cast<int>(32 * sizeof(S) / 16); ++e) dst16[e] = src16[e];
+        } else if (kT * 32 + 32 <= K) {
+#pragma unroll
+            for (int e = 0; e < 32; ++e) dst[e] = out[e];
+        } else {
+            for (int e = 0; e < 32 && kT * 32 + e < K; ++e) dst[e] = out[e];
+        }
+    }
+}
+
 }  // namespace
 }  // namespace tpq
 
@@ -530,4 +573,33 @@ TPQ_EXPORT int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const
                            int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
                            void* out, void* stream) {
     return tpq_int4_mm_ws(x, dtype, M, K, packed, inner_k_tiles, N, group, scales_and_zeros, out, nullptr, 0, stream);
+}
+
+TPQ_EXPORT int tpq_int4_dequantize(const int32_t* packed, int inner_k_tiles, int64_t N, int64_t K, int64_t group,
+                                   const void* scales_and_zeros, int dtype, void* out, void* stream) {
+    TPQ_REQUIRE(dtype == TPQ_DTYPE_F32 || dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16, TPQ_ERR_INVALID_TYPE,
+                "int4 dequantize: unsupported dtype");
+    TPQ_REQUIRE(inner_k_tiles == 2, TPQ_ERR_UNSUPPORTED, "int4 dequantize: only innerKTiles = 2 packed weights are supported");
+    TPQ_REQUIRE(group == 32 || group == 64 || group == 128, TPQ_ERR_INVALID_VALUE, "int4 dequantize: qGroupSize must be 32, 64 or 128");
+    TPQ_REQUIRE(N >= 0 && K >= 0 && N % 8 == 0, TPQ_ERR_INVALID_VALUE, "int4 dequantize: bad shape");
+    if (N == 0 || K == 0) return TPQ_OK;
+    TPQ_REQUIRE(packed && scales_and_zeros && out && aligned(packed, 16), TPQ_ERR_INVALID_VALUE, "int4 dequantize: null or unaligned pointer");
+    const int64_t k_super = (K + 31) / 32, total = N * k_super;
+    const int64_t blocks = (total + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(blocks > 65535 * 16 ? 65535 * 16 : blocks);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const auto* pp = reinterpret_cast<const uint4*>(packed);
+    const int vec = aligned(out, 16) && K % 8 == 0;  // every row segment of 32 outputs starts 16-byte aligned
+    switch (dtype) {
+        case TPQ_DTYPE_F32:
+            int4_dequantize_kernel<TPQ_DTYPE_F32><<<grid, 256, 0, s>>>(pp, static_cast<const float*>(scales_and_zeros), static_cast<float*>(out), N, K, k_super, group, total, vec);
+            break;
+        case TPQ_DTYPE_F16:
+            int4_dequantize_kernel<TPQ_DTYPE_F16><<<grid, 256, 0, s>>>(pp, static_cast<const uint16_t*>(scales_and_zeros), static_cast<uint16_t*>(out), N, K, k_super, group, total, vec);
+            break;
+        default:
+            int4_dequantize_kernel<TPQ_DTYPE_BF16><<<grid, 256, 0, s>>>(pp, static_cast<const uint16_t*>(scales_and_zeros), static_cast<uint16_t*>(out), N, K, k_super, group, total, vec);
+            break;
+    }
+    return check_launch("tpq_int4_dequantize");
 }

@@ -211,6 +211,21 @@ def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.T
     return out
 
 
+# Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM.  Measured at
+# K = 4096, N = 11008, fp16: the 16-row slabs cost about 10 us each (41 us at 64 rows), the dense route
+# 72 us at 65 rows and 75 us at 128, so the two meet near 112 rows.
+INT4_PREFILL_ROWS = 112
+
+
+def _int4_dequantize(packed: torch.Tensor, inner: int, n: int, k: int, group: int, sz: torch.Tensor) -> torch.Tensor:
+    """Dense [N, K] weight in sz.dtype: T(code - 8) * scale + zero, product and sum each rounded to T."""
+    dense = torch.empty((n, k), dtype=sz.dtype, device=packed.device)
+    with torch.cuda.device(packed.device):
+        _check(_lib.load().tpq_int4_dequantize(_ptr(packed), inner, n, k, group, _ptr(sz), _DT[sz.dtype], _ptr(dense),
+                                               _stream(packed)))
+    return dense
+
+
 def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
                         qScaleAndZeros: torch.Tensor) -> torch.Tensor:
     """``self @ W.T`` with W dequantised per group: (code - 8) * scale + zero; result in self.dtype."""
@@ -241,6 +256,13 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     x = self.contiguous()
     w = mat2.contiguous()
     sz = qScaleAndZeros.to(self.dtype).contiguous()
+    if m > INT4_PREFILL_ROWS and inner == 2:
+        # Many rows: what the reference does for every shape (QuantGemmKernels.cu:1296-1341) - dequantise
+        # the weight to a dense matrix of the activation dtype, then one plain library GEMM.  The decode
+        # kernels read the packed weight once per 16 rows, which stops paying at this point.
+        dense = _int4_dequantize(w, inner, n, k, qGroupSize, sz)
+        torch.matmul(x, dense.t(), out=out)
+        return out
     with torch.cuda.device(self.device):
         ws = _int4_workspace(self.device, n)
         _check(_lib.load().tpq_int4_mm_ws(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz),

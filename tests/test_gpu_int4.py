@@ -68,6 +68,8 @@ CASES = [  # M, N, K, group
     (2, 64, 4096, 128), (5, 24, 96, 32), (1, 16, 70, 32), (7, 136, 1024, 64),
     # matrix-core decode kernel: 5..16 rows (64-channel workgroups, partial last one), slabs of 16 plus a last row
     (16, 72, 256, 128), (9, 136, 1024, 128), (17, 64, 256, 128), (33, 40, 384, 128), (8, 200, 2048, 128),
+    # row-block kernel: 17..64 rows per launch, partial last block, 64 + 64 + 2 rows
+    (24, 136, 512, 128), (64, 72, 1024, 128), (50, 200, 256, 128), (130, 64, 384, 128), (81, 40, 1152, 128),
 ]
 
 
@@ -153,3 +155,34 @@ def test_cpu_layout_equals_torch_cpu_pack(ops):
     np.testing.assert_array_equal(host(ops._convert_weight_to_int4pack_for_cpu(dev(codes), 2)), want)
     with pytest.raises(ValueError):
         ops._convert_weight_to_int4pack_for_cpu(torch.zeros(8, 32, dtype=torch.int32, device=DEV), 2)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,K,group", [(64, 256, 128), (40, 96, 32), (136, 1024, 64), (8, 70, 32)])
+def test_dequantize_bit_exact(ops, dtype, N, K, group):
+    """Dense weight from the packed layout: the reference's dequantize kernel, bit for bit."""
+    rng = np.random.default_rng(N + K + group)
+    Kg = (K + group - 1) // group * group
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, Kg)).astype(np.float32), group)
+    codes = codes[:, :K]
+    szb = cast_bits(sz, dtype)
+    packed = oracle.int4_pack_tc(codes, 2)
+    got = ops._int4_dequantize(dev(packed), 2, packed.shape[0] * 8, K, group, dev(szb, dtype))
+    want = oracle.int4_dequantize_tc(packed, szb, dtype, K, group)
+    np.testing.assert_array_equal(host(got), want)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+def test_mm_many_rows_takes_the_dense_route(ops, dtype):
+    """More than INT4_PREFILL_ROWS rows: dequantise + library GEMM, the reference's device formulation."""
+    M, N, K, group = ops.INT4_PREFILL_ROWS + 37, 136, 512, 128
+    rng = np.random.default_rng(77)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = oracle.int4_pack_tc(codes, 2)
+    got = ops._weight_int4pack_mm(dev(xb, dtype), dev(packed), group, dev(szb, dtype)).float().cpu().numpy()
+    ref_dev = oracle.to_f32(oracle.int4_mm_tc(xb, dtype, packed, szb, group, round_w=True), dtype)
+    assert_close_norm(got, ref_dev, 1e-2, "vs reference formulation")
+    _, y64 = oracle.int4_mm_tc(xb, dtype, packed, szb, group, round_w=False, want_f64=True)
+    assert rel_err(got, y64) < {"f16": 2e-3, "bf16": 1e-2, "f32": 1e-4}[dtype]
