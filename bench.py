@@ -378,6 +378,47 @@ def main() -> int:
         extras["quantize_2048x4096_bf16_us"] = ms * 1e3
         extras["quantize_GBs"] = (3 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
 
+        # block-wise affine quantizer: the same activations in f32, one block per row -> int8 (4 + 1 bytes per
+        # element), and a 4096 x 4096 f32 weight in groups of 128 -> packed 4-bit (4 + 0.5) and back (0.5 + 4)
+        import ctypes
+        xa32 = xa_d.float()
+        shape2 = (ctypes.c_int64 * 2)(M8, K8)
+        row_block = (ctypes.c_int64 * 2)(1, K8)
+        shape_p, row_block_p = ctypes.cast(shape2, ctypes.c_void_p), ctypes.cast(row_block, ctypes.c_void_p)
+
+        def affine_rows():
+            lib.tpq_quantize_affine(xa32.data_ptr(), _lib.F32, 2, shape_p, row_block_p, a_s.data_ptr(), M8, None, 0,
+                                    _lib.STORAGE_I8, -127, 127, cq.data_ptr(), cur())
+
+        for _ in range(5):
+            affine_rows()
+        ms = time_region(affine_rows, sync, 100)
+        extras["quantize_affine_2048x4096_rows_int8_us"] = ms * 1e3
+        extras["quantize_affine_rows_GBs"] = (5 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
+        wf = torch.from_numpy(rng.normal(0, 0.02, (4096, 4096)).astype(np.float32)).to(dev)
+        gs = (wf.view(4096, 32, 128).abs().amax(dim=2) / 7.0).reshape(-1).contiguous()
+        gz = torch.full_like(gs, 8.0)
+        w4 = torch.empty((4096 * 4096 // 2,), dtype=torch.uint8, device=dev)
+        wback = torch.empty_like(wf)
+        shape_w = (ctypes.c_int64 * 2)(4096, 4096)
+        grp_block = (ctypes.c_int64 * 2)(1, 128)
+        shape_wp, grp_block_p = ctypes.cast(shape_w, ctypes.c_void_p), ctypes.cast(grp_block, ctypes.c_void_p)
+
+        def affine_q4():
+            lib.tpq_quantize_affine(wf.data_ptr(), _lib.F32, 2, shape_wp, grp_block_p, gs.data_ptr(), gs.numel(),
+                                    gz.data_ptr(), gz.numel(), _lib.STORAGE_U4X2, 0, 15, w4.data_ptr(), cur())
+
+        def affine_dq4():
+            lib.tpq_dequantize_affine(w4.data_ptr(), _lib.STORAGE_U4X2, 2, shape_wp, grp_block_p, gs.data_ptr(), gs.numel(),
+                                      gz.data_ptr(), gz.numel(), wback.data_ptr(), cur())
+
+        for fn, key in ((affine_q4, "quantize_affine_4096x4096_g128_u4"), (affine_dq4, "dequantize_affine_4096x4096_g128_u4")):
+            for _ in range(5):
+                fn()
+            ms = time_region(fn, sync, 100)
+            extras[key + "_us"] = ms * 1e3
+            extras[key + "_GBs"] = (4.5 * 4096 * 4096 + 8 * gs.numel()) / (ms * 1e-3) / 1e9
+
         # BitNet ternary: M in {1,128}, 2560 -> 6912 and 6912 -> 2560 (weights cache resident at this size)
         for (mt, kt, nt) in ((1, 2560, 6912), (1, 6912, 2560), (128, 2560, 6912), (128, 6912, 2560)):
             tern = rng.choice(np.int8([-1, 0, 1]), size=(nt, kt), p=[0.325, 0.35, 0.325])

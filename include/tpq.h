@@ -187,6 +187,41 @@ int tpq_int4_cpu_layout_to_device(const uint8_t* packed_cpu, int64_t N, int64_t 
 int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64_t K, const int8_t* w,
                            const float* scales, int64_t N, void* out, void* stream);
 
+/* Storage of quantized codes: one element per int8 / uint8 / int32, or 2 / 4 / 8 elements per byte
+ * (element i in bits (i % pack) * bits of byte i / pack, i = row-major linear index). */
+#define TPQ_STORAGE_I8 0   /* reference dtype qint8   */
+#define TPQ_STORAGE_U8 1   /* quint8   */
+#define TPQ_STORAGE_I32 2  /* qint32   */
+#define TPQ_STORAGE_U4X2 3 /* quint4x2 */
+#define TPQ_STORAGE_U2X4 4 /* quint2x4 */
+#define TPQ_STORAGE_U1X8 5 /* quint1x8 */
+
+/*
+ * Block-wise affine quantizer: code = clamp(rint(x * (1 / scale[b])) + zero_point[b], quant_min,
+ * quant_max), b = block of the element in the row-major grid of ceil(size / block_size) blocks
+ * (block_size[d] >= sizes[d]: one block along d; 1: per index; else groups).  scale 0 acts as 1.
+ * quant_min >= quant_max selects the storage's full range.
+ * x: contiguous tensor of x_dtype with `ndim` (<= 8) dimensions; `sizes` and `block_size` are HOST
+ * arrays; scales / zero_points are DEVICE f32 arrays with one entry per block or a single entry
+ * (n_zeros = 0: no zero point); out: ceil(numel * bits / 8) bytes of `storage`.
+ * Replaces quantize_affine: config/native_functions.yaml:5308-5312,
+ * p10/src/backend/cpu/QuantKernels.cpp:365-455, 579-774,
+ * p10/src/backend/cuda/AffineQuantKernels.cu:806-901.
+ */
+int tpq_quantize_affine(const void* x, int x_dtype, int ndim, const int64_t* sizes,
+                        const int64_t* block_size, const float* scales, int64_t n_scales,
+                        const float* zero_points, int64_t n_zeros, int storage, int64_t quant_min,
+                        int64_t quant_max, void* out, void* stream);
+
+/*
+ * Inverse map: out (f32, shape `sizes`) = (float(code) - zero_point[b]) * scale[b].
+ * Replaces dequantize_affine: config/native_functions.yaml:5314-5318,
+ * p10/src/backend/cpu/QuantKernels.cpp:391-404, 440-455, 776-990.
+ */
+int tpq_dequantize_affine(const void* codes, int storage, int ndim, const int64_t* sizes,
+                          const int64_t* block_size, const float* scales, int64_t n_scales,
+                          const float* zero_points, int64_t n_zeros, float* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

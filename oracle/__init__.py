@@ -311,3 +311,42 @@ def weight_int8pack_mm(x, dtype, w, scales, want_f64=False):
     lib().orc_weight_int8pack_mm(_p(x), _DT[dtype], _p(w), _p(scales), ctypes.c_int64(M), ctypes.c_int64(N),
                                  ctypes.c_int64(K), _p(out), _p(y64))
     return (out, y64) if want_f64 else out
+
+
+AFFINE_STORAGE = {"qint8": (0, np.int8, 1), "quint8": (1, np.uint8, 1), "qint32": (2, np.int32, 1),
+                  "quint4x2": (3, np.uint8, 2), "quint2x4": (4, np.uint8, 4), "quint1x8": (5, np.uint8, 8)}
+_AFFINE_BOUNDS = {"qint8": (-128, 127), "quint8": (0, 255), "qint32": (-2**31, 2**31 - 1),
+                  "quint4x2": (0, 15), "quint2x4": (0, 3), "quint1x8": (0, 1)}
+
+
+def _affine_common(shape, block_size, scales, zeros):
+    arr = ctypes.c_int64 * max(len(shape), 1)
+    scales = _c(np.asarray(scales, np.float32).reshape(-1), np.float32)
+    zeros = None if zeros is None else _c(np.asarray(zeros, np.float32).reshape(-1), np.float32)
+    return arr(*shape), arr(*block_size), scales, zeros
+
+
+def quantize_affine(x, block_size, scales, zeros, dtype, quant_min=0, quant_max=0):
+    """Codes of `dtype` ("qint8" ... "quint1x8"): an array of x's shape, or the flat packed bytes."""
+    x = _c(x, np.float32)
+    tag, code_dtype, pack = AFFINE_STORAGE[dtype]
+    lo, hi = _AFFINE_BOUNDS[dtype]
+    qmin = quant_min if quant_min < quant_max else lo   # QuantKernels.cpp:619-622
+    qmax = quant_max if quant_max > quant_min else hi
+    sizes, blocks, scales, zeros = _affine_common(x.shape, block_size, scales, zeros)
+    out = np.zeros(x.shape, code_dtype) if pack == 1 else np.zeros(((x.size + pack - 1) // pack,), np.uint8)
+    lib().orc_quantize_affine(_p(x), ctypes.c_int(x.ndim), sizes, blocks, _p(scales), ctypes.c_int64(scales.size),
+                              _p(zeros), ctypes.c_int64(0 if zeros is None else zeros.size), ctypes.c_int(tag),
+                              ctypes.c_int64(qmin), ctypes.c_int64(qmax), _p(out))
+    return out
+
+
+def dequantize_affine(codes, shape, block_size, scales, zeros, dtype):
+    tag, code_dtype, _ = AFFINE_STORAGE[dtype]
+    codes = _c(codes, code_dtype)
+    sizes, blocks, scales, zeros = _affine_common(tuple(shape), block_size, scales, zeros)
+    out = np.zeros(tuple(shape), np.float32)
+    lib().orc_dequantize_affine(_p(codes), ctypes.c_int(tag), ctypes.c_int(len(shape)), sizes, blocks, _p(scales),
+                                ctypes.c_int64(scales.size), _p(zeros), ctypes.c_int64(0 if zeros is None else zeros.size),
+                                _p(out))
+    return out

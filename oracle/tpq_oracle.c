@@ -686,3 +686,102 @@ ORC_API void orc_weight_int8pack_mm(const void* x, int dtype, const int8_t* w, c
             if (y64) y64[m * N + n] = acc64 * (double)scale[n];
         }
 }
+
+/* ------------------------------------------------------------------------ */
+/* Block-wise affine quantizer                                               */
+/* ------------------------------------------------------------------------ */
+
+/* Block of a row-major linear index in the grid of ceil(size / block) blocks
+ * (AffineGroupParams::block_of and make_affine_group_params,
+ * p10/src/backend/cpu/QuantKernels.cpp:316-360). */
+static int64_t affine_block_of(int64_t linear, int ndim, const int64_t* sizes, const int64_t* block_size) {
+    int64_t b = 0, size_stride = 1, block_stride = 1;
+    for (int d = ndim - 1; d >= 0; --d) {
+        int64_t blk = block_size[d] < sizes[d] ? block_size[d] : sizes[d];
+        if (blk <= 0) blk = 1;
+        const int64_t per_dim = (sizes[d] + blk - 1) / blk;
+        const int64_t coord = (linear / size_stride) % sizes[d];
+        b += (coord / blk) * block_stride;
+        size_stride *= sizes[d];
+        block_stride *= per_dim;
+    }
+    return b;
+}
+
+/* bits per element of a storage tag (0 int8, 1 uint8, 2 int32, 3 4-bit, 4 2-bit, 5 1-bit) */
+static int affine_bits(int storage) {
+    static const int bits[6] = {8, 8, 32, 4, 2, 1};
+    return bits[storage];
+}
+
+/*
+ * quantize_affine on float32 input.  One scale / zero point per block, or a
+ * single one for all blocks (n_scales / n_zeros == 1); n_zeros == 0: none.
+ * Byte and int32 storages: quantize_affine_kernel, QuantKernels.cpp:365-388
+ * (double position, clamp on the int64).  Packed storages:
+ * quantize_affine_subbyte_kernel, :406-438 (float position, int64 cut to its
+ * low 32 bits, clamp on the int32, low bits first).  The 2-D group kernels
+ * (:457-478, :504-537) and the device kernels (AffineQuantKernels.cu:818-884)
+ * compute the same values.
+ *
+ * Pinned by: torch.quantize_per_tensor / quantize_per_channel int_repr on the
+ * CPU (library twins for one block and for per-row blocks), the numpy closed
+ * form clamp(rint(x * (1/s)) + z) for grouped and tiled grids, the
+ * least-significant-first packing formula of
+ * test/quantization/test_native_1bit.py:43-50, and hand-computed edge cases
+ * (NaN, +-inf, 2^40, zero scale).
+ */
+ORC_API void orc_quantize_affine(const float* x, int ndim, const int64_t* sizes, const int64_t* block_size,
+                                 const float* scales, int64_t n_scales, const float* zeros, int64_t n_zeros,
+                                 int storage, int64_t qmin, int64_t qmax, void* out) {
+    int64_t numel = 1;
+    for (int d = 0; d < ndim; ++d) numel *= sizes[d];
+    const int bits = affine_bits(storage);
+    if (bits < 8) memset(out, 0, (size_t)((numel * bits + 7) / 8));
+    for (int64_t i = 0; i < numel; ++i) {
+        const int64_t b = affine_block_of(i, ndim, sizes, block_size);
+        const float s = scales[n_scales == 1 ? 0 : b];
+        const float inv = s == 0.f ? 1.f : 1.f / s;
+        const float rounded = nearbyintf(x[i] * inv);
+        const float position = n_zeros ? rounded + zeros[n_zeros == 1 ? 0 : b] : rounded;
+        const int64_t wide = (position >= -0x1p63f && position < 0x1p63f) ? (int64_t)position : INT64_MIN;
+        if (bits >= 8) {
+            int64_t q = wide < qmin ? qmin : wide > qmax ? qmax : wide;
+            if (storage == 0) ((int8_t*)out)[i] = (int8_t)q;
+            else if (storage == 1) ((uint8_t*)out)[i] = (uint8_t)q;
+            else ((int32_t*)out)[i] = (int32_t)q;
+        } else {
+            const int pack = 8 / bits;
+            int32_t q = (int32_t)(uint32_t)wide;
+            q = q < (int32_t)qmin ? (int32_t)qmin : q > (int32_t)qmax ? (int32_t)qmax : q;
+            ((uint8_t*)out)[i / pack] |= (uint8_t)((uint8_t)q << ((i % pack) * bits));
+        }
+    }
+}
+
+/*
+ * dequantize_affine: (float(code) - zero) * scale, QuantKernels.cpp:391-404
+ * (bytes, int32) and :440-455 (packed storages).
+ * Pinned by: the closed form in numpy float32, round trips of
+ * orc_quantize_affine codes, torch dequantize() of per-tensor / per-channel
+ * quantized CPU tensors.
+ */
+ORC_API void orc_dequantize_affine(const void* codes, int storage, int ndim, const int64_t* sizes,
+                                   const int64_t* block_size, const float* scales, int64_t n_scales,
+                                   const float* zeros, int64_t n_zeros, float* out) {
+    int64_t numel = 1;
+    for (int d = 0; d < ndim; ++d) numel *= sizes[d];
+    const int bits = affine_bits(storage);
+    for (int64_t i = 0; i < numel; ++i) {
+        const int64_t b = affine_block_of(i, ndim, sizes, block_size);
+        float code;
+        if (storage == 0) code = (float)((const int8_t*)codes)[i];
+        else if (storage == 1) code = (float)((const uint8_t*)codes)[i];
+        else if (storage == 2) code = (float)((const int32_t*)codes)[i];
+        else {
+            const int pack = 8 / bits;
+            code = (float)((((const uint8_t*)codes)[i / pack] >> ((i % pack) * bits)) & ((1 << bits) - 1));
+        }
+        out[i] = (code - (n_zeros ? zeros[n_zeros == 1 ? 0 : b] : 0.f)) * scales[n_scales == 1 ? 0 : b];
+    }
+}

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(HERE, "libtpq_gfx950.so")
 
 TPQ_OK, TPQ_ERR_INVALID_VALUE, TPQ_ERR_INVALID_TYPE, TPQ_ERR_RUNTIME, TPQ_ERR_UNSUPPORTED = range(5)
 F32, F16, BF16 = 0, 1, 2
+STORAGE_I8, STORAGE_U8, STORAGE_I32, STORAGE_U4X2, STORAGE_U2X4, STORAGE_U1X8 = range(6)
 
 _i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 
@@ -34,6 +35,8 @@ SIGNATURES = {
     "tpq_int4_pack_cpu_layout": [_ptr, _i64, _i64, _int, _int, _ptr, _ptr],
     "tpq_int4_cpu_layout_to_device": [_ptr, _i64, _i64, _int, _int, _ptr, _ptr],
     "tpq_weight_int8pack_mm": [_ptr, _int, _i64, _i64, _ptr, _ptr, _i64, _ptr, _ptr],
+    "tpq_quantize_affine": [_ptr, _int, _int, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _int, _i64, _i64, _ptr, _ptr],
+    "tpq_dequantize_affine": [_ptr, _int, _int, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr],
 }
 
 _lib = None

@@ -378,3 +378,113 @@ def int4pack_cpu_to_device(packed_cpu: torch.Tensor, *, block_cols: int = 64, ha
     with torch.cuda.device(p.device):
         _check(_lib.load().tpq_int4_cpu_layout_to_device(_ptr(p), N, K, int(block_cols), int(bool(half_split)), _ptr(out), _stream(p)))
     return out
+
+
+# ---- block-wise affine quantizer ----------------------------------------------------------------
+
+# quantized dtype -> (storage tag, torch dtype of the code tensor, codes per byte).  The reference's
+# quantized dtypes (p10 DType::QInt8 ... QUInt1x8) are named by string, or by the torch dtype of the
+# same name where torch has one.
+_AFFINE_STORAGE = {
+    "qint8": (_lib.STORAGE_I8, torch.int8, 1),
+    "quint8": (_lib.STORAGE_U8, torch.uint8, 1),
+    "qint32": (_lib.STORAGE_I32, torch.int32, 1),
+    "quint4x2": (_lib.STORAGE_U4X2, torch.uint8, 2),
+    "quint2x4": (_lib.STORAGE_U2X4, torch.uint8, 4),
+    "quint1x8": (_lib.STORAGE_U1X8, torch.uint8, 8),
+}
+_AFFINE_ALIASES = {torch.qint8: "qint8", torch.quint8: "quint8", torch.qint32: "qint32",
+                   torch.quint4x2: "quint4x2", torch.quint2x4: "quint2x4"}
+if hasattr(torch, "uint1"):
+    _AFFINE_ALIASES[torch.uint1] = "quint1x8"
+
+
+class PackedCodes:
+    """Codes of a packed sub-byte dtype: ``shape`` logical elements, stored low bits first in the flat
+    uint8 tensor ``data`` (element i in bits (i % pack) * bits of byte i // pack).  Stands in for the
+    reference's tensors of dtype quint4x2 / quint2x4 / quint1x8, whose storage has the same bytes."""
+
+    def __init__(self, data: torch.Tensor, shape, dtype: str):
+        self.data, self.shape, self.dtype = data, tuple(shape), dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def untyped_bytes(self) -> torch.Tensor:
+        return self.data
+
+
+def _affine_dtype_name(dtype, op: str) -> str:
+    name = _AFFINE_ALIASES.get(dtype, dtype)
+    if name not in _AFFINE_STORAGE:
+        raise TypeError(f"{op}(): expected a quantized dtype, got {dtype}")
+    return name
+
+
+def _affine_args(op, shape, block_size, scales, zero_points, device):
+    import ctypes
+    if len(block_size) != len(shape):
+        raise ValueError(f"{op}(): block_size rank must match the input rank")
+    if scales.device != device or (zero_points is not None and zero_points.numel() > 0 and zero_points.device != device):
+        raise RuntimeError(f"{op}(): scales and zero_points must be on the input device")
+    sc = scales.to(torch.float32).contiguous()
+    zp = None
+    if zero_points is not None and zero_points.numel() > 0:
+        zp = zero_points.to(torch.float32).contiguous()
+    arr = ctypes.c_int64 * max(len(shape), 1)
+    return arr(*shape), arr(*[int(b) for b in block_size]), sc, zp
+
+
+def quantize_affine(input: torch.Tensor, block_size, scales: torch.Tensor, zero_points: Optional[torch.Tensor],
+                    dtype, quant_min: int, quant_max: int):
+    """Block-wise affine quantization, ``clamp(rint(x * (1 / scale)) + zero_point)`` per block.
+
+    Returns an int8 / uint8 / int32 tensor of the input's shape, or ``PackedCodes`` for the sub-byte
+    dtypes.  Reference: ``quantize_affine`` (config/native_functions.yaml:5308,
+    p10/src/backend/cpu/QuantKernels.cpp:579-774).
+    """
+    import ctypes
+    name = _affine_dtype_name(dtype, "quantize_affine")
+    tag, code_dtype, pack = _AFFINE_STORAGE[name]
+    _require_device(input, "quantize_affine")
+    if input.dtype not in _DT:
+        input = input.to(torch.float32)
+    x = input.contiguous()
+    sizes, blocks, sc, zp = _affine_args("quantize_affine", tuple(x.shape), block_size, scales, zero_points, x.device)
+    numel = x.numel()
+    if pack == 1:
+        out = torch.empty(x.shape, dtype=code_dtype, device=x.device)
+    else:
+        out = torch.empty(((numel + pack - 1) // pack,), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(_lib.load().tpq_quantize_affine(_ptr(x), _DT[x.dtype], x.dim(), ctypes.cast(sizes, ctypes.c_void_p),
+                                               ctypes.cast(blocks, ctypes.c_void_p), _ptr(sc), sc.numel(), _ptr(zp),
+                                               0 if zp is None else zp.numel(), tag, int(quant_min), int(quant_max),
+                                               _ptr(out), _stream(x)))
+    return out if pack == 1 else PackedCodes(out, x.shape, name)
+
+
+def dequantize_affine(input, block_size, scales: torch.Tensor, zero_points: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 ``(code - zero_point) * scale`` per block; the inverse map of ``quantize_affine``.
+
+    ``input`` is an int8 / uint8 / int32 code tensor or ``PackedCodes``.  Reference:
+    ``dequantize_affine`` (config/native_functions.yaml:5314, p10/src/backend/cpu/QuantKernels.cpp:776-990).
+    """
+    import ctypes
+    if isinstance(input, PackedCodes):
+        name, codes, shape = input.dtype, input.data, input.shape
+    else:
+        by_dtype = {torch.int8: "qint8", torch.uint8: "quint8", torch.int32: "qint32"}
+        if not isinstance(input, torch.Tensor) or input.dtype not in by_dtype:
+            raise TypeError(f"dequantize_affine(): expected a quantized tensor, got {getattr(input, 'dtype', type(input))}")
+        name, codes, shape = by_dtype[input.dtype], input.contiguous(), tuple(input.shape)
+    tag = _AFFINE_STORAGE[name][0]
+    _require_device(codes, "dequantize_affine")
+    sizes, blocks, sc, zp = _affine_args("dequantize_affine", shape, block_size, scales, zero_points, codes.device)
+    out = torch.empty(shape, dtype=torch.float32, device=codes.device)
+    with torch.cuda.device(codes.device):
+        _check(_lib.load().tpq_dequantize_affine(_ptr(codes), tag, len(shape), ctypes.cast(sizes, ctypes.c_void_p),
+                                                 ctypes.cast(blocks, ctypes.c_void_p), _ptr(sc), sc.numel(), _ptr(zp),
+                                                 0 if zp is None else zp.numel(), _ptr(out), _stream(codes)))
+    return out
