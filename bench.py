@@ -337,6 +337,28 @@ def main() -> int:
             extras[f"int8pack_M{mb}_GBs"] = (N * K + 4 * N + 2 * mb * K + 2 * mb * N) / (ms * 1e-3) / 1e9
         del w8s
         torch.cuda.empty_cache()
+        # packed n-bit weight-only decode (int2 / intx / binary modules): same shape, bits per weight in
+        # {1, 2, 4, 8}, float32 (scale, zero) per group of 128; enough rotating copies to stream from HBM
+        G = K // 128
+        szf = torch.stack([torch.rand(G, N, device=dev) * 0.01, torch.full((G, N), 2.0, device=dev)], dim=-1).contiguous()
+        xb = torch.from_numpy(rng.normal(0, 1, (1, K)).astype(np.float32)).to(dev).half()
+        yb = torch.empty((1, N), dtype=torch.float16, device=dev)
+        for bits in (1, 2, 4, 8):
+            row_bytes = K * bits // 8
+            copies = max(2, min(60, (600 << 20) // (N * row_bytes)))
+            wl = [torch.randint(0, 256, (N, row_bytes), dtype=torch.uint8, device=dev) for _ in range(copies)]
+
+            def lbmm(i, wl=wl, bits=bits, copies=copies):
+                lib.tpq_lowbit_mm(xb.data_ptr(), _lib.F16, 1, K, wl[i % copies].data_ptr(), bits, 0, N, 128,
+                                  szf.data_ptr(), None, yb.data_ptr(), cur())
+
+            gl = graph_of(lambda: [lbmm(i) for i in range(2 * copies)])
+            gl.replay(); sync()
+            ms = time_region(gl.replay, sync, 1) / (2 * copies)
+            extras[f"lowbit{bits}_M1_us"] = ms * 1e3
+            extras[f"lowbit{bits}_M1_GBs"] = (N * row_bytes + 8 * G * N + 2 * K + 2 * N) / (ms * 1e-3) / 1e9
+            del wl
+        torch.cuda.empty_cache()
 
     if not args.no_extras and not args.gemv_only:
         # int8 prefill GEMM with fused dequant: M=2048, K=4096, N=4096, bf16 in/out

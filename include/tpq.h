@@ -222,6 +222,39 @@ int tpq_dequantize_affine(const void* codes, int storage, int ndim, const int64_
                           const int64_t* block_size, const float* scales, int64_t n_scales,
                           const float* zero_points, int64_t n_zeros, float* out, void* stream);
 
+/*
+ * Weight-only matmul on packed n-bit weights (1 <= bits <= 8):
+ *   out[m,n] = sum_k x[m,k] * (code[n,k] - zero[g,n]) * scale[g,n] (+ bias[n]),  g = k / group.
+ * packed: uint8 [N, ceil(K / (8 / bits))]; code i of a byte sits in bits 8 - (i+1) * bits .. when
+ * lsb_first = 0 (pack_intx / pack_int2) and in bits i * bits .. when lsb_first = 1 (pack_binary).
+ * scales_and_zeros: f32 [K / group][N][2]; bias: f32 [N] or NULL; x, out: [M,K], [M,N] of `dtype`.
+ * Replaces _intx_mm / _int2_mm / _binary_mm, which unpack, dequantize and call a float GEMM:
+ * tensorplay/ao/quantization/intx_weight_only.py:35-133, int2_weight_only.py:63-139,
+ * binary.py:50-95 (binary: scale' = 2 * scale, zero = 0.5, one group).
+ */
+int tpq_lowbit_mm(const void* x, int dtype, int64_t M, int64_t K, const uint8_t* packed, int bits,
+                  int lsb_first, int64_t N, int64_t group, const float* scales_and_zeros,
+                  const float* bias, void* out, void* stream);
+
+/*
+ * Dense [N, K] weight of `dtype` from the same packed form: (float(code) - zero) * scale
+ * (_dequantize_intx, tensorplay/ao/quantization/intx_weight_only.py:110-124).
+ */
+int tpq_lowbit_dequantize(const uint8_t* packed, int bits, int lsb_first, int64_t N, int64_t K,
+                          int64_t group, const float* scales_and_zeros, int dtype, void* out,
+                          void* stream);
+
+/*
+ * codes uint8 [rows, cols] (values < 2^bits) <-> packed uint8 [rows, ceil(cols / (8 / bits))], the
+ * last byte of a row padded with zero fields.  Replaces pack_intx / unpack_intx
+ * (tensorplay/ao/quantization/intx_weight_only.py:35-80), pack_int2 / unpack_int2
+ * (int2_weight_only.py:63-103) and, with lsb_first = 1, pack_binary / unpack_binary (binary.py:50-85).
+ */
+int tpq_lowbit_pack(const uint8_t* codes, int bits, int lsb_first, int64_t rows, int64_t cols,
+                    uint8_t* packed, void* stream);
+int tpq_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, int64_t rows, int64_t cols,
+                      uint8_t* codes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

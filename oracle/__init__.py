@@ -350,3 +350,37 @@ def dequantize_affine(codes, shape, block_size, scales, zeros, dtype):
                                 ctypes.c_int64(scales.size), _p(zeros), ctypes.c_int64(0 if zeros is None else zeros.size),
                                 _p(out))
     return out
+
+
+def lowbit_pack(codes, bits, lsb_first=False):
+    codes = _c(codes, np.uint8)
+    rows, cols = codes.shape
+    per_byte = 8 // bits
+    out = np.zeros((rows, (cols + per_byte - 1) // per_byte), np.uint8)
+    lib().orc_lowbit_pack(_p(codes), ctypes.c_int(bits), ctypes.c_int(int(lsb_first)), ctypes.c_int64(rows), ctypes.c_int64(cols), _p(out))
+    return out
+
+
+def lowbit_unpack(packed, bits, cols, lsb_first=False):
+    packed = _c(packed, np.uint8)
+    rows = packed.shape[0]
+    out = np.zeros((rows, cols), np.uint8)
+    lib().orc_lowbit_unpack(_p(packed), ctypes.c_int(bits), ctypes.c_int(int(lsb_first)), ctypes.c_int64(rows), ctypes.c_int64(cols), _p(out))
+    return out
+
+
+def lowbit_mm(x, dtype, packed, bits, sz, K, group, bias=None, lsb_first=False, want_f64=False, want_dense=False):
+    """(out, [y64], [dense]) of the packed n-bit weight-only linear; sz is float32 [K // group, N, 2]."""
+    packed = _c(packed, np.uint8)
+    sz = _c(sz, np.float32)
+    N = packed.shape[0]
+    x = None if x is None else _c(x, storage(dtype))
+    M = 0 if x is None else x.shape[0]
+    bias = None if bias is None else _c(bias, np.float32)
+    out = np.zeros((M, N), storage(dtype))
+    y64 = np.zeros((M, N), np.float64) if want_f64 else None
+    dense = np.zeros((N, K), np.float32) if want_dense else None
+    lib().orc_lowbit_mm(_p(x), _DT[dtype], _p(packed), ctypes.c_int(bits), ctypes.c_int(int(lsb_first)), _p(sz), _p(bias),
+                        ctypes.c_int64(M), ctypes.c_int64(N), ctypes.c_int64(K), ctypes.c_int64(group), _p(out), _p(y64), _p(dense))
+    res = (out,) + ((y64,) if want_f64 else ()) + ((dense,) if want_dense else ())
+    return res if len(res) > 1 else out

@@ -785,3 +785,77 @@ ORC_API void orc_dequantize_affine(const void* codes, int storage, int ndim, con
         out[i] = (code - (n_zeros ? zeros[n_zeros == 1 ? 0 : b] : 0.f)) * scales[n_scales == 1 ? 0 : b];
     }
 }
+
+/* ------------------------------------------------------------------------ */
+/* Packed n-bit weight-only linear (int2 / intx / binary modules)            */
+/* ------------------------------------------------------------------------ */
+
+/* shift of code i (0 .. 8/bits - 1) inside its byte: first code in the most
+ * significant bits (pack_intx, tensorplay/ao/quantization/intx_weight_only.py:55-58;
+ * pack_int2, int2_weight_only.py:82-87) or, lsb_first, code i in bit i * bits
+ * (pack_binary, binary.py:66-70). */
+static int lowbit_shift(int i, int bits, int lsb_first) { return lsb_first ? i * bits : 8 - (i + 1) * bits; }
+
+/*
+ * codes uint8 [rows, cols] -> packed uint8 [rows, ceil(cols / (8 / bits))], tail padded with zeros.
+ * Pinned by: a numpy restatement of the reference's strided-slice formulas, the shapes of
+ * test/quantization/test_int2_binary_modules.py:57-66, 129-137 and pack/unpack round trips.
+ */
+ORC_API void orc_lowbit_pack(const uint8_t* codes, int bits, int lsb_first, int64_t rows, int64_t cols, uint8_t* packed) {
+    const int per_byte = 8 / bits;
+    const int64_t pitch = (cols + per_byte - 1) / per_byte;
+    memset(packed, 0, (size_t)(rows * pitch));
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c)
+            packed[r * pitch + c / per_byte] |=
+                (uint8_t)((codes[r * cols + c] & ((1 << bits) - 1)) << lowbit_shift((int)(c % per_byte), bits, lsb_first));
+}
+
+/* unpack_intx (intx_weight_only.py:62-80) / unpack_int2 (int2_weight_only.py:91-103) / unpack_binary (binary.py:74-85) */
+ORC_API void orc_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, int64_t rows, int64_t cols, uint8_t* codes) {
+    const int per_byte = 8 / bits;
+    const int64_t pitch = (cols + per_byte - 1) / per_byte;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c)
+            codes[r * cols + c] =
+                (uint8_t)((packed[r * pitch + c / per_byte] >> lowbit_shift((int)(c % per_byte), bits, lsb_first)) & ((1 << bits) - 1));
+}
+
+/*
+ * _intx_mm / _int2_mm (intx_weight_only.py:110-133, int2_weight_only.py:115-139): the dense weight
+ * dq[n,k] = (float(code) - zero[g,n]) * scale[g,n] in float32, then out = x @ dq.T (+ bias).
+ * sz: float32 [K / group][N][2].  `dense` (optional) receives dq; `out` is rounded to `dtype` from a
+ * float32 fma chain over k; `y64` (optional) is the same sum in double from the float32 dq.
+ * _binary_mm (binary.py:88-95) is the case bits = 1, lsb_first, one group, scale' = 2 scale, zero = 0.5:
+ * (bit - 0.5) * 2 s = (2 bit - 1) * s exactly.
+ * Pinned by: numpy float64 x @ dq.T with dq from the closed form on independently unpacked codes; the
+ * reference test's own check (test_int2_binary_modules.py:69-89, 140-155) restated in numpy.
+ */
+ORC_API void orc_lowbit_mm(const void* x, int dtype, const uint8_t* packed, int bits, int lsb_first, const float* sz,
+                           const float* bias, int64_t M, int64_t N, int64_t K, int64_t group, void* out, double* y64,
+                           float* dense) {
+    const int per_byte = 8 / bits;
+    const int64_t pitch = (K + per_byte - 1) / per_byte;
+    for (int64_t n = 0; n < N; ++n) {
+        for (int64_t m = 0; m < (M > 0 ? M : 1); ++m) {
+            float acc = 0.0f;
+            double acc64 = 0.0;
+            for (int64_t k = 0; k < K; ++k) {
+                const int code = (packed[n * pitch + k / per_byte] >> lowbit_shift((int)(k % per_byte), bits, lsb_first)) & ((1 << bits) - 1);
+                const float* p = sz + ((k / group) * N + n) * 2;
+                const float dq = ((float)code - p[1]) * p[0];
+                if (dense && m == 0) dense[n * K + k] = dq;
+                if (M > 0) {
+                    const float xv = load_as_f32(x, dtype, m * K + k);
+                    acc = fmaf(dq, xv, acc);
+                    acc64 += (double)dq * (double)xv;
+                }
+            }
+            if (M > 0) {
+                if (bias) { acc += bias[n]; acc64 += (double)bias[n]; }
+                if (out) store_from_f32(out, dtype, m * N + n, acc);
+                if (y64) y64[m * N + n] = acc64;
+            }
+        }
+    }
+}

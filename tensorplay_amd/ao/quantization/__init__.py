@@ -11,6 +11,26 @@ from .bitnet import (  # noqa: F401
     quantize_int8_rowwise,
     unpack_ternary,
 )
+from .binary import (  # noqa: F401
+    BinaryWeightOnlyConfig,
+    WeightOnlyBinaryLinear,
+    _binary_mm,
+    _quantize_binary_weight,
+    binary_weight_only,
+    pack_binary,
+    quantize_binary_weight_only,
+    unpack_binary,
+)
+from .int2_weight_only import (  # noqa: F401
+    Int2WeightOnlyConfig,
+    WeightOnlyInt2Linear,
+    _int2_mm,
+    _quantize_int2_groupwise,
+    int2_weight_only,
+    pack_int2,
+    quantize_int2_weight_only,
+    unpack_int2,
+)
 from .int4_weight_only import (  # noqa: F401
     Int4WeightOnlyConfig,
     WeightOnlyInt4Linear,
@@ -26,5 +46,15 @@ from .int8_mixed_precision import (  # noqa: F401
     _int8_mm,
     int8_dynamic_linear,
     scaled_int8_mm,
+)
+from .intx_weight_only import (  # noqa: F401
+    IntxWeightOnlyConfig,
+    WeightOnlyIntxLinear,
+    _intx_mm,
+    _quantize_intx_groupwise,
+    intx_weight_only,
+    pack_intx,
+    quantize_intx_weight_only,
+    unpack_intx,
 )
 from .quantize_api import quantize_, register_quantize_module_handler  # noqa: F401

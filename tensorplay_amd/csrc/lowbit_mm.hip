@@ -1,0 +1,400 @@
+// Weight-only matmul for the packed n-bit weights (1 <= bits <= 8) of the reference's int2 / intx /
+// binary weight-only modules:
+//   out[m, n] = sum_k x[m, k] * (code[n, k] - zero[g, n]) * scale[g, n]  (+ bias[n]),  g = k / group
+// packed: uint8 [N, ceil(K / per_byte)], per_byte = 8 / bits codes per byte, code i of a byte in bits
+// 8 - (i + 1) * bits .. (first code in the most significant bits: pack_intx / pack_int2,
+// tensorplay/ao/quantization/intx_weight_only.py:35-59, int2_weight_only.py:63-88) or, for the 1-bit
+// sign weights, in bit i (pack_binary, binary.py:50-71).  scales_and_zeros: f32 [K / group][N][2], the
+// buffer the modules keep (intx_weight_only.py:167-170).  The reference unpacks with tensor ops,
+// dequantizes to a dense float weight and calls a float GEMM (_intx_mm, intx_weight_only.py:127-133).
+//
+// Decode kernel (fp16 activations, 1..16 rows): v_mfma_f32_16x16x16_f16 with the weights as A.  Lane
+// (i, q) owns weight row n0 + i and, per step, 32 consecutive codes of it (16 when a code has a byte
+// to itself): 4 to 16 bytes, one load.  A code becomes an fp16 number without leaving its bits: the
+// byte is copied into both halves of a dword (v_perm_b32), a mask keeps one field per half and an
+// exponent is or-ed in, chosen so that the field's position in the mantissa has weight one: a field at
+// bit p under exponent 2^(10-p) reads 2^(10-p) + code.  Two neighbouring codes per dword, so the B
+// operand is simply the activations as they lie in memory.  The offsets 2^(10-p) leave through one
+// more MFMA per four k whose A is constant (row 0: the offsets, row 1: ones -> sum of x), and a step
+// stays inside one quantization group:  y += scale * ((D - offsets) - zero * sum x).
+//
+// Everything else (fp32 / bf16 activations, odd K or group sizes) takes a plain kernel: one workgroup
+// per output channel and slab of up to 8 rows, the dequantized weight formed in fp32 exactly as the
+// reference does, fp32 fma over k.
+#include <cstdlib>
+
+#include "int4_lane.h"
+
+namespace tpq {
+namespace {
+
+// dword r of a 16-byte vector; r is a constant once the loops around the call are unrolled
+__device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
+
+template <int BITS, bool LSB>
+struct Fields {
+    static constexpr int kPerByte = 8 / BITS;
+    static constexpr int kCodes = kPerByte >= 2 ? 32 : 16;  // per lane and step
+    static constexpr int kBytes = kCodes / kPerByte;        // 4, 8 or 16
+    static constexpr int kStepK = 4 * kCodes;
+    static constexpr int kVariants = kPerByte == 8 ? 2 : 1;  // distinct offset patterns of an MFMA's four k
+    static constexpr uint32_t kField = (1u << BITS) - 1u;
+    // bit position of code i of a byte
+    static constexpr int pos(int i) { return LSB ? i * BITS : 8 - (i + 1) * BITS; }
+    // fp16 bits of 2^(10 - p): a field at bit p of the mantissa then counts in units of one
+    static constexpr uint32_t base_bits(int p) { return static_cast<uint32_t>(25 - p) << 10; }
+    // pair t = codes 2t, 2t + 1 of the lane's bytes: which byte goes to which half, masks, exponents
+    static constexpr int byte_lo(int t) { return (2 * t) / kPerByte; }
+    static constexpr int byte_hi(int t) { return (2 * t + 1) / kPerByte; }
+    static constexpr int pos_lo(int t) { return pos((2 * t) % kPerByte); }
+    static constexpr int pos_hi(int t) { return pos((2 * t + 1) % kPerByte); }
+    static constexpr uint32_t select(int t) { return 0x0C000C00u | (byte_lo(t) & 3) | ((byte_hi(t) & 3) << 16); }
+    static constexpr uint32_t mask(int t) { return (kField << pos_lo(t)) | (kField << (pos_hi(t) + 16)); }
+    static constexpr uint32_t magic(int t) { return base_bits(pos_lo(t)) | (base_bits(pos_hi(t)) << 16); }
+    static constexpr int kMagics = kPerByte >= 2 ? kPerByte / 2 : 1;  // magic(t) repeats with this period
+};
+
+// x: [M][K] fp16; packed: [N][K / per_byte]; sz: [K / group][N][2] fp32; steps = K / kStepK; a group is
+// kStepK << group_shift k.  N % 4 == 0.
+template <int BITS, bool LSB, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
+    const float* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int group_shift) {
+    using F = Fields<BITS, LSB>;
+    __shared__ float red[WAVES][4][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, q = lane >> 4;
+    const int steps = K / F::kStepK;
+    const int n0 = blockIdx.x * 16;
+    const int n_row = n0 + i < N ? n0 + i : N - 1;  // rows past N: a valid row, result dropped
+    const uint8_t* w_base = packed + static_cast<size_t>(n_row) * (K / F::kPerByte) + q * F::kBytes;
+    int n4 = n0 + 4 * q;  // this lane's four output channels
+    n4 = n4 + 4 <= N ? n4 : N - 4;
+    const float* sz_base = sz + static_cast<size_t>(n4) * 2;
+    const bool row_live = i < M;
+    // columns m >= M repeat the last row: their products are computed and never stored
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : M - 1) * K + q * F::kCodes);
+
+    // constant A of the offset MFMA: row 0 = the offsets of the four k of an MFMA, row 1 = ones
+    uint32_t a_corr[F::kVariants][2];
+#pragma unroll
+    for (int var = 0; var < F::kVariants; ++var)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int t = 2 * var + h;  // pair t of the lane's codes has the pattern of pair t + 2 * kVariants, ...
+            a_corr[var][h] = i == 0 ? F::magic(t) : i == 1 ? 0x3C003C00u : 0u;
+        }
+    uint32_t magic[F::kMagics];  // kept in VGPRs behind opaque moves: v_and_or_b32 takes one scalar operand
+#pragma unroll
+    for (int t = 0; t < F::kMagics; ++t) asm volatile("v_mov_b32 %0, %1" : "=v"(magic[t]) : "s"(F::magic(t)));
+
+    struct Step {
+        uint4 w;       // kBytes of it are used
+        uint4 p[2];    // (scale, zero) of four channels
+        uint4 xv[F::kCodes / 8];
+    };
+    auto load = [&](int s, Step& st) {
+        const uint8_t* src = w_base + static_cast<size_t>(s) * (4 * F::kBytes);
+        if constexpr (F::kBytes == 16) st.w = *reinterpret_cast<const uint4*>(src);
+        if constexpr (F::kBytes == 8) { const uint2 t = *reinterpret_cast<const uint2*>(src); st.w = make_uint4(t.x, t.y, 0, 0); }
+        if constexpr (F::kBytes == 4) st.w = make_uint4(*reinterpret_cast<const uint32_t*>(src), 0, 0, 0);
+        const uint4* prm = reinterpret_cast<const uint4*>(sz_base + static_cast<size_t>(s >> group_shift) * N * 2);
+        st.p[0] = prm[0];
+        st.p[1] = prm[1];
+#pragma unroll
+        for (int c = 0; c < F::kCodes / 8; ++c) st.xv[c] = x_base[static_cast<size_t>(s) * (F::kStepK / 8) + c];
+    };
+
+    float yacc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto compute = [&](const Step& st) {
+        float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f}, d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int u = 0; u < F::kCodes / 4; ++u) {  // MFMA u: codes 4u .. 4u+3 of the lane
+            uint32_t a[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int t = 2 * u + h;
+                const uint32_t word = dword_at(st.w, F::byte_lo(t) >> 2);
+                const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
+                a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
+            }
+            const uint32_t b0 = dword_at(st.xv[u >> 1], (2 * u) & 3), b1 = dword_at(st.xv[u >> 1], (2 * u + 1) & 3);
+            const word2_t av = {a[0], a[1]}, cv = {a_corr[u % F::kVariants][0], a_corr[u % F::kVariants][1]}, bv = {b0, b1};
+            aux = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, cv), __builtin_bit_cast(half4_t, bv), aux, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, av), __builtin_bit_cast(half4_t, bv), d, 0, 0, 0);
+        }
+        // rows 0 and 1 of the offset product sit in lanes 0..15, registers 0 and 1
+        const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint4& pv = st.p[v >> 1];
+            const float scale = __builtin_bit_cast(float, (v & 1) ? pv.z : pv.x);
+            const float zero = __builtin_bit_cast(float, (v & 1) ? pv.w : pv.y);
+            yacc[v] = __builtin_fmaf(scale, (d[v] - corr) - zero * sx, yacc[v]);
+        }
+    };
+
+    // this wavefront's steps: wave, wave + WAVES, ...; two in flight
+    Step s0, s1;
+    int s = wave;
+    if (s < steps) load(s, s0);
+    if (s + WAVES < steps) load(s + WAVES, s1);
+    for (; s + 3 * WAVES < steps; s += 2 * WAVES) {  // steady state: no branches in the body
+        compute(s0);
+        load(s + 2 * WAVES, s0);
+        compute(s1);
+        load(s + 3 * WAVES, s1);
+    }
+    if (s < steps) {
+        compute(s0);
+        if (s + 2 * WAVES < steps) load(s + 2 * WAVES, s0);
+        if (s + WAVES < steps) compute(s1);
+        if (s + 2 * WAVES < steps) compute(s0);
+    }
+
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][v][lane] = yacc[v];
+    __syncthreads();
+    if (wave == 0) {  // lane (m, q): channels n0 + 4 q + v
+        const int n = n0 + 4 * q;
+        if (row_live && n < N) {  // N % 4 == 0: all four channels exist
+            float sum[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                sum[v] = 0.0f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) sum[v] += red[w][v][lane];
+                if (bias != nullptr) sum[v] += bias[n + v];
+            }
+            const uint32_t lo = f32_to_f16_bits(sum[0]) | (static_cast<uint32_t>(f32_to_f16_bits(sum[1])) << 16);
+            const uint32_t hi = f32_to_f16_bits(sum[2]) | (static_cast<uint32_t>(f32_to_f16_bits(sum[3])) << 16);
+            *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
+        }
+    }
+}
+
+// code k of row `row` (any bits, either bit order)
+__device__ __forceinline__ int code_at(const uint8_t* row, int64_t k, int bits, int per_byte, bool lsb_first) {
+    const int i = static_cast<int>(k % per_byte);
+    const int shift = lsb_first ? i * bits : 8 - (i + 1) * bits;
+    return (row[k / per_byte] >> shift) & ((1 << bits) - 1);
+}
+
+// One workgroup per output channel n and slab of up to 8 activation rows.
+template <int DT>
+__global__ __launch_bounds__(256) void lowbit_generic_kernel(
+    const typename Elem<DT>::storage* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
+    const float* __restrict__ bias, typename Elem<DT>::storage* __restrict__ y, int64_t M, int64_t N, int64_t K,
+    int64_t group, int bits, int lsb_first) {
+    __shared__ float red[8][256 / kWave];
+    const int64_t n = blockIdx.x, m0 = static_cast<int64_t>(blockIdx.y) * 8;
+    const int rows = static_cast<int>(M - m0 < 8 ? M - m0 : 8);
+    const int per_byte = 8 / bits;
+    const uint8_t* wr = packed + n * ((K + per_byte - 1) / per_byte);
+    float acc[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) acc[b] = 0.0f;
+    for (int64_t k = threadIdx.x; k < K; k += 256) {
+        const float* p = sz + ((k / group) * N + n) * 2;
+        const float wv = (static_cast<float>(code_at(wr, k, bits, per_byte, lsb_first)) - p[1]) * p[0];
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+            if (b < rows) acc[b] = __builtin_fmaf(wv, Elem<DT>::load(x[(m0 + b) * K + k]), acc[b]);
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const float v = wave_sum(acc[b]);
+        if (lane == 0) red[b][wave] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < rows) {
+        const int b = threadIdx.x;
+        float total = (red[b][0] + red[b][1]) + (red[b][2] + red[b][3]);
+        if (bias != nullptr) total += bias[n];
+        y[(m0 + b) * N + n] = Elem<DT>::store(total);
+    }
+}
+
+// Dense [N, K] weight of `DT`: (float(code) - zero) * scale formed in fp32, then rounded once.
+template <int DT>
+__global__ __launch_bounds__(256) void lowbit_dequantize_kernel(const uint8_t* __restrict__ packed, const float* __restrict__ sz,
+                                                                typename Elem<DT>::storage* __restrict__ out, int64_t N, int64_t K,
+                                                                int64_t group, int bits, int lsb_first) {
+    const int per_byte = 8 / bits;
+    const int64_t pitch = (K + per_byte - 1) / per_byte;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < N * K;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int64_t n = idx / K, k = idx - n * K;
+        const float* p = sz + ((k / group) * N + n) * 2;
+        out[idx] = Elem<DT>::store((static_cast<float>(code_at(packed + n * pitch, k, bits, per_byte, lsb_first != 0)) - p[1]) * p[0]);
+    }
+}
+
+// codes uint8 [rows, cols] -> packed [rows, pitch]: one thread per packed byte, tail fields zero
+__global__ __launch_bounds__(256) void lowbit_pack_kernel(const uint8_t* __restrict__ codes, uint8_t* __restrict__ packed, int64_t rows,
+                                                          int64_t cols, int bits, int lsb_first) {
+    const int per_byte = 8 / bits;
+    const int64_t pitch = (cols + per_byte - 1) / per_byte;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < rows * pitch;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int64_t r = idx / pitch, b = idx - r * pitch;
+        uint32_t value = 0;
+        for (int i = 0; i < per_byte && b * per_byte + i < cols; ++i) {
+            const int shift = lsb_first ? i * bits : 8 - (i + 1) * bits;
+            value |= (codes[r * cols + b * per_byte + i] & ((1u << bits) - 1u)) << shift;
+        }
+        packed[idx] = static_cast<uint8_t>(value);
+    }
+}
+
+__global__ __launch_bounds__(256) void lowbit_unpack_kernel(const uint8_t* __restrict__ packed, uint8_t* __restrict__ codes, int64_t rows,
+                                                            int64_t cols, int bits, int lsb_first) {
+    const int per_byte = 8 / bits;
+    const int64_t pitch = (cols + per_byte - 1) / per_byte;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < rows * cols;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int64_t r = idx / cols, c = idx - r * cols;
+        codes[idx] = static_cast<uint8_t>(code_at(packed + r * pitch, c, bits, per_byte, lsb_first != 0));
+    }
+}
+
+template <int BITS, bool LSB>
+int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t M, int64_t N,
+                int64_t K, int group_shift, hipStream_t s) {
+    // wavefronts per 16-channel workgroup: each takes every WAVES-th step, two in flight
+    static const int forced = [] { const char* e = getenv("TPQ_LOWBIT_WAVES"); return e ? atoi(e) : 0; }();
+    const int64_t steps = K / Fields<BITS, LSB>::kStepK;
+    // measured at 4096 -> 11008, one row, 2 bits: 4 waves 11.1 us, 8 waves 10.4 - 11.0 us, 16 waves 14.3 us
+    const int waves = forced ? forced : steps >= 16 ? 8 : 4;
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        const dim3 grid(static_cast<unsigned>((N + 15) / 16));
+        const uint16_t* xs = static_cast<const uint16_t*>(x) + m0 * K;
+        uint16_t* ys = static_cast<uint16_t*>(out) + m0 * N;
+        const int n = static_cast<int>(N), k = static_cast<int>(K);
+        if (waves >= 16) lowbit_mfma_kernel<BITS, LSB, 16><<<grid, 16 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+        else if (waves >= 8) lowbit_mfma_kernel<BITS, LSB, 8><<<grid, 8 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+        else lowbit_mfma_kernel<BITS, LSB, 4><<<grid, 4 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+    }
+    return check_launch("tpq_lowbit_mm (mfma)");
+}
+
+template <int DT>
+int launch_generic(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t M, int64_t N,
+                   int64_t K, int64_t group, int bits, int lsb_first, hipStream_t s) {
+    using S = typename Elem<DT>::storage;
+    const int64_t slabs = (M + 7) / 8;
+    TPQ_REQUIRE(N <= 0x7FFFFFFF && slabs <= 65535, TPQ_ERR_INVALID_VALUE, "lowbit mm: shape too large");
+    lowbit_generic_kernel<DT><<<dim3(static_cast<unsigned>(N), static_cast<unsigned>(slabs)), 256, 0, s>>>(
+        static_cast<const S*>(x), packed, sz, bias, static_cast<S*>(out), M, N, K, group, bits, lsb_first);
+    return check_launch("tpq_lowbit_mm (generic)");
+}
+
+int check_lowbit(const char* op, int bits, int lsb_first, int64_t N, int64_t K, int64_t group) {
+    TPQ_REQUIRE(bits >= 1 && bits <= 8, TPQ_ERR_INVALID_VALUE, "%s: bits must be in [1, 8], got %d", op, bits);
+    TPQ_REQUIRE(lsb_first == 0 || lsb_first == 1, TPQ_ERR_INVALID_VALUE, "%s: lsb_first must be 0 or 1", op);
+    TPQ_REQUIRE(N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "%s: negative shape", op);
+    TPQ_REQUIRE(group > 0 && K % group == 0, TPQ_ERR_INVALID_VALUE, "%s: K=%lld must be divisible by groupsize=%lld", op,
+                static_cast<long long>(K), static_cast<long long>(group));
+    return TPQ_OK;
+}
+
+}  // namespace
+}  // namespace tpq
+
+using namespace tpq;
+
+TPQ_EXPORT int tpq_lowbit_mm(const void* x, int dtype, int64_t M, int64_t K, const uint8_t* packed, int bits,
+                             int lsb_first, int64_t N, int64_t group, const float* scales_and_zeros, const float* bias,
+                             void* out, void* stream) {
+    TPQ_REQUIRE(dtype == TPQ_DTYPE_F32 || dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16, TPQ_ERR_INVALID_TYPE,
+                "lowbit mm: activations must be floating point");
+    TPQ_REQUIRE(M >= 0, TPQ_ERR_INVALID_VALUE, "lowbit mm: negative shape");
+    if (int rc = check_lowbit("lowbit mm", bits, lsb_first, N, K, group)) return rc;
+    if (M == 0 || N == 0) return TPQ_OK;
+    TPQ_REQUIRE(out != nullptr, TPQ_ERR_INVALID_VALUE, "lowbit mm: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // K = 0 is an empty sum: the plain kernel then writes the bias (or zeros) and reads nothing else
+    TPQ_REQUIRE(K == 0 || (x && packed && scales_and_zeros), TPQ_ERR_INVALID_VALUE, "lowbit mm: null pointer");
+    const int per_byte = 8 / bits;
+    const int step_k = per_byte >= 2 ? 128 : 64;
+    int group_shift = -1;
+    if (group % step_k == 0) {
+        const int64_t per_group = group / step_k;
+        if ((per_group & (per_group - 1)) == 0) {
+            group_shift = 0;
+            while ((int64_t{1} << group_shift) < per_group) ++group_shift;
+        }
+    }
+    const bool fast = dtype == TPQ_DTYPE_F16 && K > 0 && group_shift >= 0 && K % step_k == 0 && N % 4 == 0 && K <= 0x7FFFFF80 &&
+                      N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(packed, 16) && aligned(scales_and_zeros, 16) && aligned(out, 8);
+    if (fast) {
+#define TPQ_LB_CASE(BITS)                                                                                                      \
+    case BITS:                                                                                                                 \
+        return lsb_first ? launch_mfma<BITS, true>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s)            \
+                         : launch_mfma<BITS, false>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s);
+        switch (bits) {
+            TPQ_LB_CASE(1)
+            TPQ_LB_CASE(2)
+            TPQ_LB_CASE(3)
+            TPQ_LB_CASE(4)
+            TPQ_LB_CASE(5)
+            TPQ_LB_CASE(6)
+            TPQ_LB_CASE(7)
+            TPQ_LB_CASE(8)
+        }
+#undef TPQ_LB_CASE
+    }
+    switch (dtype) {
+        case TPQ_DTYPE_F32: return launch_generic<TPQ_DTYPE_F32>(x, packed, scales_and_zeros, bias, out, M, N, K, group, bits, lsb_first, s);
+        case TPQ_DTYPE_F16: return launch_generic<TPQ_DTYPE_F16>(x, packed, scales_and_zeros, bias, out, M, N, K, group, bits, lsb_first, s);
+        default: return launch_generic<TPQ_DTYPE_BF16>(x, packed, scales_and_zeros, bias, out, M, N, K, group, bits, lsb_first, s);
+    }
+}
+
+TPQ_EXPORT int tpq_lowbit_dequantize(const uint8_t* packed, int bits, int lsb_first, int64_t N, int64_t K, int64_t group,
+                                     const float* scales_and_zeros, int dtype, void* out, void* stream) {
+    TPQ_REQUIRE(dtype == TPQ_DTYPE_F32 || dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16, TPQ_ERR_INVALID_TYPE,
+                "lowbit dequantize: the dense weight must be floating point");
+    if (int rc = check_lowbit("lowbit dequantize", bits, lsb_first, N, K, group)) return rc;
+    if (N == 0 || K == 0) return TPQ_OK;
+    TPQ_REQUIRE(packed && scales_and_zeros && out, TPQ_ERR_INVALID_VALUE, "lowbit dequantize: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t blocks = (N * K + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(blocks > (1 << 20) ? (1 << 20) : blocks);
+    switch (dtype) {
+        case TPQ_DTYPE_F32:
+            lowbit_dequantize_kernel<TPQ_DTYPE_F32><<<grid, 256, 0, s>>>(packed, scales_and_zeros, static_cast<float*>(out), N, K, group, bits, lsb_first);
+            break;
+        case TPQ_DTYPE_F16:
+            lowbit_dequantize_kernel<TPQ_DTYPE_F16><<<grid, 256, 0, s>>>(packed, scales_and_zeros, static_cast<uint16_t*>(out), N, K, group, bits, lsb_first);
+            break;
+        default:
+            lowbit_dequantize_kernel<TPQ_DTYPE_BF16><<<grid, 256, 0, s>>>(packed, scales_and_zeros, static_cast<uint16_t*>(out), N, K, group, bits, lsb_first);
+            break;
+    }
+    return check_launch("tpq_lowbit_dequantize");
+}
+
+TPQ_EXPORT int tpq_lowbit_pack(const uint8_t* codes, int bits, int lsb_first, int64_t rows, int64_t cols, uint8_t* packed, void* stream) {
+    if (int rc = check_lowbit("lowbit pack", bits, lsb_first, rows, cols, 1)) return rc;
+    if (rows == 0 || cols == 0) return TPQ_OK;
+    TPQ_REQUIRE(codes && packed, TPQ_ERR_INVALID_VALUE, "lowbit pack: null pointer");
+    const int per_byte = 8 / bits;
+    const int64_t blocks = (rows * ((cols + per_byte - 1) / per_byte) + 255) / 256;
+    lowbit_pack_kernel<<<static_cast<unsigned>(blocks > (1 << 20) ? (1 << 20) : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        codes, packed, rows, cols, bits, lsb_first);
+    return check_launch("tpq_lowbit_pack");
+}
+
+TPQ_EXPORT int tpq_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, int64_t rows, int64_t cols, uint8_t* codes, void* stream) {
+    if (int rc = check_lowbit("lowbit unpack", bits, lsb_first, rows, cols, 1)) return rc;
+    if (rows == 0 || cols == 0) return TPQ_OK;
+    TPQ_REQUIRE(codes && packed, TPQ_ERR_INVALID_VALUE, "lowbit unpack: null pointer");
+    const int64_t blocks = (rows * cols + 255) / 256;
+    lowbit_unpack_kernel<<<static_cast<unsigned>(blocks > (1 << 20) ? (1 << 20) : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        packed, codes, rows, cols, bits, lsb_first);
+    return check_launch("tpq_lowbit_unpack");
+}

@@ -488,3 +488,94 @@ def dequantize_affine(input, block_size, scales: torch.Tensor, zero_points: Opti
                                                  ctypes.cast(blocks, ctypes.c_void_p), _ptr(sc), sc.numel(), _ptr(zp),
                                                  0 if zp is None else zp.numel(), _ptr(out), _stream(codes)))
     return out
+
+
+# ---- packed n-bit weight-only linear (int2 / intx / binary modules) ------------------------------
+
+LOWBIT_PREFILL_ROWS = 64  # above this many activation rows the weight is dequantised once for the library GEMM
+
+
+def _lowbit_codes(t: torch.Tensor, what: str) -> torch.Tensor:
+    _require_device(t, what)
+    if t.dtype not in (torch.uint8, torch.int8):
+        t = t.to(torch.uint8)
+    return t.contiguous().view(torch.uint8)
+
+
+def pack_lowbit(codes: torch.Tensor, bits: int, lsb_first: bool = False) -> torch.Tensor:
+    """uint8 [..., ceil(cols / (8 // bits))]: ``8 // bits`` codes per byte, the first in the most
+    significant bits (``pack_intx``) or, ``lsb_first``, code i in bit i (``pack_binary``)."""
+    if not 1 <= bits <= 8:
+        raise ValueError(f"bits must be in [1, 8], got {bits}")
+    c = _lowbit_codes(codes, "pack_lowbit")
+    cols = c.shape[-1]
+    rows = c.numel() // cols if cols else 0
+    per_byte = 8 // bits
+    out = torch.empty((*c.shape[:-1], (cols + per_byte - 1) // per_byte), dtype=torch.uint8, device=c.device)
+    with torch.cuda.device(c.device):
+        _check(_lib.load().tpq_lowbit_pack(_ptr(c), bits, int(lsb_first), rows, cols, _ptr(out), _stream(c)))
+    return out
+
+
+def unpack_lowbit(packed: torch.Tensor, bits: int, columns: int, lsb_first: bool = False) -> torch.Tensor:
+    """uint8 codes [..., columns] of a tensor written by ``pack_lowbit``."""
+    if not 1 <= bits <= 8:
+        raise ValueError(f"bits must be in [1, 8], got {bits}")
+    p = _lowbit_codes(packed, "unpack_lowbit")
+    per_byte = 8 // bits
+    if p.shape[-1] != (columns + per_byte - 1) // per_byte:
+        raise ValueError(f"unpack: {p.shape[-1]} bytes per row do not hold {columns} {bits}-bit codes")
+    rows = p.numel() // p.shape[-1] if p.shape[-1] else 0
+    out = torch.empty((*p.shape[:-1], columns), dtype=torch.uint8, device=p.device)
+    with torch.cuda.device(p.device):
+        _check(_lib.load().tpq_lowbit_unpack(_ptr(p), bits, int(lsb_first), rows, columns, _ptr(out), _stream(p)))
+    return out
+
+
+def _lowbit_operands(packed, bits, columns, scales_and_zeros, what):
+    _require_device(packed, what)
+    if packed.dim() != 2 or packed.dtype != torch.uint8:
+        raise TypeError(f"{what}: expected a 2-D uint8 packed weight")
+    per_byte = 8 // bits
+    if packed.shape[1] != (columns + per_byte - 1) // per_byte:
+        raise ValueError(f"{what}: {packed.shape[1]} bytes per row do not hold {columns} {bits}-bit codes")
+    n = packed.shape[0]
+    if scales_and_zeros.dim() != 3 or scales_and_zeros.shape[1] != n or scales_and_zeros.shape[2] != 2 or scales_and_zeros.shape[0] < 1:
+        raise ValueError(f"{what}: scales_and_zeros must be [K / groupsize, N, 2]")
+    if columns % scales_and_zeros.shape[0]:
+        raise ValueError(f"{what}: K={columns} must be divisible by the number of groups {scales_and_zeros.shape[0]}")
+    return packed.contiguous(), scales_and_zeros.to(torch.float32).contiguous(), n, columns // scales_and_zeros.shape[0]
+
+
+def _lowbit_dequantize(packed, bits, columns, scales_and_zeros, dtype=torch.float32, lsb_first=False) -> torch.Tensor:
+    """Dense [N, K] weight ``(code - zero) * scale`` of ``dtype`` (``_dequantize_intx``)."""
+    w, sz, n, group = _lowbit_operands(packed, bits, columns, scales_and_zeros, "_lowbit_dequantize")
+    out = torch.empty((n, columns), dtype=dtype, device=w.device)
+    with torch.cuda.device(w.device):
+        _check(_lib.load().tpq_lowbit_dequantize(_ptr(w), bits, int(lsb_first), n, columns, group, _ptr(sz), _DT[dtype],
+                                                 _ptr(out), _stream(w)))
+    return out
+
+
+def _lowbit_mm(input: torch.Tensor, packed: torch.Tensor, bits: int, columns: int, scales_and_zeros: torch.Tensor,
+               bias: Optional[torch.Tensor] = None, lsb_first: bool = False) -> torch.Tensor:
+    """``input @ dequantize(packed).T (+ bias)`` for a packed n-bit weight, without the dense weight
+    (``_intx_mm`` / ``_int2_mm`` / ``_binary_mm`` of the reference).  input [M, K] f32 / f16 / bf16."""
+    if input.dim() != 2 or input.shape[1] != columns:
+        raise ValueError(f"_lowbit_mm: expected activations [M, {columns}]")
+    if input.dtype not in _DT:
+        raise TypeError("_lowbit_mm: activations must be float32, float16 or bfloat16")
+    _require_device(input, "_lowbit_mm")
+    w, sz, n, group = _lowbit_operands(packed, bits, columns, scales_and_zeros, "_lowbit_mm")
+    x = input.contiguous()
+    m = x.shape[0]
+    b = None if bias is None else bias.to(torch.float32).contiguous()
+    if m > LOWBIT_PREFILL_ROWS:
+        dense = _lowbit_dequantize(w, bits, columns, sz, x.dtype, lsb_first)
+        out = torch.matmul(x, dense.t())
+        return out if b is None else out + b.to(out.dtype)
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(_lib.load().tpq_lowbit_mm(_ptr(x), _DT[x.dtype], m, columns, _ptr(w), bits, int(lsb_first), n, group,
+                                         _ptr(sz), _ptr(b), _ptr(out), _stream(x)))
+    return out

@@ -1,0 +1,256 @@
+"""Packed n-bit weight-only linear (int2 / intx / binary modules of the reference).
+
+CPU: the oracle against numpy restatements of the reference's strided-slice pack / unpack formulas
+(tensorplay/ao/quantization/intx_weight_only.py:35-80, binary.py:50-85) and against x @ dq.T in
+float64.  GPU: the HIP kernels against the oracle: packing bit-exact, the dense weight bit-exact, the
+matmul within the reference tests' own 1e-5 for float32 (test_int2_binary_modules.py:69-89) and 1e-3
+of the float64 sums for fp16.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+
+def ref_pack_msb_first(codes, bits):
+    """pack_intx: per_byte codes per byte, shift 8 - (i + 1) * bits, zero padded."""
+    per_byte = 8 // bits
+    rows, cols = codes.shape
+    padded = -(-cols // per_byte) * per_byte
+    x = np.zeros((rows, padded), np.int32)
+    x[:, :cols] = codes
+    out = np.zeros((rows, padded // per_byte), np.int32)
+    for i in range(per_byte):
+        out |= (x[:, i::per_byte] & ((1 << bits) - 1)) << (8 - (i + 1) * bits)
+    return out.astype(np.uint8)
+
+
+def ref_pack_binary(codes):
+    """pack_binary: code i of each group of eight in bit i."""
+    rows, cols = codes.shape
+    padded = -(-cols // 8) * 8
+    x = np.zeros((rows, padded), np.uint8)
+    x[:, :cols] = codes
+    return sum(((x[:, i::8] & 1) << i) for i in range(8)).astype(np.uint8)
+
+
+def dense_weight(codes, sz, group):
+    """(code - zero) * scale in float32 with sz [G, N, 2]."""
+    s = np.repeat(sz[:, :, 0].T, group, axis=1)
+    z = np.repeat(sz[:, :, 1].T, group, axis=1)
+    return ((codes.astype(np.float32) - z) * s).astype(np.float32)
+
+
+def make_case(rng, bits, N, K, group):
+    codes = rng.integers(0, 1 << bits, (N, K)).astype(np.uint8)
+    sz = np.stack([rng.uniform(0.01, 0.2, (K // group, N)), rng.integers(0, 1 << bits, (K // group, N)).astype(np.float64)],
+                  axis=-1).astype(np.float32)
+    return codes, sz
+
+
+# ---------------------------------------------------------------------------------------------
+# oracle (CPU)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bits", range(1, 9))
+@pytest.mark.parametrize("shape", [(5, 10), (4, 16), (3, 1), (7, 33)])
+def test_oracle_pack_matches_reference_formula(bits, shape):
+    rng = np.random.default_rng(bits * 100 + shape[1])
+    codes = rng.integers(0, 1 << bits, shape).astype(np.uint8)
+    packed = oracle.lowbit_pack(codes, bits)
+    np.testing.assert_array_equal(packed, ref_pack_msb_first(codes, bits))
+    np.testing.assert_array_equal(oracle.lowbit_unpack(packed, bits, shape[1]), codes)
+
+
+def test_oracle_pack_shapes_of_the_reference_tests():
+    rng = np.random.default_rng(0)
+    c2 = rng.integers(0, 4, (5, 10)).astype(np.uint8)
+    assert oracle.lowbit_pack(c2, 2).shape == (5, 3)        # test_int2_binary_modules.py:57-66
+    c1 = rng.integers(0, 2, (4, 10)).astype(np.uint8)
+    p1 = oracle.lowbit_pack(c1, 1, lsb_first=True)
+    assert p1.shape == (4, 2)                               # :129-137
+    np.testing.assert_array_equal(p1, ref_pack_binary(c1))
+    np.testing.assert_array_equal(oracle.lowbit_unpack(p1, 1, 10, lsb_first=True), c1)
+    # one byte by hand: codes 3,0,2,1 -> 0b11001001
+    np.testing.assert_array_equal(oracle.lowbit_pack(np.array([[3, 0, 2, 1]], np.uint8), 2), [[0b11001001]])
+    np.testing.assert_array_equal(oracle.lowbit_pack(np.array([[1, 0, 0, 1, 0, 0, 0, 1]], np.uint8), 1, lsb_first=True), [[0b10001001]])
+
+
+@pytest.mark.parametrize("bits", range(1, 9))
+def test_oracle_mm_matches_float64_product(bits):
+    rng = np.random.default_rng(40 + bits)
+    N, K, group, M = 12, 48, 16, 3
+    codes, sz = make_case(rng, bits, N, K, group)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out, y64, dense = oracle.lowbit_mm(x, "f32", ref_pack_msb_first(codes, bits), bits, sz, K, group, bias=bias,
+                                       want_f64=True, want_dense=True)
+    dq = dense_weight(codes, sz, group)
+    np.testing.assert_array_equal(dense, dq)
+    want = x.astype(np.float64) @ dq.astype(np.float64).T + bias
+    np.testing.assert_allclose(y64, want, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-5)
+
+
+def test_oracle_binary_is_the_sign_times_scale():
+    rng = np.random.default_rng(7)
+    N, K = 6, 20
+    bits01 = rng.integers(0, 2, (N, K)).astype(np.uint8)
+    scale = rng.uniform(0.1, 1.0, (N, 1)).astype(np.float32)
+    sz = np.stack([2 * scale[:, 0], np.full(N, 0.5, np.float32)], axis=-1)[None]
+    dense = oracle.lowbit_mm(None, "f32", ref_pack_binary(bits01), 1, sz, K, K, lsb_first=True, want_dense=True)[1]
+    np.testing.assert_array_equal(dense, (bits01.astype(np.float32) * 2 - 1) * scale)   # binary.py:92-94
+
+
+# ---------------------------------------------------------------------------------------------
+# HIP against the oracle (GPU)
+# ---------------------------------------------------------------------------------------------
+
+DEV = "cuda:0"
+
+
+def rel_err(got, want):
+    return float(np.abs(got.astype(np.float64) - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits", range(1, 9))
+@pytest.mark.parametrize("shape", [(5, 10), (64, 256), (3, 1), (130, 77)])
+def test_gpu_pack_unpack_bit_exact(bits, shape):
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(bits + shape[1])
+    codes = rng.integers(0, 1 << bits, shape).astype(np.uint8)
+    for lsb in ((False, True) if bits == 1 else (False,)):
+        packed = ops.pack_lowbit(torch.from_numpy(codes).to(DEV), bits, lsb_first=lsb)
+        np.testing.assert_array_equal(packed.cpu().numpy(), oracle.lowbit_pack(codes, bits, lsb_first=lsb))
+        back = ops.unpack_lowbit(packed, bits, shape[1], lsb_first=lsb)
+        np.testing.assert_array_equal(back.cpu().numpy(), codes)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits", range(1, 9))
+@pytest.mark.parametrize("N,K,group,M", [(32, 16, 8, 3), (10, 48, 16, 9), (7, 33, 11, 1)])
+def test_gpu_mm_float32_small_shapes(bits, N, K, group, M):
+    """The shapes of the reference's module tests (K=16, N=32, B=3, groupsize 8) and odd ones: plain kernel."""
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(bits * 7 + K)
+    codes, sz = make_case(rng, bits, N, K, group)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    packed = oracle.lowbit_pack(codes, bits)
+    want = oracle.lowbit_mm(x, "f32", packed, bits, sz, K, group, bias=bias, want_f64=True)[1]
+    got = ops._lowbit_mm(torch.from_numpy(x).to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV),
+                         torch.from_numpy(bias).to(DEV))
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,lsb", [(b, False) for b in range(1, 9)] + [(1, True)])
+@pytest.mark.parametrize("N,K,group,M", [(64, 256, 128, 1), (36, 512, 256, 3), (48, 1024, 128, 16), (16, 384, 128, 17), (20, 128, 128, 2)])
+def test_gpu_mm_fp16_decode_kernel(bits, lsb, N, K, group, M):
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(bits * 13 + K + M)
+    codes, sz = make_case(rng, bits, N, K, group)
+    x16 = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).half()
+    bias = rng.standard_normal(N).astype(np.float32) if M % 2 else None
+    packed = oracle.lowbit_pack(codes, bits, lsb_first=lsb)
+    want = oracle.lowbit_mm(x16.view(torch.int16).numpy().view(np.uint16), "f16", packed, bits, sz, K, group, bias=bias,
+                            lsb_first=lsb, want_f64=True)[1]
+    got = ops._lowbit_mm(x16.to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV),
+                         None if bias is None else torch.from_numpy(bias).to(DEV), lsb_first=lsb)
+    assert got.dtype == torch.float16 and got.shape == (M, N)
+    assert rel_err(got.float().cpu().numpy(), want) < 1e-3   # fp16 output rounding is 5e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tdtype", [torch.bfloat16, torch.float16])
+def test_gpu_mm_other_routes(tdtype):
+    """bf16 activations, and N % 4 != 0 / groups that the decode kernel does not take: plain kernel."""
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(5)
+    N, K, group, M = 18, 256, 64, 5
+    codes, sz = make_case(rng, 2, N, K, group)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(tdtype)
+    packed = oracle.lowbit_pack(codes, 2)
+    want = x.double().numpy() @ dense_weight(codes, sz, group).astype(np.float64).T
+    got = ops._lowbit_mm(x.to(DEV), torch.from_numpy(packed).to(DEV), 2, K, torch.from_numpy(sz).to(DEV))
+    assert rel_err(got.float().cpu().numpy(), want) < (1e-2 if tdtype == torch.bfloat16 else 1e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 8])
+def test_gpu_dequantize_bit_exact_and_many_rows(bits):
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(60 + bits)
+    N, K, group = 40, 256, 128
+    codes, sz = make_case(rng, bits, N, K, group)
+    packed = torch.from_numpy(oracle.lowbit_pack(codes, bits)).to(DEV)
+    dense = ops._lowbit_dequantize(packed, bits, K, torch.from_numpy(sz).to(DEV), torch.float32)
+    np.testing.assert_array_equal(dense.cpu().numpy(), dense_weight(codes, sz, group))
+    dense16 = ops._lowbit_dequantize(packed, bits, K, torch.from_numpy(sz).to(DEV), torch.float16)
+    np.testing.assert_array_equal(dense16.cpu().numpy(), dense_weight(codes, sz, group).astype(np.float16))
+    M = ops.LOWBIT_PREFILL_ROWS + 5   # dequantise + library GEMM
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32))
+    got = ops._lowbit_mm(x.to(DEV), packed, bits, K, torch.from_numpy(sz).to(DEV))
+    want = x.double().numpy() @ dense_weight(codes, sz, group).astype(np.float64).T
+    assert rel_err(got.cpu().numpy(), want) < 1e-5
+
+
+@pytest.mark.gpu
+def test_gpu_modules_follow_the_reference_tests():
+    """from_float + forward against the manual group-wise formula, as test_int2_binary_modules.py:69-89, 140-155."""
+    import torch.nn as nn
+    from tensorplay_amd.ao import quantization as q
+    torch.manual_seed(0)
+    x = torch.randn(3, 16, device=DEV)
+    lin = nn.Linear(16, 32, bias=False).to(DEV)
+
+    mod = q.WeightOnlyInt2Linear.from_float(lin, groupsize=8)
+    assert mod.weight.dtype == torch.uint8 and mod.weight.shape == (32, 4) and mod.scales_and_zeros.shape == (2, 32, 2)
+    scale = mod.scales_and_zeros[..., 0].t().contiguous().repeat_interleave(8, dim=-1)
+    zero = mod.scales_and_zeros[..., 1].t().contiguous().repeat_interleave(8, dim=-1)
+    dq = (q.unpack_int2(mod.weight, 16).float() - zero) * scale
+    torch.testing.assert_close(mod(x), x @ dq.T, atol=1e-5, rtol=1e-5)
+    assert set(dq.div(scale).round().unique().tolist()) <= {-2.0, -1.0, 0.0, 1.0}
+
+    modb = q.WeightOnlyBinaryLinear.from_float(lin)
+    assert modb.weight.shape == (32, 2) and modb.scale.shape == (32, 1)
+    dqb = (q.unpack_binary(modb.weight, 16).float() * 2.0 - 1.0) * modb.scale
+    torch.testing.assert_close(modb(x), x @ dqb.T, atol=1e-5, rtol=1e-5)
+    assert float((dqb.abs() - modb.scale).abs().max()) < 1e-5
+
+    for bits in (1, 3, 4, 8):
+        modx = q.WeightOnlyIntxLinear.from_float(nn.Linear(16, 32, bias=True).to(DEV), bits=bits, groupsize=8)
+        s = modx.scales_and_zeros[..., 0].t().contiguous().repeat_interleave(8, dim=-1)
+        z = modx.scales_and_zeros[..., 1].t().contiguous().repeat_interleave(8, dim=-1)
+        codes = q.unpack_intx(modx.weight, bits, 16).view(torch.uint8).float()
+        torch.testing.assert_close(modx(x), x @ ((codes - z) * s).T + modx.bias, atol=1e-5, rtol=1e-5)
+
+    model = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Linear(32, 8)).to(DEV)
+    qmodel = q.quantize_(model, q.int2_weight_only(groupsize=8))
+    assert isinstance(qmodel[0], q.WeightOnlyInt2Linear) and isinstance(qmodel[2], q.WeightOnlyInt2Linear)
+    assert qmodel(x).shape == (3, 8)
+    assert isinstance(q.quantize_binary_weight_only(nn.Sequential(nn.Linear(16, 16)).to(DEV))[0], q.WeightOnlyBinaryLinear)
+    assert isinstance(q.quantize_intx_weight_only(nn.Sequential(nn.Linear(16, 16)).to(DEV), bits=3, groupsize=8)[0], q.WeightOnlyIntxLinear)
+
+
+@pytest.mark.gpu
+def test_gpu_full_size_int2_decode_linearity():
+    """4096 -> 11008 at 2 bits, fp16, one row: the sum of two activation vectors maps to the sum of the outputs
+    (up to fp16 rounding), and a slice of channels matches the oracle."""
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(77)
+    N, K, group = 11008, 4096, 128
+    codes, sz = make_case(rng, 2, N, K, group)
+    sz[..., 0] *= 0.1
+    packed = oracle.lowbit_pack(codes, 2)
+    xa = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).half()
+    xb = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).half()
+    args = (torch.from_numpy(packed).to(DEV), 2, K, torch.from_numpy(sz).to(DEV))
+    ya, yb = ops._lowbit_mm(xa.to(DEV), *args).float(), ops._lowbit_mm(xb.to(DEV), *args).float()
+    yab = ops._lowbit_mm((xa.float() + xb.float()).half().to(DEV), *args).float()
+    assert float((yab - (ya + yb)).abs().max() / (ya + yb).abs().max()) < 5e-3
+    rows = slice(5000, 5064)
+    want = oracle.lowbit_mm(xa.view(torch.int16).numpy().view(np.uint16), "f16", packed[rows], 2, sz[:, rows], K, group, want_f64=True)[1]
+    assert rel_err(ya[:, rows].cpu().numpy(), want) < 1e-3
