@@ -234,7 +234,7 @@ def main() -> int:
     x_d = torch.from_numpy(x).to(dev).half()
     sz_d = torch.from_numpy(sz).to(dev).half().contiguous()
     packed0 = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(dev), 2)
-    copies = 26  # 26 x (22.5 + 1.4) MB = 622 MB: far beyond L2 + the 256 MB last-level cache
+    copies = 64  # 64 x (22.5 + 1.4) MB = 1.53 GB: far beyond L2 + the 256 MB last-level cache
     packs = [packed0] + [packed0.clone() for _ in range(copies - 1)]
     szs = [sz_d] + [sz_d.clone() for _ in range(copies - 1)]
     y_d = torch.empty((M, N), dtype=torch.float16, device=dev)
@@ -280,6 +280,9 @@ def main() -> int:
     gbs = GEMV_BYTES / (ms_per_step * 1e-3) / 1e9
 
     extras = {"gemv_max_rel_err_vs_fp64": gpu_err, "graph_wall_ms_per_step": wall_ms / steps}
+    if not args.no_extras:  # the same graph seven more times: median step time
+        reps = sorted(time_region(g.replay, sync, 1) / steps for _ in range(7))
+        extras["int4_gemv_us_median_of_7_replays"] = reps[3] * 1e3
     if args.calibrate_copy:
         src_c = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst_c = torch.empty_like(src_c)
@@ -345,16 +348,16 @@ def main() -> int:
         yb = torch.empty((1, N), dtype=torch.float16, device=dev)
         for bits in (1, 2, 4, 8):
             row_bytes = K * bits // 8
-            copies = max(2, min(60, (600 << 20) // (N * row_bytes)))
-            wl = [torch.randint(0, 256, (N, row_bytes), dtype=torch.uint8, device=dev) for _ in range(copies)]
+            n_copies = max(2, min(60, (600 << 20) // (N * row_bytes)))
+            wl = [torch.randint(0, 256, (N, row_bytes), dtype=torch.uint8, device=dev) for _ in range(n_copies)]
 
-            def lbmm(i, wl=wl, bits=bits, copies=copies):
-                lib.tpq_lowbit_mm(xb.data_ptr(), _lib.F16, 1, K, wl[i % copies].data_ptr(), bits, 0, N, 128,
+            def lbmm(i, wl=wl, bits=bits, n_copies=n_copies):
+                lib.tpq_lowbit_mm(xb.data_ptr(), _lib.F16, 1, K, wl[i % n_copies].data_ptr(), bits, 0, N, 128,
                                   szf.data_ptr(), None, yb.data_ptr(), cur())
 
-            gl = graph_of(lambda: [lbmm(i) for i in range(2 * copies)])
+            gl = graph_of(lambda: [lbmm(i) for i in range(2 * n_copies)])
             gl.replay(); sync()
-            ms = time_region(gl.replay, sync, 1) / (2 * copies)
+            ms = time_region(gl.replay, sync, 1) / (2 * n_copies)
             extras[f"lowbit{bits}_M1_us"] = ms * 1e3
             extras[f"lowbit{bits}_M1_GBs"] = (N * row_bytes + 8 * G * N + 2 * K + 2 * N) / (ms * 1e-3) / 1e9
             del wl
