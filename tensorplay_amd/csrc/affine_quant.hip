@@ -399,8 +399,8 @@ __global__ __launch_bounds__(256) void dequantize_pieces_kernel(const void* __re
         for (int j = 0; j < kFlight; ++j) {
             const int64_t p = p0 + j * stride;
             if (p < pieces)
-                reinterpret_cast<float4*>(out)[p] = make_float4(dequantize_one(q[j][0], scale[j], zero[j]), dequantize_one(q[j][1], scale[j], zero[j]),
-                                                                 dequantize_one(q[j][2], scale[j], zero[j]), dequantize_one(q[j][3], scale[j], zero[j]));
+                nt_store(reinterpret_cast<float4*>(out) + p, dequantize_one(q[j][0], scale[j], zero[j]), dequantize_one(q[j][1], scale[j], zero[j]),
+                         dequantize_one(q[j][2], scale[j], zero[j]), dequantize_one(q[j][3], scale[j], zero[j]));
         }
     }
 }
@@ -408,10 +408,11 @@ __global__ __launch_bounds__(256) void dequantize_pieces_kernel(const void* __re
 template <int DT>
 __device__ __forceinline__ void load_piece_floats(const void* x, int64_t p, float v[4]) {
     if constexpr (DT == TPQ_DTYPE_F32) {
-        const float4 t = static_cast<const float4*>(x)[p];
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        const uint4 t = nt_load(static_cast<const uint4*>(x) + p);
+        v[0] = __builtin_bit_cast(float, t.x); v[1] = __builtin_bit_cast(float, t.y);
+        v[2] = __builtin_bit_cast(float, t.z); v[3] = __builtin_bit_cast(float, t.w);
     } else {
-        const uint2 t = static_cast<const uint2*>(x)[p];
+        const uint2 t = nt_load(static_cast<const uint2*>(x) + p);
         v[0] = Elem<DT>::load(static_cast<uint16_t>(t.x)); v[1] = Elem<DT>::load(static_cast<uint16_t>(t.x >> 16));
         v[2] = Elem<DT>::load(static_cast<uint16_t>(t.y)); v[3] = Elem<DT>::load(static_cast<uint16_t>(t.y >> 16));
     }

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     auto load = [&](int s, Step& st) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            st.w[b] = w_base[b][static_cast<size_t>(s) * 32];                       // four k-tiles further per step
+            st.w[b] = nt_load(w_base[b] + static_cast<size_t>(s) * 32);             // four k-tiles further per step
             st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
         }
 #pragma unroll

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
     auto issue = [&](Chunk<MROWS, kGroups>& ch, int chunk) {
         chunk = chunk < n_chunks ? chunk : n_chunks - 1;  // past the end: harmless re-read, never used
 #pragma unroll
-        for (int i = 0; i < kChunkKT; ++i) ch.q[i] = wp[static_cast<size_t>(chunk * kChunkKT + i) * 8];
+        for (int i = 0; i < kChunkKT; ++i) ch.q[i] = nt_load(wp + static_cast<size_t>(chunk * kChunkKT + i) * 8);
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) ch.p[g] = szp[static_cast<size_t>(chunk * kGroups + g) * N];
 #pragma unroll

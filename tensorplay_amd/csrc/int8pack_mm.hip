@@ -48,8 +48,8 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
         uint4 xv[4];
     };
     auto load = [&](int s, Step& st) {
-        st.w[0] = w_base[s * 8];
-        st.w[1] = w_base[s * 8 + 1];
+        st.w[0] = nt_load(w_base + s * 8);
+        st.w[1] = nt_load(w_base + s * 8 + 1);
 #pragma unroll
         for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
     };

@@ -96,9 +96,9 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     };
     auto load = [&](int s, Step& st) {
         const uint8_t* src = w_base + static_cast<size_t>(s) * (4 * F::kBytes);
-        if constexpr (F::kBytes == 16) st.w = *reinterpret_cast<const uint4*>(src);
-        if constexpr (F::kBytes == 8) { const uint2 t = *reinterpret_cast<const uint2*>(src); st.w = make_uint4(t.x, t.y, 0, 0); }
-        if constexpr (F::kBytes == 4) st.w = make_uint4(*reinterpret_cast<const uint32_t*>(src), 0, 0, 0);
+        if constexpr (F::kBytes == 16) st.w = nt_load(reinterpret_cast<const uint4*>(src));
+        if constexpr (F::kBytes == 8) { const uint2 t = nt_load(reinterpret_cast<const uint2*>(src)); st.w = make_uint4(t.x, t.y, 0, 0); }
+        if constexpr (F::kBytes == 4) st.w = make_uint4(nt_load(reinterpret_cast<const uint32_t*>(src)), 0, 0, 0);
         const uint4* prm = reinterpret_cast<const uint4*>(sz_base + static_cast<size_t>(s >> group_shift) * N * 2);
         st.p[0] = prm[0];
         st.p[1] = prm[1];

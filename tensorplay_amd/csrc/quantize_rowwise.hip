@@ -70,12 +70,13 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
 template <int DT>
 __device__ __forceinline__ void load_chunk(const typename Elem<DT>::storage* p, float (&v)[kVec]) {
     if constexpr (DT == TPQ_DTYPE_F32) {
-        const float4 a = reinterpret_cast<const float4*>(p)[0];
-        const float4 b = reinterpret_cast<const float4*>(p)[1];
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        const uint4 a = nt_load(reinterpret_cast<const uint4*>(p)), b = nt_load(reinterpret_cast<const uint4*>(p) + 1);
+        v[0] = __builtin_bit_cast(float, a.x); v[1] = __builtin_bit_cast(float, a.y);
+        v[2] = __builtin_bit_cast(float, a.z); v[3] = __builtin_bit_cast(float, a.w);
+        v[4] = __builtin_bit_cast(float, b.x); v[5] = __builtin_bit_cast(float, b.y);
+        v[6] = __builtin_bit_cast(float, b.z); v[7] = __builtin_bit_cast(float, b.w);
     } else {
-        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint4 raw = nt_load(reinterpret_cast<const uint4*>(p));
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {

