@@ -87,7 +87,7 @@ __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
 #pragma unroll
         for (int i = 0; i < kChunkKT; ++i) ch.q[i] = nt_load(wp + static_cast<size_t>(chunk * kChunkKT + i) * 8);
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) ch.p[g] = szp[static_cast<size_t>(chunk * kGroups + g) * N];
+        for (int g = 0; g < kGroups; ++g) ch.p[g] = nt_load(szp + static_cast<size_t>(chunk * kGroups + g) * N);
 #pragma unroll
         for (int m = 0; m < MROWS; ++m) ch.xw[m] = x[static_cast<size_t>(m) * words_per_row + chunk * 64 + lane];
     };

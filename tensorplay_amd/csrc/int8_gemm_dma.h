@@ -501,7 +501,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         const char* srcp = lds_bytes + row * kPitch + col * sizeof(out_t);
         out_t* dstp = tile.out + static_cast<size_t>(m) * N + n;
         if (vector_stores && n + kPerChunk <= N) {
-            *reinterpret_cast<uint4*>(dstp) = *reinterpret_cast<const uint4*>(srcp);
+            nt_store(reinterpret_cast<uint4*>(dstp), *reinterpret_cast<const uint4*>(srcp));  // written once, read by a later kernel
         } else {
             for (int e = 0; e < kPerChunk && n + e < N; ++e) dstp[e] = reinterpret_cast<const out_t*>(srcp)[e];
         }

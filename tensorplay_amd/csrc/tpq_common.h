@@ -97,6 +97,12 @@ __device__ __forceinline__ void nt_store(float4* p, float a, float b, float c, f
     __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
 }
 
+__device__ __forceinline__ void nt_store(uint4* p, const uint4& v) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const u4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<u4*>(p));
+}
+
 // ---- 64-lane reductions -----------------------------------------------------
 
 __device__ __forceinline__ float wave_max(float v) {
