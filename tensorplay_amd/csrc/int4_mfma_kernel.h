@@ -83,8 +83,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         sz_base[b] = sz + n4;
     }
     const bool row_live = i < M;
-    // columns m >= M repeat the last row: their products are computed and never stored
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : M - 1) * K) + q * 4;
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 4;
 
     // constant A of the correction MFMA: row 0 = offset + 8 of the pair parity, row 1 = ones
     uint32_t a_corr_even = 0, a_corr_odd = 0;
@@ -105,8 +104,10 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
             st.w[b] = nt_load(w_base[b] + static_cast<size_t>(s) * 32);             // four k-tiles further per step
             st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
         }
+        if (row_live) {  // columns m >= M keep the zeros they start with: no load, nothing stored
 #pragma unroll
-        for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
+            for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
+        }
     };
 
     float yacc[NB][4];
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     };
 
     // this wavefront's steps: wave, wave + WAVES, ...; two in flight
-    Step s0, s1;
+    Step s0 = {}, s1 = {};
     int s = wave;
     if (s < steps) load(s, s0);
     if (s + WAVES < steps) load(s + WAVES, s1);
