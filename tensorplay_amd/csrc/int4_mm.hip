@@ -400,7 +400,8 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     // but only when N still yields enough of them to fill the chip.  Measured (us, weights from
     // HBM): N=11008 K=4096: 4 rows 9.6 (16 ch, 8 waves); 8 rows 10.9 (64 ch) vs 11.3 (16 ch);
     // 16 rows 11.8 (64 ch) vs 16.7 (16 ch).  N=4096 K=4096: 8 rows 5.7 (16 ch) vs 9.9 (64 ch).
-    int nb = (rows > 4 && N >= 8192) ? 4 : 1;
+    // 4 rows at N=11008: 32 ch x 4 waves 9.06, 64 ch x 4 waves 9.32, 16 ch x 8 waves 9.68 us
+    int nb = N >= 8192 ? (rows > 4 ? 4 : 2) : 1;
     if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
     int waves = nb == 1 && rows <= 8 ? 8 : 4;
     if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
