@@ -34,9 +34,9 @@ INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 M, K, N, GROUP = 1, 4096, 11008, 128
 GEMV_BYTES = N * K // 2 + (K // GROUP) * N * 4 + 2 * M * K + 2 * M * N   # 23,983,616
 # HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
-# by what the same counter reads for a 256 MiB device copy (--calibrate-copy): 11770.35 KiB x 1.99981
+# by what the same counter reads for a 256 MiB device copy (--calibrate-copy): 11770.35 KiB x 1.99973
 # fetched + 21.50 KiB x 1.0 written.  Summary: profiles/int4_decode_gemv_M1_K4096_N11008.md
-MEASURED_TRAFFIC_BYTES = 24_125_400
+MEASURED_TRAFFIC_BYTES = 24_120_100
 
 
 def asym_quant_int4(w, group):
@@ -108,7 +108,27 @@ def cpu_baseline(x16, codes, sz16, want, budget_s=12.0):
             break
     pool.shutdown()
     per_call = dt / calls
+    # the library twin the reference benchmarks its CPU op against (test_native_operator_families.py:579-599):
+    # PyTorch's own CPU int4 kernel on the same codes, default thread count, a few seconds
+    twin = None
+    try:
+        import torch
+
+        if hasattr(torch, "_weight_int4pack_mm_for_cpu"):
+            szt = torch.from_numpy(sz16.view(np.float16).astype(np.float32)).half()
+            xt = torch.from_numpy(x16.view(np.float16).copy())
+            pk = torch._convert_weight_to_int4pack_for_cpu(torch.from_numpy(codes.astype(np.int32)), 1)
+            torch._weight_int4pack_mm_for_cpu(xt, pk, GROUP, szt)
+            t1 = time.perf_counter()
+            n_twin = 0
+            while time.perf_counter() - t1 < 3.0:
+                torch._weight_int4pack_mm_for_cpu(xt, pk, GROUP, szt)
+                n_twin += 1
+            twin = {"GBs": round(GEMV_BYTES / ((time.perf_counter() - t1) / n_twin) / 1e9, 3), "threads": torch.get_num_threads()}
+    except Exception as exc:  # the twin is a side figure: never fail the benchmark over it
+        twin = {"error": str(exc)[:120]}
     return {
+        "torch_cpu_twin": twin,
         "value": round(GEMV_BYTES / per_call / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
