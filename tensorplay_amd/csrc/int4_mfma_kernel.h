@@ -2,19 +2,21 @@
 // group a multiple of 128, K % 128 == 0): every packed byte is read once for
 // all rows, and the multiply-accumulate work leaves the vector ALU.
 //
-// v_mfma_f32_16x16x16 computes D[i][j] += sum_k A[i][k] B[k][j] with lane
-// l = (i or j) + 16 q holding the four k-slots 4q..4q+3 of its row / column.
+// v_mfma_f32_16x16x32 computes D[i][j] += sum_k A[i][k] B[k][j] with lane
+// l = (i or j) + 16 q holding the eight k-slots 8q..8q+7 of its row / column.
 // Which actual k sits in a slot is free as long as A and B agree, and that is
 // what makes the packed layout usable without any shuffle:
 //   * A = weights.  Lane (i, q) owns row n0 + i and, in a step of four k-tiles
 //     (128 k), the k-tile 4 s + q: one 16-byte load = the row's four words =
 //     all 32 k of that tile.  A word unpacks in place into four 16-bit pairs
-//     (magic + code, see int4_lane.h); pair j of words r and r + 1 is k = 2r + 8j
-//     .. + 3, the A operand of one MFMA, eight MFMAs per step and 16 rows.
+//     (magic + code, see int4_lane.h); pair j of word r is k = 2r + 8j, + 1, and
+//     pair j of the four words is the A operand of MFMA j: four MFMAs per step
+//     and 16 rows.
 //   * B = activations.  Lane (m, q) loads the 64 bytes x[m][32 (4s+q) .. +32)
-//     and the operand of MFMA u is simply dwords 2u and 2u + 1 of them, the same
-//     four k as the weight pairs.  Columns m >= M repeat row M-1 and are dropped.
-//   * One more MFMA per four k with a constant A (row 0: the magic offsets + 8,
+//     and the operand of MFMA j is simply dwords 4j .. 4j+3 of them (k = 8j ..
+//     8j+7, the same eight k as the weight pairs), one 16-byte load.  Columns
+//     m >= M stay zero and are dropped.
+//   * One more MFMA per eight k with a constant A (row 0: the magic offsets + 8,
 //     row 1: ones) yields, per activation row, corr = sum x (offset + 8) and
 //     sx = sum x over the step; they come out in lanes 0..15 and are broadcast
 //     with two cross-lane reads.
@@ -34,22 +36,24 @@ namespace {
 // dword r of a 16-byte vector; r is a constant once the loops around the call are unrolled
 __device__ __forceinline__ uint32_t dword_of(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
 
+typedef uint32_t word4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+
 template <int DT>
 struct MfmaLane;
 template <>
 struct MfmaLane<TPQ_DTYPE_F16> {
     static constexpr uint32_t kOffEven = 0x64086408u, kOffOdd = 0x54805480u, kOnes = 0x3C003C00u;  // 1032, 72, 1
-    static __device__ __forceinline__ float4_t mfma(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
-        const word2_t a = {a0, a1}, b = {b0, b1};
-        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
+    static __device__ __forceinline__ float4_t mfma(const word4_t& a, const word4_t& b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
     }
 };
 template <>
 struct MfmaLane<TPQ_DTYPE_BF16> {
     static constexpr uint32_t kOffEven = 0x43084308u, kOffOdd = 0x43084308u, kOnes = 0x3F803F80u;  // 136, 136, 1
-    static __device__ __forceinline__ float4_t mfma(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
-        const word2_t a = {a0, a1}, b = {b0, b1};
-        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+    static __device__ __forceinline__ float4_t mfma(const word4_t& a, const word4_t& b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a), __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
     }
 };
 
@@ -117,7 +121,6 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         for (int v = 0; v < 4; ++v) yacc[b][v] = 0.0f;
 
     auto compute = [&](const Step& st) {
-        auto xd = [&](int k) { return dword_of(st.xv[k >> 2], k & 3); };  // dword k of the lane's 64 activation bytes
         // the correction product and the weight products alternate, so that no MFMA waits for
         // the one issued just before it
         float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -129,15 +132,19 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int r = 0; r < 4; ++r) L::template unpack<true>(dword_of(st.w[b], r), v[b][r], magic_even, magic_odd);
-        // MFMA u covers k = 4u .. 4u+3 of the k-tile: B is dwords 2u, 2u+1 of the activations (adjacent
-        // registers of one load), A is pair j = u/2 of words r0 = 2 (u%2) and r0 + 1.
+        // MFMA u (16x16x32) covers pair u of the four words of the lane's k-tile: k = 2 r + 8 u, + 1 for
+        // r = 0..3, which are dwords 4u .. 4u+3 of the activations, one 16-byte load.
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int r0 = 2 * (u & 1), j = u >> 1;
-            const bool odd = j & 1;
-            aux = ML::mfma(odd ? a_corr_odd : a_corr_even, odd ? a_corr_odd : a_corr_even, xd(2 * u), xd(2 * u + 1), aux);
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t off = (u & 1) ? a_corr_odd : a_corr_even;
+            const word4_t xb = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
+            const word4_t ac = {off, off, off, off};
+            aux = ML::mfma(ac, xb, aux);
 #pragma unroll
-            for (int b = 0; b < NB; ++b) d[b] = ML::mfma(v[b][r0][j], v[b][r0 + 1][j], xd(2 * u), xd(2 * u + 1), d[b]);
+            for (int b = 0; b < NB; ++b) {
+                const word4_t aw = {v[b][0][u], v[b][1][u], v[b][2][u], v[b][3][u]};
+                d[b] = ML::mfma(aw, xb, d[b]);
+            }
         }
         // rows 0 and 1 of the correction product sit in lanes 0..15, registers 0 and 1
         const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);

@@ -8,14 +8,14 @@
 // buffer the modules keep (intx_weight_only.py:167-170).  The reference unpacks with tensor ops,
 // dequantizes to a dense float weight and calls a float GEMM (_intx_mm, intx_weight_only.py:127-133).
 //
-// Decode kernel (fp16 activations, 1..16 rows): v_mfma_f32_16x16x16_f16 with the weights as A.  Lane
+// Decode kernel (fp16 activations, 1..16 rows): v_mfma_f32_16x16x32_f16 with the weights as A.  Lane
 // (i, q) owns weight row n0 + i and, per step, 32 consecutive codes of it (16 when a code has a byte
 // to itself): 4 to 16 bytes, one load.  A code becomes an fp16 number without leaving its bits: the
 // byte is copied into both halves of a dword (v_perm_b32), a mask keeps one field per half and an
 // exponent is or-ed in, chosen so that the field's position in the mantissa has weight one: a field at
 // bit p under exponent 2^(10-p) reads 2^(10-p) + code.  Two neighbouring codes per dword, so the B
 // operand is simply the activations as they lie in memory.  The offsets 2^(10-p) leave through one
-// more MFMA per four k whose A is constant (row 0: the offsets, row 1: ones -> sum of x), and a step
+// more MFMA per eight k whose A is constant (row 0: the offsets, row 1: ones -> sum of x), and a step
 // stays inside one quantization group:  y += scale * ((D - offsets) - zero * sum x).
 //
 // Everything else (fp32 / bf16 activations, odd K or group sizes) takes a plain kernel: one workgroup
@@ -28,6 +28,9 @@
 namespace tpq {
 namespace {
 
+typedef uint32_t word4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
 // dword r of a 16-byte vector; r is a constant once the loops around the call are unrolled
 __device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
 
@@ -37,7 +40,6 @@ struct Fields {
     static constexpr int kCodes = kPerByte >= 2 ? 32 : 16;  // per lane and step
     static constexpr int kBytes = kCodes / kPerByte;        // 4, 8 or 16
     static constexpr int kStepK = 4 * kCodes;
-    static constexpr int kVariants = kPerByte == 8 ? 2 : 1;  // distinct offset patterns of an MFMA's four k
     static constexpr uint32_t kField = (1u << BITS) - 1u;
     // bit position of code i of a byte
     static constexpr int pos(int i) { return LSB ? i * BITS : 8 - (i + 1) * BITS; }
@@ -76,15 +78,11 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     // columns m >= M repeat the last row: their products are computed and never stored
     const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : M - 1) * K + q * F::kCodes);
 
-    // constant A of the offset MFMA: row 0 = the offsets of the four k of an MFMA, row 1 = ones
-    uint32_t a_corr[F::kVariants][2];
+    // constant A of the offset MFMA: row 0 = the offsets of the eight k of an MFMA (pairs 0..3 of the
+    // lane's codes: the pattern repeats every byte, so every MFMA has the same), row 1 = ones
+    uint32_t a_corr[4];
 #pragma unroll
-    for (int var = 0; var < F::kVariants; ++var)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int t = 2 * var + h;  // pair t of the lane's codes has the pattern of pair t + 2 * kVariants, ...
-            a_corr[var][h] = i == 0 ? F::magic(t) : i == 1 ? 0x3C003C00u : 0u;
-        }
+    for (int h = 0; h < 4; ++h) a_corr[h] = i == 0 ? F::magic(h) : i == 1 ? 0x3C003C00u : 0u;
     uint32_t magic[F::kMagics];  // kept in VGPRs behind opaque moves: v_and_or_b32 takes one scalar operand
 #pragma unroll
     for (int t = 0; t < F::kMagics; ++t) asm volatile("v_mov_b32 %0, %1" : "=v"(magic[t]) : "s"(F::magic(t)));
@@ -110,19 +108,19 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     auto compute = [&](const Step& st) {
         float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f}, d = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int u = 0; u < F::kCodes / 4; ++u) {  // MFMA u: codes 4u .. 4u+3 of the lane
-            uint32_t a[2];
+        for (int u = 0; u < F::kCodes / 8; ++u) {  // MFMA u (16x16x32): codes 8u .. 8u+7 of the lane
+            uint32_t a[4];
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int t = 2 * u + h;
+            for (int h = 0; h < 4; ++h) {
+                const int t = 4 * u + h;
                 const uint32_t word = dword_at(st.w, F::byte_lo(t) >> 2);
                 const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
                 a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
             }
-            const uint32_t b0 = dword_at(st.xv[u >> 1], (2 * u) & 3), b1 = dword_at(st.xv[u >> 1], (2 * u + 1) & 3);
-            const word2_t av = {a[0], a[1]}, cv = {a_corr[u % F::kVariants][0], a_corr[u % F::kVariants][1]}, bv = {b0, b1};
-            aux = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, cv), __builtin_bit_cast(half4_t, bv), aux, 0, 0, 0);
-            d = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, av), __builtin_bit_cast(half4_t, bv), d, 0, 0, 0);
+            const word4_t av = {a[0], a[1], a[2], a[3]}, cv = {a_corr[0], a_corr[1], a_corr[2], a_corr[3]};
+            const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};  // the same eight k of the activations
+            aux = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, cv), __builtin_bit_cast(half8_t, bv), aux, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
         }
         // rows 0 and 1 of the offset product sit in lanes 0..15, registers 0 and 1
         const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
