@@ -3,7 +3,7 @@
 // activations converted to fp32, fp32 accumulation, per-row scale applied to the sum).
 //
 // Decode kernel (fp16 activations, K % 128 == 0, 1..16 rows per launch), bandwidth bound at one byte
-// per weight: v_mfma_f32_16x16x16_f16 with the weights as A and the activations as B, as in the int4
+// per weight: v_mfma_f32_16x16x32_f16 with the weights as A and the activations as B, as in the int4
 // decode kernel for several rows.  Lane (i, q) owns weight row n0 + i and, in a step of 128 k, the 32
 // bytes at k = 128 s + 32 q: two 16-byte loads, whole 128-byte lines per row and step.  Every dword
 // (four int8) becomes two fp16 pairs: xor 0x80808080 turns the bytes into b + 128, v_perm_b32 drops
@@ -20,6 +20,9 @@ namespace {
 
 constexpr int kI8Waves = 2;
 constexpr int kI8Ring = 2;  // steps in flight per wavefront
+
+typedef uint32_t word4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
 
@@ -56,16 +59,20 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
     float4_t d0 = {0.0f, 0.0f, 0.0f, 0.0f}, d1 = {0.0f, 0.0f, 0.0f, 0.0f};
     auto compute = [&](const Step& st) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {  // MFMA u: k = 4u .. 4u+3 of the lane's 32
-            const uint32_t t = dword_at(st.w[u >> 2], u & 3) ^ 0x80808080u;
-            const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
-            const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
-            const uint32_t a0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
-            const uint32_t a1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
-            const uint32_t b0 = dword_at(st.xv[u >> 1], (2 * u) & 3), b1 = dword_at(st.xv[u >> 1], (2 * u + 1) & 3);
-            const word2_t a = {a0, a1}, b = {b0, b1};
-            if (u & 1) d1 = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), d1, 0, 0, 0);
-            else d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), d0, 0, 0, 0);
+        for (int u = 0; u < 4; ++u) {  // MFMA u (16x16x32): k = 8u .. 8u+7 of the lane's 32
+            uint32_t a[4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t t = dword_at(st.w[u >> 1], (2 * u + h) & 3) ^ 0x80808080u;
+                const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
+                const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
+                a[2 * h] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
+                a[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
+            }
+            const word4_t av = {a[0], a[1], a[2], a[3]};
+            const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
+            if (u & 1) d1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d1, 0, 0, 0);
+            else d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d0, 0, 0, 0);
         }
     };
 
