@@ -517,13 +517,8 @@ int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
     auto kernel = int8_gemm_dma_kernel<Tile, KSPLIT>;
-    static bool configured = false;  // per instantiation: raise the dynamic LDS limit once
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-        if (e != hipSuccess) return fail(TPQ_ERR_RUNTIME, "int8 gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};  // per instantiation
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int8 gemm")) return rc;
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
     kernel<<<dim3(static_cast<unsigned>(tiles)), 256 * KSPLIT, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
                                                                  static_cast<int>(K), tile, vector_stores);

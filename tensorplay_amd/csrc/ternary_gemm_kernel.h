@@ -136,13 +136,8 @@ int launch_ternary_gemm_tile(const int8_t* x, const uint8_t* packed, int64_t M, 
     constexpr size_t part_bytes = static_cast<size_t>(16 - BM / 32) * 16 * kWave * sizeof(int);
     constexpr size_t smem = stage_bytes > part_bytes ? stage_bytes : part_bytes;
     auto kernel = ternary_gemm_m128_kernel<BM, Epilogue>;
-    static bool configured = false;  // per instantiation: raise the dynamic LDS limit once
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-        if (e != hipSuccess) return fail(TPQ_ERR_RUNTIME, "ternary gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};  // per instantiation
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "ternary gemm")) return rc;
     const int64_t gx = (N + kTgN - 1) / kTgN, gy = (M + BM - 1) / BM;
     TPQ_REQUIRE(gx <= 0x7FFFFFFF && gy <= 65535, TPQ_ERR_INVALID_VALUE, "ternary gemm: shape too large");
     kernel<<<dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)), kTgThreads, smem, s>>>(

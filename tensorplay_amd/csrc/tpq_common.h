@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -29,6 +30,19 @@ inline int check_launch(const char* what) {
     do {                                                \
         if (!(cond)) return ::tpq::fail(code, __VA_ARGS__); \
     } while (0)
+
+// Raises a kernel's dynamic LDS limit once per device; `done` is a bit per device id, one
+// word per kernel instantiation.  Safe to call from several threads.
+inline int ensure_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint64_t>& done, const char* what) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(TPQ_ERR_RUNTIME, "%s: no current device", what);
+    const uint64_t bit = uint64_t{1} << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return TPQ_OK;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+    if (e != hipSuccess) return fail(TPQ_ERR_RUNTIME, "%s: cannot reserve %zu bytes of LDS: %s", what, bytes, hipGetErrorString(e));
+    done.fetch_or(bit, std::memory_order_release);
+    return TPQ_OK;
+}
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
