@@ -92,5 +92,58 @@ for K in (3, 31, 32, 65):
     v[f"packed_K{K}_offsets"] = wcodes.astype(np.int64).sum(1)
     v[f"packed_K{K}_acc"] = (xcodes.astype(np.int64) @ wcodes.astype(np.int64).T).astype(np.int32)
 
+# ---- int8 weight-only matmul: the literal example of test/test_mps.py:1052-1061 and a seeded case --
+a_lit = np.array([[1., 2., 3., 4.], [-1., 0.5, 2., -3.]], np.float32)
+w_lit = np.array([[1, -2, 3, 4], [0, 5, -6, 7], [8, -9, 10, -11]], np.int8)
+s_lit = np.array([0.5, 0.25, 2.0], np.float32)
+v.update(int8pack_lit_a=a_lit, int8pack_lit_w=w_lit, int8pack_lit_s=s_lit,
+         int8pack_lit_y=((a_lit @ w_lit.astype(np.float32).T) * s_lit).astype(np.float32))
+rng = np.random.default_rng(901)
+pa = rng.normal(0, 1, (3, 256)).astype(np.float32)
+pw = rng.integers(-128, 128, (40, 256)).astype(np.int8)
+ps = rng.uniform(0.001, 0.02, 40).astype(np.float32)
+v.update(int8pack_a=pa, int8pack_w=pw, int8pack_s=ps,
+         int8pack_y_f64=(pa.astype(np.float64) @ pw.astype(np.float64).T) * ps.astype(np.float64))
+
+# ---- quantize_affine: PyTorch CPU twins (one block, per-row blocks) and the grouped closed form -----
+rng = np.random.default_rng(902)
+qa = (rng.standard_normal((6, 40)) * 30).astype(np.float32)
+qa[0, :8] = np.array([-.5, .5, 1.5, 2.5, 3.5, 4.5, 7.5, 15.5], np.float32) * np.float32(0.37)  # ties
+v["affine_x"] = qa
+v["affine_tensor_scale"], v["affine_tensor_zero"] = np.float32(0.37), np.float32(3)
+for name, tdt in (("qint8", torch.qint8), ("quint8", torch.quint8)):
+    q = torch.quantize_per_tensor(torch.from_numpy(qa), 0.37, 3, tdt)
+    v[f"affine_tensor_{name}"] = q.int_repr().numpy()
+    v[f"affine_tensor_{name}_back"] = q.dequantize().numpy()
+row_s = rng.uniform(0.05, 0.9, 6).astype(np.float32)
+row_z = rng.integers(-4, 5, 6).astype(np.float32)
+q = torch.quantize_per_channel(torch.from_numpy(qa), torch.from_numpy(row_s).double(), torch.from_numpy(row_z).long(), 0, torch.qint8)
+v.update(affine_row_scale=row_s, affine_row_zero=row_z, affine_row_qint8=q.int_repr().numpy(), affine_row_back=q.dequantize().numpy())
+grp_s = rng.uniform(0.5, 4.0, (6, 5)).astype(np.float32)   # groups of 8 along the rows
+grp_z = np.full((6, 5), 8.0, np.float32)
+inv = (np.float32(1) / grp_s).astype(np.float32)
+pos = np.rint((qa.reshape(6, 5, 8) * inv[:, :, None]).astype(np.float32)) + grp_z[:, :, None]
+codes4 = np.clip(pos, 0, 15).astype(np.uint8).reshape(6, 40)
+v.update(affine_group_scale=grp_s, affine_group_zero=grp_z, affine_group_u4_codes=codes4,
+         affine_group_u4_packed=(codes4.reshape(-1)[0::2] | (codes4.reshape(-1)[1::2] << 4)).astype(np.uint8),  # low bits first
+         affine_group_u4_back=((codes4.reshape(6, 5, 8).astype(np.float32) - grp_z[:, :, None]) * grp_s[:, :, None]).reshape(6, 40).astype(np.float32))
+
+# ---- packed n-bit weight-only linear: the reference's pack formulas and x @ dq.T --------------------
+rng = np.random.default_rng(903)
+for bits in (1, 2, 4):
+    per_byte = 8 // bits
+    lc = rng.integers(0, 1 << bits, (12, 40)).astype(np.int32)
+    packed = np.zeros((12, 40 // per_byte), np.int32)
+    for i in range(per_byte):  # pack_intx: code i of a byte at shift 8 - (i + 1) * bits
+        packed |= (lc[:, i::per_byte] & ((1 << bits) - 1)) << (8 - (i + 1) * bits)
+    lsz = np.stack([rng.uniform(0.01, 0.2, (5, 12)), rng.integers(0, 1 << bits, (5, 12)).astype(np.float64)], axis=-1).astype(np.float32)
+    dq = ((lc.astype(np.float32) - np.repeat(lsz[:, :, 1].T, 8, axis=1)) * np.repeat(lsz[:, :, 0].T, 8, axis=1)).astype(np.float32)
+    lx = rng.standard_normal((3, 40)).astype(np.float32)
+    v.update({f"lowbit{bits}_codes": lc.astype(np.uint8), f"lowbit{bits}_packed": packed.astype(np.uint8), f"lowbit{bits}_sz": lsz,
+              f"lowbit{bits}_x": lx, f"lowbit{bits}_dense": dq, f"lowbit{bits}_y_f64": lx.astype(np.float64) @ dq.astype(np.float64).T})
+sign = rng.integers(0, 2, (4, 10)).astype(np.uint8)       # pack_binary: code i of a byte in bit i, zero padded
+padded = np.zeros((4, 16), np.uint8); padded[:, :10] = sign
+v.update(binary_codes=sign, binary_packed=sum(((padded[:, i::8] & 1) << i) for i in range(8)).astype(np.uint8))
+
 np.savez_compressed(OUT, **v)
 print(OUT, os.path.getsize(OUT), "bytes,", len(v), "arrays")

@@ -135,3 +135,75 @@ def test_gpu_packed_linear_special_case(K):
     x, w = G[f"packed_K{K}_x"].reshape(-1, K), G[f"packed_K{K}_w"]
     acc = ops._int_mm(dev(x), dev(w).t())
     np.testing.assert_array_equal(host(acc), G[f"packed_K{K}_acc"].reshape(-1, 7))
+
+
+# ---- the rows next to the path: int8 weight-only, affine quantizer, packed n-bit linears ------------
+
+def test_oracle_int8pack():
+    np.testing.assert_allclose(oracle.to_f32(oracle.weight_int8pack_mm(G["int8pack_lit_a"], "f32", G["int8pack_lit_w"], G["int8pack_lit_s"]), "f32"),
+                               G["int8pack_lit_y"], atol=1e-5)
+    got = oracle.to_f32(oracle.weight_int8pack_mm(G["int8pack_a"], "f32", G["int8pack_w"], G["int8pack_s"]), "f32")
+    np.testing.assert_allclose(got, G["int8pack_y_f64"], rtol=1e-5, atol=1e-5)
+
+
+def _affine_cases():
+    x = G["affine_x"]
+    yield "qint8", x.shape, [G["affine_tensor_scale"]], [G["affine_tensor_zero"]], G["affine_tensor_qint8"], G["affine_tensor_qint8_back"]
+    yield "quint8", x.shape, [G["affine_tensor_scale"]], [G["affine_tensor_zero"]], G["affine_tensor_quint8"], G["affine_tensor_quint8_back"]
+    yield "qint8", (1, x.shape[1]), G["affine_row_scale"], G["affine_row_zero"], G["affine_row_qint8"], G["affine_row_back"]
+    yield "quint4x2", (1, 8), G["affine_group_scale"], G["affine_group_zero"], G["affine_group_u4_packed"], G["affine_group_u4_back"]
+
+
+def test_oracle_affine():
+    x = G["affine_x"]
+    for dtype, block, scales, zeros, want, back in _affine_cases():
+        got = oracle.quantize_affine(x, block, scales, zeros, dtype)
+        np.testing.assert_array_equal(got, want)
+        np.testing.assert_array_equal(oracle.dequantize_affine(got, x.shape, block, scales, zeros, dtype), back)
+
+
+def test_oracle_lowbit():
+    for bits in (1, 2, 4):
+        np.testing.assert_array_equal(oracle.lowbit_pack(G[f"lowbit{bits}_codes"], bits), G[f"lowbit{bits}_packed"])
+        out, y64, dense = oracle.lowbit_mm(G[f"lowbit{bits}_x"], "f32", G[f"lowbit{bits}_packed"], bits, G[f"lowbit{bits}_sz"], 40, 8,
+                                           want_f64=True, want_dense=True)
+        np.testing.assert_array_equal(dense, G[f"lowbit{bits}_dense"])
+        np.testing.assert_allclose(y64, G[f"lowbit{bits}_y_f64"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_array_equal(oracle.lowbit_pack(G["binary_codes"], 1, lsb_first=True), G["binary_packed"])
+
+
+@pytest.mark.gpu
+def test_gpu_int8pack():
+    from gpu_util import dev, host
+    from tensorplay_amd import ops
+    np.testing.assert_allclose(host(ops._weight_int8pack_mm(dev(G["int8pack_lit_a"]), dev(G["int8pack_lit_w"]), dev(G["int8pack_lit_s"]))),
+                               G["int8pack_lit_y"], atol=1e-5)
+    got = host(ops._weight_int8pack_mm(dev(G["int8pack_a"]), dev(G["int8pack_w"]), dev(G["int8pack_s"])))
+    np.testing.assert_allclose(got, G["int8pack_y_f64"], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_gpu_affine():
+    from gpu_util import dev, host
+    from tensorplay_amd import ops
+    x = dev(G["affine_x"])
+    for dtype, block, scales, zeros, want, back in _affine_cases():
+        sc, zp = dev(np.asarray(scales, np.float32)), dev(np.asarray(zeros, np.float32))
+        q = ops.quantize_affine(x, list(block), sc, zp, dtype, 0, 0)
+        raw = q.data if isinstance(q, ops.PackedCodes) else q
+        np.testing.assert_array_equal(host(raw), want)
+        np.testing.assert_array_equal(host(ops.dequantize_affine(q, list(block), sc, zp)), back)
+
+
+@pytest.mark.gpu
+def test_gpu_lowbit():
+    from gpu_util import dev, host
+    from tensorplay_amd import ops
+    for bits in (1, 2, 4):
+        packed = ops.pack_lowbit(dev(G[f"lowbit{bits}_codes"]), bits)
+        np.testing.assert_array_equal(host(packed), G[f"lowbit{bits}_packed"])
+        sz = dev(G[f"lowbit{bits}_sz"])
+        np.testing.assert_array_equal(host(ops._lowbit_dequantize(packed, bits, 40, sz)), G[f"lowbit{bits}_dense"])
+        np.testing.assert_allclose(host(ops._lowbit_mm(dev(G[f"lowbit{bits}_x"]), packed, bits, 40, sz)), G[f"lowbit{bits}_y_f64"],
+                                   rtol=1e-5, atol=1e-5)
+    np.testing.assert_array_equal(host(ops.pack_lowbit(dev(G["binary_codes"]), 1, lsb_first=True)), G["binary_packed"])
