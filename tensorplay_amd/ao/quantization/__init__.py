@@ -39,6 +39,17 @@ from .int4_weight_only import (  # noqa: F401
     _quantize_int4_groupwise,
     int4_weight_only,
 )
+from .int8_dyn_act_lowbit import (  # noqa: F401
+    Int8DynActBinaryWeightLinear,
+    Int8DynActInt2WeightLinear,
+    Int8DynActInt4WeightLinear,
+    Int8DynamicActivationBinaryWeightConfig,
+    Int8DynamicActivationInt2WeightConfig,
+    Int8DynamicActivationInt4WeightConfig,
+    int8_dynamic_activation_binary_weight,
+    int8_dynamic_activation_int2_weight,
+    int8_dynamic_activation_int4_weight,
+)
 from .int8_mixed_precision import (  # noqa: F401
     Int8DynamicLinear,
     Int8DynamicLinearConfig,

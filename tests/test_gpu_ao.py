@@ -141,3 +141,64 @@ def test_quantize_swaps_int4_modules():
     y = model(x)
     assert y.shape == dense.shape
     assert (y.float() - dense.float()).abs().max().item() < 0.25 * dense.float().abs().max().item() + 0.05
+
+
+# ---- int8 dynamic activation x low-bit weight linears (reference test/quantization/test_int8_dyn_act_lowbit.py) ----
+
+def _two_layer():
+    import torch.nn as nn
+    return nn.Sequential(nn.Linear(64, 64, bias=False), nn.ReLU(), nn.Linear(64, 16, bias=False))
+
+
+@pytest.mark.gpu
+def test_8da4w_8da2w_8da1w_forward_close_to_float():
+    from tensorplay_amd.ao import quantization as q
+    torch.manual_seed(0)
+    x = torch.randn(4, 64, device="cuda:0")
+    for cfg, cls, check in ((q.int8_dynamic_activation_int4_weight(), q.Int8DynActInt4WeightLinear, "rel"),
+                            (q.int8_dynamic_activation_int2_weight(), q.Int8DynActInt2WeightLinear, "rel"),
+                            (q.int8_dynamic_activation_binary_weight(), q.Int8DynActBinaryWeightLinear, "cos")):
+        m = _two_layer().to("cuda:0")
+        ref = m(x)
+        qm = q.quantize_(m, cfg)
+        assert isinstance(qm[0], cls)
+        out = qm(x)
+        assert out.shape == (4, 16)
+        if check == "rel":   # reference :30-42
+            assert ((out - ref).abs().mean() / ref.abs().mean()).item() < (0.25 if cls is q.Int8DynActInt4WeightLinear else 1.0)
+        else:                # reference :45-59
+            assert ((out.reshape(-1) @ ref.reshape(-1)).abs() / (out.norm() * ref.norm())).item() > 0.5
+
+
+@pytest.mark.gpu
+def test_8da2w_matches_its_integer_formula_and_ste_gradients():
+    """Forward equals (x_i8 . codes) * x_scale * w_scale bit for bit; backward is the straight-through
+    estimator (reference :62-75)."""
+    from tensorplay_amd import ops
+    from tensorplay_amd.ao import quantization as q
+    torch.manual_seed(1)
+    x = torch.randn(3, 8, device="cuda:0", requires_grad=True)
+    mod = q.Int8DynActInt2WeightLinear(8, 5, bias=False).to("cuda:0")
+    out = mod(x)
+    xq, xs = ops._quantize_int8_rowwise(x.detach(), 1e-5)
+    wq, ws = ops._quantize_int2_rowwise(mod.weight.detach(), 1e-8)
+    want = (xq.double() @ wq.double().T).float() * xs[:, None] * ws[None, :]
+    assert torch.equal(out.detach(), want)
+    out.sum().backward()
+    assert mod.weight.grad.shape == (5, 8)
+    torch.testing.assert_close(x.grad, torch.ones_like(out) @ mod.weight.detach(), atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.gpu
+def test_lowbit_quantize_kernels_match_reference_formulas():
+    """reference test_int8_dyn_act_lowbit.py:95-110"""
+    from tensorplay_amd import ops
+    torch.manual_seed(3)
+    w = torch.randn(6, 16, device="cuda:0")
+    codes, scales = ops._quantize_int2_rowwise(w, 1e-8)
+    scale_ref = w.abs().amax(dim=-1, keepdim=True) / 2.0
+    assert bool((codes == (w / scale_ref).round().clamp(-2, 1)).all())
+    assert float((scales.unsqueeze(-1) - scale_ref).abs().max()) < 1e-6
+    codes_b, scales_b = ops._quantize_binary_rowwise(w, 1e-8)
+    assert bool((codes_b == torch.where(w >= 0, 1, -1).to(torch.int8)).all())
+    assert float((scales_b.unsqueeze(-1) - w.abs().amax(dim=-1, keepdim=True)).abs().max()) < 1e-6
