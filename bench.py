@@ -193,7 +193,35 @@ def decoder_layer_share(dev, rng_seed=5):
         xn = F.rms_norm(x, (d,), n2, 1e-5)
         return r + L["down"](F.silu(L["gate"](xn)) * L["up"](xn))
 
+    from tensorplay_amd import ops as tops
+
+    def layer_fused(L, x):
+        """The same layer with the two fusions around the MLP matmuls: residual add in the epilogue of the
+        o and down projections, gate and up in one launch with the SwiGLU epilogue."""
+        xf = x.view(B, d)
+        xn = F.rms_norm(xf, (d,), n1, 1e-5)
+        q = L["q"](xn).view(B, 1, H, D).transpose(1, 2)
+        k = L["k"](xn).view(B, 1, H, D).transpose(1, 2)
+        v = L["v"](xn).view(B, 1, H, D).transpose(1, 2)
+        q, k = rope(q), rope(k)
+        kc[:, :, T:T + 1] = k
+        vc[:, :, T:T + 1] = v
+        a = F.scaled_dot_product_attention(q, kc, vc).transpose(1, 2).reshape(B, H * D)
+        x1 = tops.int4pack_mm_add(a, L["o"].weight, 128, L["o"].scales_and_zeros, xf)
+        xn = F.rms_norm(x1, (d,), n2, 1e-5)
+        h = tops.int4pack_mm_swiglu(xn, L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros, L["up"].scales_and_zeros)
+        return tops.int4pack_mm_add(h, L["down"].weight, 128, L["down"].scales_and_zeros, x1).view(B, 1, d)
+
     xin = {n: torch.randn(B, 1, k, device=dev, generator=gen).half() for n, (_, k) in shapes.items()}
+    res_d = torch.randn(B, d, device=dev, generator=gen).half()
+
+    def linears_fused(L):
+        for name in ("q", "k", "v"):
+            L[name](xin[name])
+        tops.int4pack_mm_add(xin["o"].view(B, d), L["o"].weight, 128, L["o"].scales_and_zeros, res_d)
+        tops.int4pack_mm_swiglu(xin["gate"].view(B, d), L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros,
+                                L["up"].scales_and_zeros)
+        tops.int4pack_mm_add(xin["down"].view(B, inter), L["down"].weight, 128, L["down"].scales_and_zeros, res_d)
 
     def linears(L):
         for name in shapes:
@@ -203,10 +231,17 @@ def decoder_layer_share(dev, rng_seed=5):
     out = layer(layers[0], x0)
     torch.cuda.synchronize()
     assert torch.isfinite(out).all()
+    out_f = layer_fused(layers[0], x0)
+    torch.cuda.synchronize()
+    fused_diff = float((out_f.float() - out.float()).abs().max() / out.float().abs().max())
+    assert fused_diff < 2e-2, fused_diff
     g_layer = graph_of(lambda: [layer(layers[i % copies], x0) for i in range(reps)])
     g_lin = graph_of(lambda: [linears(layers[i % copies]) for i in range(reps)])
-    res = {}
-    for key, g in (("layer_decode_b8_kv2048_us", g_layer), ("layer_int4_linears_us", g_lin)):
+    g_layer_f = graph_of(lambda: [layer_fused(layers[i % copies], x0) for i in range(reps)])
+    g_lin_f = graph_of(lambda: [linears_fused(layers[i % copies]) for i in range(reps)])
+    res = {"layer_fused_vs_unfused_max_rel_diff": fused_diff}
+    for key, g in (("layer_decode_b8_kv2048_us", g_layer), ("layer_int4_linears_us", g_lin),
+                   ("layer_decode_fused_mlp_us", g_layer_f), ("layer_int4_linears_fused_us", g_lin_f)):
         g.replay(); torch.cuda.synchronize()
         ts = [time_region(g.replay, torch.cuda.synchronize, 1) / reps for _ in range(5)]
         res[key] = sorted(ts)[2] * 1e3

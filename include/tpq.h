@@ -151,6 +151,24 @@ int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packe
                    int32_t* acc_out, void* stream);
 
 /*
+ * Two fusions around the decode matmul for the MLP of a decoder layer (float16 / bfloat16
+ * activations, innerKTiles = 2, group 128, K % 128 == 0; anything else returns TPQ_ERR_UNSUPPORTED
+ * and the caller runs the separate ops).  Both round exactly where the separate ops would.
+ *   tpq_int4_mm_add:    out = T(T(x . W^T) + residual)            (residual, out: [M, N] of dtype)
+ *   tpq_int4_mm_swiglu: out = silu_mul(T(x . Wgate^T), T(x . Wup^T)) = T(g * sigmoid(g) * u) in fp32
+ * They stand for _weight_int4pack_mm followed by add, and for two _weight_int4pack_mm calls
+ * followed by silu_mul (config/native_functions.yaml:6071-6075,
+ * p10/src/backend/cpu/PointwiseKernels.cpp:1466-1540), the sequence of the reference's decoder layer
+ * (benchmark/bench_llama_e2e.py:140-144).
+ */
+int tpq_int4_mm_add(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
+                    int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
+                    const void* residual, void* out, void* stream);
+int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed_gate,
+                       const int32_t* packed_up, int inner_k_tiles, int64_t N, int64_t group,
+                       const void* sz_gate, const void* sz_up, void* out, void* stream);
+
+/*
  * Dense weight [N, K] of `dtype` from the packed device layout: W = T(code - 8) * scale + zero, the
  * product and the sum each rounded to T.  The reference runs this before its library GEMM
  * (int4_tc_dequantize_kernel, p10/src/backend/cuda/QuantGemmKernels.cu:1170-1202, 1296-1341); the

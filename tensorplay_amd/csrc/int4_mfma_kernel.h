@@ -57,13 +57,28 @@ struct MfmaLane<TPQ_DTYPE_BF16> {
     }
 };
 
+// SwiGLU gate of two rounded outputs, as the unfused sequence computes it: silu_mul on the 16-bit
+// results in fp32, gate * sigmoid(gate) * up, rounded once (reference: silu_mul_loop,
+// p10/src/backend/cpu/PointwiseKernels.cpp:1466-1478).
+template <int DT>
+__device__ __forceinline__ uint16_t swiglu_of(float gate_sum, float up_sum) {
+    using L = Lane16<DT>;
+    const float g = Elem<DT>::load(L::out(gate_sum)), u = Elem<DT>::load(L::out(up_sum));
+    const float sigmoid = __fdiv_rn(1.0f, 1.0f + expf(-g));
+    return L::out(g * sigmoid * u);
+}
+
 // x: [M][K] 16-bit; packed: [N/8][K/32][8] x 16 bytes; sz: [K/group][N] words (scale, zero);
 // steps = K / 128; a group is 128 << group_shift k.
-//
-template <int DT, int NB, int WAVES>
+// PAIR (NB = 2): the two blocks are the same 16 channels of two weights (packed / sz: gate, packed_b /
+// sz_b: up) and the output is silu_mul(gate, up).  residual (plain mode, may be null): [M][N], added to
+// the rounded output.
+template <int DT, int NB, int WAVES, bool PAIR = false>
 __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
-    uint16_t* __restrict__ y, int M, int N, int K, int group_shift) {
+    uint16_t* __restrict__ y, int M, int N, int K, int group_shift, const uint4* __restrict__ packed_b,
+    const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual) {
+    static_assert(!PAIR || NB == 2, "a pair is two blocks");
     using L = Lane16<DT>;
     using ML = MfmaLane<DT>;
     __shared__ float red[WAVES][NB][4][kWave];
@@ -72,19 +87,20 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int k_super = K / 32, steps = K / 128, n_tiles = N / 8;
-    const int n0 = blockIdx.x * (16 * NB);
+    const int n0 = blockIdx.x * (PAIR ? 16 : 16 * NB);
 
     // per-lane bases
     const uint4* w_base[NB];
     const uint32_t* sz_base[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-        int tile = (n0 + 16 * b + i) >> 3;                 // tile of row n0 + 16 b + i
+        const int nb0 = PAIR ? n0 : n0 + 16 * b;           // first channel of block b
+        int tile = (nb0 + i) >> 3;                         // tile of row nb0 + i
         tile = tile < n_tiles ? tile : n_tiles - 1;        // rows past N: any valid tile, result dropped
-        w_base[b] = packed + (static_cast<size_t>(tile) * k_super + q) * 8 + (i & 7);
-        int n4 = n0 + 16 * b + 4 * q;                      // this lane's four output channels
+        w_base[b] = (PAIR && b == 1 ? packed_b : packed) + (static_cast<size_t>(tile) * k_super + q) * 8 + (i & 7);
+        int n4 = nb0 + 4 * q;                              // this lane's four output channels
         n4 = n4 + 4 <= N ? n4 : N - 4;
-        sz_base[b] = sz + n4;
+        sz_base[b] = (PAIR && b == 1 ? sz_b : sz) + n4;
     }
     const bool row_live = i < M;
     const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 4;
@@ -181,6 +197,26 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
 #pragma unroll
         for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = yacc[b][v];
     __syncthreads();
+    if constexpr (PAIR) {
+        if (wave == 0) {  // lane (m, q): channels n0 + 4 q + v of both weights
+            float sum[2][4];
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    sum[b][v] = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) sum[b][v] += red[w][b][v][lane];
+                }
+            const int n = n0 + 4 * q;
+            if (row_live && n < N) {
+                const uint32_t lo = swiglu_of<DT>(sum[0][0], sum[1][0]) | (static_cast<uint32_t>(swiglu_of<DT>(sum[0][1], sum[1][1])) << 16);
+                const uint32_t hi = swiglu_of<DT>(sum[0][2], sum[1][2]) | (static_cast<uint32_t>(swiglu_of<DT>(sum[0][3], sum[1][3])) << 16);
+                *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
+            }
+        }
+        return;
+    }
     // wavefront w finishes block b = w, w + W, ...: lane (m, q) stores channels n0 + 16 b + 4 q + v
     for (int b = wave; b < NB; b += WAVES) {
         float sum[4];
@@ -192,9 +228,18 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         }
         const int n = n0 + 16 * b + 4 * q;
         if (row_live && n < N) {  // N % 8 == 0 and n % 4 == 0: all four channels exist
-            const uint32_t lo = L::out(sum[0]) | (static_cast<uint32_t>(L::out(sum[1])) << 16);
-            const uint32_t hi = L::out(sum[2]) | (static_cast<uint32_t>(L::out(sum[3])) << 16);
-            *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
+            uint16_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = L::out(sum[v]);
+            if (residual != nullptr) {  // the rounded output plus the residual, rounded again: what a separate add does
+                const uint2 r = *reinterpret_cast<const uint2*>(residual + static_cast<size_t>(i) * N + n);
+                const uint16_t rv[4] = {static_cast<uint16_t>(r.x), static_cast<uint16_t>(r.x >> 16), static_cast<uint16_t>(r.y),
+                                        static_cast<uint16_t>(r.y >> 16)};
+#pragma unroll
+                for (int v = 0; v < 4; ++v) o[v] = L::out(Elem<DT>::load(o[v]) + Elem<DT>::load(rv[v]));
+            }
+            *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) =
+                make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
         }
     }
 }

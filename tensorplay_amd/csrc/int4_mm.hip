@@ -389,13 +389,15 @@ bool launch_stream(const void* x, const int32_t* packed, const void* sz, void* y
 }
 
 // Up to 16 rows per launch on the matrix cores; false if the shape does not fit that kernel.
+// residual (may be null): [rows][N] added to the rounded output; it forces this kernel for one row too.
 template <int DT>
 bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void* sz, void* y, int N, int K,
-                      int group, hipStream_t s, int* rc) {
+                      int group, hipStream_t s, int* rc, const void* residual = nullptr) {
     if ((group != 128 && group != 256) || !aligned(sz, 16) || !aligned(y, 8)) return false;
+    if (residual != nullptr && !aligned(residual, 8)) return false;
     const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
-    if (force && force[0] == 'd') return false;
-    if (rows == 1 && !(force && force[0] == 'm')) return false;
+    if (force && force[0] == 'd' && residual == nullptr) return false;
+    if (rows == 1 && residual == nullptr && !(force && force[0] == 'm')) return false;
     // Every workgroup reads all of x from cache, so many rows want wide workgroups (64 channels),
     // but only when N still yields enough of them to fill the chip.  Measured (us, weights from
     // HBM): N=11008 K=4096: 4 rows 9.6 (16 ch, 8 waves); 8 rows 10.9 (64 ch) vs 11.3 (16 ch);
@@ -411,7 +413,8 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     auto* yp = static_cast<uint16_t*>(y);
     const int shift = group == 128 ? 0 : 1;  // a group is 128 << shift k (128 or 256)
 #define TPQ_MFMA(NBV, WV) \
-    int4_mfma_kernel<DT, NBV, WV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>(xp, pp, sp, yp, rows, N, K, shift)
+    int4_mfma_kernel<DT, NBV, WV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \
+        xp, pp, sp, yp, rows, N, K, shift, nullptr, nullptr, static_cast<const uint16_t*>(residual))
     if (waves == 16 && nb == 1) {
         TPQ_MFMA(1, 16);
     } else if (waves == 8) {
@@ -422,6 +425,38 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
 #undef TPQ_MFMA
     *rc = check_launch("tpq_int4_mm (mfma)");
     return true;
+}
+
+// gate / up pair with the SwiGLU epilogue, and the plain product plus a residual: slabs of 16 rows
+template <int DT>
+int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz, const int32_t* packed_b, const void* sz_b,
+                 const void* residual, void* y, int N, int K, int group, hipStream_t s) {
+    const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        const char* xs = static_cast<const char*>(x) + m0 * row_x;
+        char* ys = static_cast<char*>(y) + m0 * row_y;
+        int rc = TPQ_OK;
+        if (packed_b != nullptr) {
+            static const int pair_waves = [] { const char* e = std::getenv("TPQ_INT4_PAIR_WAVES"); return e ? std::atoi(e) : 4; }();
+            const auto* xp = reinterpret_cast<const uint16_t*>(xs);
+            const auto* pa = reinterpret_cast<const uint4*>(packed);
+            const auto* pb = reinterpret_cast<const uint4*>(packed_b);
+            const auto* sa = static_cast<const uint32_t*>(sz);
+            const auto* sb = static_cast<const uint32_t*>(sz_b);
+            auto* yp = reinterpret_cast<uint16_t*>(ys);
+            const dim3 grid((N + 15) / 16);
+            if (pair_waves == 8)
+                int4_mfma_kernel<DT, 2, 8, true><<<grid, dim3(8 * kWave), 0, s>>>(xp, pa, sa, yp, rows, N, K, group == 128 ? 0 : 1, pb, sb, nullptr);
+            else
+                int4_mfma_kernel<DT, 2, 4, true><<<grid, dim3(4 * kWave), 0, s>>>(xp, pa, sa, yp, rows, N, K, group == 128 ? 0 : 1, pb, sb, nullptr);
+            rc = check_launch("tpq_int4_mm_swiglu");
+        } else if (!launch_mfma_rows<DT>(xs, rows, packed, sz, ys, N, K, group, s, &rc, static_cast<const char*>(residual) + m0 * row_y)) {
+            return fail(TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_add: this shape or alignment is not built");
+        }
+        if (rc != TPQ_OK) return rc;
+    }
+    return TPQ_OK;
 }
 
 template <int DT>
@@ -603,4 +638,47 @@ TPQ_EXPORT int tpq_int4_dequantize(const int32_t* packed, int inner_k_tiles, int
             break;
     }
     return check_launch("tpq_int4_dequantize");
+}
+
+namespace {
+// shapes the fused entry points are built for: what the matrix-core decode kernel takes
+int check_fused(const char* op, int dtype, int64_t M, int64_t K, int inner_k_tiles, int64_t N, int64_t group) {
+    TPQ_REQUIRE(dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16, TPQ_ERR_UNSUPPORTED, "%s: float16 / bfloat16 activations only", op);
+    TPQ_REQUIRE(inner_k_tiles == 2, TPQ_ERR_UNSUPPORTED, "%s: only innerKTiles = 2 packed weights are supported", op);
+    TPQ_REQUIRE(group == 128, TPQ_ERR_UNSUPPORTED, "%s: qGroupSize must be 128", op);
+    TPQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && N % 8 == 0, TPQ_ERR_INVALID_VALUE, "%s: K dimension does not match packed B", op);
+    TPQ_REQUIRE(K % 128 == 0 && N <= 0x7FFFFFF8 && K <= 0x7FFFFFE0, TPQ_ERR_UNSUPPORTED, "%s: K must be a multiple of 128", op);
+    return TPQ_OK;
+}
+}  // namespace
+
+TPQ_EXPORT int tpq_int4_mm_add(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed, int inner_k_tiles,
+                               int64_t N, int64_t group, const void* scales_and_zeros, const void* residual, void* out,
+                               void* stream) {
+    if (int rc = check_fused("tpq_int4_mm_add", dtype, M, K, inner_k_tiles, N, group)) return rc;
+    if (M == 0 || N == 0) return TPQ_OK;
+    TPQ_REQUIRE(K > 0, TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_add: K = 0 is not built");
+    TPQ_REQUIRE(x && packed && scales_and_zeros && residual && out, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_add: null pointer");
+    TPQ_REQUIRE(aligned(x, 16) && aligned(packed, 16) && aligned(scales_and_zeros, 16) && aligned(residual, 8) && aligned(out, 8) && N % 4 == 0,
+                TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_add: unaligned operand");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == TPQ_DTYPE_F16)
+        return launch_fused<TPQ_DTYPE_F16>(x, M, packed, scales_and_zeros, nullptr, nullptr, residual, out, (int)N, (int)K, (int)group, s);
+    return launch_fused<TPQ_DTYPE_BF16>(x, M, packed, scales_and_zeros, nullptr, nullptr, residual, out, (int)N, (int)K, (int)group, s);
+}
+
+TPQ_EXPORT int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed_gate,
+                                  const int32_t* packed_up, int inner_k_tiles, int64_t N, int64_t group,
+                                  const void* sz_gate, const void* sz_up, void* out, void* stream) {
+    if (int rc = check_fused("tpq_int4_mm_swiglu", dtype, M, K, inner_k_tiles, N, group)) return rc;
+    if (M == 0 || N == 0) return TPQ_OK;
+    TPQ_REQUIRE(K > 0, TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_swiglu: K = 0 is not built");
+    TPQ_REQUIRE(x && packed_gate && packed_up && sz_gate && sz_up && out, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_swiglu: null pointer");
+    TPQ_REQUIRE(aligned(x, 16) && aligned(packed_gate, 16) && aligned(packed_up, 16) && aligned(sz_gate, 16) && aligned(sz_up, 16) &&
+                    aligned(out, 8),
+                TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_swiglu: unaligned operand");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == TPQ_DTYPE_F16)
+        return launch_fused<TPQ_DTYPE_F16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s);
+    return launch_fused<TPQ_DTYPE_BF16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s);
 }

@@ -579,3 +579,62 @@ def _lowbit_mm(input: torch.Tensor, packed: torch.Tensor, bits: int, columns: in
         _check(_lib.load().tpq_lowbit_mm(_ptr(x), _DT[x.dtype], m, columns, _ptr(w), bits, int(lsb_first), n, group,
                                          _ptr(sz), _ptr(b), _ptr(out), _stream(x)))
     return out
+
+
+# ---- fusions around the int4 decode matmul (MLP of a decoder layer) -------------------------------
+
+def _fused_int4_operands(x, packed, group, sz, what):
+    if packed.dtype != torch.int32 or packed.dim() != 4 or packed.size(2) != 32:
+        raise TypeError(f"{what}: packed weight must be 4-D int32 in the tensor-core B layout")
+    if x.dim() != 2 or x.dtype not in _DT:
+        raise ValueError(f"{what}: expected 2-D float activations [m,k]")
+    _require_device(x, what)
+    inner, n = packed.size(3) * 2, packed.size(0) * 8
+    if tuple(sz.shape) != ((x.shape[1] + group - 1) // group, n, 2):
+        raise ValueError(f"{what}: qScaleAndZeros must be [K/group, N, 2]")
+    return x.contiguous(), packed.contiguous(), sz.to(x.dtype).contiguous(), inner, n
+
+
+def int4pack_mm_add(input: torch.Tensor, mat2: torch.Tensor, qGroupSize: int, qScaleAndZeros: torch.Tensor,
+                    residual: torch.Tensor) -> torch.Tensor:
+    """``residual + _weight_int4pack_mm(input, mat2, qGroupSize, qScaleAndZeros)`` in one launch, rounded
+    where the two separate ops round.  Shapes the fused kernel does not take run the two ops."""
+    x, w, sz, inner, n = _fused_int4_operands(input, mat2, qGroupSize, qScaleAndZeros, "int4pack_mm_add")
+    m, k = x.shape
+    if tuple(residual.shape) != (m, n) or residual.dtype != x.dtype:
+        raise ValueError("int4pack_mm_add: residual must be [m, n] of the activation dtype")
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if m == 0 or n == 0:
+        return out
+    r = residual.contiguous()
+    with torch.cuda.device(x.device):
+        status = _lib.load().tpq_int4_mm_add(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz), _ptr(r),
+                                             _ptr(out), _stream(x))
+    if status == _lib.TPQ_ERR_UNSUPPORTED:
+        return r + _weight_int4pack_mm(x, w, qGroupSize, sz)
+    _check(status)
+    return out
+
+
+def int4pack_mm_swiglu(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, qGroupSize: int,
+                       gate_scale_and_zeros: torch.Tensor, up_scale_and_zeros: torch.Tensor) -> torch.Tensor:
+    """``silu_mul(_weight_int4pack_mm(input, gate, ...), _weight_int4pack_mm(input, up, ...))`` in one launch
+    (the reference's ``silu_mul``: gate * sigmoid(gate) * up in float32, rounded once).  Shapes the fused kernel
+    does not take run the separate ops."""
+    x, wg, szg, inner, n = _fused_int4_operands(input, gate, qGroupSize, gate_scale_and_zeros, "int4pack_mm_swiglu")
+    _, wu, szu, inner_u, n_u = _fused_int4_operands(input, up, qGroupSize, up_scale_and_zeros, "int4pack_mm_swiglu")
+    if (inner_u, n_u) != (inner, n) or wu.shape != wg.shape:
+        raise ValueError("int4pack_mm_swiglu: gate and up must have the same packed shape")
+    m, k = x.shape
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if m == 0 or n == 0:
+        return out
+    with torch.cuda.device(x.device):
+        status = _lib.load().tpq_int4_mm_swiglu(_ptr(x), _DT[x.dtype], m, k, _ptr(wg), _ptr(wu), inner, n, qGroupSize, _ptr(szg),
+                                                _ptr(szu), _ptr(out), _stream(x))
+    if status == _lib.TPQ_ERR_UNSUPPORTED:
+        g = _weight_int4pack_mm(x, wg, qGroupSize, szg).float()
+        u = _weight_int4pack_mm(x, wu, qGroupSize, szu).float()
+        return (g * torch.sigmoid(g) * u).to(x.dtype)
+    _check(status)
+    return out

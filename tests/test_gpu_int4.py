@@ -186,3 +186,65 @@ def test_mm_many_rows_takes_the_dense_route(ops, dtype):
     assert_close_norm(got, ref_dev, 1e-2, "vs reference formulation")
     _, y64 = oracle.int4_mm_tc(xb, dtype, packed, szb, group, round_w=False, want_f64=True)
     assert rel_err(got, y64) < {"f16": 2e-3, "bf16": 1e-2, "f32": 1e-4}[dtype]
+
+
+# ---- fusions around the decode matmul --------------------------------------------------------------
+
+def _fused_case(rng, M, N, K, tdt):
+    codes = rng.integers(0, 16, (N, K)).astype(np.int32)
+    sz = np.stack([rng.uniform(0.005, 0.02, (K // 128, N)), rng.uniform(-0.05, 0.05, (K // 128, N))], axis=-1).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(tdt)
+    return codes, torch.from_numpy(sz).to(tdt), x
+
+
+@pytest.mark.parametrize("tdt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 4096, 1024), (19, 48, 384)])
+def test_mm_add_equals_the_two_ops(ops, tdt, M, N, K):
+    """out = residual + x.W^T with both roundings of the separate ops: equal bit for bit whenever the matmul
+    runs on the same kernel (rows > 1), within one rounding of it otherwise."""
+    rng = np.random.default_rng(M * 1000 + N)
+    codes, sz, x = _fused_case(rng, M, N, K, tdt)
+    packed = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(DEV), 2)
+    res = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32)).to(tdt).to(DEV)
+    got = ops.int4pack_mm_add(x.to(DEV), packed, 128, sz.to(DEV), res)
+    want = res + ops._weight_int4pack_mm(x.to(DEV), packed, 128, sz.to(DEV))
+    if M > 1 and M % 16 != 1:
+        assert torch.equal(got, want)
+    else:
+        assert_close_norm(got.float().cpu().numpy(), want.float().cpu().numpy(), 4e-3 if tdt == torch.float16 else 2e-2)
+
+
+@pytest.mark.parametrize("tdt,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 1024, 1024), (19, 48, 384)])
+def test_mm_swiglu_against_oracle(ops, tdt, tol, M, N, K):
+    """silu_mul(T(x.Wg^T), T(x.Wu^T)): the oracle's two device-layout products rounded to T, then
+    gate * sigmoid(gate) * up in float32 (p10/src/backend/cpu/PointwiseKernels.cpp:1466-1478)."""
+    rng = np.random.default_rng(M * 77 + N)
+    tag = "f16" if tdt == torch.float16 else "bf16"
+    cg, szg, x = _fused_case(rng, M, N, K, tdt)
+    cu, szu, _ = _fused_case(rng, M, N, K, tdt)
+    pg = ops._convert_weight_to_int4pack(torch.from_numpy(cg).to(DEV), 2)
+    pu = ops._convert_weight_to_int4pack(torch.from_numpy(cu).to(DEV), 2)
+    got = ops.int4pack_mm_swiglu(x.to(DEV), pg, pu, 128, szg.to(DEV), szu.to(DEV))
+    g = ops._weight_int4pack_mm(x.to(DEV), pg, 128, szg.to(DEV)).float()
+    u = ops._weight_int4pack_mm(x.to(DEV), pu, 128, szu.to(DEV)).float()
+    unfused = (g * torch.sigmoid(g) * u).to(tdt)
+    assert_close_norm(got.float().cpu().numpy(), unfused.float().cpu().numpy(), tol)
+    # and against the CPU oracle's products
+    og = oracle.to_f32(oracle.int4_mm_tc(host(x), tag, oracle.int4_pack_tc(cg, 2), host(szg), 128), tag)
+    ou = oracle.to_f32(oracle.int4_mm_tc(host(x), tag, oracle.int4_pack_tc(cu, 2), host(szu), 128), tag)
+    want = og * (1.0 / (1.0 + np.exp(-og))) * ou
+    assert_close_norm(got.float().cpu().numpy(), want, 2 * tol)
+
+
+def test_fused_entry_points_fall_back_for_other_shapes(ops):
+    rng = np.random.default_rng(5)
+    codes = rng.integers(0, 16, (32, 128)).astype(np.int32)
+    packed = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(DEV), 2)
+    sz = torch.rand(4, 32, 2, device=DEV).half() * 0.01   # groups of 32: not a fused shape
+    x = torch.randn(3, 128, device=DEV).half()
+    res = torch.randn(3, 32, device=DEV).half()
+    assert torch.equal(ops.int4pack_mm_add(x, packed, 32, sz, res), res + ops._weight_int4pack_mm(x, packed, 32, sz))
+    out = ops.int4pack_mm_swiglu(x, packed, packed, 32, sz, sz)
+    g = ops._weight_int4pack_mm(x, packed, 32, sz).float()
+    assert torch.equal(out, (g * torch.sigmoid(g) * g).half())
