@@ -11,8 +11,9 @@
 // leaves b exactly.  The products are exact and accumulate in fp32 over the whole K range, two
 // accumulators taking turns; the per-row scale multiplies the final sum.
 //
-// Everything else (bf16 / fp32 activations, other K, unaligned pointers) takes a plain kernel: one
-// workgroup per output channel and slab of up to 8 rows, fp32 fma over k, block reduction.
+// Everything else (bf16 / fp32 activations, other K) takes the vector kernel below (wavefront = four channels,
+// eight k per lane and turn, fp32 fma), and K % 8 != 0 or unaligned pointers a plain one: one workgroup per
+// output channel and slab of up to 8 rows, block reduction.
 #include "int4_lane.h"
 
 namespace tpq {
@@ -112,6 +113,52 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
     }
 }
 
+// Any floating activation dtype, K % 8 == 0, 16-byte aligned rows: a wavefront owns four consecutive output
+// channels and a slab of up to four activation rows; a lane takes eight consecutive k per turn (8 bytes of
+// each weight row, 16 or 32 bytes of each activation row), fp32 fma, one wavefront reduction at the end.
+constexpr int kVecChannels = 4, kVecRows = 4;
+
+template <int DT>
+__global__ __launch_bounds__(256) void int8pack_vector_kernel(
+    const typename Elem<DT>::storage* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
+    typename Elem<DT>::storage* __restrict__ y, int64_t M, int64_t N, int64_t K) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int64_t n0 = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * kVecChannels, m0 = static_cast<int64_t>(blockIdx.y) * kVecRows;
+    if (n0 >= N) return;
+    const int rows = static_cast<int>(M - m0 < kVecRows ? M - m0 : kVecRows);
+    float acc[kVecChannels][kVecRows];
+#pragma unroll
+    for (int c = 0; c < kVecChannels; ++c)
+#pragma unroll
+        for (int r = 0; r < kVecRows; ++r) acc[c][r] = 0.0f;
+    for (int64_t k = static_cast<int64_t>(lane) * 8; k < K; k += kWave * 8) {
+        float xv[kVecRows][8];
+#pragma unroll
+        for (int r = 0; r < kVecRows; ++r)
+            if (r < rows) load_eight<DT>(x + (m0 + r) * K + k, xv[r]);
+#pragma unroll
+        for (int c = 0; c < kVecChannels; ++c) {
+            const int64_t n = n0 + c < N ? n0 + c : N - 1;  // channels past N: a valid row, result dropped
+            const uint2 raw = nt_load(reinterpret_cast<const uint2*>(w + n * K + k));
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t word = e < 4 ? raw.x : raw.y;
+                const float wv = static_cast<float>(static_cast<int8_t>(word >> (8 * (e & 3))));
+#pragma unroll
+                for (int r = 0; r < kVecRows; ++r)
+                    if (r < rows) acc[c][r] = __builtin_fmaf(wv, xv[r][e], acc[c][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < kVecChannels; ++c)
+#pragma unroll
+        for (int r = 0; r < kVecRows; ++r) {
+            const float total = wave_sum(acc[c][r]);
+            if (lane == 0 && r < rows && n0 + c < N) y[(m0 + r) * N + n0 + c] = Elem<DT>::store(__fmul_rn(total, scale[n0 + c]));
+        }
+}
+
 // One workgroup per output channel n and slab of up to 8 activation rows.
 template <int DT>
 __global__ __launch_bounds__(256) void int8pack_generic_kernel(
@@ -149,6 +196,13 @@ __global__ __launch_bounds__(256) void int8pack_generic_kernel(
 template <int DT>
 int launch_generic(const void* x, const int8_t* w, const float* scale, void* y, int64_t M, int64_t N, int64_t K, hipStream_t s) {
     using S = typename Elem<DT>::storage;
+    if (K % 8 == 0 && aligned(x, 32) && aligned(w, 8)) {
+        const int64_t gx = (N + 4 * kVecChannels - 1) / (4 * kVecChannels), gy = (M + kVecRows - 1) / kVecRows;
+        TPQ_REQUIRE(gx <= 0x7FFFFFFF && gy <= 65535, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): shape too large");
+        int8pack_vector_kernel<DT><<<dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)), 256, 0, s>>>(
+            static_cast<const S*>(x), w, scale, static_cast<S*>(y), M, N, K);
+        return check_launch("_weight_int8pack_mm (vector)");
+    }
     const int64_t slabs = (M + 7) / 8;
     TPQ_REQUIRE(N <= 0x7FFFFFFF && slabs <= 65535, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): shape too large");
     int8pack_generic_kernel<DT><<<dim3(static_cast<unsigned>(N), static_cast<unsigned>(slabs)), 256, 0, s>>>(

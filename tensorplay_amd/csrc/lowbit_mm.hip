@@ -18,9 +18,10 @@
 // more MFMA per eight k whose A is constant (row 0: the offsets, row 1: ones -> sum of x), and a step
 // stays inside one quantization group:  y += scale * ((D - offsets) - zero * sum x).
 //
-// Everything else (fp32 / bf16 activations, odd K or group sizes) takes a plain kernel: one workgroup
-// per output channel and slab of up to 8 rows, the dequantized weight formed in fp32 exactly as the
-// reference does, fp32 fma over k.
+// Everything else (fp32 / bf16 activations, other group sizes) takes the vector kernel below (wavefront = four
+// channels, eight k per lane and turn), and K or group sizes that are not multiples of 8 a plain one: one
+// workgroup per output channel and slab of up to 8 rows; both form the dequantized weight in fp32 exactly as the
+// reference does and accumulate with fp32 fma.
 #include <cstdlib>
 
 #include "int4_lane.h"
@@ -179,6 +180,69 @@ __device__ __forceinline__ int code_at(const uint8_t* row, int64_t k, int bits, 
     return (row[k / per_byte] >> shift) & ((1 << bits) - 1);
 }
 
+// Any floating activation dtype and bit width, K % 8 == 0, group % 8 == 0, aligned rows: a wavefront owns
+// four consecutive output channels and a slab of up to four activation rows; a lane takes eight consecutive k
+// per turn (1 to 8 bytes of each weight row), forms (code - zero) * scale in fp32 as the reference does, fp32
+// fma, one wavefront reduction at the end.
+constexpr int kVecChannels = 4, kVecRows = 4;
+
+template <int DT>
+__global__ __launch_bounds__(256) void lowbit_vector_kernel(
+    const typename Elem<DT>::storage* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
+    const float* __restrict__ bias, typename Elem<DT>::storage* __restrict__ y, int64_t M, int64_t N, int64_t K,
+    int64_t group, int bits, int lsb_first) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int64_t n0 = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * kVecChannels, m0 = static_cast<int64_t>(blockIdx.y) * kVecRows;
+    if (n0 >= N) return;
+    const int rows = static_cast<int>(M - m0 < kVecRows ? M - m0 : kVecRows);
+    const int per_byte = 8 / bits, bytes = 8 / per_byte;  // bytes holding eight codes: 1, 2, 4 or 8
+    const int pb_shift = per_byte == 8 ? 3 : per_byte == 4 ? 2 : per_byte == 2 ? 1 : 0;
+    const int64_t pitch = K >> pb_shift;
+    const uint32_t field = (1u << bits) - 1u;
+    float acc[kVecChannels][kVecRows];
+#pragma unroll
+    for (int c = 0; c < kVecChannels; ++c)
+#pragma unroll
+        for (int r = 0; r < kVecRows; ++r) acc[c][r] = 0.0f;
+    for (int64_t k = static_cast<int64_t>(lane) * 8; k < K; k += kWave * 8) {
+        float xv[kVecRows][8];
+#pragma unroll
+        for (int r = 0; r < kVecRows; ++r)
+            if (r < rows) load_eight<DT>(x + (m0 + r) * K + k, xv[r]);
+        const int64_t g = k / group;
+#pragma unroll
+        for (int c = 0; c < kVecChannels; ++c) {
+            const int64_t n = n0 + c < N ? n0 + c : N - 1;  // channels past N: a valid row, result dropped
+            const uint8_t* src = packed + n * pitch + (k >> pb_shift);
+            uint64_t raw;
+            if (bytes == 8) { const uint2 t = nt_load(reinterpret_cast<const uint2*>(src)); raw = t.x | (static_cast<uint64_t>(t.y) << 32); }
+            else if (bytes == 4) raw = nt_load(reinterpret_cast<const uint32_t*>(src));
+            else if (bytes == 2) raw = *reinterpret_cast<const uint16_t*>(src);
+            else raw = *src;
+            const float2 p = *reinterpret_cast<const float2*>(sz + (g * N + n) * 2);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int i = e & (per_byte - 1);  // per_byte is 1, 2, 4 or 8
+                const int shift = 8 * (e >> pb_shift) + (lsb_first ? i * bits : 8 - (i + 1) * bits);
+                const float wv = (static_cast<float>(static_cast<uint32_t>(raw >> shift) & field) - p.y) * p.x;
+#pragma unroll
+                for (int r = 0; r < kVecRows; ++r)
+                    if (r < rows) acc[c][r] = __builtin_fmaf(wv, xv[r][e], acc[c][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < kVecChannels; ++c)
+#pragma unroll
+        for (int r = 0; r < kVecRows; ++r) {
+            float total = wave_sum(acc[c][r]);
+            if (lane == 0 && r < rows && n0 + c < N) {
+                if (bias != nullptr) total += bias[n0 + c];
+                y[(m0 + r) * N + n0 + c] = Elem<DT>::store(total);
+            }
+        }
+}
+
 // One workgroup per output channel n and slab of up to 8 activation rows.
 template <int DT>
 __global__ __launch_bounds__(256) void lowbit_generic_kernel(
@@ -283,6 +347,13 @@ template <int DT>
 int launch_generic(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t M, int64_t N,
                    int64_t K, int64_t group, int bits, int lsb_first, hipStream_t s) {
     using S = typename Elem<DT>::storage;
+    if (K > 0 && K % 8 == 0 && group % 8 == 0 && aligned(x, 32) && aligned(packed, 8) && aligned(sz, 8)) {
+        const int64_t gx = (N + 4 * kVecChannels - 1) / (4 * kVecChannels), gy = (M + kVecRows - 1) / kVecRows;
+        TPQ_REQUIRE(gx <= 0x7FFFFFFF && gy <= 65535, TPQ_ERR_INVALID_VALUE, "lowbit mm: shape too large");
+        lowbit_vector_kernel<DT><<<dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)), 256, 0, s>>>(
+            static_cast<const S*>(x), packed, sz, bias, static_cast<S*>(out), M, N, K, group, bits, lsb_first);
+        return check_launch("tpq_lowbit_mm (vector)");
+    }
     const int64_t slabs = (M + 7) / 8;
     TPQ_REQUIRE(N <= 0x7FFFFFFF && slabs <= 65535, TPQ_ERR_INVALID_VALUE, "lowbit mm: shape too large");
     lowbit_generic_kernel<DT><<<dim3(static_cast<unsigned>(N), static_cast<unsigned>(slabs)), 256, 0, s>>>(

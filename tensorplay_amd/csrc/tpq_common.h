@@ -117,6 +117,26 @@ __device__ __forceinline__ void nt_store(uint4* p, const uint4& v) {
     __builtin_nontemporal_store(t, reinterpret_cast<u4*>(p));
 }
 
+// ---- eight consecutive activations as floats ----------------------------------------------------
+
+// p is 16-byte aligned (32 for fp32)
+template <int DT>
+__device__ __forceinline__ void load_eight(const typename Elem<DT>::storage* p, float (&v)[8]) {
+    if constexpr (DT == TPQ_DTYPE_F32) {
+        const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = Elem<DT>::load(static_cast<uint16_t>(w[i] & 0xFFFFu));
+            v[2 * i + 1] = Elem<DT>::load(static_cast<uint16_t>(w[i] >> 16));
+        }
+    }
+}
+
 // ---- 64-lane reductions -----------------------------------------------------
 
 __device__ __forceinline__ float wave_max(float v) {
