@@ -2,13 +2,14 @@
 // (reference: _weight_int8pack_mm, p10/src/backend/cuda/QuantGemmKernels.cu:86-180, 339-405:
 // activations converted to fp32, fp32 accumulation, per-row scale applied to the sum).
 //
-// Decode kernel (fp16 activations, K % 128 == 0, 1..16 rows per launch), bandwidth bound at one byte
+// Decode kernel (fp16 / bf16 activations, K % 128 == 0, 1..16 rows per launch), bandwidth bound at one byte
 // per weight: v_mfma_f32_16x16x32_f16 with the weights as A and the activations as B, as in the int4
 // decode kernel for several rows.  Lane (i, q) owns weight row n0 + i and, in a step of 128 k, the 32
 // bytes at k = 128 s + 32 q: two 16-byte loads, whole 128-byte lines per row and step.  Every dword
 // (four int8) becomes two fp16 pairs: xor 0x80808080 turns the bytes into b + 128, v_perm_b32 drops
 // each next to the exponent byte 0x64 (fp16 1024 + 128 + b), and one packed fp16 subtract of 1152
-// leaves b exactly.  The products are exact and accumulate in fp32 over the whole K range, two
+// leaves b exactly (bf16: a sign-extending byte-to-float conversion per code, upper halves packed by
+// v_perm_b32).  The products are exact and accumulate in fp32 over the whole K range, two
 // accumulators taking turns; the per-row scale multiplies the final sum.
 //
 // Everything else (bf16 / fp32 activations, other K) takes the vector kernel below (wavefront = four channels,
@@ -27,7 +28,10 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r == 0 ? q.x : r == 1 ? q.y : r == 2 ? q.z : q.w; }
 
-// x: [M][K] fp16; w: [N][K] int8; scale: [N] fp32; steps = K / 128
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+
+// x: [M][K] fp16 or bf16; w: [N][K] int8; scale: [N] fp32; steps = K / 128
+template <int DT>
 __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
     const uint16_t* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
     uint16_t* __restrict__ y, int M, int N, int K) {
@@ -64,16 +68,30 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
             uint32_t a[4];
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const uint32_t t = dword_at(st.w[u >> 1], (2 * u + h) & 3) ^ 0x80808080u;
-                const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
-                const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
-                a[2 * h] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
-                a[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
+                const uint32_t word = dword_at(st.w[u >> 1], (2 * u + h) & 3);
+                if constexpr (DT == TPQ_DTYPE_F16) {
+                    const uint32_t t = word ^ 0x80808080u;
+                    const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
+                    const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
+                    a[2 * h] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
+                    a[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
+                } else {
+                    // bf16 is the upper half of a float and an int8 has eight significant bits: convert each
+                    // byte (sign-extending byte select) and keep the upper halves, exact
+                    uint32_t f[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) f[e] = __builtin_bit_cast(uint32_t, static_cast<float>(static_cast<int8_t>(word >> (8 * e))));
+                    a[2 * h] = __builtin_amdgcn_perm(f[1], f[0], 0x07060302u);      // (bf16 b0, bf16 b1)
+                    a[2 * h + 1] = __builtin_amdgcn_perm(f[3], f[2], 0x07060302u);  // (bf16 b2, bf16 b3)
+                }
             }
             const word4_t av = {a[0], a[1], a[2], a[3]};
             const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
-            if (u & 1) d1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d1, 0, 0, 0);
-            else d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d0, 0, 0, 0);
+            float4_t& d = (u & 1) ? d1 : d0;
+            if constexpr (DT == TPQ_DTYPE_F16)
+                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
+            else
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), d, 0, 0, 0);
         }
     };
 
@@ -108,7 +126,7 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
         if (i < M) {
 #pragma unroll
             for (int v = 0; v < 4; ++v)
-                if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = f32_to_f16_bits(__fmul_rn(sum[v], scale[n + v]));
+                if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = Elem<DT>::store(__fmul_rn(sum[v], scale[n + v]));
         }
     }
 }
@@ -223,12 +241,16 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
     if (M == 0 || N == 0 || K == 0) return TPQ_OK;  // the reference returns an uninitialised [B, N] here
     TPQ_REQUIRE(x && w && scales && out, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == TPQ_DTYPE_F16 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
+    if (dtype != TPQ_DTYPE_F32 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
-            int8pack_mfma_kernel<<<dim3(static_cast<unsigned>((N + 15) / 16)), kI8Waves * kWave, 0, s>>>(
-                static_cast<const uint16_t*>(x) + m0 * K, w, scales, static_cast<uint16_t*>(out) + m0 * N, rows,
-                static_cast<int>(N), static_cast<int>(K));
+            const dim3 grid(static_cast<unsigned>((N + 15) / 16));
+            const auto* xs = static_cast<const uint16_t*>(x) + m0 * K;
+            auto* ys = static_cast<uint16_t*>(out) + m0 * N;
+            if (dtype == TPQ_DTYPE_F16)
+                int8pack_mfma_kernel<TPQ_DTYPE_F16><<<grid, kI8Waves * kWave, 0, s>>>(xs, w, scales, ys, rows, static_cast<int>(N), static_cast<int>(K));
+            else
+                int8pack_mfma_kernel<TPQ_DTYPE_BF16><<<grid, kI8Waves * kWave, 0, s>>>(xs, w, scales, ys, rows, static_cast<int>(N), static_cast<int>(K));
         }
         return check_launch("_weight_int8pack_mm (mfma)");
     }
