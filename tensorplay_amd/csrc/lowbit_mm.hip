@@ -8,7 +8,8 @@
 // buffer the modules keep (intx_weight_only.py:167-170).  The reference unpacks with tensor ops,
 // dequantizes to a dense float weight and calls a float GEMM (_intx_mm, intx_weight_only.py:127-133).
 //
-// Decode kernel (fp16 activations, 1..16 rows): v_mfma_f32_16x16x32_f16 with the weights as A.  Lane
+// Decode kernel (fp16 / bf16 activations, 1..16 rows): v_mfma_f32_16x16x32 with the weights as A (fp16 below;
+// bf16 converts each code to float and keeps the upper half).  Lane
 // (i, q) owns weight row n0 + i and, per step, 32 consecutive codes of it (16 when a code has a byte
 // to itself): 4 to 16 bytes, one load.  A code becomes an fp16 number without leaving its bits: the
 // byte is copied into both halves of a dword (v_perm_b32), a mask keeps one field per half and an
@@ -57,9 +58,14 @@ struct Fields {
     static constexpr int kMagics = kPerByte >= 2 ? kPerByte / 2 : 1;  // magic(t) repeats with this period
 };
 
-// x: [M][K] fp16; packed: [N][K / per_byte]; sz: [K / group][N][2] fp32; steps = K / kStepK; a group is
-// kStepK << group_shift k.  N % 4 == 0.
-template <int BITS, bool LSB, int WAVES>
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+
+// x: [M][K] fp16 or bf16; packed: [N][K / per_byte]; sz: [K / group][N][2] fp32; steps = K / kStepK; a group
+// is kStepK << group_shift k.  N % 4 == 0.
+// bf16 has seven mantissa bits, too few for the exponent trick: there a code is cut out of its dword,
+// converted to float (exact) and the upper halves of two floats are packed; no offsets to take out, the
+// constant-A MFMA only sums x.
+template <int DT, int BITS, bool LSB, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
     const float* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int group_shift) {
@@ -83,7 +89,10 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     // lane's codes: the pattern repeats every byte, so every MFMA has the same), row 1 = ones
     uint32_t a_corr[4];
 #pragma unroll
-    for (int h = 0; h < 4; ++h) a_corr[h] = i == 0 ? F::magic(h) : i == 1 ? 0x3C003C00u : 0u;
+    for (int h = 0; h < 4; ++h) {
+        if constexpr (DT == TPQ_DTYPE_F16) a_corr[h] = i == 0 ? F::magic(h) : i == 1 ? 0x3C003C00u : 0u;
+        else a_corr[h] = i == 1 ? 0x3F803F80u : 0u;
+    }
     uint32_t magic[F::kMagics];  // kept in VGPRs behind opaque moves: v_and_or_b32 takes one scalar operand
 #pragma unroll
     for (int t = 0; t < F::kMagics; ++t) asm volatile("v_mov_b32 %0, %1" : "=v"(magic[t]) : "s"(F::magic(t)));
@@ -115,13 +124,24 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
             for (int h = 0; h < 4; ++h) {
                 const int t = 4 * u + h;
                 const uint32_t word = dword_at(st.w, F::byte_lo(t) >> 2);
-                const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
-                a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
+                if constexpr (DT == TPQ_DTYPE_F16) {
+                    const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
+                    a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
+                } else {
+                    const float lo = static_cast<float>((word >> (8 * (F::byte_lo(t) & 3) + F::pos_lo(t))) & F::kField);
+                    const float hi = static_cast<float>((word >> (8 * (F::byte_hi(t) & 3) + F::pos_hi(t))) & F::kField);
+                    a[h] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+                }
             }
             const word4_t av = {a[0], a[1], a[2], a[3]}, cv = {a_corr[0], a_corr[1], a_corr[2], a_corr[3]};
             const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};  // the same eight k of the activations
-            aux = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, cv), __builtin_bit_cast(half8_t, bv), aux, 0, 0, 0);
-            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
+            if constexpr (DT == TPQ_DTYPE_F16) {
+                aux = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, cv), __builtin_bit_cast(half8_t, bv), aux, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
+            } else {
+                aux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, cv), __builtin_bit_cast(bf8_t, bv), aux, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), d, 0, 0, 0);
+            }
         }
         // rows 0 and 1 of the offset product sit in lanes 0..15, registers 0 and 1
         const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
@@ -166,8 +186,8 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
                 for (int w = 0; w < WAVES; ++w) sum[v] += red[w][v][lane];
                 if (bias != nullptr) sum[v] += bias[n + v];
             }
-            const uint32_t lo = f32_to_f16_bits(sum[0]) | (static_cast<uint32_t>(f32_to_f16_bits(sum[1])) << 16);
-            const uint32_t hi = f32_to_f16_bits(sum[2]) | (static_cast<uint32_t>(f32_to_f16_bits(sum[3])) << 16);
+            const uint32_t lo = Elem<DT>::store(sum[0]) | (static_cast<uint32_t>(Elem<DT>::store(sum[1])) << 16);
+            const uint32_t hi = Elem<DT>::store(sum[2]) | (static_cast<uint32_t>(Elem<DT>::store(sum[3])) << 16);
             *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
         }
     }
@@ -322,7 +342,7 @@ __global__ __launch_bounds__(256) void lowbit_unpack_kernel(const uint8_t* __res
     }
 }
 
-template <int BITS, bool LSB>
+template <int DT, int BITS, bool LSB>
 int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t M, int64_t N,
                 int64_t K, int group_shift, hipStream_t s) {
     // wavefronts per 16-channel workgroup: each takes every WAVES-th step, two in flight
@@ -336,9 +356,9 @@ int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const flo
         const uint16_t* xs = static_cast<const uint16_t*>(x) + m0 * K;
         uint16_t* ys = static_cast<uint16_t*>(out) + m0 * N;
         const int n = static_cast<int>(N), k = static_cast<int>(K);
-        if (waves >= 16) lowbit_mfma_kernel<BITS, LSB, 16><<<grid, 16 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
-        else if (waves >= 8) lowbit_mfma_kernel<BITS, LSB, 8><<<grid, 8 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
-        else lowbit_mfma_kernel<BITS, LSB, 4><<<grid, 4 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+        if (waves >= 16) lowbit_mfma_kernel<DT, BITS, LSB, 16><<<grid, 16 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+        else if (waves >= 8) lowbit_mfma_kernel<DT, BITS, LSB, 8><<<grid, 8 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+        else lowbit_mfma_kernel<DT, BITS, LSB, 4><<<grid, 4 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
     }
     return check_launch("tpq_lowbit_mm (mfma)");
 }
@@ -397,13 +417,16 @@ TPQ_EXPORT int tpq_lowbit_mm(const void* x, int dtype, int64_t M, int64_t K, con
             while ((int64_t{1} << group_shift) < per_group) ++group_shift;
         }
     }
-    const bool fast = dtype == TPQ_DTYPE_F16 && K > 0 && group_shift >= 0 && K % step_k == 0 && N % 4 == 0 && K <= 0x7FFFFF80 &&
+    const bool fast = dtype != TPQ_DTYPE_F32 && K > 0 && group_shift >= 0 && K % step_k == 0 && N % 4 == 0 && K <= 0x7FFFFF80 &&
                       N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(packed, 16) && aligned(scales_and_zeros, 16) && aligned(out, 8);
     if (fast) {
 #define TPQ_LB_CASE(BITS)                                                                                                      \
     case BITS:                                                                                                                 \
-        return lsb_first ? launch_mfma<BITS, true>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s)            \
-                         : launch_mfma<BITS, false>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s);
+        if (dtype == TPQ_DTYPE_F16)                                                                                            \
+            return lsb_first ? launch_mfma<TPQ_DTYPE_F16, BITS, true>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s) \
+                             : launch_mfma<TPQ_DTYPE_F16, BITS, false>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s); \
+        return lsb_first ? launch_mfma<TPQ_DTYPE_BF16, BITS, true>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s) \
+                         : launch_mfma<TPQ_DTYPE_BF16, BITS, false>(x, packed, scales_and_zeros, bias, out, M, N, K, group_shift, s);
         switch (bits) {
             TPQ_LB_CASE(1)
             TPQ_LB_CASE(2)

@@ -148,19 +148,20 @@ def test_gpu_mm_float32_small_shapes(bits, N, K, group, M):
 @pytest.mark.gpu
 @pytest.mark.parametrize("bits,lsb", [(b, False) for b in range(1, 9)] + [(1, True)])
 @pytest.mark.parametrize("N,K,group,M", [(64, 256, 128, 1), (36, 512, 256, 3), (48, 1024, 128, 16), (16, 384, 128, 17), (20, 128, 128, 2)])
-def test_gpu_mm_fp16_decode_kernel(bits, lsb, N, K, group, M):
+@pytest.mark.parametrize("tdt,tag,tol", [(torch.float16, "f16", 1e-3), (torch.bfloat16, "bf16", 8e-3)])  # output rounding 5e-4 / 4e-3
+def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
     from tensorplay_amd import ops
     rng = np.random.default_rng(bits * 13 + K + M)
     codes, sz = make_case(rng, bits, N, K, group)
-    x16 = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).half()
+    x16 = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(tdt)
     bias = rng.standard_normal(N).astype(np.float32) if M % 2 else None
     packed = oracle.lowbit_pack(codes, bits, lsb_first=lsb)
-    want = oracle.lowbit_mm(x16.view(torch.int16).numpy().view(np.uint16), "f16", packed, bits, sz, K, group, bias=bias,
+    want = oracle.lowbit_mm(x16.view(torch.int16).numpy().view(np.uint16), tag, packed, bits, sz, K, group, bias=bias,
                             lsb_first=lsb, want_f64=True)[1]
     got = ops._lowbit_mm(x16.to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV),
                          None if bias is None else torch.from_numpy(bias).to(DEV), lsb_first=lsb)
-    assert got.dtype == torch.float16 and got.shape == (M, N)
-    assert rel_err(got.float().cpu().numpy(), want) < 1e-3   # fp16 output rounding is 5e-4
+    assert got.dtype == tdt and got.shape == (M, N)
+    assert rel_err(got.float().cpu().numpy(), want) < tol
 
 
 @pytest.mark.gpu
