@@ -73,12 +73,19 @@ __device__ __forceinline__ uint16_t swiglu_of(float gate_sum, float up_sum) {
 // PAIR (NB = 2): the two blocks are the same 16 channels of two weights (packed / sz: gate, packed_b /
 // sz_b: up) and the output is silu_mul(gate, up).  residual (plain mode, may be null): [M][N], added to
 // the rounded output.
-template <int DT, int NB, int WAVES, bool PAIR = false>
+// GKT = k-tiles (of 32) per quantization group: 4 stands for groups of 128 k and more (above).  Groups of 32
+// or 64 k (GKT = 1, 2; fp16 only) differ between the four lanes an MFMA adds up, so there the weights are
+// dequantized in registers before the product, with the packed fp16 operations and roundings of the reference's
+// own dense weight, T(code - 8) * scale + zero (int4_tc_dequantize_kernel, QuantGemmKernels.cu:1170-1202):
+// three packed operations per pair, no offset MFMA, no per-step epilogue.
+template <int DT, int NB, int WAVES, bool PAIR = false, int GKT = 4>
 __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
     uint16_t* __restrict__ y, int M, int N, int K, int group_shift, const uint4* __restrict__ packed_b,
     const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual) {
     static_assert(!PAIR || NB == 2, "a pair is two blocks");
+    static_assert(GKT == 4 || (DT == TPQ_DTYPE_F16 && !PAIR), "in-register dequantization is built for fp16");
+    constexpr bool DEQ = GKT < 4;
     using L = Lane16<DT>;
     using ML = MfmaLane<DT>;
     __shared__ float red[WAVES][NB][4][kWave];
@@ -101,6 +108,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         int n4 = nb0 + 4 * q;                              // this lane's four output channels
         n4 = n4 + 4 <= N ? n4 : N - 4;
         sz_base[b] = (PAIR && b == 1 ? sz_b : sz) + n4;
+        if constexpr (DEQ) sz_base[b] = sz + ((nb0 + i) < N ? nb0 + i : N - 1);  // (scale, zero) of this lane's weight row
     }
     const bool row_live = i < M;
     const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 4;
@@ -122,7 +130,8 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             st.w[b] = nt_load(w_base[b] + static_cast<size_t>(s) * 32);             // four k-tiles further per step
-            st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
+            if constexpr (DEQ) st.p[b].x = sz_base[b][static_cast<size_t>((4 * s + q) / GKT) * N];  // group of k-tile 4 s + q
+            else st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
         }
         if (row_live) {  // columns m >= M keep the zeros they start with: no load, nothing stored
 #pragma unroll
@@ -148,6 +157,23 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int r = 0; r < 4; ++r) L::template unpack<true>(dword_of(st.w[b], r), v[b][r], magic_even, magic_odd);
+        if constexpr (DEQ) {
+            const half2_t off_even = {static_cast<_Float16>(1032.0f), static_cast<_Float16>(1032.0f)};  // magic + 8
+            const half2_t off_odd = {static_cast<_Float16>(72.0f), static_cast<_Float16>(72.0f)};
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint32_t pw = st.p[b].x;  // (scale, zero) of the lane's row and k-tile
+                const half2_t s2 = __builtin_bit_cast(half2_t, (pw & 0xFFFFu) | (pw << 16));
+                const half2_t z2 = __builtin_bit_cast(half2_t, (pw >> 16) | (pw & 0xFFFF0000u));
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const half2_t code = __builtin_bit_cast(half2_t, v[b][r][j]) - ((j & 1) ? off_odd : off_even);  // exact
+                        v[b][r][j] = __builtin_bit_cast(uint32_t, code * s2 + z2);  // rounded after the product and after the sum
+                    }
+            }
+        }
         // MFMA u (16x16x32) covers pair u of the four words of the lane's k-tile: k = 2 r + 8 u, + 1 for
         // r = 0..3, which are dwords 4u .. 4u+3 of the activations, one 16-byte load.
 #pragma unroll
@@ -155,12 +181,19 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
             const uint32_t off = (u & 1) ? a_corr_odd : a_corr_even;
             const word4_t xb = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
             const word4_t ac = {off, off, off, off};
-            aux = ML::mfma(ac, xb, aux);
+            if constexpr (!DEQ) aux = ML::mfma(ac, xb, aux);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const word4_t aw = {v[b][0][u], v[b][1][u], v[b][2][u], v[b][3][u]};
                 d[b] = ML::mfma(aw, xb, d[b]);
             }
+        }
+        if constexpr (DEQ) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) yacc[b][v] += d[b][v];
+            return;
         }
         // rows 0 and 1 of the correction product sit in lanes 0..15, registers 0 and 1
         const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);

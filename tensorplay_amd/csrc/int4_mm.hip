@@ -393,7 +393,8 @@ bool launch_stream(const void* x, const int32_t* packed, const void* sz, void* y
 template <int DT>
 bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void* sz, void* y, int N, int K,
                       int group, hipStream_t s, int* rc, const void* residual = nullptr) {
-    if ((group != 128 && group != 256) || !aligned(sz, 16) || !aligned(y, 8)) return false;
+    const bool deq = (group == 32 || group == 64) && DT == TPQ_DTYPE_F16 && residual == nullptr;  // dequantized in registers
+    if ((group != 128 && group != 256 && !deq) || !aligned(sz, 16) || !aligned(y, 8)) return false;
     if (residual != nullptr && !aligned(residual, 8)) return false;
     const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
     if (force && force[0] == 'd' && residual == nullptr) return false;
@@ -412,6 +413,19 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     const auto* sp = static_cast<const uint32_t*>(sz);
     auto* yp = static_cast<uint16_t*>(y);
     const int shift = group == 128 ? 0 : 1;  // a group is 128 << shift k (128 or 256)
+    if constexpr (DT == TPQ_DTYPE_F16) {
+        if (deq) {
+#define TPQ_MFMA_DEQ(NBV, WV, GKTV)                                                                                       \
+    int4_mfma_kernel<DT, NBV, WV, false, GKTV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \
+        xp, pp, sp, yp, rows, N, K, 0, nullptr, nullptr, nullptr)
+            const bool wide = N >= 8192;  // as for groups of 128: 32-channel workgroups at wide N, 8 wavefronts otherwise
+            if (group == 32) { if (wide) TPQ_MFMA_DEQ(2, 4, 1); else TPQ_MFMA_DEQ(1, 8, 1); }
+            else { if (wide) TPQ_MFMA_DEQ(2, 4, 2); else TPQ_MFMA_DEQ(1, 8, 2); }
+#undef TPQ_MFMA_DEQ
+            *rc = check_launch("tpq_int4_mm (mfma, small groups)");
+            return true;
+        }
+    }
 #define TPQ_MFMA(NBV, WV) \
     int4_mfma_kernel<DT, NBV, WV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \
         xp, pp, sp, yp, rows, N, K, shift, nullptr, nullptr, static_cast<const uint16_t*>(residual))
