@@ -49,3 +49,13 @@ def test_argument_validation_needs_no_gpu():
     assert lib.tpq_quantize_rowwise(None, 0, 0, 16, 1e-5, 127.0, -127, 127, 0, None, None, None) == _lib.TPQ_OK
     assert lib.tpq_int_mm(None, 0, None, 1, 1, None, 0, 4, 4, None) == _lib.TPQ_OK
     assert lib.tpq_ternary_mm(None, None, None, 1.0, None, 0, 4, 4, None, 0, None, None) == _lib.TPQ_OK
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark is a one-GPU program: any other --gpus value exits with a message and status 2."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 2 and "ONE GPU" in run.stderr
