@@ -3,6 +3,7 @@
 // int8_gemm_kernel.h, shared with the ternary matmul.
 #include <cstdlib>
 
+#include "int8_decode_kernel.h"
 #include "int8_gemm_dma.h"
 
 namespace tpq {
@@ -15,9 +16,23 @@ TileDequant<DT> to_tile(const EpilogueDequant<DT>& ep) {
     return TileDequant<DT>{ep.out, ep.rs, ep.cs, ep.bias};
 }
 
+// the epilogue of a slab of rows starting at m0: same operation, pointers moved to that row
+inline EpilogueInt32 rebase_rows(const EpilogueInt32& ep, int64_t m0, int64_t N) { return EpilogueInt32{ep.c + m0 * N}; }
+template <int DT>
+EpilogueDequant<DT> rebase_rows(const EpilogueDequant<DT>& ep, int64_t m0, int64_t N) {
+    return EpilogueDequant<DT>{ep.out + m0 * N, ep.rs + m0, ep.cs, ep.bias};
+}
+
 template <class Epilogue>
 int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
     const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
+    // a few rows: stream the weight once per 16 rows through the decode kernel.  K = N = 4096: 16 rows 7.3 us,
+    // 32 rows 13.2 us, 48 rows 20.0 us, against 21.3 / 22.7 / 22.7 us for the tiled kernels
+    static const int decode_rows = [] { const char* e = std::getenv("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : 48; }();
+    if (M <= decode_rows && int8_decode_ok(a, w, M, N, K) && !(force && force[0] == 'r'))
+        return launch_int8_decode(a, w, M, N, K, ep, [N](const Epilogue& e, int64_t m0) { return rebase_rows(e, m0, N); }, s);
+    // The ring-buffered kernel also wins when its 256 x 128 tiles fill only part of the chip: at K = N = 4096,
+    // M = 512 / 1024 it takes 27.9 / 29.5 us against 33.9 / 39.4 us for the register-staged kernel on 128 x 64 tiles.
     if (dma_path_ok(M, K) && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
     return launch_mfma(a, w, M, N, K, ep, s);
 }
