@@ -205,6 +205,15 @@ int tpq_int4_cpu_layout_to_device(const uint8_t* packed_cpu, int64_t N, int64_t 
 int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64_t K, const int8_t* w,
                            const float* scales, int64_t N, void* out, void* stream);
 
+/*
+ * Dense [N, K] weight of `dtype` from the int8 weight and its per-row scales: T(float(w) * scale[n]).
+ * For many activation rows the host op multiplies this with a library GEMM instead of streaming the
+ * int8 weight once per 16 rows (the reference's device op runs its batched GEMV at every size,
+ * p10/src/backend/cuda/QuantGemmKernels.cu:345-405).
+ */
+int tpq_int8pack_dequantize(const int8_t* w, const float* scales, int64_t N, int64_t K, int dtype,
+                            void* out, void* stream);
+
 /* Storage of quantized codes: one element per int8 / uint8 / int32, or 2 / 4 / 8 elements per byte
  * (element i in bits (i % pack) * bits of byte i / pack, i = row-major linear index). */
 #define TPQ_STORAGE_I8 0   /* reference dtype qint8   */

@@ -37,6 +37,7 @@ SIGNATURES = {
     "tpq_int4_pack_cpu_layout": [_ptr, _i64, _i64, _int, _int, _ptr, _ptr],
     "tpq_int4_cpu_layout_to_device": [_ptr, _i64, _i64, _int, _int, _ptr, _ptr],
     "tpq_weight_int8pack_mm": [_ptr, _int, _i64, _i64, _ptr, _ptr, _i64, _ptr, _ptr],
+    "tpq_int8pack_dequantize": [_ptr, _ptr, _i64, _i64, _int, _ptr, _ptr],
     "tpq_quantize_affine": [_ptr, _int, _int, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _int, _i64, _i64, _ptr, _ptr],
     "tpq_lowbit_mm": [_ptr, _int, _i64, _i64, _ptr, _int, _int, _i64, _i64, _ptr, _ptr, _ptr, _ptr],
     "tpq_lowbit_dequantize": [_ptr, _int, _int, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],

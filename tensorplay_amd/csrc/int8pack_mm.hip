@@ -228,10 +228,56 @@ int launch_generic(const void* x, const int8_t* w, const float* scale, void* y, 
     return check_launch("_weight_int8pack_mm (generic)");
 }
 
+// Dense [N, K] weight of `DT`: T(float(w) * scale[n]), one rounding; thread = 16 consecutive k of a row
+// (K % 16 == 0) or, for other K, one element.
+template <int DT>
+__global__ __launch_bounds__(256) void int8pack_dequantize_kernel(const int8_t* __restrict__ w, const float* __restrict__ scale,
+                                                                  typename Elem<DT>::storage* __restrict__ out, int64_t N, int64_t K,
+                                                                  int vectors) {
+    using S = typename Elem<DT>::storage;
+    if (vectors) {
+        const int64_t chunks = N * K / 16;
+        for (int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; c < chunks; c += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+            const float sc = scale[(c * 16) / K];
+            const uint4 raw = nt_load(reinterpret_cast<const uint4*>(w) + c);
+            const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+            __attribute__((aligned(16))) S o[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                o[e] = Elem<DT>::store(__fmul_rn(static_cast<float>(static_cast<int8_t>(words[e >> 2] >> (8 * (e & 3)))), sc));
+            uint4* dst = reinterpret_cast<uint4*>(out + c * 16);
+#pragma unroll
+            for (int e = 0; e < static_cast<int>(16 * sizeof(S) / 16); ++e) dst[e] = reinterpret_cast<const uint4*>(o)[e];
+        }
+    } else {
+        for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < N * K; i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+            out[i] = Elem<DT>::store(__fmul_rn(static_cast<float>(w[i]), scale[i / K]));
+    }
+}
+
 }  // namespace
 }  // namespace tpq
 
 using namespace tpq;
+
+TPQ_EXPORT int tpq_int8pack_dequantize(const int8_t* w, const float* scales, int64_t N, int64_t K, int dtype, void* out, void* stream) {
+    TPQ_REQUIRE(dtype == TPQ_DTYPE_F32 || dtype == TPQ_DTYPE_F16 || dtype == TPQ_DTYPE_BF16, TPQ_ERR_INVALID_TYPE,
+                "int8pack dequantize: the dense weight must be floating point");
+    TPQ_REQUIRE(N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "int8pack dequantize: negative shape");
+    if (N == 0 || K == 0) return TPQ_OK;
+    TPQ_REQUIRE(w && scales && out, TPQ_ERR_INVALID_VALUE, "int8pack dequantize: null pointer");
+    const int vectors = K % 16 == 0 && aligned(w, 16) && aligned(out, 16);
+    const int64_t items = vectors ? N * K / 16 : N * K;
+    const int64_t blocks = (items + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(blocks > (1 << 20) ? (1 << 20) : blocks);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case TPQ_DTYPE_F32: int8pack_dequantize_kernel<TPQ_DTYPE_F32><<<grid, 256, 0, s>>>(w, scales, static_cast<float*>(out), N, K, vectors); break;
+        case TPQ_DTYPE_F16: int8pack_dequantize_kernel<TPQ_DTYPE_F16><<<grid, 256, 0, s>>>(w, scales, static_cast<uint16_t*>(out), N, K, vectors); break;
+        default: int8pack_dequantize_kernel<TPQ_DTYPE_BF16><<<grid, 256, 0, s>>>(w, scales, static_cast<uint16_t*>(out), N, K, vectors); break;
+    }
+    return check_launch("tpq_int8pack_dequantize");
+}
 
 TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64_t K, const int8_t* w,
                                       const float* scales, int64_t N, void* out, void* stream) {

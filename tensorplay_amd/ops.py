@@ -326,6 +326,12 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
     return (out, acc) if return_acc else out
 
 
+# Above this many activation rows _weight_int8pack_mm dequantises and calls the library GEMM.  Measured at
+# K = 4096, N = 11008, fp16 (eager): the 16-row slabs cost about 20 us each (62 us at 48 rows), the dense route
+# 53 us at 128 rows and 203 us at 2048.
+INT8PACK_PREFILL_ROWS = 40
+
+
 def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
     """``(self @ mat2.T) * scales``: activations [B,K] float, int8 weight [N,K], per-row scales [N];
     fp32 accumulation, result in the activation dtype (reference: QuantGemmKernels.cu:345-405)."""
@@ -348,6 +354,13 @@ def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Te
     x, w = self.contiguous(), mat2.contiguous()
     sc = scales.to(torch.float32).contiguous()
     with torch.cuda.device(x.device):
+        if B > INT8PACK_PREFILL_ROWS:
+            # Many rows: the decode kernel streams the weight once per 16 rows, which stops paying here.  One pass
+            # writes the dense weight T(w * scale) and a library GEMM does the rest.
+            dense = torch.empty((N, K), dtype=x.dtype, device=x.device)
+            _check(_lib.load().tpq_int8pack_dequantize(_ptr(w), _ptr(sc), N, K, _DT[x.dtype], _ptr(dense), _stream(x)))
+            torch.matmul(x, dense.t(), out=out)
+            return out
         _check(_lib.load().tpq_weight_int8pack_mm(_ptr(x), _DT[x.dtype], B, K, _ptr(w), _ptr(sc), N, _ptr(out), _stream(x)))
     return out
 

@@ -84,3 +84,22 @@ def test_gpu_all_positive_activations_full_width():
     got = ops._weight_int8pack_mm(dev(xb, "f16"), dev(w), dev(s)).float().cpu().numpy()
     _, y64 = oracle.weight_int8pack_mm(xb, "f16", w, s, want_f64=True)
     assert rel_err(got, y64) < 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+def test_gpu_many_rows_take_the_dense_route(dtype):
+    """More rows than INT8PACK_PREFILL_ROWS: dense weight T(w * scale) + library GEMM, within the same bounds."""
+    import torch
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(77)
+    M, K, N = ops.INT8PACK_PREFILL_ROWS + 9, 272, 40
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.integers(-128, 128, (N, K)).astype(np.int8)
+    s = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
+    xt = torch.from_numpy(x).to(tdt)
+    got = ops._weight_int8pack_mm(xt.to("cuda:0"), torch.from_numpy(w).to("cuda:0"), torch.from_numpy(s).to("cuda:0"))
+    y64 = (xt.double().numpy() @ w.astype(np.float64).T) * s.astype(np.float64)
+    assert got.dtype == tdt and got.shape == (M, N)
+    assert rel_err(got.float().cpu().numpy(), y64) < {"f32": 1e-4, "f16": 2e-3, "bf16": 1.6e-2}[dtype]
