@@ -20,6 +20,8 @@
 // expands the 2-bit chunks to int8 on their way into LDS.
 //
 // Anything else: one thread per output.
+#include <cstdlib>
+
 #include "int8_gemm_kernel.h"
 #include "ternary_gemm_kernel.h"
 
@@ -115,7 +117,16 @@ template <class Epilogue>
 int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N, int64_t K,
                    Epilogue ep, hipStream_t s) {
     const bool sizes_ok = M <= 0x7FFFFFFF && N <= 0x7FFFFFFF && K <= 0x7FFFFFFF;
-    if (sizes_ok && M <= 8 && K % 64 == 0 && aligned(x, 16) && aligned(packed, 16)) {
+    // the tile kernel below takes over where it is faster and its shape conditions hold
+    // Measured at 2560 -> 6912 / 6912 -> 2560 (216 / 80 tiles of 32 channels): the decode kernel takes 7, 7.5, 9.4, 11.4 us
+    // for 1..4 rows and twice that for 5..8, the tile kernel 9.3 / 18.3 us for any row count up to 128.
+    static const int forced_decode_rows = [] { const char* e = std::getenv("TPQ_TERNARY_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
+    // ... and stays ahead of the 256 x 128-tile kernel at every larger row count tried (512 rows: 30 / 33 us against
+    // 54 / 103 us; 2048 rows: 100 / 85 us against 111 / 112 us), so there is no upper limit by default.
+    static const int64_t gemm_rows = [] { const char* e = std::getenv("TPQ_TERNARY_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{1} << 40; }();
+    const int decode_rows = forced_decode_rows >= 0 ? forced_decode_rows : ((N + kTgN - 1) / kTgN >= 128 ? 3 : 6);
+    const bool gemm_ok = sizes_ok && M <= gemm_rows && K % kTgStage == 0 && aligned(x, 16) && aligned(packed, 4);
+    if (sizes_ok && M <= 8 && (M <= decode_rows || !gemm_ok) && K % 64 == 0 && aligned(x, 16) && aligned(packed, 16)) {
         const int waves = static_cast<int>((N + kRowsPerWave - 1) / kRowsPerWave);
         const dim3 grid((waves + 3) / 4);
         for (int m0 = 0; m0 < M; m0 += 4) {
@@ -129,8 +140,7 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
         }
         return check_launch("tpq_ternary_mm (decode)");
     }
-    if (sizes_ok && M <= 256 && ternary_gemm_m128_ok(M, K) && aligned(x, 16) && aligned(packed, 4))
-        return launch_ternary_gemm_m128(x, packed, M, N, K, ep, s);
+    if (gemm_ok) return launch_ternary_gemm_m128(x, packed, M, N, K, ep, s);
     if (sizes_ok && K % 16 == 0 && aligned(x, 16) && aligned(packed, 4))
         return launch_mfma<true>(x, packed, M, N, K, ep, s);
     const int64_t blocks = (M * N + 255) / 256;

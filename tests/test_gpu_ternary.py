@@ -45,7 +45,9 @@ def test_unpack_every_byte_value(ops):
 # (M, K, N): decode kernel, matrix-core kernel, generic kernel
 CASES = [(1, 2560, 6912), (1, 6912, 2560), (4, 2560, 256), (8, 128, 67), (5, 64, 9), (128, 2560, 6912),
          (128, 6912, 2560), (16, 256, 100), (33, 48, 70), (3, 9, 5), (2, 10, 4), (9, 2560, 130),
-         (200, 512, 70), (97, 256, 33), (300, 256, 64)]
+         (200, 512, 70), (97, 256, 33), (300, 256, 64),
+         # tile kernel below nine rows (many / few tiles of 32 channels) and beyond 256 rows
+         (4, 256, 4200), (7, 512, 72), (8, 768, 40), (513, 512, 100), (700, 256, 4160)]
 
 
 @pytest.mark.parametrize("M,K,N", CASES)
