@@ -1,10 +1,12 @@
 // Fused row-wise signed quantizer for gfx950.
 //
-// One 256-thread workgroup per row.  The row is read from HBM once, kept in
+// One 256-thread workgroup per row (rows of up to 1024 elements: a lane group of 8..64 lanes per
+// row, several rows per workgroup).  The row is read from HBM once, kept in
 // registers (8 elements per 16/32-byte vector load, up to 8 such chunks per
 // lane), reduced to its absolute maximum with a 64-lane butterfly and one LDS
 // exchange between the four wavefronts, and written back as int8 codes with
-// 8-byte stores.  Rows longer than the register budget (K > 16384) or rows
+// 8-byte stores (rows of more than 16384 elements: 1024 threads).  Rows longer than the register budget
+// (K > 65536) or rows
 // that cannot be vector-loaded (K % 8 != 0) take the streaming kernel, which
 // reads the row a second time (the second read comes from L2).
 //
@@ -55,7 +57,8 @@ __device__ __forceinline__ void quantize_eight(const float (&v)[kVec], float sca
     }
 }
 
-// Block-wide max over 256 threads; every thread gets the result.
+// Block-wide max over THREADS threads; every thread gets the result.
+template <int THREADS = kThreads>
 __device__ __forceinline__ float block_max(float v, float* smem) {
     v = wave_max(v);
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
@@ -63,7 +66,7 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
     __syncthreads();
     float r = smem[0];
 #pragma unroll
-    for (int w = 1; w < kThreads / kWave; ++w) r = fmaxf(r, smem[w]);
+    for (int w = 1; w < THREADS / kWave; ++w) r = fmaxf(r, smem[w]);
     return r;
 }
 
@@ -86,12 +89,12 @@ __device__ __forceinline__ void load_chunk(const typename Elem<DT>::storage* p, 
     }
 }
 
-// Row cached in registers: CHUNKS * 256 * 8 >= K, K % 8 == 0.
-template <int DT, int CHUNKS>
-__global__ __launch_bounds__(kThreads) void quantize_rows_cached(
+// Row cached in registers: CHUNKS * THREADS * 8 >= K, K % 8 == 0.
+template <int DT, int CHUNKS, int THREADS = kThreads>
+__global__ __launch_bounds__(THREADS) void quantize_rows_cached(
     const typename Elem<DT>::storage* __restrict__ x, int8_t* __restrict__ codes,
     float* __restrict__ scales, int K, QParams p) {
-    __shared__ float smem[kThreads / kWave];
+    __shared__ float smem[THREADS / kWave];
     const int64_t row = blockIdx.x;
     const auto* xr = x + row * K;
     int8_t* cr = codes + row * K;
@@ -100,14 +103,14 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_cached(
     float absmax = 0.0f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
-        const int k0 = (c * kThreads + threadIdx.x) * kVec;
+        const int k0 = (c * THREADS + threadIdx.x) * kVec;
         if (k0 < K) {
             load_chunk<DT>(xr + k0, v[c]);
 #pragma unroll
             for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
         }
     }
-    absmax = block_max(absmax, smem);
+    absmax = block_max<THREADS>(absmax, smem);
     const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
     if (threadIdx.x == 0) scales[row] = scale;
     // the shortcut needs |quotient| <= 128 and a finite reciprocal: true for every scale the formula
@@ -117,8 +120,61 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_cached(
 
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
-        const int k0 = (c * kThreads + threadIdx.x) * kVec;
+        const int k0 = (c * THREADS + threadIdx.x) * kVec;
         if (k0 < K) {
+            int code[kVec];
+            if (shortcut) {
+                quantize_eight(v[c], scale, inv_scale, p, code);
+            } else {
+#pragma unroll
+                for (int i = 0; i < kVec; ++i) code[i] = quantize_one(v[c][i], scale, p);
+            }
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                lo |= (static_cast<uint32_t>(code[i]) & 0xFFu) << (8 * i);
+                hi |= (static_cast<uint32_t>(code[i + 4]) & 0xFFu) << (8 * i);
+            }
+            *reinterpret_cast<uint2*>(cr + k0) = make_uint2(lo, hi);
+        }
+    }
+}
+
+// Short rows (K <= LANES * CHUNKS * 8, K % 8 == 0): LANES lanes of a wavefront per row, so a workgroup
+// takes 256 / LANES rows and no lane idles; the maximum is a butterfly inside the lane group, no LDS.
+template <int DT, int LANES, int CHUNKS>
+__global__ __launch_bounds__(kThreads) void quantize_rows_subwave(
+    const typename Elem<DT>::storage* __restrict__ x, int8_t* __restrict__ codes,
+    float* __restrict__ scales, int64_t M, int K, QParams p) {
+    constexpr int kRows = kThreads / LANES;
+    const int sub = threadIdx.x % LANES;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRows + threadIdx.x / LANES;
+    const bool live = row < M;  // dead lanes still take part in the butterfly
+    const auto* xr = x + (live ? row : 0) * K;
+    int8_t* cr = codes + (live ? row : 0) * K;
+
+    float v[CHUNKS][kVec];
+    float absmax = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k0 = (c * LANES + sub) * kVec;
+        if (live && k0 < K) {
+            load_chunk<DT>(xr + k0, v[c]);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
+        }
+    }
+#pragma unroll
+    for (int off = LANES / 2; off >= 1; off >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, off));
+    const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
+    if (live && sub == 0) scales[row] = scale;
+    const float inv_scale = __fdiv_rn(1.0f, scale);
+    const bool shortcut = !p.sign_mode && p.divisor <= 128.0f && inv_scale < 3.0e38f && absmax <= 3.0e38f;  // as above
+
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int k0 = (c * LANES + sub) * kVec;
+        if (live && k0 < K) {
             int code[kVec];
             if (shortcut) {
                 quantize_eight(v[c], scale, inv_scale, p, code);
@@ -161,14 +217,29 @@ int launch(const void* x, int64_t M, int64_t K, const QParams& p, int8_t* codes,
     using S = typename Elem<DT>::storage;
     const S* xp = static_cast<const S*>(x);
     const dim3 grid(static_cast<unsigned>(M)), block(kThreads);
-    const bool vec_ok = (K % kVec == 0) && aligned(x, 16) && aligned(codes, 8) && K <= 8 * kThreads * kVec;
-    if (vec_ok) {
+    const bool vec_ok = (K % kVec == 0) && aligned(x, 16) && aligned(codes, 8) && K <= 8 * 1024 * kVec;
+    if (vec_ok && K <= 1024) {
+        const int k = static_cast<int>(K);
+        auto run = [&](auto lanes, auto chunks) {
+            constexpr int L = decltype(lanes)::value, C = decltype(chunks)::value;
+            const dim3 g(static_cast<unsigned>((M + kThreads / L - 1) / (kThreads / L)));
+            quantize_rows_subwave<DT, L, C><<<g, block, 0, stream>>>(xp, codes, scales, M, k, p);
+        };
+        using std::integral_constant;
+        if (K <= 64) run(integral_constant<int, 8>{}, integral_constant<int, 1>{});
+        else if (K <= 128) run(integral_constant<int, 16>{}, integral_constant<int, 1>{});
+        else if (K <= 256) run(integral_constant<int, 32>{}, integral_constant<int, 1>{});
+        else if (K <= 512) run(integral_constant<int, 64>{}, integral_constant<int, 1>{});
+        else run(integral_constant<int, 64>{}, integral_constant<int, 2>{});
+    } else if (vec_ok) {
         const int chunks = static_cast<int>((K + kThreads * kVec - 1) / (kThreads * kVec));
         const int k = static_cast<int>(K);
         if (chunks <= 1) quantize_rows_cached<DT, 1><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
         else if (chunks <= 2) quantize_rows_cached<DT, 2><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
         else if (chunks <= 4) quantize_rows_cached<DT, 4><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
-        else quantize_rows_cached<DT, 8><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
+        else if (chunks <= 8) quantize_rows_cached<DT, 8><<<grid, block, 0, stream>>>(xp, codes, scales, k, p);
+        else if (chunks <= 16) quantize_rows_cached<DT, 4, 1024><<<grid, 1024, 0, stream>>>(xp, codes, scales, k, p);
+        else quantize_rows_cached<DT, 8, 1024><<<grid, 1024, 0, stream>>>(xp, codes, scales, k, p);
     } else {
         quantize_rows_streaming<DT><<<grid, block, 0, stream>>>(xp, codes, scales, K, p);
     }

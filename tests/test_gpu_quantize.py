@@ -17,7 +17,9 @@ def ops():
 
 
 SHAPES = [(1, 1), (3, 5), (16, 1024), (7, 2560), (1, 6912), (5, 4099), (4, 8), (2, 16384), (2, 20000),
-          (3, 16392), (128, 6912), (300, 2048), (2048, 4096)]
+          (3, 16392), (128, 6912), (300, 2048), (2048, 4096),
+          (1000, 64), (77, 56), (33, 128), (5, 200), (129, 512), (9, 264), (70, 1000), (4097, 1024), (3, 1032),
+          (3, 28672), (2, 65536), (2, 65544), (5, 40000)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
