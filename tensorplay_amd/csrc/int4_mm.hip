@@ -398,15 +398,20 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     if (residual != nullptr && !aligned(residual, 8)) return false;
     const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
     if (force && force[0] == 'd' && residual == nullptr) return false;
-    if (rows == 1 && residual == nullptr && !(force && force[0] == 'm')) return false;
-    // Every workgroup reads all of x from cache, so many rows want wide workgroups (64 channels),
-    // but only when N still yields enough of them to fill the chip.  Measured (us, weights from
-    // HBM): N=11008 K=4096: 4 rows 9.6 (16 ch, 8 waves); 8 rows 10.9 (64 ch) vs 11.3 (16 ch);
-    // 16 rows 11.8 (64 ch) vs 16.7 (16 ch).  N=4096 K=4096: 8 rows 5.7 (16 ch) vs 9.9 (64 ch).
-    // 4 rows at N=11008: 32 ch x 4 waves 9.06, 64 ch x 4 waves 9.32, 16 ch x 8 waves 9.68 us
-    int nb = N >= 8192 ? (rows > 4 ? 4 : 2) : 1;
+    // One row: the column-per-lane kernel wins only where N is wide enough to fill the chip with its
+    // 64-column workgroups (measured: N = 11008, K = 4096: 7.1 us against 8.5 us here; N = 4096,
+    // K = 11008: 12.5 against 9.7; N = 8192, K = 28672: 32.8 against 26.4).
+    if (rows == 1 && residual == nullptr && N >= 10240 && !(force && force[0] == 'm')) return false;
+    // Channels per workgroup (16 nb) and wavefronts per workgroup, from a sweep over model shapes
+    // (K 4096..28672, 2..16 rows).  Every workgroup reads all of x from cache, so many rows want wide
+    // workgroups, but only when N still yields enough of them to fill the chip:
+    //   N = 4096:  16 ch x 8 waves always (8 rows: 5.3 us against 6.0 for 32 ch, 8.5 for 64 ch)
+    //   N = 6144, 8192:  32 ch x 8 waves (8192 x 8192, 8 rows: 9.8 us against 13.4 for 16 ch, 14.6 for 64 ch)
+    //   N >= 11008:  32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (11008 x 4096, 16 rows: 9.7 us
+    //                against 12.2 for 32 ch and 14.9 for 16 ch)
+    int nb = N > 5120 ? (N < 10240 ? 2 : (rows > 4 ? 4 : 2)) : 1;
     if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
-    int waves = nb == 1 && rows <= 8 ? 8 : 4;
+    int waves = N < 10240 ? 8 : 4;
     if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
@@ -418,9 +423,14 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
 #define TPQ_MFMA_DEQ(NBV, WV, GKTV)                                                                                       \
     int4_mfma_kernel<DT, NBV, WV, false, GKTV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \
         xp, pp, sp, yp, rows, N, K, 0, nullptr, nullptr, nullptr)
-            const bool wide = N >= 8192;  // as for groups of 128: 32-channel workgroups at wide N, 8 wavefronts otherwise
-            if (group == 32) { if (wide) TPQ_MFMA_DEQ(2, 4, 1); else TPQ_MFMA_DEQ(1, 8, 1); }
-            else { if (wide) TPQ_MFMA_DEQ(2, 4, 2); else TPQ_MFMA_DEQ(1, 8, 2); }
+            // same shapes of workgroup as for groups of 128
+            if (group == 32) {
+                if (nb == 1) TPQ_MFMA_DEQ(1, 8, 1); else if (nb == 2 && waves == 8) TPQ_MFMA_DEQ(2, 8, 1);
+                else if (nb == 2) TPQ_MFMA_DEQ(2, 4, 1); else TPQ_MFMA_DEQ(4, 4, 1);
+            } else {
+                if (nb == 1) TPQ_MFMA_DEQ(1, 8, 2); else if (nb == 2 && waves == 8) TPQ_MFMA_DEQ(2, 8, 2);
+                else if (nb == 2) TPQ_MFMA_DEQ(2, 4, 2); else TPQ_MFMA_DEQ(4, 4, 2);
+            }
 #undef TPQ_MFMA_DEQ
             *rc = check_launch("tpq_int4_mm (mfma, small groups)");
             return true;
