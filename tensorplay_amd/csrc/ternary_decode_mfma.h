@@ -1,0 +1,156 @@
+// Ternary-weight product for a few activation rows (1..16 per launch: decode batches of the BitNet
+// linear), K % 256 == 0.  The packed weight is streamed once whatever the row count:
+// v_mfma_i32_16x16x64_i8 with the WEIGHTS as the A operand, NB blocks of 16 channels per workgroup.
+// Lane (i, q) owns weight row n0 + i and, in a step of 256 k, the 16 packed bytes (64 codes) at
+// k = 256 s + 64 q: one 16-byte load, four MFMAs (one per packed dword).
+//
+// Expanding a packed dword w (bytes b = 0..3, the code of k = 4 b + j in bits 7-2j..6-2j of byte b) the
+// cheap way gives the codes of ONE field position per register: (w >> (6 - 2 j)) & 0x03030303 holds
+// the four codes k = j, 4 + j, 8 + j, 12 + j as bytes, and v_perm_b32 with those bytes as selectors
+// into the table {0, 1, -2, -1} sign-extends them: 3 instructions per int8 dword.  Which k sits in
+// which slot of the MFMA is free as long as both operands agree, so the activations are brought into
+// the same order instead: lane (m, q) loads x[m][256 s + 64 q .. + 64) as four 16-byte chunks and
+// transposes each as a 4 x 4 byte matrix (8 v_perm_b32), once for all NB channel blocks.
+// D comes out as lane (m, q) x channels 4 q + v of a block in int32, exact; the wavefronts of a
+// workgroup take the steps round-robin and add their partial sums through LDS.  Columns m >= M stay
+// zero and load nothing.
+#pragma once
+
+#include "int8_gemm_kernel.h"
+
+namespace tpq {
+namespace {
+
+// 16 consecutive int8 (k0 .. k0 + 15) -> register j holds k0 + j, 4 + j, 8 + j, 12 + j
+__device__ __forceinline__ v4i transpose_4x4_bytes(const uint4 r) {
+    const uint32_t lo01 = __builtin_amdgcn_perm(r.y, r.x, 0x05010400u), hi01 = __builtin_amdgcn_perm(r.y, r.x, 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(r.w, r.z, 0x05010400u), hi23 = __builtin_amdgcn_perm(r.w, r.z, 0x07030602u);
+    v4i out;
+    out[0] = static_cast<int>(__builtin_amdgcn_perm(lo23, lo01, 0x05040100u));
+    out[1] = static_cast<int>(__builtin_amdgcn_perm(lo23, lo01, 0x07060302u));
+    out[2] = static_cast<int>(__builtin_amdgcn_perm(hi23, hi01, 0x05040100u));
+    out[3] = static_cast<int>(__builtin_amdgcn_perm(hi23, hi01, 0x07060302u));
+    return out;
+}
+
+// one packed dword (16 codes) -> register j holds the codes of field position j of its four bytes
+__device__ __forceinline__ v4i ternary_fields_to_i8(uint32_t w) {
+    constexpr uint32_t kTable = 0xFFFE0100u;  // selector 0..3 -> 0, 1, -2, -1
+    v4i out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        out[j] = static_cast<int>(__builtin_amdgcn_perm(0u, kTable, (w >> (6 - 2 * j)) & 0x03030303u));
+    return out;
+}
+
+template <int NB, int WAVES, class Epilogue>
+__global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(const int8_t* __restrict__ x, const uint8_t* __restrict__ packed,
+                                                                           int m_base, int M, int N, int K, Epilogue ep) {
+    __shared__ int red[WAVES][NB][4][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, q = lane >> 4;
+    const int steps = K / 256;
+    const int n0 = blockIdx.x * (16 * NB);
+    const bool row_live = i < M;
+    const size_t bpr = static_cast<size_t>(K) >> 2;
+    const uint4* w_base[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int n = n0 + 16 * b + i;
+        w_base[b] = reinterpret_cast<const uint4*>(packed + static_cast<size_t>(n < N ? n : N - 1) * bpr) + q;  // rows past N: a valid row, result dropped
+    }
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m_base + (row_live ? i : 0)) * K) + q * 4;
+
+    struct Step {
+        uint4 w[NB];
+        uint4 xv[4];
+    };
+    auto load = [&](int s, Step& st) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) st.w[b] = nt_load(w_base[b] + s * 4);
+        if (row_live) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) st.xv[d] = x_base[s * 16 + d];
+        }
+    };
+    v4i acc[NB][2] = {};  // two accumulators per block taking turns
+    auto compute = [&](const Step& st) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const v4i xb = transpose_4x4_bytes(st.xv[d]);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint32_t word = d == 0 ? st.w[b].x : d == 1 ? st.w[b].y : d == 2 ? st.w[b].z : st.w[b].w;
+                acc[b][d & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ternary_fields_to_i8(word), xb, acc[b][d & 1], 0, 0, 0);
+            }
+        }
+    };
+
+    // this wavefront's steps: wave, wave + WAVES, ...; four in flight (a step is 16 NB + 64 bytes per lane)
+    constexpr int kRing = 4;
+    Step ring[kRing] = {};
+#pragma unroll
+    for (int r = 0; r < kRing; ++r)
+        if (wave + r * WAVES < steps) load(wave + r * WAVES, ring[r]);
+    for (int base = wave; base < steps; base += kRing * WAVES) {
+#pragma unroll
+        for (int r = 0; r < kRing; ++r) {
+            const int s = base + r * WAVES;
+            if (s < steps) {
+                compute(ring[r]);
+                if (s + kRing * WAVES < steps) load(s + kRing * WAVES, ring[r]);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = acc[b][0][v] + acc[b][1][v];
+    __syncthreads();
+    if (wave == 0 && row_live) {  // lane (m, q): channels n0 + 16 b + 4 q + v
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                int sum = 0;
+#pragma unroll
+                for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b][v][lane];
+                const int n = n0 + 16 * b + 4 * q + v;
+                if (n < N) ep.store(static_cast<int64_t>(m_base + i) * N + n, m_base + i, n, sum);
+            }
+    }
+}
+
+inline bool ternary_decode_mfma_ok(const void* x, const void* packed, int64_t M, int64_t N, int64_t K) {
+    return M >= 1 && N >= 1 && K >= 256 && K % 256 == 0 && aligned(x, 16) && aligned(packed, 16) && M <= 0x7FFFFFF0 && N <= 0x7FFFFFF0 &&
+           K <= 0x7FFFFF00;
+}
+
+// slabs of 16 rows
+template <class Epilogue>
+int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
+    static const int forced_nb = [] { const char* e = std::getenv("TPQ_TERNARY_NB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_waves = [] { const char* e = std::getenv("TPQ_TERNARY_WAVES"); return e ? std::atoi(e) : 0; }();
+    // Workgroup shape from a sweep over model shapes (K 2560..28672, 1..16 rows), about 2000..4000 wavefronts in all:
+    //   N < 8192: 16 channels x 8 wavefronts (4096 x 4096, 8 rows: 5.0 us; 32 channels: 6.6)
+    //   N < 10240: 32 x 8 (8192 x 28672 -> 8192, 16 rows: 26.4 us; 16 channels: 36.3)
+    //   N < 16384: 16 x 4 (4096 -> 11008, 2 rows: 6.7 us; 8 wavefronts 7.6, 32 channels 7.9)
+    //   above: 32 x 4 (8192 -> 28672, 8 rows: 24.3 us; 16 channels 28.2, 8 wavefronts 29.4)
+    const int nb = forced_nb ? forced_nb : ((N >= 8192 && N < 10240) || N >= 16384 ? 2 : 1);
+    const int waves = forced_waves ? forced_waves : (N < 10240 ? 8 : 4);
+    const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        const int mb = static_cast<int>(m0), n = static_cast<int>(N), k = static_cast<int>(K);
+        if (nb == 2 && waves == 8) ternary_decode_mfma_kernel<2, 8, Epilogue><<<grid, 8 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
+        else if (nb == 2) ternary_decode_mfma_kernel<2, 4, Epilogue><<<grid, 4 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
+        else if (waves == 8) ternary_decode_mfma_kernel<1, 8, Epilogue><<<grid, 8 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
+        else ternary_decode_mfma_kernel<1, 4, Epilogue><<<grid, 4 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
+    }
+    return check_launch("tpq_ternary_mm (mfma decode)");
+}
+
+}  // namespace
+}  // namespace tpq

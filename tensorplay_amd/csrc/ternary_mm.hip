@@ -7,7 +7,9 @@
 // weight is ever materialised (the reference unpacks to int8 on every call,
 // tensorplay/ao/quantization/bitnet.py:233).
 //
-// Decode kernel (M <= 8): one wavefront per 4 weight rows, lane l owns the
+// Up to 32 rows with K % 256 == 0: the matrix-core decode kernel of ternary_decode_mfma.h.
+//
+// Dot-product decode kernel (M <= 8, other K % 64 == 0): one wavefront per 4 weight rows, lane l owns the
 // 16-byte chunks l, l+64, ... of each row (64 codes per chunk, 1 KB per
 // wavefront load).  For field position q of every byte,
 //   f = (w >> (6-2q)) & 0x03030303  are four unsigned codes, and
@@ -16,14 +18,15 @@
 // (a 4x4 byte transpose of the activation chunk, done once per wavefront and
 // reused for its rows).  v_dot4_i32_i8 does the multiply-adds.
 //
-// Prefill (M > 8, K % 16 == 0): the int8 matrix-core GEMM with a loader that
-// expands the 2-bit chunks to int8 on their way into LDS.
+// More rows: the tile kernel of ternary_gemm_kernel.h (K % 256 == 0), else (K % 16 == 0) the int8
+// matrix-core GEMM with a loader that expands the 2-bit chunks to int8 on their way into LDS.
 //
 // Anything else: one thread per output.
 #include <cstdlib>
 
 #include "int8_gemm_kernel.h"
 #include "ternary_gemm_kernel.h"
+#include "ternary_decode_mfma.h"
 
 namespace tpq {
 namespace {
@@ -125,6 +128,13 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
     // 54 / 103 us; 2048 rows: 100 / 85 us against 111 / 112 us), so there is no upper limit by default.
     static const int64_t gemm_rows = [] { const char* e = std::getenv("TPQ_TERNARY_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{1} << 40; }();
     const int decode_rows = forced_decode_rows >= 0 ? forced_decode_rows : ((N + kTgN - 1) / kTgN >= 128 ? 3 : 6);
+    // Up to 32 rows, in slabs of 16: the weight streamed once per slab through the matrix cores.  Measured against the
+    // kernels below over K, N = 1024..28672: one row 4.3..19.8 us (the dot-product kernel 4.7..19.2), 16 rows
+    // 5.2..29.6 us (the tile kernel 9.3..75 us for any row count up to 128; two slabs stay below it, three do not).
+    static const int mfma_min = [] { const char* e = std::getenv("TPQ_TERNARY_MFMA_MIN"); return e ? std::atoi(e) : 1; }();
+    static const int mfma_rows = [] { const char* e = std::getenv("TPQ_TERNARY_MFMA_ROWS"); return e ? std::atoi(e) : 32; }();
+    if (forced_decode_rows < 0 && M >= mfma_min && M <= mfma_rows && ternary_decode_mfma_ok(x, packed, M, N, K))
+        return launch_ternary_decode_mfma(x, packed, M, N, K, ep, s);
     const bool gemm_ok = sizes_ok && M <= gemm_rows && K % kTgStage == 0 && aligned(x, 16) && aligned(packed, 4);
     if (sizes_ok && M <= 8 && (M <= decode_rows || !gemm_ok) && K % 64 == 0 && aligned(x, 16) && aligned(packed, 16)) {
         const int waves = static_cast<int>((N + kRowsPerWave - 1) / kRowsPerWave);

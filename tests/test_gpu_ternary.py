@@ -47,7 +47,10 @@ CASES = [(1, 2560, 6912), (1, 6912, 2560), (4, 2560, 256), (8, 128, 67), (5, 64,
          (128, 6912, 2560), (16, 256, 100), (33, 48, 70), (3, 9, 5), (2, 10, 4), (9, 2560, 130),
          (200, 512, 70), (97, 256, 33), (300, 256, 64),
          # tile kernel below nine rows (many / few tiles of 32 channels) and beyond 256 rows
-         (4, 256, 4200), (7, 512, 72), (8, 768, 40), (513, 512, 100), (700, 256, 4160)]
+         (4, 256, 4200), (7, 512, 72), (8, 768, 40), (513, 512, 100), (700, 256, 4160),
+         # matrix-core decode kernel: each workgroup shape (by N), ragged N, one and two slabs of rows
+         (1, 4096, 4100), (2, 2560, 8200), (16, 512, 8192), (3, 1024, 11010), (15, 256, 16390), (17, 768, 50),
+         (32, 512, 8208), (31, 6912, 2560), (12, 256, 1), (1, 256, 17)]
 
 
 @pytest.mark.parametrize("M,K,N", CASES)
