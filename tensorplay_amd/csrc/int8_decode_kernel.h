@@ -1,5 +1,5 @@
-// int8 x int8 product for a few activation rows (1..16 per launch: decode batches of the dynamic int8
-// linear), K % 128 == 0.  At these sizes the product is a stream over the weight, one byte per element,
+// int8 x int8 product for a few activation rows (1..16 MB per launch: decode batches of the dynamic int8
+// linear), K % 128 == 0, NB blocks of 16 channels per workgroup.  At these sizes the product is a stream over the weight, one byte per element,
 // and what matters is reading it once at full rate: v_mfma_i32_16x16x64_i8 with the WEIGHTS as the A
 // operand, exactly as the weight-only decode kernels do.  Lane (i, q) owns weight row n0 + i and, in a
 // step of 128 k, the 32 bytes at k = 128 s + 32 q: two 16-byte loads, each the A operand of one MFMA
@@ -10,45 +10,67 @@
 // partial sums through LDS.  Columns m >= M stay zero and load nothing.
 #pragma once
 
+#include <cstdlib>
+
 #include "int8_gemm_kernel.h"
 
 namespace tpq {
 namespace {
 
-template <int WAVES, class Epilogue>
+template <int NB, int MB, int WAVES, class Epilogue>
 __global__ __launch_bounds__(WAVES * kWave) void int8_decode_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ w,
                                                                    int M, int N, int K, Epilogue ep) {
-    __shared__ int red[WAVES][4][kWave];
+    __shared__ int red[WAVES][NB * MB][4][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int steps = K / 128;
-    const int n0 = blockIdx.x * 16;
-    const int n_row = n0 + i < N ? n0 + i : N - 1;  // rows past N: a valid row, result dropped
-    const bool row_live = i < M;
-    const uint4* w_base = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n_row) * K) + q * 2;
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 2;
+    const int n0 = blockIdx.x * (16 * NB);
+    const uint4* w_base[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int n = n0 + 16 * b + i;
+        w_base[b] = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n < N ? n : N - 1) * K) + q * 2;  // rows past N: a valid row, result dropped
+    }
+    bool row_live[MB];
+    const uint4* x_base[MB];
+#pragma unroll
+    for (int r = 0; r < MB; ++r) {
+        row_live[r] = 16 * r + i < M;
+        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live[r] ? 16 * r + i : 0) * K) + q * 2;
+    }
 
     struct Step {
-        uint4 w[2];
-        uint4 xv[2];
+        uint4 w[NB][2];
+        uint4 xv[MB][2];
     };
     auto load = [&](int s, Step& st) {
-        st.w[0] = nt_load(w_base + s * 8);
-        st.w[1] = nt_load(w_base + s * 8 + 1);
-        if (row_live) {
-            st.xv[0] = x_base[s * 8];
-            st.xv[1] = x_base[s * 8 + 1];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            st.w[b][0] = nt_load(w_base[b] + s * 8);
+            st.w[b][1] = nt_load(w_base[b] + s * 8 + 1);
         }
+#pragma unroll
+        for (int r = 0; r < MB; ++r)
+            if (row_live[r]) {
+                st.xv[r][0] = x_base[r][s * 8];
+                st.xv[r][1] = x_base[r][s * 8 + 1];
+            }
     };
-    v4i d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};  // two accumulators taking turns
+    v4i d[NB][MB][2] = {};  // two accumulators per output block taking turns
     auto compute = [&](const Step& st) {
-        d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, st.w[0]), __builtin_bit_cast(v4i, st.xv[0]), d0, 0, 0, 0);
-        d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, st.w[1]), __builtin_bit_cast(v4i, st.xv[1]), d1, 0, 0, 0);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int r = 0; r < MB; ++r)
+                    d[b][r][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, st.w[b][h]), __builtin_bit_cast(v4i, st.xv[r][h]),
+                                                                      d[b][r][h], 0, 0, 0);
     };
 
-    // this wavefront's steps: wave, wave + WAVES, ...; four in flight (a step is 64 bytes per lane)
-    constexpr int kRing = 4;
+    // this wavefront's steps: wave, wave + WAVES, ...; RING in flight (a step is 32 (NB + MB) bytes per lane)
+    constexpr int kRing = NB + MB >= 4 ? 2 : 4;
     Step ring[kRing] = {};
 #pragma unroll
     for (int r = 0; r < kRing; ++r)
@@ -65,17 +87,25 @@ __global__ __launch_bounds__(WAVES * kWave) void int8_decode_kernel(const int8_t
     }
 
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][v][lane] = d0[v] + d1[v];
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < MB; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][b * MB + r][v][lane] = d[b][r][0][v] + d[b][r][1][v];
     __syncthreads();
-    if (wave == 0 && row_live) {  // lane (m, q): channels n0 + 4 q + v
+    if (wave == 0) {  // lane (m, q): rows 16 r + m, channels n0 + 16 b + 4 q + v
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            int sum = 0;
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][v][lane];
-            const int n = n0 + 4 * q + v;
-            if (n < N) ep.store(static_cast<int64_t>(i) * N + n, i, n, sum);
-        }
+            for (int r = 0; r < MB; ++r)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    int sum = 0;
+#pragma unroll
+                    for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b * MB + r][v][lane];
+                    const int n = n0 + 16 * b + 4 * q + v, m = 16 * r + i;
+                    if (row_live[r] && n < N) ep.store(static_cast<int64_t>(m) * N + n, m, n, sum);
+                }
     }
 }
 
@@ -83,18 +113,34 @@ inline bool int8_decode_ok(const void* a, const void* w, int64_t M, int64_t N, i
     return M >= 1 && K >= 128 && K % 128 == 0 && aligned(a, 16) && aligned(w, 16) && N <= 0x7FFFFFF0 && K <= 0x7FFFFF80;
 }
 
-// slabs of 16 rows; the epilogue sees row indices of the whole problem through `rebase`
+// slabs of 32 rows (16 for what is left); the epilogue sees row indices of the whole problem through `rebase`
 template <class Epilogue, class Rebase>
 int launch_int8_decode(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, Rebase rebase, hipStream_t s) {
+    static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT8_DECODE_NB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_mb = [] { const char* e = std::getenv("TPQ_INT8_DECODE_MB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT8_DECODE_WAVES"); return e ? std::atoi(e) : 0; }();
     const int steps = static_cast<int>(K / 128);
-    for (int64_t m0 = 0; m0 < M; m0 += 16) {
-        const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
-        const dim3 grid(static_cast<unsigned>((N + 15) / 16));
+    const int n = static_cast<int>(N), k = static_cast<int>(K);
+    for (int64_t m0 = 0; m0 < M;) {
+        const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
+        const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
+        const int rows = left < 16 * mb ? left : 16 * mb;
+        // Workgroup shape from a sweep over model shapes (K, N = 1024..28672): 32 channels pay from 8 rows on where
+        // N gives a whole number of rounds of workgroups (8192 x 8192, 32 rows: 22.4 us against 26.3; 28672 -> 8192:
+        // 69 against 86), never for one row or narrow N (4096 x 4096, 16 rows: 9.3 us against 6.9).
+        const bool wide = rows >= 8 && ((N >= 6144 && N < 10240) || N >= 16384);
+        const int nb = forced_nb ? forced_nb : (wide ? 2 : 1);
+        const int waves = forced_waves ? forced_waves : (nb == 2 ? 8 : mb == 2 ? 4 : steps >= 32 ? 8 : 4);
+        const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
         const Epilogue slab = rebase(ep, m0);
-        if (steps >= 32)
-            int8_decode_kernel<8, Epilogue><<<grid, 8 * kWave, 0, s>>>(a + m0 * K, w, rows, static_cast<int>(N), static_cast<int>(K), slab);
-        else
-            int8_decode_kernel<4, Epilogue><<<grid, 4 * kWave, 0, s>>>(a + m0 * K, w, rows, static_cast<int>(N), static_cast<int>(K), slab);
+        const int8_t* xs = a + m0 * K;
+#define TPQ_I8DEC(NBV, MBV, WV) int8_decode_kernel<NBV, MBV, WV, Epilogue><<<grid, WV * kWave, 0, s>>>(xs, w, rows, n, k, slab)
+        if (nb == 2 && mb == 2) { if (waves == 8) TPQ_I8DEC(2, 2, 8); else TPQ_I8DEC(2, 2, 4); }
+        else if (nb == 2) { if (waves == 8) TPQ_I8DEC(2, 1, 8); else TPQ_I8DEC(2, 1, 4); }
+        else if (mb == 2) { if (waves == 8) TPQ_I8DEC(1, 2, 8); else TPQ_I8DEC(1, 2, 4); }
+        else { if (waves == 8) TPQ_I8DEC(1, 1, 8); else TPQ_I8DEC(1, 1, 4); }
+#undef TPQ_I8DEC
+        m0 += rows;
     }
     return check_launch("int8 decode gemm");
 }

@@ -26,9 +26,12 @@ EpilogueDequant<DT> rebase_rows(const EpilogueDequant<DT>& ep, int64_t m0, int64
 template <class Epilogue>
 int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
     const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
-    // a few rows: stream the weight once per 16 rows through the decode kernel.  K = N = 4096: 16 rows 7.3 us,
-    // 32 rows 13.2 us, 48 rows 20.0 us, against 21.3 / 22.7 / 22.7 us for the tiled kernels
-    static const int decode_rows = [] { const char* e = std::getenv("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : 48; }();
+    // a few rows: stream the weight once per 32 rows through the decode kernel.  K = N = 4096: 16 rows 6.9 us,
+    // 32 rows 9.1 us, 64 rows 17.8 us, against 27.5 us for the tiled kernels below at any of these row counts
+    // (28672 -> 8192: 61 / 69 / 138 us against 182 us; 4096 -> 11008: 15 / 21 / 41 us against 31 / 31 / 32 us)
+    // Wide N gives the tiled kernel enough tiles earlier (8192 -> 28672: 99 us at 65 rows against 133 at 48).
+    static const int forced_decode_rows = [] { const char* e = std::getenv("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
+    const int decode_rows = forced_decode_rows >= 0 ? forced_decode_rows : (N >= 10240 ? 32 : 64);
     if (M <= decode_rows && int8_decode_ok(a, w, M, N, K) && !(force && force[0] == 'r'))
         return launch_int8_decode(a, w, M, N, K, ep, [N](const Epilogue& e, int64_t m0) { return rebase_rows(e, m0, N); }, s);
     // The ring-buffered kernel also wins when its 256 x 128 tiles fill only part of the chip: at K = N = 4096,
