@@ -1,4 +1,4 @@
-// Ternary-weight product for a few activation rows (1..16 per launch: decode batches of the BitNet
+// Ternary-weight product for a few activation rows (1..16 MB per launch: decode batches of the BitNet
 // linear), K % 256 == 0.  The packed weight is streamed once whatever the row count:
 // v_mfma_i32_16x16x64_i8 with the WEIGHTS as the A operand, NB blocks of 16 channels per workgroup.
 // Lane (i, q) owns weight row n0 + i and, in a step of 256 k, the 16 packed bytes (64 codes) at
@@ -15,6 +15,8 @@
 // workgroup take the steps round-robin and add their partial sums through LDS.  Columns m >= M stay
 // zero and load nothing.
 #pragma once
+
+#include <cstdlib>
 
 #include "int8_gemm_kernel.h"
 
@@ -43,16 +45,15 @@ __device__ __forceinline__ v4i ternary_fields_to_i8(uint32_t w) {
     return out;
 }
 
-template <int NB, int WAVES, class Epilogue>
+template <int NB, int MB, int WAVES, class Epilogue>
 __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(const int8_t* __restrict__ x, const uint8_t* __restrict__ packed,
                                                                            int m_base, int M, int N, int K, Epilogue ep) {
-    __shared__ int red[WAVES][NB][4][kWave];
+    __shared__ int red[WAVES][NB * MB][4][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int steps = K / 256;
     const int n0 = blockIdx.x * (16 * NB);
-    const bool row_live = i < M;
     const size_t bpr = static_cast<size_t>(K) >> 2;
     const uint4* w_base[NB];
 #pragma unroll
@@ -60,35 +61,47 @@ __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(cons
         const int n = n0 + 16 * b + i;
         w_base[b] = reinterpret_cast<const uint4*>(packed + static_cast<size_t>(n < N ? n : N - 1) * bpr) + q;  // rows past N: a valid row, result dropped
     }
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m_base + (row_live ? i : 0)) * K) + q * 4;
+    bool row_live[MB];
+    const uint4* x_base[MB];
+#pragma unroll
+    for (int r = 0; r < MB; ++r) {
+        row_live[r] = 16 * r + i < M;
+        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m_base + (row_live[r] ? 16 * r + i : 0)) * K) + q * 4;
+    }
 
     struct Step {
         uint4 w[NB];
-        uint4 xv[4];
+        uint4 xv[MB][4];
     };
     auto load = [&](int s, Step& st) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) st.w[b] = nt_load(w_base[b] + s * 4);
-        if (row_live) {
 #pragma unroll
-            for (int d = 0; d < 4; ++d) st.xv[d] = x_base[s * 16 + d];
-        }
+        for (int r = 0; r < MB; ++r)
+            if (row_live[r]) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) st.xv[r][d] = x_base[r][s * 16 + d];
+            }
     };
-    v4i acc[NB][2] = {};  // two accumulators per block taking turns
+    v4i acc[NB][MB][2] = {};  // two accumulators per output block taking turns
     auto compute = [&](const Step& st) {
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            const v4i xb = transpose_4x4_bytes(st.xv[d]);
+            v4i xb[MB];
+#pragma unroll
+            for (int r = 0; r < MB; ++r) xb[r] = transpose_4x4_bytes(st.xv[r][d]);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const uint32_t word = d == 0 ? st.w[b].x : d == 1 ? st.w[b].y : d == 2 ? st.w[b].z : st.w[b].w;
-                acc[b][d & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ternary_fields_to_i8(word), xb, acc[b][d & 1], 0, 0, 0);
+                const v4i codes = ternary_fields_to_i8(word);
+#pragma unroll
+                for (int r = 0; r < MB; ++r) acc[b][r][d & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(codes, xb[r], acc[b][r][d & 1], 0, 0, 0);
             }
         }
     };
 
-    // this wavefront's steps: wave, wave + WAVES, ...; four in flight (a step is 16 NB + 64 bytes per lane)
-    constexpr int kRing = 4;
+    // this wavefront's steps: wave, wave + WAVES, ...; RING in flight (a step is 16 NB + 64 MB bytes per lane)
+    constexpr int kRing = MB >= 2 ? 2 : 4;
     Step ring[kRing] = {};
 #pragma unroll
     for (int r = 0; r < kRing; ++r)
@@ -107,19 +120,23 @@ __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(cons
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = acc[b][0][v] + acc[b][1][v];
+        for (int r = 0; r < MB; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][b * MB + r][v][lane] = acc[b][r][0][v] + acc[b][r][1][v];
     __syncthreads();
-    if (wave == 0 && row_live) {  // lane (m, q): channels n0 + 16 b + 4 q + v
+    if (wave == 0) {  // lane (m, q): rows 16 r + m, channels n0 + 16 b + 4 q + v
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                int sum = 0;
+            for (int r = 0; r < MB; ++r)
 #pragma unroll
-                for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b][v][lane];
-                const int n = n0 + 16 * b + 4 * q + v;
-                if (n < N) ep.store(static_cast<int64_t>(m_base + i) * N + n, m_base + i, n, sum);
-            }
+                for (int v = 0; v < 4; ++v) {
+                    int sum = 0;
+#pragma unroll
+                    for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b * MB + r][v][lane];
+                    const int n = n0 + 16 * b + 4 * q + v, m = m_base + 16 * r + i;
+                    if (row_live[r] && n < N) ep.store(static_cast<int64_t>(m) * N + n, m, n, sum);
+                }
     }
 }
 
@@ -128,10 +145,11 @@ inline bool ternary_decode_mfma_ok(const void* x, const void* packed, int64_t M,
            K <= 0x7FFFFF00;
 }
 
-// slabs of 16 rows
+// slabs of 32 rows (16 for what is left)
 template <class Epilogue>
 int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
     static const int forced_nb = [] { const char* e = std::getenv("TPQ_TERNARY_NB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_mb = [] { const char* e = std::getenv("TPQ_TERNARY_MB"); return e ? std::atoi(e) : 0; }();
     static const int forced_waves = [] { const char* e = std::getenv("TPQ_TERNARY_WAVES"); return e ? std::atoi(e) : 0; }();
     // Workgroup shape from a sweep over model shapes (K 2560..28672, 1..16 rows), about 2000..4000 wavefronts in all:
     //   N < 8192: 16 channels x 8 wavefronts (4096 x 4096, 8 rows: 5.0 us; 32 channels: 6.6)
@@ -141,13 +159,19 @@ int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M
     const int nb = forced_nb ? forced_nb : ((N >= 8192 && N < 10240) || N >= 16384 ? 2 : 1);
     const int waves = forced_waves ? forced_waves : (N < 10240 ? 8 : 4);
     const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
-    for (int64_t m0 = 0; m0 < M; m0 += 16) {
-        const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
-        const int mb = static_cast<int>(m0), n = static_cast<int>(N), k = static_cast<int>(K);
-        if (nb == 2 && waves == 8) ternary_decode_mfma_kernel<2, 8, Epilogue><<<grid, 8 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
-        else if (nb == 2) ternary_decode_mfma_kernel<2, 4, Epilogue><<<grid, 4 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
-        else if (waves == 8) ternary_decode_mfma_kernel<1, 8, Epilogue><<<grid, 8 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
-        else ternary_decode_mfma_kernel<1, 4, Epilogue><<<grid, 4 * kWave, 0, s>>>(x, packed, mb, rows, n, k, ep);
+    const int n = static_cast<int>(N), k = static_cast<int>(K);
+    for (int64_t m0 = 0; m0 < M;) {
+        const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
+        const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
+        const int rows = left < 16 * mb ? left : 16 * mb;
+        const int base = static_cast<int>(m0);
+#define TPQ_TDEC(NBV, MBV, WV) ternary_decode_mfma_kernel<NBV, MBV, WV, Epilogue><<<grid, WV * kWave, 0, s>>>(x, packed, base, rows, n, k, ep)
+        if (nb == 2 && mb == 2) { if (waves == 8) TPQ_TDEC(2, 2, 8); else TPQ_TDEC(2, 2, 4); }
+        else if (nb == 2) { if (waves == 8) TPQ_TDEC(2, 1, 8); else TPQ_TDEC(2, 1, 4); }
+        else if (mb == 2) { if (waves == 8) TPQ_TDEC(1, 2, 8); else TPQ_TDEC(1, 2, 4); }
+        else { if (waves == 8) TPQ_TDEC(1, 1, 8); else TPQ_TDEC(1, 1, 4); }
+#undef TPQ_TDEC
+        m0 += rows;
     }
     return check_launch("tpq_ternary_mm (mfma decode)");
 }
