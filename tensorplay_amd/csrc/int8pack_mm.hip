@@ -4,7 +4,8 @@
 //
 // Decode kernel (fp16 / bf16 activations, K % 128 == 0, 1..16 rows per launch), bandwidth bound at one byte
 // per weight: v_mfma_f32_16x16x32_f16 with the weights as A and the activations as B, as in the int4
-// decode kernel for several rows.  Lane (i, q) owns weight row n0 + i and, in a step of 128 k, the 32
+// decode kernel for several rows (NB blocks of 16 channels and 4 or 8 wavefronts per workgroup, chosen by N).
+// Lane (i, q) owns weight row n0 + i and, in a step of 128 k, the 32
 // bytes at k = 128 s + 32 q: two 16-byte loads, whole 128-byte lines per row and step.  Every dword
 // (four int8) becomes two fp16 pairs: xor 0x80808080 turns the bytes into b + 128, v_perm_b32 drops
 // each next to the exponent byte 0x64 (fp16 1024 + 128 + b), and one packed fp16 subtract of 1152
@@ -15,12 +16,13 @@
 // Everything else (bf16 / fp32 activations, other K) takes the vector kernel below (wavefront = four channels,
 // eight k per lane and turn, fp32 fma), and K % 8 != 0 or unaligned pointers a plain one: one workgroup per
 // output channel and slab of up to 8 rows, block reduction.
+#include <cstdlib>
+
 #include "int4_lane.h"
 
 namespace tpq {
 namespace {
 
-constexpr int kI8Waves = 2;
 constexpr int kI8Ring = 2;  // steps in flight per wavefront
 
 typedef uint32_t word4_t __attribute__((ext_vector_type(4)));
@@ -30,21 +32,25 @@ __device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r =
 
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 
-// x: [M][K] fp16 or bf16; w: [N][K] int8; scale: [N] fp32; steps = K / 128
-template <int DT>
-__global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
+// x: [M][K] fp16 or bf16; w: [N][K] int8; scale: [N] fp32; steps = K / 128; NB blocks of 16 channels per workgroup
+template <int DT, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
     const uint16_t* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
     uint16_t* __restrict__ y, int M, int N, int K) {
-    __shared__ float red[kI8Waves][4][kWave];
+    __shared__ float red[WAVES][NB][4][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int steps = K / 128;
-    const int n0 = blockIdx.x * 16;
-    const int n_row = n0 + i < N ? n0 + i : N - 1;  // rows past N: a valid row, result dropped
-    const uint4* w_base = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n_row) * K) + q * 2;
-    // columns m >= M repeat the last row: their products are computed and never stored
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(i < M ? i : M - 1) * K) + q * 4;
+    const int n0 = blockIdx.x * (16 * NB);
+    const uint4* w_base[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int n = n0 + 16 * b + i;
+        w_base[b] = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n < N ? n : N - 1) * K) + q * 2;  // rows past N: a valid row, result dropped
+    }
+    const bool row_live = i < M;  // columns m >= M stay zero and load nothing
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 4;
 
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     const h2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
@@ -52,82 +58,89 @@ __global__ __launch_bounds__(kI8Waves * kWave) void int8pack_mfma_kernel(
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(0x64646464u));
 
     struct Step {
-        uint4 w[2];
+        uint4 w[NB][2];
         uint4 xv[4];
     };
     auto load = [&](int s, Step& st) {
-        st.w[0] = nt_load(w_base + s * 8);
-        st.w[1] = nt_load(w_base + s * 8 + 1);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
+        for (int b = 0; b < NB; ++b) {
+            st.w[b][0] = nt_load(w_base[b] + s * 8);
+            st.w[b][1] = nt_load(w_base[b] + s * 8 + 1);
+        }
+        if (row_live) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
+        }
     };
-    float4_t d0 = {0.0f, 0.0f, 0.0f, 0.0f}, d1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    float4_t d[NB][2] = {};  // two accumulators per block taking turns
     auto compute = [&](const Step& st) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {  // MFMA u (16x16x32): k = 8u .. 8u+7 of the lane's 32
-            uint32_t a[4];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t word = dword_at(st.w[u >> 1], (2 * u + h) & 3);
-                if constexpr (DT == TPQ_DTYPE_F16) {
-                    const uint32_t t = word ^ 0x80808080u;
-                    const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
-                    const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
-                    a[2 * h] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
-                    a[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
-                } else {
-                    // bf16 is the upper half of a float and an int8 has eight significant bits: convert each
-                    // byte (sign-extending byte select) and keep the upper halves, exact
-                    uint32_t f[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) f[e] = __builtin_bit_cast(uint32_t, static_cast<float>(static_cast<int8_t>(word >> (8 * e))));
-                    a[2 * h] = __builtin_amdgcn_perm(f[1], f[0], 0x07060302u);      // (bf16 b0, bf16 b1)
-                    a[2 * h + 1] = __builtin_amdgcn_perm(f[3], f[2], 0x07060302u);  // (bf16 b2, bf16 b3)
-                }
-            }
-            const word4_t av = {a[0], a[1], a[2], a[3]};
             const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
-            float4_t& d = (u & 1) ? d1 : d0;
-            if constexpr (DT == TPQ_DTYPE_F16)
-                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
-            else
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), d, 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                uint32_t a[4];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const uint32_t word = dword_at(st.w[b][u >> 1], (2 * u + h) & 3);
+                    if constexpr (DT == TPQ_DTYPE_F16) {
+                        const uint32_t t = word ^ 0x80808080u;
+                        const uint32_t lo = __builtin_amdgcn_perm(magic, t, 0x04010400u);  // (1152 + b0, 1152 + b1)
+                        const uint32_t hi = __builtin_amdgcn_perm(magic, t, 0x04030402u);  // (1152 + b2, 1152 + b3)
+                        a[2 * h] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, lo) - bias);
+                        a[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, hi) - bias);
+                    } else {
+                        // bf16 is the upper half of a float and an int8 has eight significant bits: convert each
+                        // byte (sign-extending byte select) and keep the upper halves, exact
+                        uint32_t f[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) f[e] = __builtin_bit_cast(uint32_t, static_cast<float>(static_cast<int8_t>(word >> (8 * e))));
+                        a[2 * h] = __builtin_amdgcn_perm(f[1], f[0], 0x07060302u);      // (bf16 b0, bf16 b1)
+                        a[2 * h + 1] = __builtin_amdgcn_perm(f[3], f[2], 0x07060302u);  // (bf16 b2, bf16 b3)
+                    }
+                }
+                const word4_t av = {a[0], a[1], a[2], a[3]};
+                float4_t& acc = d[b][u & 1];
+                if constexpr (DT == TPQ_DTYPE_F16)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), acc, 0, 0, 0);
+                else
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), acc, 0, 0, 0);
+            }
         }
     };
 
     // this wavefront's steps: wave, wave + W, ...; kI8Ring of them in flight
-    Step ring[kI8Ring];
+    Step ring[kI8Ring] = {};
 #pragma unroll
     for (int r = 0; r < kI8Ring; ++r)
-        if (wave + r * kI8Waves < steps) load(wave + r * kI8Waves, ring[r]);
-    for (int base = wave; base < steps; base += kI8Ring * kI8Waves) {
+        if (wave + r * WAVES < steps) load(wave + r * WAVES, ring[r]);
+    for (int base = wave; base < steps; base += kI8Ring * WAVES) {
 #pragma unroll
         for (int r = 0; r < kI8Ring; ++r) {
-            const int s = base + r * kI8Waves;
+            const int s = base + r * WAVES;
             if (s < steps) {
                 compute(ring[r]);
-                if (s + kI8Ring * kI8Waves < steps) load(s + kI8Ring * kI8Waves, ring[r]);
+                if (s + kI8Ring * WAVES < steps) load(s + kI8Ring * WAVES, ring[r]);
             }
         }
     }
 
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][v][lane] = d0[v] + d1[v];
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = d[b][0][v] + d[b][1][v];
     __syncthreads();
-    if (wave == 0) {  // lane (m, q): channels n0 + 4 q + v
-        const int n = n0 + 4 * q;
-        float sum[4];
+    if (wave == 0 && row_live) {  // lane (m, q): channels n0 + 16 b + 4 q + v
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            sum[v] = 0.0f;
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int ww = 0; ww < kI8Waves; ++ww) sum[v] += red[ww][v][lane];
-        }
-        if (i < M) {
+            for (int v = 0; v < 4; ++v) {
+                float sum = 0.0f;
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = Elem<DT>::store(__fmul_rn(sum[v], scale[n + v]));
-        }
+                for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b][v][lane];
+                const int n = n0 + 16 * b + 4 * q + v;
+                if (n < N) y[static_cast<size_t>(i) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
+            }
     }
 }
 
@@ -288,15 +301,26 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
     TPQ_REQUIRE(x && w && scales && out, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype != TPQ_DTYPE_F32 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
+        static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT8PACK_NB"); return e ? std::atoi(e) : 0; }();
+        static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_WAVES"); return e ? std::atoi(e) : 0; }();
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
-            const dim3 grid(static_cast<unsigned>((N + 15) / 16));
+            // Workgroup shape from a sweep over model shapes (K, N = 1024..28672; 1, 8, 16 rows): 16 channels x 8
+            // wavefronts (4096 x 4096, one row: 6.4 us; 2 wavefronts 9.5); 32 channels where N gives whole rounds of
+            // workgroups and from 8 rows on at N >= 16384 (28672 -> 8192, 16 rows: 72 us against 88).
+            const bool wide = (N >= 8192 && N < 10240) || (N >= 16384 && rows >= 8);
+            const int nb = forced_nb ? forced_nb : (wide ? 2 : 1);
+            const int waves = forced_waves ? forced_waves : (N >= 16384 && !wide ? 4 : 8);
+            const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
             const auto* xs = static_cast<const uint16_t*>(x) + m0 * K;
             auto* ys = static_cast<uint16_t*>(out) + m0 * N;
-            if (dtype == TPQ_DTYPE_F16)
-                int8pack_mfma_kernel<TPQ_DTYPE_F16><<<grid, kI8Waves * kWave, 0, s>>>(xs, w, scales, ys, rows, static_cast<int>(N), static_cast<int>(K));
-            else
-                int8pack_mfma_kernel<TPQ_DTYPE_BF16><<<grid, kI8Waves * kWave, 0, s>>>(xs, w, scales, ys, rows, static_cast<int>(N), static_cast<int>(K));
+            const int n = static_cast<int>(N), k = static_cast<int>(K);
+#define TPQ_I8P(DTV, NBV, WV) int8pack_mfma_kernel<DTV, NBV, WV><<<grid, WV * kWave, 0, s>>>(xs, w, scales, ys, rows, n, k)
+#define TPQ_I8P_DT(NBV, WV) do { if (dtype == TPQ_DTYPE_F16) TPQ_I8P(TPQ_DTYPE_F16, NBV, WV); else TPQ_I8P(TPQ_DTYPE_BF16, NBV, WV); } while (0)
+            if (nb == 2) { if (waves == 8) TPQ_I8P_DT(2, 8); else if (waves == 4) TPQ_I8P_DT(2, 4); else TPQ_I8P_DT(2, 2); }
+            else { if (waves == 8) TPQ_I8P_DT(1, 8); else if (waves == 4) TPQ_I8P_DT(1, 4); else TPQ_I8P_DT(1, 2); }
+#undef TPQ_I8P_DT
+#undef TPQ_I8P
         }
         return check_launch("_weight_int8pack_mm (mfma)");
     }
