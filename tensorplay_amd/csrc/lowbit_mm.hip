@@ -82,8 +82,8 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     n4 = n4 + 4 <= N ? n4 : N - 4;
     const float* sz_base = sz + static_cast<size_t>(n4) * 2;
     const bool row_live = i < M;
-    // columns m >= M repeat the last row: their products are computed and never stored
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : M - 1) * K + q * F::kCodes);
+    // columns m >= M stay zero and load nothing
+    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K + q * F::kCodes);
 
     // constant A of the offset MFMA: row 0 = the offsets of the eight k of an MFMA (pairs 0..3 of the
     // lane's codes: the pattern repeats every byte, so every MFMA has the same), row 1 = ones
@@ -110,8 +110,10 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
         const uint4* prm = reinterpret_cast<const uint4*>(sz_base + static_cast<size_t>(s >> group_shift) * N * 2);
         st.p[0] = prm[0];
         st.p[1] = prm[1];
+        if (row_live) {
 #pragma unroll
-        for (int c = 0; c < F::kCodes / 8; ++c) st.xv[c] = x_base[static_cast<size_t>(s) * (F::kStepK / 8) + c];
+            for (int c = 0; c < F::kCodes / 8; ++c) st.xv[c] = x_base[static_cast<size_t>(s) * (F::kStepK / 8) + c];
+        }
     };
 
     float yacc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     };
 
     // this wavefront's steps: wave, wave + WAVES, ...; two in flight
-    Step s0, s1;
+    Step s0 = {}, s1 = {};
     int s = wave;
     if (s < steps) load(s, s0);
     if (s + WAVES < steps) load(s + WAVES, s1);
