@@ -74,17 +74,18 @@ __device__ __forceinline__ uint16_t swiglu_of(float gate_sum, float up_sum) {
 // sz_b: up) and the output is silu_mul(gate, up).  residual (plain mode, may be null): [M][N], added to
 // the rounded output.
 // GKT = k-tiles (of 32) per quantization group: 4 stands for groups of 128 k and more (above).  Groups of 32
-// or 64 k (GKT = 1, 2; fp16 only) differ between the four lanes an MFMA adds up, so there the weights are
-// dequantized in registers before the product, with the packed fp16 operations and roundings of the reference's
-// own dense weight, T(code - 8) * scale + zero (int4_tc_dequantize_kernel, QuantGemmKernels.cu:1170-1202):
-// three packed operations per pair, no offset MFMA, no per-step epilogue.
+// or 64 k (GKT = 1, 2) differ between the four lanes an MFMA adds up, so there the weights are dequantized in
+// registers before the product, no offset MFMA, no per-step epilogue.  fp16: the packed fp16 operations and
+// roundings of the reference's own dense weight, T(code - 8) * scale + zero (int4_tc_dequantize_kernel,
+// QuantGemmKernels.cu:1170-1202), three packed operations per pair.  bf16 (no packed bf16 arithmetic): one fp32
+// fma per code and one rounding to bf16, five operations per pair.
 template <int DT, int NB, int WAVES, bool PAIR = false, int GKT = 4>
 __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
     uint16_t* __restrict__ y, int M, int N, int K, int group_shift, const uint4* __restrict__ packed_b,
     const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual) {
     static_assert(!PAIR || NB == 2, "a pair is two blocks");
-    static_assert(GKT == 4 || (DT == TPQ_DTYPE_F16 && !PAIR), "in-register dequantization is built for fp16");
+    static_assert(GKT == 4 || !PAIR, "in-register dequantization is not built for the pair");
     constexpr bool DEQ = GKT < 4;
     using L = Lane16<DT>;
     using ML = MfmaLane<DT>;
@@ -157,7 +158,27 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int r = 0; r < 4; ++r) L::template unpack<true>(dword_of(st.w[b], r), v[b][r], magic_even, magic_odd);
-        if constexpr (DEQ) {
+        if constexpr (DEQ && DT == TPQ_DTYPE_BF16) {
+            // a pair is (128 + code) twice in bf16: widen both halves (a shift, a mask), one fp32 fma each with
+            // zero - 136 scale folded into the addend, and one v_cvt_pk_bf16_f32 back: round-to-nearest-even once
+            typedef float f2_t __attribute__((ext_vector_type(2)));
+            typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint32_t pw = st.p[b].x;  // (scale, zero) of the lane's row and k-tile
+                const float sc = L::lo(pw), zc = __builtin_fmaf(-136.0f, sc, L::hi(pw));
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t pv = v[b][r][j];
+                        const f2_t f = {__builtin_fmaf(__builtin_bit_cast(float, pv << 16), sc, zc),
+                                        __builtin_fmaf(__builtin_bit_cast(float, pv & 0xFFFF0000u), sc, zc)};
+                        v[b][r][j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf2_t));
+                    }
+            }
+        }
+        if constexpr (DEQ && DT == TPQ_DTYPE_F16) {
             const half2_t off_even = {static_cast<_Float16>(1032.0f), static_cast<_Float16>(1032.0f)};  // magic + 8
             const half2_t off_odd = {static_cast<_Float16>(72.0f), static_cast<_Float16>(72.0f)};
 #pragma unroll

@@ -393,7 +393,7 @@ bool launch_stream(const void* x, const int32_t* packed, const void* sz, void* y
 template <int DT>
 bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void* sz, void* y, int N, int K,
                       int group, hipStream_t s, int* rc, const void* residual = nullptr) {
-    const bool deq = (group == 32 || group == 64) && DT == TPQ_DTYPE_F16 && residual == nullptr;  // dequantized in registers
+    const bool deq = (group == 32 || group == 64) && residual == nullptr;  // dequantized in registers
     if ((group != 128 && group != 256 && !deq) || !aligned(sz, 16) || !aligned(y, 8)) return false;
     if (residual != nullptr && !aligned(residual, 8)) return false;
     const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
@@ -418,7 +418,7 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     const auto* sp = static_cast<const uint32_t*>(sz);
     auto* yp = static_cast<uint16_t*>(y);
     const int shift = group == 128 ? 0 : 1;  // a group is 128 << shift k (128 or 256)
-    if constexpr (DT == TPQ_DTYPE_F16) {
+    {
         if (deq) {
 #define TPQ_MFMA_DEQ(NBV, WV, GKTV)                                                                                       \
     int4_mfma_kernel<DT, NBV, WV, false, GKTV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \

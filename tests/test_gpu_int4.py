@@ -70,8 +70,9 @@ CASES = [  # M, N, K, group
     (16, 72, 256, 128), (9, 136, 1024, 128), (17, 64, 256, 128), (33, 40, 384, 128), (8, 200, 2048, 128),
     # row-block kernel: 17..64 rows per launch, partial last block, 64 + 64 + 2 rows
     (24, 136, 512, 128), (64, 72, 1024, 128), (50, 200, 256, 128), (130, 64, 384, 128), (81, 40, 1152, 128),
-    # groups of 32 / 64 with several rows: dequantized in registers (fp16), narrow and wide N
+    # groups of 32 / 64: dequantized in registers (fp16, bf16), every shape of workgroup (by N and rows), one row too
     (4, 8200, 256, 32), (12, 8192, 384, 64), (2, 48, 640, 32), (16, 24, 128, 64),
+    (9, 6152, 256, 32), (16, 10248, 128, 64), (1, 4104, 256, 32), (3, 10240, 256, 32), (1, 10240, 128, 64),
 ]
 
 
