@@ -88,6 +88,20 @@ int tpq_int8_mm_dequant(const int8_t* a, const int8_t* w, const float* row_scale
                         int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
+ * The same operation with a caller-provided workspace (16-byte aligned).  With few output tiles and a long K
+ * (a few hundred rows against a square weight) the k range is cut into slices, one workgroup each, whose exact
+ * integer partial sums go to the workspace; a second kernel adds them and applies the scales.  The result is
+ * bit-identical to tpq_int8_mm_dequant (same reference lines).  tpq_int8_mm_workspace_bytes says how many
+ * bytes the shape can use (0: the workspace would not be used); a NULL or smaller workspace falls back to
+ * tpq_int8_mm_dequant.
+ */
+int64_t tpq_int8_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const float* row_scale,
+                           const float* col_scale, const float* bias, void* out, int out_dtype,
+                           int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                           void* stream);
+
+/*
  * int32 codes [N,K] in 0..15 -> int32 [ceil(N/8)][ceil(K/(16 I))][32][I/2],
  * the packed layout of the reference's device op (I = inner_k_tiles in {2,4,8}).
  * Replaces _convert_weight_to_int4pack: config/native_functions.yaml:7991,

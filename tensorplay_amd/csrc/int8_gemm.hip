@@ -2,6 +2,7 @@
 // int8 GEMM + dequant; the matrix-core kernel itself lives in
 // int8_gemm_kernel.h, shared with the ternary matmul.
 #include <cstdlib>
+#include <type_traits>
 
 #include "int8_decode_kernel.h"
 #include "int8_gemm_dma.h"
@@ -23,6 +24,57 @@ EpilogueDequant<DT> rebase_rows(const EpilogueDequant<DT>& ep, int64_t m0, int64
     return EpilogueDequant<DT>{ep.out + m0 * N, ep.rs + m0, ep.cs, ep.bias};
 }
 
+// Up to this many rows the decode kernel streams the weight once per 32 rows.
+inline int int8_decode_rows(int64_t N) {
+    static const int forced = [] { const char* e = std::getenv("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
+    return forced >= 0 ? forced : (N >= 10240 ? 32 : 64);
+}
+
+// Slices of the k range the tiled kernel would be cut into for this shape (1: not cut); see dma_slices.
+// With a workspace at hand the decode kernel keeps only what it does in one pass (32 rows): two passes cost more
+// than the sliced kernel (K = N = 8192, 48 rows: 41 us against 28).
+inline int int8_slices(const void* a, const void* w, int64_t M, int64_t N, int64_t K) {
+    const char* force = std::getenv("TPQ_INT8_KERNEL");
+    if (K <= 0 || !mfma_path_ok(a, w, M, N, K) || (force && force[0] == 'r')) return 1;
+    const int decode_rows = int8_decode_rows(N) < 32 ? int8_decode_rows(N) : 32;
+    if (M <= decode_rows && int8_decode_ok(a, w, M, N, K)) return 1;
+    return dma_slices(M, N, K);
+}
+
+// partial [slices][M][N] int32 -> out: acc = sum of the slices (exact), then (float(acc) * rs[m]) * cs[n] (+ bias[n]),
+// the arithmetic of the fused epilogues
+template <int DT>
+__global__ __launch_bounds__(256) void int8_finish_kernel(const int32_t* __restrict__ partial, int slices, const float* __restrict__ rs,
+                                                          const float* __restrict__ cs, const float* __restrict__ bias,
+                                                          typename Elem<DT>::storage* __restrict__ out, int64_t M, int64_t N) {
+    const int64_t total = M * N, stride = static_cast<int64_t>(gridDim.x) * 256;
+    const bool has_bias = bias != nullptr;
+    if (N % 4 == 0) {  // four consecutive columns of one row per thread
+        for (int64_t q = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; q < total / 4; q += stride) {
+            const int64_t idx = q * 4, m = idx / N, n = idx - m * N;
+            int4 v = make_int4(0, 0, 0, 0);
+            for (int z = 0; z < slices; ++z) {
+                const uint4 p = nt_load(reinterpret_cast<const uint4*>(partial + z * total + idx));
+                v.x += static_cast<int>(p.x); v.y += static_cast<int>(p.y); v.z += static_cast<int>(p.z); v.w += static_cast<int>(p.w);
+            }
+            const float4 c = *reinterpret_cast<const float4*>(cs + n);
+            const float4 b = has_bias ? *reinterpret_cast<const float4*>(bias + n) : make_float4(0, 0, 0, 0);
+            const float r = rs[m];
+            out[idx] = TileDequant<DT>::convert(v.x, r, c.x, b.x, has_bias);
+            out[idx + 1] = TileDequant<DT>::convert(v.y, r, c.y, b.y, has_bias);
+            out[idx + 2] = TileDequant<DT>::convert(v.z, r, c.z, b.z, has_bias);
+            out[idx + 3] = TileDequant<DT>::convert(v.w, r, c.w, b.w, has_bias);
+        }
+        return;
+    }
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += stride) {
+        const int64_t m = idx / N, n = idx - m * N;
+        int acc = 0;
+        for (int z = 0; z < slices; ++z) acc += partial[z * total + idx];
+        out[idx] = TileDequant<DT>::convert(acc, rs[m], cs[n], has_bias ? bias[n] : 0.0f, has_bias);
+    }
+}
+
 template <class Epilogue>
 int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
     const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
@@ -30,13 +82,12 @@ int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t 
     // 32 rows 9.1 us, 64 rows 17.8 us, against 27.5 us for the tiled kernels below at any of these row counts
     // (28672 -> 8192: 61 / 69 / 138 us against 182 us; 4096 -> 11008: 15 / 21 / 41 us against 31 / 31 / 32 us)
     // Wide N gives the tiled kernel enough tiles earlier (8192 -> 28672: 99 us at 65 rows against 133 at 48).
-    static const int forced_decode_rows = [] { const char* e = std::getenv("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
-    const int decode_rows = forced_decode_rows >= 0 ? forced_decode_rows : (N >= 10240 ? 32 : 64);
+    const int decode_rows = int8_decode_rows(N);
     if (M <= decode_rows && int8_decode_ok(a, w, M, N, K) && !(force && force[0] == 'r'))
         return launch_int8_decode(a, w, M, N, K, ep, [N](const Epilogue& e, int64_t m0) { return rebase_rows(e, m0, N); }, s);
     // The ring-buffered kernel also wins when its 256 x 128 tiles fill only part of the chip: at K = N = 4096,
     // M = 512 / 1024 it takes 27.9 / 29.5 us against 33.9 / 39.4 us for the register-staged kernel on 128 x 64 tiles.
-    if (dma_path_ok(M, K) && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
+    if (dma_path_ok(M, N, K) && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
     return launch_mfma(a, w, M, N, K, ep, s);
 }
 
@@ -129,4 +180,35 @@ TPQ_EXPORT int tpq_int8_mm_dequant(const int8_t* a, const int8_t* w, const float
         default: TPQ_DISPATCH(TPQ_DTYPE_BF16)
     }
 #undef TPQ_DISPATCH
+}
+
+TPQ_EXPORT int64_t tpq_int8_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    // operand alignment is checked again at the call; a 16-byte aligned pair stands in for it here
+    const int slices = int8_slices(reinterpret_cast<const void*>(16), reinterpret_cast<const void*>(16), M, N, K);
+    return slices >= 2 ? slices * M * N * 4 : 0;
+}
+
+TPQ_EXPORT int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const float* row_scale, const float* col_scale,
+                                      const float* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                      void* workspace, int64_t workspace_bytes, void* stream) {
+    const int slices = (M > 0 && N > 0 && K > 0 && a && w) ? int8_slices(a, w, M, N, K) : 1;
+    if (slices < 2 || workspace == nullptr || workspace_bytes < slices * M * N * 4 || !aligned(workspace, 16) || (M * N) % 4 != 0 ||
+        !aligned(col_scale, 16) || !aligned(bias, 16))
+        return tpq_int8_mm_dequant(a, w, row_scale, col_scale, bias, out, out_dtype, M, N, K, stream);
+    TPQ_REQUIRE(out_dtype == TPQ_DTYPE_F32 || out_dtype == TPQ_DTYPE_F16 || out_dtype == TPQ_DTYPE_BF16,
+                TPQ_ERR_INVALID_TYPE, "int8_mm_dequant: unsupported output dtype");
+    TPQ_REQUIRE(out && row_scale && col_scale, TPQ_ERR_INVALID_VALUE, "int8_mm_dequant: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int32_t* acc = static_cast<int32_t*>(workspace);  // [slices][M][N]; M N % 4 == 0 keeps every matrix 16-byte aligned
+    if (int rc = launch_dma_sliced(a, w, M, N, K, acc, slices, s)) return rc;
+    const int64_t items = N % 4 == 0 ? M * N / 4 : M * N;
+    const int64_t blocks = (items + 255) / 256;
+    const unsigned grid = static_cast<unsigned>(blocks > 4096 ? 4096 : blocks);
+    switch (out_dtype) {
+        case TPQ_DTYPE_F32: int8_finish_kernel<TPQ_DTYPE_F32><<<grid, 256, 0, s>>>(acc, slices, row_scale, col_scale, bias, static_cast<float*>(out), M, N); break;
+        case TPQ_DTYPE_F16: int8_finish_kernel<TPQ_DTYPE_F16><<<grid, 256, 0, s>>>(acc, slices, row_scale, col_scale, bias, static_cast<uint16_t*>(out), M, N); break;
+        default: int8_finish_kernel<TPQ_DTYPE_BF16><<<grid, 256, 0, s>>>(acc, slices, row_scale, col_scale, bias, static_cast<uint16_t*>(out), M, N); break;
+    }
+    return check_launch("int8_mm_dequant (finish)");
 }

@@ -120,7 +120,7 @@ constexpr int kDmaStages = 3;
 template <class Tile, int KSPLIT>
 __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
                                                             const int8_t* __restrict__ W, int M, int N,
-                                                            int K, Tile tile, int vector_stores) {
+                                                            int K, Tile tile, int vector_stores, int slices) {
     using out_t = typename Tile::out_t;
     constexpr int BM = 256, BN = 128, WM = 128, WN = 64, TM = 4, TN = 2;
     constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;    // 48 KB
@@ -158,7 +158,11 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         }
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int nk = K / kDmaRowBytes;
+    // blockIdx.y = slice of the k range (whole stages, every slice at least one: the launcher sees to it);
+    // slice z writes its sums to the z-th [M][N] matrix of the destination
+    const int nk_all = K / kDmaRowBytes, nk_slice = (nk_all + slices - 1) / slices;
+    const int kt0 = blockIdx.y * nk_slice;
+    const int nk = nk_all - kt0 < nk_slice ? nk_all - kt0 : nk_slice;
 
     if (Tile::kScaled && tid < BN) {  // column scales and bias of this tile: read once, used in the epilogue
         const int n = n0 + tid < N ? n0 + tid : N - 1;
@@ -176,11 +180,11 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         if (row < BM) {
             int gr = m0 + row;
             gr = gr < M ? gr : M - 1;
-            src[i] = A + static_cast<size_t>(gr) * K + chunk * 16;
+            src[i] = A + static_cast<size_t>(gr) * K + chunk * 16 + static_cast<size_t>(kt0) * kDmaRowBytes;
         } else {
             int gr = n0 + row - BM;
             gr = gr < N ? gr : N - 1;
-            src[i] = W + static_cast<size_t>(gr) * K + chunk * 16;
+            src[i] = W + static_cast<size_t>(gr) * K + chunk * 16 + static_cast<size_t>(kt0) * kDmaRowBytes;
         }
     }
     // loads FIRST, FIRST+1 of this wavefront's six
@@ -499,7 +503,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         const int m = m0 + row, n = n0 + col;
         if (m >= M || n >= N) continue;
         const char* srcp = lds_bytes + row * kPitch + col * sizeof(out_t);
-        out_t* dstp = tile.out + static_cast<size_t>(m) * N + n;
+        out_t* dstp = tile.out + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
         if (vector_stores && n + kPerChunk <= N) {
             nt_store(reinterpret_cast<uint4*>(dstp), *reinterpret_cast<const uint4*>(srcp));  // written once, read by a later kernel
         } else {
@@ -509,10 +513,11 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
 }
 
 // K must be a multiple of the 128-byte stage.
-inline bool dma_path_ok(int64_t M, int64_t K) { return M > 128 && K % kDmaRowBytes == 0; }
+// Up to 128 rows the 256-row tiles are half empty: worth it only where N alone yields tiles for the whole chip.
+inline bool dma_path_ok(int64_t M, int64_t N, int64_t K) { return (M > 128 || (M > 32 && N >= 16384)) && K % kDmaRowBytes == 0; }
 
 template <int KSPLIT, class Tile>
-int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
     constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + 2 * 128 * sizeof(float);
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
@@ -520,17 +525,40 @@ int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int
     static std::atomic<uint64_t> configured{0};  // per instantiation
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int8 gemm")) return rc;
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
-    kernel<<<dim3(static_cast<unsigned>(tiles)), 256 * KSPLIT, smem, s>>>(a, w, static_cast<int>(M), static_cast<int>(N),
-                                                                 static_cast<int>(K), tile, vector_stores);
+    kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), 256 * KSPLIT, smem, s>>>(
+        a, w, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), tile, vector_stores, slices);
     return check_launch("int8 mfma gemm (dma)");
 }
 
 // TPQ_INT8_KSPLIT=1 selects the four-wavefront variant for comparison runs.
 template <class Tile>
-int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s) {
+int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
     const char* env = std::getenv("TPQ_INT8_KSPLIT");
-    if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s);
-    return launch_dma_split<2>(a, w, M, N, K, tile, s);
+    if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s, slices);
+    return launch_dma_split<2>(a, w, M, N, K, tile, s, slices);
+}
+
+// Few output tiles and a long k range (a few hundred rows against a square weight): each tile's k range is cut
+// into slices of whole stages, one workgroup per slice, each writing its exact partial sums to a matrix of its
+// own; a second kernel adds them.  How many slices: enough workgroups for the chip, at least four stages each
+// and none empty; 1 = not worth it.
+inline int dma_slices(int64_t M, int64_t N, int64_t K) {
+    static const int forced = [] { const char* e = std::getenv("TPQ_INT8_SLICES"); return e ? std::atoi(e) : 0; }();
+    if (M < 1 || K % kDmaRowBytes != 0) return 1;
+    const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128), nk = K / kDmaRowBytes;
+    static const int min_stages = [] { const char* e = std::getenv("TPQ_INT8_SLICE_STAGES"); return e ? std::atoi(e) : 4; }();
+    static const int target = [] { const char* e = std::getenv("TPQ_INT8_SLICE_TARGET"); return e ? std::atoi(e) : 256; }();
+    int64_t slices = forced ? forced : target / tiles;
+    if (slices > nk / min_stages) slices = nk / min_stages;
+    if (slices < 2) return 1;
+    const int64_t per = (nk + slices - 1) / slices;
+    return static_cast<int>((nk + per - 1) / per);  // drop slices that would start past the end
+}
+
+// partial [slices][M][N] int32 (16-byte aligned) := the slices of A W^T
+inline int launch_dma_sliced(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, int32_t* partial, int slices, hipStream_t s) {
+    const TileInt32 tile{partial, nullptr, nullptr, nullptr};
+    return launch_dma(a, w, M, N, K, tile, s, slices);
 }
 
 }  // namespace

@@ -169,9 +169,18 @@ def int8_mm_dequant(A_i8: torch.Tensor, B_t_i8: torch.Tensor, row_scale: torch.T
     b = None if bias is None else bias.contiguous().to(torch.float32)
     if b is not None and b.numel() != N:
         raise ValueError("int8_mm_dequant: bias must have one value per output channel")
+    lib = _lib.load()
     with torch.cuda.device(a.device):
-        _check(_lib.load().tpq_int8_mm_dequant(_ptr(a), _ptr(w), _ptr(rs), _ptr(cs), _ptr(b), _ptr(out),
-                                               _DT[out_dtype], M, N, K, _stream(a)))
+        # a few hundred rows against a long K: the library cuts the k range into slices that meet in an int32
+        # scratch matrix (same bits as the single launch); it says for which shapes that pays
+        scratch_bytes = int(lib.tpq_int8_mm_workspace_bytes(M, N, K))
+        if scratch_bytes:
+            scratch = torch.empty(scratch_bytes // 4, dtype=torch.int32, device=a.device)
+            _check(lib.tpq_int8_mm_dequant_ws(_ptr(a), _ptr(w), _ptr(rs), _ptr(cs), _ptr(b), _ptr(out), _DT[out_dtype],
+                                              M, N, K, _ptr(scratch), scratch_bytes, _stream(a)))
+        else:
+            _check(lib.tpq_int8_mm_dequant(_ptr(a), _ptr(w), _ptr(rs), _ptr(cs), _ptr(b), _ptr(out),
+                                           _DT[out_dtype], M, N, K, _stream(a)))
     return out
 
 

@@ -25,7 +25,9 @@ SHAPES = [(5, 7, 3), (1, 1, 1), (64, 12, 32), (16, 1024, 1024), (64, 128, 32), (
           (129, 64, 65), (256, 4096, 128), (300, 208, 200), (128, 2560, 6912 // 8), (513, 80, 257),
           # decode kernel: 1..64 rows in slabs of 32 / 16, K a multiple of 128, ragged N, both widths of workgroup
           (1, 128, 40), (17, 256, 24), (48, 384, 72), (33, 4096, 100), (7, 11008, 64),
-          (64, 256, 6150), (49, 128, 8200), (8, 384, 16400), (31, 256, 6144), (16, 128, 9000), (64, 512, 17)]
+          (64, 256, 6150), (49, 128, 8200), (8, 384, 16400), (31, 256, 6144), (16, 128, 9000), (64, 512, 17),
+          # tiled kernel with the k range in slices (few tiles, long K), ragged last slice
+          (130, 1024, 200), (300, 2048, 136), (65, 1152, 64), (257, 1280, 100), (33, 1024, 10248)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -84,7 +86,8 @@ def test_rescale_bit_exact(ops):
 
 
 @pytest.mark.parametrize("out_dtype", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("shape", [(16, 1024, 1024), (300, 208, 200), (5, 7, 3), (256, 512, 384), (40, 256, 36), (1, 4096, 64), (50, 256, 6160), (9, 128, 16390)])
+@pytest.mark.parametrize("shape", [(16, 1024, 1024), (300, 208, 200), (5, 7, 3), (256, 512, 384), (40, 256, 36), (1, 4096, 64), (50, 256, 6160), (9, 128, 16390),
+                                   (130, 1024, 200), (300, 2048, 136), (65, 1152, 66), (257, 1280, 100)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_fused_dequant_bit_exact(ops, out_dtype, shape, with_bias):
     from gpu_util import TORCH_DT
