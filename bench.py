@@ -444,6 +444,28 @@ def main() -> int:
         fused_chk = ((acc_chk.float() * a_s[:64, None]) * w_s[None, :]).bfloat16()
         extras["int8_gemm_rows_checked_equal"] = bool(torch.equal(fused_chk, out8[:64]))
 
+        # the same product for decode batches and short prompts (16 / 128 rows): the decode kernel, and the tiled
+        # kernel with its k range in slices (workspace entry point), weights rotating through 30 copies (0.5 GB)
+        w_rot = [w_q.clone() for _ in range(30)]
+        for m_small in (16, 128):
+            a_small, s_small = a_q[:m_small].contiguous(), a_s[:m_small].contiguous()
+            out_small = torch.empty((m_small, N8), dtype=torch.bfloat16, device=dev)
+            ws_bytes = int(lib.tpq_int8_mm_workspace_bytes(m_small, N8, K8))
+            scratch = torch.empty(max(ws_bytes, 16) // 4, dtype=torch.int32, device=dev)
+
+            def gemm_small(i, a_small=a_small, s_small=s_small, out_small=out_small, m_small=m_small, scratch=scratch, ws_bytes=ws_bytes):
+                lib.tpq_int8_mm_dequant_ws(a_small.data_ptr(), w_rot[i % 30].data_ptr(), s_small.data_ptr(), w_s.data_ptr(), None,
+                                           out_small.data_ptr(), _lib.BF16, m_small, N8, K8, scratch.data_ptr(), ws_bytes, cur())
+
+            gemm_small(0); sync()
+            gs8 = graph_of(lambda: [gemm_small(i) for i in range(120)])
+            gs8.replay(); sync()
+            ms = time_region(gs8.replay, sync, 1) / 120
+            extras[f"int8_gemm_{m_small}x4096x4096_us"] = ms * 1e3
+            extras[f"int8_gemm_{m_small}x4096x4096_weight_GBs"] = N8 * K8 / (ms * 1e-3) / 1e9
+            extras[f"int8_gemm_{m_small}_rows_equal_big_gemm"] = bool(torch.equal(out_small, out8[:m_small]))
+        del w_rot
+
         # activation quantizer on the same activations: 2*M*K + M*K + 4*M bytes
         cq = torch.empty((M8, K8), dtype=torch.int8, device=dev)
         sq = torch.empty((M8,), dtype=torch.float32, device=dev)
@@ -500,7 +522,7 @@ def main() -> int:
             extras[key + "_GBs"] = (4.5 * 4096 * 4096 + 8 * gs.numel()) / (ms * 1e-3) / 1e9
 
         # BitNet ternary: M in {1,128}, 2560 -> 6912 and 6912 -> 2560 (weights cache resident at this size)
-        for (mt, kt, nt) in ((1, 2560, 6912), (1, 6912, 2560), (128, 2560, 6912), (128, 6912, 2560)):
+        for (mt, kt, nt) in ((1, 2560, 6912), (1, 6912, 2560), (8, 2560, 6912), (8, 6912, 2560), (128, 2560, 6912), (128, 6912, 2560)):
             tern = rng.choice(np.int8([-1, 0, 1]), size=(nt, kt), p=[0.325, 0.35, 0.325])
             pk = ops.pack_ternary(torch.from_numpy(tern).to(dev))
             xt = torch.from_numpy(rng.normal(0, 1, (mt, kt)).astype(np.float32)).to(dev)
@@ -516,7 +538,7 @@ def main() -> int:
             ms = time_region(gt.replay, sync, 1) / 200
             key = f"ternary_M{mt}_{kt}x{nt}"
             extras[key + "_us"] = ms * 1e3
-            if mt == 1:
+            if mt <= 8:
                 extras[key + "_GBs_cache_resident"] = (nt * kt // 4 + mt * kt + 4 * mt + 2 * mt * nt) / (ms * 1e-3) / 1e9
             else:
                 extras[key + "_TOPS"] = 2.0 * mt * nt * kt / (ms * 1e-3) / 1e12
