@@ -1,4 +1,4 @@
-// int4 decode kernel for 1..16 activation rows on the matrix cores (fp16 / bf16,
+// int4 decode kernel for 1..16 (MB = 2: ..32) activation rows on the matrix cores (fp16 / bf16,
 // group a multiple of 128, K % 128 == 0): every packed byte is read once for
 // all rows, and the multiply-accumulate work leaves the vector ALU.
 //
@@ -79,17 +79,19 @@ __device__ __forceinline__ uint16_t swiglu_of(float gate_sum, float up_sum) {
 // roundings of the reference's own dense weight, T(code - 8) * scale + zero (int4_tc_dequantize_kernel,
 // QuantGemmKernels.cu:1170-1202), three packed operations per pair.  bf16 (no packed bf16 arithmetic): one fp32
 // fma per code and one rounding to bf16, five operations per pair.
-template <int DT, int NB, int WAVES, bool PAIR = false, int GKT = 4>
+// MB = blocks of 16 activation rows per launch (1 or 2): the unpacked weights of a step feed MB column blocks.
+template <int DT, int NB, int WAVES, bool PAIR = false, int GKT = 4, int MB = 1>
 __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
     uint16_t* __restrict__ y, int M, int N, int K, int group_shift, const uint4* __restrict__ packed_b,
     const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual) {
     static_assert(!PAIR || NB == 2, "a pair is two blocks");
     static_assert(GKT == 4 || !PAIR, "in-register dequantization is not built for the pair");
+    static_assert(MB == 1 || !PAIR, "the pair takes 16 rows");
     constexpr bool DEQ = GKT < 4;
     using L = Lane16<DT>;
     using ML = MfmaLane<DT>;
-    __shared__ float red[WAVES][NB][4][kWave];
+    __shared__ float red[WAVES][NB * MB][4][kWave];
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -111,8 +113,13 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         sz_base[b] = (PAIR && b == 1 ? sz_b : sz) + n4;
         if constexpr (DEQ) sz_base[b] = sz + ((nb0 + i) < N ? nb0 + i : N - 1);  // (scale, zero) of this lane's weight row
     }
-    const bool row_live = i < M;
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 4;
+    bool row_live[MB];
+    const uint4* x_base[MB];
+#pragma unroll
+    for (int r = 0; r < MB; ++r) {
+        row_live[r] = 16 * r + i < M;
+        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live[r] ? 16 * r + i : 0) * K) + q * 4;
+    }
 
     // constant A of the correction MFMA: row 0 = offset + 8 of the pair parity, row 1 = ones
     uint32_t a_corr_even = 0, a_corr_odd = 0;
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     struct Step {
         uint4 w[NB];
         uint4 p[NB];
-        uint4 xv[4];
+        uint4 xv[MB][4];
     };
     auto load = [&](int s, Step& st) {
 #pragma unroll
@@ -134,25 +141,33 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
             if constexpr (DEQ) st.p[b].x = sz_base[b][static_cast<size_t>((4 * s + q) / GKT) * N];  // group of k-tile 4 s + q
             else st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
         }
-        if (row_live) {  // columns m >= M keep the zeros they start with: no load, nothing stored
 #pragma unroll
-            for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
-        }
+        for (int r = 0; r < MB; ++r)
+            if (row_live[r]) {  // columns m >= M keep the zeros they start with: no load, nothing stored
+#pragma unroll
+                for (int c = 0; c < 4; ++c) st.xv[r][c] = x_base[r][s * 16 + c];
+            }
     };
 
-    float yacc[NB][4];
+    float yacc[NB][MB][4];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) yacc[b][v] = 0.0f;
+        for (int r = 0; r < MB; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) yacc[b][r][v] = 0.0f;
 
     auto compute = [&](const Step& st) {
         // the correction product and the weight products alternate, so that no MFMA waits for
         // the one issued just before it
-        float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f};
-        float4_t d[NB];
+        float4_t aux[MB];
+        float4_t d[NB][MB];
 #pragma unroll
-        for (int b = 0; b < NB; ++b) d[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int r = 0; r < MB; ++r) {
+            aux[r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int b = 0; b < NB; ++b) d[b][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
         uint32_t v[NB][4][4];  // [block][word r][pair j] = codes at k = 2 r + 8 j, + 1 of the lane's k-tile
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -200,30 +215,41 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const uint32_t off = (u & 1) ? a_corr_odd : a_corr_even;
-            const word4_t xb = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
+            word4_t xb[MB];
+#pragma unroll
+            for (int r = 0; r < MB; ++r) xb[r] = word4_t{st.xv[r][u].x, st.xv[r][u].y, st.xv[r][u].z, st.xv[r][u].w};
             const word4_t ac = {off, off, off, off};
-            if constexpr (!DEQ) aux = ML::mfma(ac, xb, aux);
+            if constexpr (!DEQ) {
+#pragma unroll
+                for (int r = 0; r < MB; ++r) aux[r] = ML::mfma(ac, xb[r], aux[r]);
+            }
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const word4_t aw = {v[b][0][u], v[b][1][u], v[b][2][u], v[b][3][u]};
-                d[b] = ML::mfma(aw, xb, d[b]);
+#pragma unroll
+                for (int r = 0; r < MB; ++r) d[b][r] = ML::mfma(aw, xb[r], d[b][r]);
             }
         }
         if constexpr (DEQ) {
 #pragma unroll
             for (int b = 0; b < NB; ++b)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) yacc[b][v] += d[b][v];
+                for (int r = 0; r < MB; ++r)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) yacc[b][r][v] += d[b][r][v];
             return;
         }
-        // rows 0 and 1 of the correction product sit in lanes 0..15, registers 0 and 1
-        const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
 #pragma unroll
-        for (int b = 0; b < NB; ++b) {
+        for (int r = 0; r < MB; ++r) {
+            // rows 0 and 1 of the correction product sit in lanes 0..15, registers 0 and 1
+            const float corr = __shfl(aux[r][0], i, kWave), sx = __shfl(aux[r][1], i, kWave);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint32_t pw = dword_of(st.p[b], v);  // (scale, zero) of channel n0 + 16 b + 4 q + v
-                yacc[b][v] = __builtin_fmaf(L::lo(pw), d[b][v] - corr, __builtin_fmaf(L::hi(pw), sx, yacc[b][v]));
+            for (int b = 0; b < NB; ++b) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const uint32_t pw = dword_of(st.p[b], v);  // (scale, zero) of channel n0 + 16 b + 4 q + v
+                    yacc[b][r][v] = __builtin_fmaf(L::lo(pw), d[b][r][v] - corr, __builtin_fmaf(L::hi(pw), sx, yacc[b][r][v]));
+                }
             }
         }
     };
@@ -249,7 +275,9 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = yacc[b][v];
+        for (int r = 0; r < MB; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][b * MB + r][v][lane] = yacc[b][r][v];
     __syncthreads();
     if constexpr (PAIR) {
         if (wave == 0) {  // lane (m, q): channels n0 + 4 q + v of both weights
@@ -263,7 +291,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
                     for (int w = 0; w < WAVES; ++w) sum[b][v] += red[w][b][v][lane];
                 }
             const int n = n0 + 4 * q;
-            if (row_live && n < N) {
+            if (row_live[0] && n < N) {
                 const uint32_t lo = swiglu_of<DT>(sum[0][0], sum[1][0]) | (static_cast<uint32_t>(swiglu_of<DT>(sum[0][1], sum[1][1])) << 16);
                 const uint32_t hi = swiglu_of<DT>(sum[0][2], sum[1][2]) | (static_cast<uint32_t>(swiglu_of<DT>(sum[0][3], sum[1][3])) << 16);
                 *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
@@ -271,28 +299,31 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
         }
         return;
     }
-    // wavefront w finishes block b = w, w + W, ...: lane (m, q) stores channels n0 + 16 b + 4 q + v
-    for (int b = wave; b < NB; b += WAVES) {
+    // wavefront w finishes output block w, w + W, ... (block = channel block b x row block r): lane (m, q) stores
+    // row 16 r + m, channels n0 + 16 b + 4 q + v
+    for (int blk = wave; blk < NB * MB; blk += WAVES) {
+        const int b = blk / MB, r = blk % MB;
         float sum[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             sum[v] = 0.0f;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) sum[v] += red[w][b][v][lane];
+            for (int w = 0; w < WAVES; ++w) sum[v] += red[w][blk][v][lane];
         }
         const int n = n0 + 16 * b + 4 * q;
-        if (row_live && n < N) {  // N % 8 == 0 and n % 4 == 0: all four channels exist
+        const int row = 16 * r + i;
+        if (row < M && n < N) {  // N % 8 == 0 and n % 4 == 0: all four channels exist
             uint16_t o[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[v] = L::out(sum[v]);
             if (residual != nullptr) {  // the rounded output plus the residual, rounded again: what a separate add does
-                const uint2 r = *reinterpret_cast<const uint2*>(residual + static_cast<size_t>(i) * N + n);
-                const uint16_t rv[4] = {static_cast<uint16_t>(r.x), static_cast<uint16_t>(r.x >> 16), static_cast<uint16_t>(r.y),
-                                        static_cast<uint16_t>(r.y >> 16)};
+                const uint2 rw = *reinterpret_cast<const uint2*>(residual + static_cast<size_t>(row) * N + n);
+                const uint16_t rv[4] = {static_cast<uint16_t>(rw.x), static_cast<uint16_t>(rw.x >> 16), static_cast<uint16_t>(rw.y),
+                                        static_cast<uint16_t>(rw.y >> 16)};
 #pragma unroll
                 for (int v = 0; v < 4; ++v) o[v] = L::out(Elem<DT>::load(o[v]) + Elem<DT>::load(rv[v]));
             }
-            *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) =
+            *reinterpret_cast<uint2*>(y + static_cast<size_t>(row) * N + n) =
                 make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
         }
     }

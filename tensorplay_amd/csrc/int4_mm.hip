@@ -436,6 +436,16 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
             return true;
         }
     }
+    if (rows > 16) {  // 17..32 rows: two row blocks per workgroup share the unpacked weights
+        if (deq) return false;
+#define TPQ_MFMA2(NBV, WV) \
+    int4_mfma_kernel<DT, NBV, WV, false, 4, 2><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \
+        xp, pp, sp, yp, rows, N, K, shift, nullptr, nullptr, static_cast<const uint16_t*>(residual))
+        if (nb == 1) TPQ_MFMA2(1, 8); else if (nb == 2 && waves == 8) TPQ_MFMA2(2, 8); else if (nb == 2) TPQ_MFMA2(2, 4); else TPQ_MFMA2(4, 4);
+#undef TPQ_MFMA2
+        *rc = check_launch("tpq_int4_mm (mfma, 32 rows)");
+        return true;
+    }
 #define TPQ_MFMA(NBV, WV) \
     int4_mfma_kernel<DT, NBV, WV><<<dim3((N + 16 * NBV - 1) / (16 * NBV)), dim3(WV * kWave), 0, s>>>( \
         xp, pp, sp, yp, rows, N, K, shift, nullptr, nullptr, static_cast<const uint16_t*>(residual))
@@ -486,15 +496,18 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
 template <int DT>
 int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* sz, void* y, int N,
                   int K, int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
-    {   // slabs of 16 rows on the matrix cores where the shape allows
+    {   // slabs of 32 rows (16 with groups of 32 / 64) on the matrix cores where the shape allows
+        static const int slab_rows = [] { const char* e = std::getenv("TPQ_INT4_SLAB_ROWS"); return e ? std::atoi(e) : 32; }();
         const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;
+        const int slab = (group == 32 || group == 64) ? 16 : slab_rows;
         int64_t m0 = 0;
-        for (; m0 < M; m0 += 16) {
-            const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        while (m0 < M) {
+            const int rows = static_cast<int>(M - m0 < slab ? M - m0 : slab);
             int rc;
             if (!launch_mfma_rows<DT>(static_cast<const char*>(x) + m0 * row_x, rows, packed, sz,
                                       static_cast<char*>(y) + m0 * row_y, N, K, group, s, &rc)) break;
             if (rc != TPQ_OK) return rc;
+            m0 += rows;
         }
         if (m0 >= M) return TPQ_OK;
         x = static_cast<const char*>(x) + m0 * row_x;  // what is left (a single last row, or everything) takes the paths below

@@ -220,10 +220,12 @@ def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.T
     return out
 
 
-# Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM.  Measured at
-# K = 4096, N = 11008, fp16: the 16-row slabs cost about 10 us each (41 us at 64 rows), the dense route
-# 72 us at 65 rows and 75 us at 128, so the two meet near 112 rows.
-INT4_PREFILL_ROWS = 112
+# Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM.  Measured (fp16): at
+# K = 4096, N = 11008 the 32-row slabs cost about 13.5 us each (54 us at 128 rows, 79 us at 192), the dense route
+# 74 us at 128 rows and 81 us at 192; at K = N = 4096: 41.5 / 61 us against 44 / 50 us.  So the two meet near 128
+# rows for N below 8192 and near 176 rows above.
+INT4_PREFILL_ROWS = 128
+INT4_PREFILL_ROWS_WIDE = 176
 
 
 def _int4_dequantize(packed: torch.Tensor, inner: int, n: int, k: int, group: int, sz: torch.Tensor) -> torch.Tensor:
@@ -265,10 +267,10 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     x = self.contiguous()
     w = mat2.contiguous()
     sz = qScaleAndZeros.to(self.dtype).contiguous()
-    if m > INT4_PREFILL_ROWS and inner == 2:
+    if m > (INT4_PREFILL_ROWS_WIDE if n >= 8192 else INT4_PREFILL_ROWS) and inner == 2:
         # Many rows: what the reference does for every shape (QuantGemmKernels.cu:1296-1341) - dequantise
         # the weight to a dense matrix of the activation dtype, then one plain library GEMM.  The decode
-        # kernels read the packed weight once per 16 rows, which stops paying at this point.
+        # kernels read the packed weight once per 32 rows, which stops paying at this point.
         dense = _int4_dequantize(w, inner, n, k, qGroupSize, sz)
         torch.matmul(x, dense.t(), out=out)
         return out

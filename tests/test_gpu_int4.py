@@ -68,8 +68,9 @@ CASES = [  # M, N, K, group
     (2, 64, 4096, 128), (5, 24, 96, 32), (1, 16, 70, 32), (7, 136, 1024, 64),
     # matrix-core decode kernel: 5..16 rows (64-channel workgroups, partial last one), slabs of 16 plus a last row
     (16, 72, 256, 128), (9, 136, 1024, 128), (17, 64, 256, 128), (33, 40, 384, 128), (8, 200, 2048, 128),
-    # row-block kernel: 17..64 rows per launch, partial last block, 64 + 64 + 2 rows
+    # slabs of 32 rows (two row blocks per workgroup), partial last block, every width of workgroup
     (24, 136, 512, 128), (64, 72, 1024, 128), (50, 200, 256, 128), (130, 64, 384, 128), (81, 40, 1152, 128),
+    (32, 6152, 256, 128), (31, 10248, 128, 128), (19, 5128, 256, 128), (128, 8200, 128, 128),
     # groups of 32 / 64: dequantized in registers (fp16, bf16), every shape of workgroup (by N and rows), one row too
     (4, 8200, 256, 32), (12, 8192, 384, 64), (2, 48, 640, 32), (16, 24, 128, 64),
     (9, 6152, 256, 32), (16, 10248, 128, 64), (1, 4104, 256, 32), (3, 10240, 256, 32), (1, 10240, 128, 64),
