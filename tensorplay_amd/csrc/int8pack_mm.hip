@@ -32,12 +32,13 @@ __device__ __forceinline__ uint32_t dword_at(const uint4& q, int r) { return r =
 
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 
-// x: [M][K] fp16 or bf16; w: [N][K] int8; scale: [N] fp32; steps = K / 128; NB blocks of 16 channels per workgroup
-template <int DT, int NB, int WAVES>
+// x: [M][K] fp16 or bf16; w: [N][K] int8; scale: [N] fp32; steps = K / 128; NB blocks of 16 channels and MB blocks
+// of 16 activation rows per workgroup (the converted weights of a step feed every row block)
+template <int DT, int NB, int MB, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
     const uint16_t* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
     uint16_t* __restrict__ y, int M, int N, int K) {
-    __shared__ float red[WAVES][NB][4][kWave];
+    __shared__ float red[WAVES][NB * MB][4][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
@@ -49,8 +50,13 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
         const int n = n0 + 16 * b + i;
         w_base[b] = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n < N ? n : N - 1) * K) + q * 2;  // rows past N: a valid row, result dropped
     }
-    const bool row_live = i < M;  // columns m >= M stay zero and load nothing
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K) + q * 4;
+    bool row_live[MB];  // columns m >= M stay zero and load nothing
+    const uint4* x_base[MB];
+#pragma unroll
+    for (int r = 0; r < MB; ++r) {
+        row_live[r] = 16 * r + i < M;
+        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live[r] ? 16 * r + i : 0) * K) + q * 4;
+    }
 
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     const h2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
@@ -59,7 +65,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
 
     struct Step {
         uint4 w[NB][2];
-        uint4 xv[4];
+        uint4 xv[MB][4];
     };
     auto load = [&](int s, Step& st) {
 #pragma unroll
@@ -67,16 +73,20 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
             st.w[b][0] = nt_load(w_base[b] + s * 8);
             st.w[b][1] = nt_load(w_base[b] + s * 8 + 1);
         }
-        if (row_live) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) st.xv[c] = x_base[s * 16 + c];
-        }
+        for (int r = 0; r < MB; ++r)
+            if (row_live[r]) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) st.xv[r][c] = x_base[r][s * 16 + c];
+            }
     };
-    float4_t d[NB][2] = {};  // two accumulators per block taking turns
+    float4_t d[NB][MB][2] = {};  // two accumulators per output block taking turns
     auto compute = [&](const Step& st) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {  // MFMA u (16x16x32): k = 8u .. 8u+7 of the lane's 32
-            const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};
+            word4_t bv[MB];
+#pragma unroll
+            for (int r = 0; r < MB; ++r) bv[r] = word4_t{st.xv[r][u].x, st.xv[r][u].y, st.xv[r][u].z, st.xv[r][u].w};
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 uint32_t a[4];
@@ -100,11 +110,14 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
                     }
                 }
                 const word4_t av = {a[0], a[1], a[2], a[3]};
-                float4_t& acc = d[b][u & 1];
-                if constexpr (DT == TPQ_DTYPE_F16)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), acc, 0, 0, 0);
-                else
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), acc, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < MB; ++r) {
+                    float4_t& acc = d[b][r][u & 1];
+                    if constexpr (DT == TPQ_DTYPE_F16)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv[r]), acc, 0, 0, 0);
+                    else
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv[r]), acc, 0, 0, 0);
+                }
             }
         }
     };
@@ -128,19 +141,23 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[wave][b][v][lane] = d[b][0][v] + d[b][1][v];
+        for (int r = 0; r < MB; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][b * MB + r][v][lane] = d[b][r][0][v] + d[b][r][1][v];
     __syncthreads();
-    if (wave == 0 && row_live) {  // lane (m, q): channels n0 + 16 b + 4 q + v
+    if (wave == 0) {  // lane (m, q): rows 16 r + m, channels n0 + 16 b + 4 q + v
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                float sum = 0.0f;
+            for (int r = 0; r < MB; ++r)
 #pragma unroll
-                for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b][v][lane];
-                const int n = n0 + 16 * b + 4 * q + v;
-                if (n < N) y[static_cast<size_t>(i) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
-            }
+                for (int v = 0; v < 4; ++v) {
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b * MB + r][v][lane];
+                    const int n = n0 + 16 * b + 4 * q + v;
+                    if (row_live[r] && n < N) y[static_cast<size_t>(16 * r + i) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
+                }
     }
 }
 
@@ -303,8 +320,11 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
     if (dtype != TPQ_DTYPE_F32 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
         static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT8PACK_NB"); return e ? std::atoi(e) : 0; }();
         static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_WAVES"); return e ? std::atoi(e) : 0; }();
-        for (int64_t m0 = 0; m0 < M; m0 += 16) {
-            const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        static const int forced_mb = [] { const char* e = std::getenv("TPQ_INT8PACK_MB"); return e ? std::atoi(e) : 0; }();
+        for (int64_t m0 = 0; m0 < M;) {
+            const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
+            const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
+            const int rows = left < 16 * mb ? left : 16 * mb;
             // Workgroup shape from a sweep over model shapes (K, N = 1024..28672; 1, 8, 16 rows): 16 channels x 8
             // wavefronts (4096 x 4096, one row: 6.4 us; 2 wavefronts 9.5); 32 channels where N gives whole rounds of
             // workgroups and from 8 rows on at N >= 16384 (28672 -> 8192, 16 rows: 72 us against 88).
@@ -315,12 +335,16 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
             const auto* xs = static_cast<const uint16_t*>(x) + m0 * K;
             auto* ys = static_cast<uint16_t*>(out) + m0 * N;
             const int n = static_cast<int>(N), k = static_cast<int>(K);
-#define TPQ_I8P(DTV, NBV, WV) int8pack_mfma_kernel<DTV, NBV, WV><<<grid, WV * kWave, 0, s>>>(xs, w, scales, ys, rows, n, k)
-#define TPQ_I8P_DT(NBV, WV) do { if (dtype == TPQ_DTYPE_F16) TPQ_I8P(TPQ_DTYPE_F16, NBV, WV); else TPQ_I8P(TPQ_DTYPE_BF16, NBV, WV); } while (0)
-            if (nb == 2) { if (waves == 8) TPQ_I8P_DT(2, 8); else if (waves == 4) TPQ_I8P_DT(2, 4); else TPQ_I8P_DT(2, 2); }
-            else { if (waves == 8) TPQ_I8P_DT(1, 8); else if (waves == 4) TPQ_I8P_DT(1, 4); else TPQ_I8P_DT(1, 2); }
+#define TPQ_I8P(DTV, NBV, MBV, WV) int8pack_mfma_kernel<DTV, NBV, MBV, WV><<<grid, WV * kWave, 0, s>>>(xs, w, scales, ys, rows, n, k)
+#define TPQ_I8P_DT(NBV, MBV, WV) do { if (dtype == TPQ_DTYPE_F16) TPQ_I8P(TPQ_DTYPE_F16, NBV, MBV, WV); else TPQ_I8P(TPQ_DTYPE_BF16, NBV, MBV, WV); } while (0)
+            if (mb == 2) {
+                if (nb == 2) { if (waves == 4) TPQ_I8P_DT(2, 2, 4); else TPQ_I8P_DT(2, 2, 8); }
+                else { if (waves == 4) TPQ_I8P_DT(1, 2, 4); else TPQ_I8P_DT(1, 2, 8); }
+            } else if (nb == 2) { if (waves == 8) TPQ_I8P_DT(2, 1, 8); else if (waves == 4) TPQ_I8P_DT(2, 1, 4); else TPQ_I8P_DT(2, 1, 2); }
+            else { if (waves == 8) TPQ_I8P_DT(1, 1, 8); else if (waves == 4) TPQ_I8P_DT(1, 1, 4); else TPQ_I8P_DT(1, 1, 2); }
 #undef TPQ_I8P_DT
 #undef TPQ_I8P
+            m0 += rows;
         }
         return check_launch("_weight_int8pack_mm (mfma)");
     }

@@ -337,10 +337,11 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
     return (out, acc) if return_acc else out
 
 
-# Above this many activation rows _weight_int8pack_mm dequantises and calls the library GEMM.  Measured at
-# K = 4096, N = 11008, fp16 (eager): the 16-row slabs cost about 20 us each (62 us at 48 rows), the dense route
-# 53 us at 128 rows and 203 us at 2048.
-INT8PACK_PREFILL_ROWS = 40
+# Above this many activation rows _weight_int8pack_mm dequantises and calls the library GEMM.  Measured (fp16, us,
+# 32-row slabs against the dense route): K = 4096, N = 11008: 33 / 44 at 32 rows, 53 / 46 at 48; K = N = 4096: 26 / 33
+# at 64 rows, 39 / 41 at 96; K = N = 8192: 58 / 65 at 64 rows, 86 / 69 at 96.
+INT8PACK_PREFILL_ROWS = 64
+INT8PACK_PREFILL_ROWS_WIDE = 40  # N >= 10240
 
 
 def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
@@ -365,8 +366,8 @@ def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Te
     x, w = self.contiguous(), mat2.contiguous()
     sc = scales.to(torch.float32).contiguous()
     with torch.cuda.device(x.device):
-        if B > INT8PACK_PREFILL_ROWS:
-            # Many rows: the decode kernel streams the weight once per 16 rows, which stops paying here.  One pass
+        if B > (INT8PACK_PREFILL_ROWS_WIDE if N >= 10240 else INT8PACK_PREFILL_ROWS):
+            # Many rows: the decode kernel streams the weight once per 32 rows, which stops paying here.  One pass
             # writes the dense weight T(w * scale) and a library GEMM does the rest.
             dense = torch.empty((N, K), dtype=x.dtype, device=x.device)
             _check(_lib.load().tpq_int8pack_dequantize(_ptr(w), _ptr(sc), N, K, _DT[x.dtype], _ptr(dense), _stream(x)))

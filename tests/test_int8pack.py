@@ -30,7 +30,9 @@ def test_oracle_literal_and_closed_form():
     assert rel_err(oracle.to_f32(oracle.weight_int8pack_mm(x, "f32", w, s), "f32"), want) < 1e-5
 
 
-CASES = [(1, 4096, 512), (4, 1024, 136), (16, 256, 40), (17, 384, 72), (2, 100, 9), (8, 16, 3), (33, 128, 24), (1, 11008, 256)]
+CASES = [(1, 4096, 512), (4, 1024, 136), (16, 256, 40), (17, 384, 72), (2, 100, 9), (8, 16, 3), (33, 128, 24), (1, 11008, 256),
+         # every shape of workgroup of the decode kernel: 16 / 32 channels, 16 / 32 rows per pass, ragged N
+         (32, 256, 8200), (64, 128, 50), (9, 128, 16390), (3, 256, 16400), (24, 384, 10250), (40, 128, 10240)]
 
 
 @pytest.mark.gpu
