@@ -226,6 +226,9 @@ def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.T
 # rows for N below 8192 and near 176 rows above.
 INT4_PREFILL_ROWS = 128
 INT4_PREFILL_ROWS_WIDE = 176
+# float32 activations have no matrix-core decode kernel: the per-row kernel costs about 16 us a row at K = 4096,
+# N = 11008 (71 us at 4 rows, 253 us at 16), the dense float32 route 95 us at 16 rows and 134 us at 64.
+INT4_PREFILL_ROWS_F32 = 4
 
 
 def _int4_dequantize(packed: torch.Tensor, inner: int, n: int, k: int, group: int, sz: torch.Tensor) -> torch.Tensor:
@@ -267,7 +270,11 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     x = self.contiguous()
     w = mat2.contiguous()
     sz = qScaleAndZeros.to(self.dtype).contiguous()
-    if m > (INT4_PREFILL_ROWS_WIDE if n >= 8192 else INT4_PREFILL_ROWS) and inner == 2:
+    if self.dtype == torch.float32:
+        prefill_rows = INT4_PREFILL_ROWS_F32
+    else:
+        prefill_rows = INT4_PREFILL_ROWS_WIDE if n >= 8192 else INT4_PREFILL_ROWS
+    if m > prefill_rows and inner == 2:
         # Many rows: what the reference does for every shape (QuantGemmKernels.cu:1296-1341) - dequantise
         # the weight to a dense matrix of the activation dtype, then one plain library GEMM.  The decode
         # kernels read the packed weight once per 32 rows, which stops paying at this point.
