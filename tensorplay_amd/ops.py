@@ -349,6 +349,7 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
 # at 64 rows, 39 / 41 at 96; K = N = 8192: 58 / 65 at 64 rows, 86 / 69 at 96.
 INT8PACK_PREFILL_ROWS = 64
 INT8PACK_PREFILL_ROWS_WIDE = 40  # N >= 10240
+INT8PACK_PREFILL_ROWS_F32 = 24  # float32 activations (per-row kernel): 64 / 89 us at 16 rows, 119 / 94 us at 32
 
 
 def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
@@ -373,7 +374,7 @@ def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Te
     x, w = self.contiguous(), mat2.contiguous()
     sc = scales.to(torch.float32).contiguous()
     with torch.cuda.device(x.device):
-        if B > (INT8PACK_PREFILL_ROWS_WIDE if N >= 10240 else INT8PACK_PREFILL_ROWS):
+        if B > (INT8PACK_PREFILL_ROWS_F32 if x.dtype == torch.float32 else INT8PACK_PREFILL_ROWS_WIDE if N >= 10240 else INT8PACK_PREFILL_ROWS):
             # Many rows: the decode kernel streams the weight once per 32 rows, which stops paying here.  One pass
             # writes the dense weight T(w * scale) and a library GEMM does the rest.
             dense = torch.empty((N, K), dtype=x.dtype, device=x.device)
@@ -525,6 +526,7 @@ def dequantize_affine(input, block_size, scales: torch.Tensor, zero_points: Opti
 # ---- packed n-bit weight-only linear (int2 / intx / binary modules) ------------------------------
 
 LOWBIT_PREFILL_ROWS = 64  # above this many activation rows the weight is dequantised once for the library GEMM
+LOWBIT_PREFILL_ROWS_F32 = 40  # float32 activations (per-row kernel): 144 / 165 us at 32 rows, 278 / 192 us at 64 (K = 4096, N = 11008)
 
 
 def _lowbit_codes(t: torch.Tensor, what: str) -> torch.Tensor:
@@ -602,7 +604,7 @@ def _lowbit_mm(input: torch.Tensor, packed: torch.Tensor, bits: int, columns: in
     x = input.contiguous()
     m = x.shape[0]
     b = None if bias is None else bias.to(torch.float32).contiguous()
-    if m > LOWBIT_PREFILL_ROWS:
+    if m > (LOWBIT_PREFILL_ROWS_F32 if x.dtype == torch.float32 else LOWBIT_PREFILL_ROWS):
         dense = _lowbit_dequantize(w, bits, columns, sz, x.dtype, lsb_first)
         out = torch.matmul(x, dense.t())
         return out if b is None else out + b.to(out.dtype)
