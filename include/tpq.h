@@ -96,6 +96,10 @@ int tpq_int8_mm_dequant(const int8_t* a, const int8_t* w, const float* row_scale
  * tpq_int8_mm_dequant.
  */
 int64_t tpq_int8_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+/* tpq_int_mm (same reference lines: p10/src/backend/cuda/IntMM.cu:344-454) with the same optional workspace. */
+int tpq_int_mm_ws(const void* a, int a_unsigned, const int8_t* b, int64_t b_stride_k,
+                  int64_t b_stride_n, int32_t* c, int64_t M, int64_t K, int64_t N,
+                  void* workspace, int64_t workspace_bytes, void* stream);
 int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const float* row_scale,
                            const float* col_scale, const float* bias, void* out, int out_dtype,
                            int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,

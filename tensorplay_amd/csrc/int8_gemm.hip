@@ -75,6 +75,19 @@ __global__ __launch_bounds__(256) void int8_finish_kernel(const int32_t* __restr
     }
 }
 
+// c [M][N] = sum of the slices (exact)
+__global__ __launch_bounds__(256) void int32_sum_slices_kernel(const int32_t* __restrict__ partial, int slices, int32_t* __restrict__ c, int64_t total) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t q = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; q < total / 4; q += stride) {  // total % 4 == 0
+        int4 v = make_int4(0, 0, 0, 0);
+        for (int z = 0; z < slices; ++z) {
+            const uint4 p = nt_load(reinterpret_cast<const uint4*>(partial + z * total) + q);
+            v.x += static_cast<int>(p.x); v.y += static_cast<int>(p.y); v.z += static_cast<int>(p.z); v.w += static_cast<int>(p.w);
+        }
+        reinterpret_cast<int4*>(c)[q] = v;
+    }
+}
+
 template <class Epilogue>
 int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
     const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
@@ -211,4 +224,19 @@ TPQ_EXPORT int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const fl
         default: int8_finish_kernel<TPQ_DTYPE_BF16><<<grid, 256, 0, s>>>(acc, slices, row_scale, col_scale, bias, static_cast<uint16_t*>(out), M, N); break;
     }
     return check_launch("int8_mm_dequant (finish)");
+}
+
+TPQ_EXPORT int tpq_int_mm_ws(const void* a, int a_unsigned, const int8_t* b, int64_t b_stride_k, int64_t b_stride_n, int32_t* c,
+                             int64_t M, int64_t K, int64_t N, void* workspace, int64_t workspace_bytes, void* stream) {
+    const bool sliceable = M > 0 && N > 0 && K > 0 && a && b && c && !a_unsigned && b_stride_k == 1 && b_stride_n == K;
+    const int slices = sliceable ? int8_slices(a, b, M, N, K) : 1;
+    if (slices < 2 || workspace == nullptr || workspace_bytes < slices * M * N * 4 || !aligned(workspace, 16) || (M * N) % 4 != 0 ||
+        !aligned(c, 16))
+        return tpq_int_mm(a, a_unsigned, b, b_stride_k, b_stride_n, c, M, K, N, stream);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int32_t* partial = static_cast<int32_t*>(workspace);
+    if (int rc = launch_dma_sliced(static_cast<const int8_t*>(a), b, M, N, K, partial, slices, s)) return rc;
+    const int64_t blocks = (M * N / 4 + 255) / 256;
+    int32_sum_slices_kernel<<<static_cast<unsigned>(blocks > 4096 ? 4096 : blocks), 256, 0, s>>>(partial, slices, c, M * N);
+    return check_launch("_int_mm (sum of slices)");
 }

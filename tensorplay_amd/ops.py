@@ -114,9 +114,17 @@ def _int_mm(self: torch.Tensor, mat2: torch.Tensor, *, out: Optional[torch.Tenso
         else:
             b = mat2.contiguous()
             sbk, sbn = N, 1
+        lib = _lib.load()
         with torch.cuda.device(self.device):
-            _check(_lib.load().tpq_int_mm(_ptr(a), int(a.dtype == torch.uint8), _ptr(b), sbk, sbn, _ptr(dst),
-                                          M, K, N, _stream(self)))
+            # a few hundred rows against a long K: slices of the k range meet in a scratch matrix (same bits)
+            scratch_bytes = int(lib.tpq_int8_mm_workspace_bytes(M, N, K)) if (sbk == 1 and a.dtype == torch.int8) else 0
+            if scratch_bytes:
+                scratch = torch.empty(scratch_bytes // 4, dtype=torch.int32, device=self.device)
+                _check(lib.tpq_int_mm_ws(_ptr(a), 0, _ptr(b), sbk, sbn, _ptr(dst), M, K, N, _ptr(scratch), scratch_bytes,
+                                         _stream(self)))
+            else:
+                _check(lib.tpq_int_mm(_ptr(a), int(a.dtype == torch.uint8), _ptr(b), sbk, sbn, _ptr(dst),
+                                      M, K, N, _stream(self)))
     if out is not None and dst is not out:
         out.copy_(dst)
     return out if out is not None else dst
