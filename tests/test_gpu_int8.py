@@ -64,6 +64,29 @@ def test_int_mm_unsigned_lhs_out_and_empty(ops):
         ops._int_mm(torch.zeros(2, 3, dtype=torch.int8, device=DEV), torch.zeros(2, 2, dtype=torch.int8, device=DEV))
 
 
+@pytest.mark.parametrize("shape", [(32, 4096, 11008), (128, 4096, 4096), (48, 11008, 4096), (512, 4096, 4096)])
+def test_int_mm_decode_and_sliced_kernels_at_model_sizes(ops, shape):
+    """The decode kernel (32 rows per pass, both widths of workgroup) and the sliced tiled kernel at real layer sizes,
+    with the extremes in: exact against numpy, and against the un-sliced single launch through the C ABI."""
+    M, K, N = shape
+    rng = np.random.default_rng(M + K + N)
+    a = _rand_i8(rng, (M, K))
+    w = _rand_i8(rng, (N, K))
+    a[0, :] = -128
+    w[N - 1, :] = -128
+    a[M - 1, ::2] = 127
+    want = a.astype(np.int32) @ w.astype(np.int32).T
+    ad, wd = dev(a), dev(w)
+    got = ops._int_mm(ad, wd.t())
+    np.testing.assert_array_equal(host(got), want)
+    from tensorplay_amd import _lib
+    plain = torch.empty((M, N), dtype=torch.int32, device=DEV)
+    rc = _lib.load().tpq_int_mm(ad.data_ptr(), 0, wd.data_ptr(), 1, K, plain.data_ptr(), M, K, N,
+                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert torch.equal(plain, got)
+
+
 def test_int_mm_extreme_values(ops):
     K = 6912
     a = np.full((130, K), -128, np.int8)

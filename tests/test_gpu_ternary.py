@@ -73,6 +73,21 @@ def test_ternary_mm_exact(ops, M, K, N):
         np.testing.assert_array_equal(host(g16), w16)
 
 
+@pytest.mark.parametrize("M,K,N", [(16, 2560, 6912), (32, 6912, 2560), (8, 8192, 28672)])
+def test_ternary_decode_kernel_at_model_sizes(ops, M, K, N):
+    """The matrix-core decode kernel at real layer sizes, any byte value in the packed weight: exact accumulators,
+    and linear in the activations (x and -x give opposite sums)."""
+    rng = np.random.default_rng(M + K + N)
+    packed = rng.integers(0, 256, size=(N, K // 4)).astype(np.uint8)
+    x = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+    rs = np.ones(M, np.float32)
+    _, want_acc = oracle.ternary_mm(x, rs, packed, 1.0, K)
+    _, acc = ops.ternary_mm(dev(x), dev(rs), dev(packed), 1.0, K, return_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    _, neg = ops.ternary_mm(dev((-x).astype(np.int8)), dev(rs), dev(packed), 1.0, K, return_acc=True)
+    assert torch.equal(neg, -acc)
+
+
 def test_ternary_mm_arbitrary_bytes_and_extremes(ops):
     """Any byte is a legal packed value (0b10 decodes to -2); activations at the int8 extremes."""
     rng = np.random.default_rng(8)
