@@ -38,6 +38,7 @@
 
 #include "int4_lane.h"
 #include "int4_mfma_kernel.h"
+#include "int4_gemm_kernel.h"
 
 namespace tpq {
 namespace {
@@ -496,6 +497,11 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
 template <int DT>
 int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* sz, void* y, int N,
                   int K, int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
+    // Many rows: the tiled kernel, the packed weight read once per 128 rows.  Measured against the 32-row slabs below
+    // (us, fp16): K = 4096, N = 11008: 43 / 55 at 128 rows, 62 / 107 at 256, 258 / 821 at 2048; K = N = 8192:
+    // 77 / 81 at 128, 82 / 157 at 256; at 96 rows the slabs still win (42 against 43, 63 against 77).
+    static const int64_t gemm_rows = [] { const char* e = std::getenv("TPQ_INT4_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{113}; }();
+    if (M >= gemm_rows && int4_gemm_ok(x, packed, sz, y, M, N, K, group)) return launch_int4_gemm<DT>(x, packed, sz, y, M, N, K, group, s);
     {   // slabs of 32 rows (16 with groups of 32 / 64) on the matrix cores where the shape allows
         static const int slab_rows = [] { const char* e = std::getenv("TPQ_INT4_SLAB_ROWS"); return e ? std::atoi(e) : 32; }();
         const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;

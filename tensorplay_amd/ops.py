@@ -228,12 +228,17 @@ def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.T
     return out
 
 
-# Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM.  Measured (fp16): at
-# K = 4096, N = 11008 the 32-row slabs cost about 13.5 us each (54 us at 128 rows, 79 us at 192), the dense route
-# 74 us at 128 rows and 81 us at 192; at K = N = 4096: 41.5 / 61 us against 44 / 50 us.  So the two meet near 128
-# rows for N below 8192 and near 176 rows above.
-INT4_PREFILL_ROWS = 128
-INT4_PREFILL_ROWS_WIDE = 176
+# Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM; below, the library's own
+# kernels read the packed weight (decode kernels up to 112 rows, a tiled kernel above).  Measured (fp16, us, tiled kernel
+# against the dense route): K = 4096, N = 11008: 62 / 89 at 256 rows, 72 / 99 at 512, 141 / 131 at 1024; K = N = 8192:
+# 121 / 141 at 512, 140 / 190 at 1024, 300 / 262 at 2048; K = N = 4096: 42 / 43 at 256, 63 / 45 at 384;
+# K = 11008, N = 4096: 100 / 95 at 256.
+# bfloat16 pays ten vector operations per pair of weights for the dense weight's two roundings (fp16: three packed
+# ones), so the tiled kernel hands over earlier: K = 4096, N = 11008: 69 / 89 at 256 rows, 101 / 89 at 384.
+INT4_PREFILL_ROWS = 256
+INT4_PREFILL_ROWS_WIDE = 768  # N >= 8192
+INT4_PREFILL_ROWS_BF16 = 128
+INT4_PREFILL_ROWS_BF16_WIDE = 256
 # float32 activations have no matrix-core decode kernel: the per-row kernel costs about 16 us a row at K = 4096,
 # N = 11008 (71 us at 4 rows, 253 us at 16), the dense float32 route 95 us at 16 rows and 134 us at 64.
 INT4_PREFILL_ROWS_F32 = 4
@@ -280,6 +285,8 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     sz = qScaleAndZeros.to(self.dtype).contiguous()
     if self.dtype == torch.float32:
         prefill_rows = INT4_PREFILL_ROWS_F32
+    elif self.dtype == torch.bfloat16:
+        prefill_rows = INT4_PREFILL_ROWS_BF16_WIDE if n >= 8192 else INT4_PREFILL_ROWS_BF16
     else:
         prefill_rows = INT4_PREFILL_ROWS_WIDE if n >= 8192 else INT4_PREFILL_ROWS
     if m > prefill_rows and inner == 2:

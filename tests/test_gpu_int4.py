@@ -102,6 +102,34 @@ def test_mm_matches_oracle(ops, dtype, M, N, K, group):
     assert rel_err(got32, y64) < tol
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,group", [(113, 136, 512, 128), (128, 72, 128, 128), (200, 8200, 256, 64), (257, 264, 384, 32),
+                                         (300, 520, 1024, 128), (640, 8, 256, 128), (129, 4096, 4096, 128)])
+def test_mm_tiled_kernel_matches_oracle(ops, dtype, M, N, K, group):
+    """113 rows and more through the C ABI: the tiled kernel (both shapes of workgroup, ragged M and N, every group size),
+    against the oracle to the bounds of test_mm_matches_oracle, and against the decode kernels' rows."""
+    from tensorplay_amd import _lib
+    rng = np.random.default_rng(M * 7 + N * 3 + K + group)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = oracle.int4_pack_tc(codes, 2)
+    xd, pd, sd = dev(xb, dtype), dev(packed), dev(szb, dtype)
+    out = torch.empty((M, N), dtype=TORCH_DT[dtype], device=DEV)
+    tag = {"f16": _lib.F16, "bf16": _lib.BF16}[dtype]
+    rc = _lib.load().tpq_int4_mm(xd.data_ptr(), tag, M, K, pd.data_ptr(), 2, N, group, sd.data_ptr(), out.data_ptr(),
+                                 torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    got32 = out.float().cpu().numpy()
+    ref_dev = oracle.to_f32(oracle.int4_mm_tc(xb, dtype, packed, szb, group, round_w=True), dtype)
+    _, y64 = oracle.int4_mm_tc(xb, dtype, packed, szb, group, round_w=False, want_f64=True)
+    assert_close_norm(got32, ref_dev, 1.5e-2 if dtype == "bf16" and M * N > 50000 else 1e-2, "vs reference formulation")
+    assert rel_err(got32, y64) < {"f16": 1e-3, "bf16": 1e-2}[dtype]
+    few = ops._weight_int4pack_mm(xd[:16], pd, group, sd).float().cpu().numpy()   # the decode kernel on the first rows
+    # two kernels, each within its bound of the oracle (bf16: the decode kernel rounds small-group weights once, this one twice)
+    assert_close_norm(got32[:16], few, 2e-2 if dtype == "bf16" else 1e-2, "vs the decode kernel")
+
+
 @pytest.mark.parametrize("M", [1, 4, 16])
 def test_mm_config2_full_size(ops, M):
     """M x 4096 x 11008, group 128, fp16: the decode configuration at its real size."""
