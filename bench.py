@@ -360,8 +360,8 @@ def main() -> int:
         ms = time_region(gc.replay, sync, 1) / 500
         extras["int4_gemv_cache_resident_us"] = ms * 1e3
         extras["int4_gemv_cache_resident_GBs"] = GEMV_BYTES / (ms * 1e-3) / 1e9
-        # batched decode M = 4, 16 (rotating weights)
-        for mb in (4, 16):
+        # batched decode M = 4, 16, 32 (decode kernels) and 256 rows (tiled kernel), rotating weights
+        for mb in (4, 16, 32, 256):
             xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
             yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
 
@@ -369,9 +369,14 @@ def main() -> int:
                 lib.tpq_int4_mm_ws(xb.data_ptr(), _lib.F16, mb, K, packs[i % copies].data_ptr(), 2, N, GROUP,
                                    szs[i % copies].data_ptr(), yb.data_ptr(), ws.data_ptr(), ws.numel(), cur())
 
-            gb = graph_of(lambda: [gemv_b(i) for i in range(260)])
+            n_b = 260 if mb <= 32 else 64
+            gb = graph_of(lambda: [gemv_b(i) for i in range(n_b)])
             gb.replay(); sync()
-            ms = time_region(gb.replay, sync, 1) / 260
+            ms = time_region(gb.replay, sync, 1) / n_b
+            if mb >= 128:
+                extras[f"int4_gemm_M{mb}_us"] = ms * 1e3
+                extras[f"int4_gemm_M{mb}_TFLOPs"] = 2.0 * mb * N * K / (ms * 1e-3) / 1e12
+                continue
             bytes_b = N * K // 2 + (K // GROUP) * N * 4 + 2 * mb * K + 2 * mb * N
             extras[f"int4_gemv_M{mb}_us"] = ms * 1e3
             extras[f"int4_gemv_M{mb}_GBs"] = bytes_b / (ms * 1e-3) / 1e9
