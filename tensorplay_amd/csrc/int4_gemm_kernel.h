@@ -62,7 +62,10 @@ struct DensePair<TPQ_DTYPE_BF16> {
     }
 };
 
-template <int DT, int NB, int WAVES, int GKT>
+// RSPLIT: the wavefronts of a workgroup form RSPLIT groups that share the channels and split the eight row blocks
+// (each dequantizes the weights again, but there are RSPLIT times the wavefronts per SIMD to overlap loads, vector
+// work and MFMAs when the grid is small).
+template <int DT, int NB, int WAVES, int GKT, int RSPLIT>
 __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t* __restrict__ x, const uint4* __restrict__ packed,
                                                                  const uint32_t* __restrict__ sz, uint16_t* __restrict__ y, int M, int N,
                                                                  int K) {
@@ -78,7 +81,9 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int k_super = K / 32, steps = K / 128, n_tiles = N / 8;
-    const int n0 = blockIdx.x * (16 * NB * WAVES) + wave * (16 * NB);  // first channel of this wavefront
+    constexpr int kChannelWaves = WAVES / RSPLIT, kRowBlocks = kGemmRowBlocks / RSPLIT;
+    const int cw = wave % kChannelWaves, rp = wave / kChannelWaves;    // channel position, row part
+    const int n0 = blockIdx.x * (16 * NB * kChannelWaves) + cw * (16 * NB);  // first channel of this wavefront
     const int m0 = blockIdx.y * kGemmRows;
     const int rows_here = M - m0 < kGemmRows ? M - m0 : kGemmRows;
 
@@ -103,7 +108,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
         x_src[j] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m0 + (x_live[j] ? row : 0)) * K) + col;
         x_dst[j] = row * kGemmPitch + col * 16;
     }
-    const int frag_base = i * kGemmPitch + q * 64;  // + rb * 16 * pitch + u * 16
+    const int frag_base = (rp * kRowBlocks * 16 + i) * kGemmPitch + q * 64;  // + rb * 16 * pitch + u * 16
 
     uint32_t magic_even, magic_odd;  // kept in VGPRs behind an opaque move: v_and_or_b32 takes one literal only
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic_even) : "s"(L::kMagicEven));
@@ -130,11 +135,11 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
         for (int j = 0; j < kChunks; ++j) *reinterpret_cast<uint4*>(lds + buf * kGemmStageBytes + x_dst[j]) = xr[set][j];
     };
 
-    float4_t acc[NB][kGemmRowBlocks];
+    float4_t acc[NB][kRowBlocks];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int rb = 0; rb < kGemmRowBlocks; ++rb) acc[b][rb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int rb = 0; rb < kRowBlocks; ++rb) acc[b][rb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     // (always_inline: a call would put every captured array into scratch memory)
     auto compute = [&](const Weights& st, int buf) __attribute__((always_inline)) {
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
 #pragma unroll
-            for (int rb = 0; rb < kGemmRowBlocks; ++rb) {  // rows past M are zeros in LDS: no branch, so the reads run ahead of the MFMAs
+            for (int rb = 0; rb < kRowBlocks; ++rb) {  // rows past M are zeros in LDS: no branch, so the reads run ahead of the MFMAs
                 const uint4 f = *reinterpret_cast<const uint4*>(stage + rb * (16 * kGemmPitch) + u * 16);
                 const word4_t xb = {f.x, f.y, f.z, f.w};
 #pragma unroll
@@ -203,8 +208,8 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
         const int n = n0 + 16 * b + 4 * q;
         if (n >= N) continue;  // N % 8 == 0 and n % 4 == 0: all four channels exist
 #pragma unroll
-        for (int rb = 0; rb < kGemmRowBlocks; ++rb) {
-            const int row = 16 * rb + i;
+        for (int rb = 0; rb < kRowBlocks; ++rb) {
+            const int row = 16 * (rp * kRowBlocks + rb) + i;
             if (row < rows_here) {
                 const float4_t d = acc[b][rb];
                 const uint32_t lo = L::out(d[0]) | (static_cast<uint32_t>(L::out(d[1])) << 16);
@@ -221,18 +226,19 @@ inline bool int4_gemm_ok(const void* x, const void* packed, const void* sz, cons
            (M + kGemmRows - 1) / kGemmRows <= 65535;
 }
 
-template <int DT, int NB, int WAVES>
+template <int DT, int NB, int WAVES, int RSPLIT>
 int launch_int4_gemm_shape(const void* x, const int32_t* packed, const void* sz, void* y, int64_t M, int64_t N, int64_t K, int group,
                            hipStream_t s) {
     constexpr size_t smem = 2 * static_cast<size_t>(kGemmStageBytes);
-    const dim3 grid(static_cast<unsigned>((N + 16 * NB * WAVES - 1) / (16 * NB * WAVES)), static_cast<unsigned>((M + kGemmRows - 1) / kGemmRows));
+    constexpr int kChannels = 16 * NB * (WAVES / RSPLIT);
+    const dim3 grid(static_cast<unsigned>((N + kChannels - 1) / kChannels), static_cast<unsigned>((M + kGemmRows - 1) / kGemmRows));
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
     const auto* sp = static_cast<const uint32_t*>(sz);
     auto* yp = static_cast<uint16_t*>(y);
 #define TPQ_GEMM4(GKTV)                                                                                                      \
     {                                                                                                                        \
-        auto kernel = int4_gemm_kernel<DT, NB, WAVES, GKTV>;                                                                 \
+        auto kernel = int4_gemm_kernel<DT, NB, WAVES, GKTV, RSPLIT>;                                                                 \
         static std::atomic<uint64_t> configured{0};                                                                          \
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int4 gemm")) return rc;    \
         kernel<<<grid, WAVES * kWave, smem, s>>>(xp, pp, sp, yp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K)); \
@@ -246,14 +252,32 @@ template <int DT>
 int launch_int4_gemm(const void* x, const int32_t* packed, const void* sz, void* y, int64_t M, int64_t N, int64_t K, int group, hipStream_t s) {
     static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT4_GEMM_NB"); return e ? std::atoi(e) : 0; }();
     static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT4_GEMM_WAVES"); return e ? std::atoi(e) : 0; }();
-    // Up to 256 rows there are few workgroups: 64 channels each (4 wavefronts x 16); more rows: 256 channels (8 x 32),
-    // which halves the LDS reads per product.
-    const int nb = forced_nb ? forced_nb : (M <= 256 ? 1 : 2);
-    const int waves = forced_waves ? forced_waves : (M <= 256 ? 4 : 8);
-    if (nb == 4) return launch_int4_gemm_shape<DT, 4, 4>(x, packed, sz, y, M, N, K, group, s);
-    if (nb == 2 && waves == 8) return launch_int4_gemm_shape<DT, 2, 8>(x, packed, sz, y, M, N, K, group, s);
-    if (nb == 2) return launch_int4_gemm_shape<DT, 2, 4>(x, packed, sz, y, M, N, K, group, s);
-    return launch_int4_gemm_shape<DT, 1, 4>(x, packed, sz, y, M, N, K, group, s);
+    static const int forced_rsplit = [] { const char* e = std::getenv("TPQ_INT4_GEMM_RSPLIT"); return e ? std::atoi(e) : 0; }();
+    // Eight wavefronts per workgroup.  Few workgroups (up to 256 rows): two groups of four share the channels and split
+    // the rows, 64 channels per workgroup while that gives at most one workgroup per compute unit, else 128; more rows:
+    // 256 channels, which halves the LDS reads per product.  Measured (us, fp16): 4096 -> 11008: 128 rows 37.5 (42.2
+    // without the split), 256 rows 53.9 with 128 channels (62.6 with 64), 512 rows 74.3 (98.1 with 64 channels);
+    // 8192 x 8192, 256 rows: 73 with 64 channels (256 workgroups), 93 with 128.
+    const bool few = M <= 256;
+    const int64_t narrow_groups = ((N + 63) / 64) * ((M + kGemmRows - 1) / kGemmRows);
+    const int nb = forced_nb ? forced_nb : (few && narrow_groups <= 256 ? 1 : 2);
+    const int waves = forced_waves ? forced_waves : 8;
+    const int rsplit = forced_rsplit ? forced_rsplit : (few ? 2 : 1);
+    if (rsplit == 4 && waves == 16) {
+        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 16, 4>(x, packed, sz, y, M, N, K, group, s);
+        return launch_int4_gemm_shape<DT, 1, 16, 4>(x, packed, sz, y, M, N, K, group, s);
+    }
+    if (rsplit == 2 && waves == 16) {
+        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 16, 2>(x, packed, sz, y, M, N, K, group, s);
+        return launch_int4_gemm_shape<DT, 1, 16, 2>(x, packed, sz, y, M, N, K, group, s);
+    }
+    if (rsplit == 2) {
+        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 8, 2>(x, packed, sz, y, M, N, K, group, s);
+        return launch_int4_gemm_shape<DT, 1, 8, 2>(x, packed, sz, y, M, N, K, group, s);
+    }
+    if (nb == 2 && waves == 8) return launch_int4_gemm_shape<DT, 2, 8, 1>(x, packed, sz, y, M, N, K, group, s);
+    if (nb == 2) return launch_int4_gemm_shape<DT, 2, 4, 1>(x, packed, sz, y, M, N, K, group, s);
+    return launch_int4_gemm_shape<DT, 1, 4, 1>(x, packed, sz, y, M, N, K, group, s);
 }
 
 }  // namespace
