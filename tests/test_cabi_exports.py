@@ -51,6 +51,26 @@ def test_argument_validation_needs_no_gpu():
     assert lib.tpq_ternary_mm(None, None, None, 1.0, None, 0, 4, 4, None, 0, None, None) == _lib.TPQ_OK
 
 
+def test_int8_workspace_sizing_is_host_logic():
+    """tpq_int8_mm_workspace_bytes: slices x M x N x 4 bytes where the k range is cut, 0 where one launch does it."""
+    from tensorplay_amd import _lib
+
+    lib = _lib.load()
+    ws = lib.tpq_int8_mm_workspace_bytes
+    assert ws(16, 4096, 4096) == 0            # decode kernel
+    assert ws(32, 4096, 4096) == 0
+    assert ws(2048, 4096, 4096) == 0          # 256 tiles fill the chip
+    assert ws(128, 4096, 4096) == 8 * 128 * 4096 * 4     # 32 tiles of 256 x 128 -> 8 slices of 4 stages
+    assert ws(512, 4096, 4096) == 4 * 512 * 4096 * 4     # 64 tiles -> 4 slices
+    assert ws(128, 4096, 512) == 0            # K of four stages: nothing to cut
+    assert ws(128, 4096, 4100) == 0           # K not a multiple of the stage
+    assert ws(0, 4096, 4096) == 0 and ws(128, 0, 4096) == 0
+    # a NULL workspace is the plain entry point: same argument checks, no launch for empty problems
+    assert lib.tpq_int8_mm_dequant_ws(None, None, None, None, None, None, 0, 0, 8, 8, None, 0, None) == _lib.TPQ_OK
+    assert lib.tpq_int8_mm_dequant_ws(None, None, None, None, None, None, 7, 4, 8, 8, None, 0, None) == _lib.TPQ_ERR_INVALID_TYPE
+    assert lib.tpq_int_mm_ws(None, 0, None, 1, 1, None, 0, 4, 4, None, 0, None) == _lib.TPQ_OK
+
+
 def test_bench_refuses_more_than_one_gpu():
     """The benchmark is a one-GPU program: any other --gpus value exits with a message and status 2."""
     import os
