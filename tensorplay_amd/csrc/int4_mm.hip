@@ -408,11 +408,14 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     // workgroups, but only when N still yields enough of them to fill the chip:
     //   N = 4096:  16 ch x 8 waves always (8 rows: 5.3 us against 6.0 for 32 ch, 8.5 for 64 ch)
     //   N = 6144, 8192:  32 ch x 8 waves (8192 x 8192, 8 rows: 9.8 us against 13.4 for 16 ch, 14.6 for 64 ch)
-    //   N >= 11008:  32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (11008 x 4096, 16 rows: 9.7 us
-    //                against 12.2 for 32 ch and 14.9 for 16 ch)
-    int nb = N > 5120 ? (N < 10240 ? 2 : (rows > 4 ? 4 : 2)) : 1;
+    //   N = 10240 .. 28672:  64 ch x 8 waves up to 12 rows (4096 -> 11008: 8.0 / 8.1 / 8.4 / 9.0 us at 2 / 4 / 8 / 12
+    //                rows against 8.4 / 8.5 / 9.0 / 9.3 for the next best; 8192 -> 28672, 8 rows: 27.4 against 30.4),
+    //                64 ch x 4 waves above (16 rows: 9.7 us against 12.3 for 32 ch)
+    //   N > 28672:   32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (4096 -> 32000, 4 rows: 16.2 against 16.6)
+    const bool wide = N >= 10240 && N <= 28672 && rows <= 12;
+    int nb = N > 5120 ? (N < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
     if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
-    int waves = N < 10240 ? 8 : 4;
+    int waves = N < 10240 || wide ? 8 : 4;
     if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
@@ -453,7 +456,7 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     if (waves == 16 && nb == 1) {
         TPQ_MFMA(1, 16);
     } else if (waves == 8) {
-        if (nb == 1) TPQ_MFMA(1, 8); else TPQ_MFMA(2, 8);
+        if (nb == 1) TPQ_MFMA(1, 8); else if (nb == 2) TPQ_MFMA(2, 8); else TPQ_MFMA(4, 8);
     } else {
         if (nb == 1) TPQ_MFMA(1, 4); else if (nb == 2) TPQ_MFMA(2, 4); else TPQ_MFMA(4, 4);
     }
