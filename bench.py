@@ -445,6 +445,18 @@ def main() -> int:
         extras["int8_gemm_2048x4096x4096_us"] = ms * 1e3
         extras["int8_gemm_TOPS"] = tops
         extras["int8_gemm_frac_of_mfma_peak"] = tops / INT8_PEAK_TOPS
+        # the vendor library's int8 GEMM on the same operands (torch._int_mm -> hipBLASLt), for scale: it
+        # writes raw int32 sums, without the dequant epilogue that the kernel above includes
+        try:
+            w_qt = w_q.t()
+            for _ in range(5):
+                torch._int_mm(a_q, w_qt)
+            ms_lib = time_region(lambda: torch._int_mm(a_q, w_qt), sync, 50)
+            extras["int8_gemm_vendor_int_mm_us"] = ms_lib * 1e3
+            extras["int8_gemm_vendor_int_mm_TOPS"] = 2.0 * M8 * N8 * K8 / (ms_lib * 1e-3) / 1e12
+        except Exception as exc:  # the library may lack the shape: a comparison figure only
+            extras["int8_gemm_vendor_int_mm_us"] = None
+            extras["int8_gemm_vendor_note"] = str(exc)[:80]
         acc_chk = (a_q[:64].double() @ w_q.double().t())
         fused_chk = ((acc_chk.float() * a_s[:64, None]) * w_s[None, :]).bfloat16()
         extras["int8_gemm_rows_checked_equal"] = bool(torch.equal(fused_chk, out8[:64]))

@@ -604,6 +604,79 @@ __global__ __launch_bounds__(256) void int4_dequantize_kernel(const uint4* __res
     }
 }
 
+// The same dense weight with row-contiguous stores, for K % 32 == 0 and a 16-byte aligned destination.  A thread
+// produces the E = 16 / sizeof(T) consecutive outputs of one 16-byte store: piece p of the 32 k of (row, k-tile).
+// The P = 32 / E threads of a k-tile load the same 16 bytes (one request to the cache) and each cuts out its own
+// nibbles; 32 consecutive threads cover 32 E consecutive k of one row, so every store instruction writes whole
+// cache lines, and the eight rows of a tile are taken by the same workgroup, which reads each packed line once.
+template <int DT>
+__global__ __launch_bounds__(256) void int4_dequantize_rows_kernel(const uint4* __restrict__ packed,
+                                                                   const typename Elem<DT>::storage* __restrict__ sz,
+                                                                   typename Elem<DT>::storage* __restrict__ W, int N, int K,
+                                                                   int k_super, int group_tiles, int chunks_per_row) {
+    using S = typename Elem<DT>::storage;
+    constexpr int E = 16 / sizeof(S), P = 32 / E, kTilesPerGroup = 32 / P;  // k-tiles per workgroup and row
+    const int nT = blockIdx.x / chunks_per_row, chunk = blockIdx.x - nT * chunks_per_row;
+    const int r = threadIdx.x >> 5, q = threadIdx.x & 31;
+    const int kT = chunk * kTilesPerGroup + q / P, p = q % P;
+    if (kT >= k_super) return;
+    const int n = nT * 8 + r;
+    const uint4 w = packed[(static_cast<size_t>(nT) * k_super + kT) * 8 + r];  // the line serves all eight rows: plain load
+    const size_t szi = (static_cast<size_t>(kT / group_tiles) * N + n) * 2;
+    const float scale = Elem<DT>::load(sz[szi]), zero = Elem<DT>::load(sz[szi + 1]);
+    auto code_of = [&](int e) {
+        // k = p E + e inside the tile sits in word (k % 8) / 2, nibble k / 8 (+ 4 for odd k)
+        const int k = p * E + e;
+        const int t4 = (k & 7) >> 1;
+        const uint32_t word = t4 == 0 ? w.x : t4 == 1 ? w.y : t4 == 2 ? w.z : w.w;
+        return static_cast<float>(static_cast<int>((word >> (4 * (k >> 3) + 16 * (k & 1))) & 15u) - 8);
+    };
+    uint32_t words[4];
+    if constexpr (DT == TPQ_DTYPE_BF16) {
+        // both roundings with the hardware's packed conversion (round to nearest even); a NaN takes the
+        // pattern 0x7FC0 that the scalar conversion gives it
+        typedef float f2_t __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int e = 0; e < E; e += 2) {
+            const f2_t prod = {__fmul_rn(code_of(e), scale), __fmul_rn(code_of(e + 1), scale)};
+            const uint32_t pb = __builtin_bit_cast(uint32_t, __builtin_convertvector(prod, bf2_t));
+            const f2_t sum = {__fadd_rn(__builtin_bit_cast(float, pb << 16), zero), __fadd_rn(__builtin_bit_cast(float, pb & 0xFFFF0000u), zero)};
+            uint32_t sb = __builtin_bit_cast(uint32_t, __builtin_convertvector(sum, bf2_t));
+            if (sum.x != sum.x) sb = (sb & 0xFFFF0000u) | 0x7FC0u;
+            if (sum.y != sum.y) sb = (sb & 0x0000FFFFu) | 0x7FC00000u;
+            words[e / 2] = sb;
+        }
+    } else {
+        S out[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float prod = Elem<DT>::load(Elem<DT>::store(__fmul_rn(code_of(e), scale)));
+            out[e] = Elem<DT>::store(__fadd_rn(prod, zero));
+        }
+        if constexpr (sizeof(S) == 2) {
+#pragma unroll
+            for (int e = 0; e < E; e += 2) words[e / 2] = out[e] | (static_cast<uint32_t>(out[e + 1]) << 16);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) words[e] = __builtin_bit_cast(uint32_t, out[e]);
+        }
+    }
+    const uint4 v = make_uint4(words[0], words[1], words[2], words[3]);
+    *reinterpret_cast<uint4*>(W + static_cast<size_t>(n) * K + kT * 32 + p * E) = v;
+}
+
+template <int DT>
+void launch_dequantize_rows(const uint4* packed, const void* sz, void* out, int64_t N, int64_t K, int64_t group, hipStream_t s) {
+    using S = typename Elem<DT>::storage;
+    constexpr int kTilesPerGroup = 32 / (32 / (16 / static_cast<int>(sizeof(S))));
+    const int k_super = static_cast<int>(K / 32);
+    const int chunks = (k_super + kTilesPerGroup - 1) / kTilesPerGroup;
+    int4_dequantize_rows_kernel<DT><<<dim3(static_cast<unsigned>((N / 8) * chunks)), 256, 0, s>>>(
+        packed, static_cast<const S*>(sz), static_cast<S*>(out), static_cast<int>(N), static_cast<int>(K), k_super,
+        static_cast<int>(group / 32), chunks);
+}
+
 }  // namespace
 }  // namespace tpq
 
@@ -672,6 +745,14 @@ TPQ_EXPORT int tpq_int4_dequantize(const int32_t* packed, int inner_k_tiles, int
     hipStream_t s = static_cast<hipStream_t>(stream);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
     const int vec = aligned(out, 16) && K % 8 == 0;  // every row segment of 32 outputs starts 16-byte aligned
+    if (vec && K % 32 == 0 && N * K <= 0x7FFFFFFF && (N / 8) * ((K / 32 + 3) / 4) <= 0x7FFFFFFF && aligned(scales_and_zeros, 4)) {
+        switch (dtype) {
+            case TPQ_DTYPE_F32: launch_dequantize_rows<TPQ_DTYPE_F32>(pp, scales_and_zeros, out, N, K, group, s); break;
+            case TPQ_DTYPE_F16: launch_dequantize_rows<TPQ_DTYPE_F16>(pp, scales_and_zeros, out, N, K, group, s); break;
+            default: launch_dequantize_rows<TPQ_DTYPE_BF16>(pp, scales_and_zeros, out, N, K, group, s); break;
+        }
+        return check_launch("tpq_int4_dequantize");
+    }
     switch (dtype) {
         case TPQ_DTYPE_F32:
             int4_dequantize_kernel<TPQ_DTYPE_F32><<<grid, 256, 0, s>>>(pp, static_cast<const float*>(scales_and_zeros), static_cast<float*>(out), N, K, k_super, group, total, vec);

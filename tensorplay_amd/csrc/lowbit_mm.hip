@@ -316,6 +316,47 @@ __global__ __launch_bounds__(256) void lowbit_dequantize_kernel(const uint8_t* _
     }
 }
 
+// The same for K % 8 == 0 and group % 8 == 0 with aligned rows: a thread takes eight consecutive k of one row, i.e.
+// `bytes` = 1, 2, 4 or 8 packed bytes in one load, one (scale, zero) pair, and 16 (two-byte T) or 32 contiguous output
+// bytes; a wavefront reads and writes contiguous runs of a row.
+template <int DT>
+__global__ __launch_bounds__(256) void lowbit_dequantize_vec_kernel(const uint8_t* __restrict__ packed, const float* __restrict__ sz,
+                                                                    typename Elem<DT>::storage* __restrict__ out, int64_t N, int64_t K,
+                                                                    int64_t group, int bits, int lsb_first) {
+    using S = typename Elem<DT>::storage;
+    const int per_byte = 8 / bits, bytes = 8 / per_byte;
+    const int pb_shift = per_byte == 8 ? 3 : per_byte == 4 ? 2 : per_byte == 2 ? 1 : 0;
+    const int64_t pitch = K >> pb_shift, per_row = K >> 3, total = N * per_row;
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int64_t n = idx / per_row, k0 = (idx - n * per_row) * 8;
+        const uint8_t* src = packed + n * pitch + (k0 >> pb_shift);
+        uint64_t v;
+        if (bytes == 8) v = *reinterpret_cast<const uint64_t*>(src);
+        else if (bytes == 4) v = *reinterpret_cast<const uint32_t*>(src);
+        else if (bytes == 2) v = *reinterpret_cast<const uint16_t*>(src);
+        else v = *src;
+        const float2 p = *reinterpret_cast<const float2*>(sz + ((k0 / group) * N + n) * 2);  // (scale, zero)
+        S o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int field = i & (per_byte - 1);
+            const int shift = 8 * (i >> pb_shift) + (lsb_first ? field * bits : 8 - (field + 1) * bits);
+            const uint32_t code = static_cast<uint32_t>(v >> shift) & mask;
+            o[i] = Elem<DT>::store((static_cast<float>(code) - p.y) * p.x);
+        }
+        S* dst = out + n * K + k0;
+        if constexpr (sizeof(S) == 2) {
+            *reinterpret_cast<uint4*>(dst) = make_uint4(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16),
+                                                        o[4] | (static_cast<uint32_t>(o[5]) << 16), o[6] | (static_cast<uint32_t>(o[7]) << 16));
+        } else {
+            reinterpret_cast<float4*>(dst)[0] = make_float4(o[0], o[1], o[2], o[3]);
+            reinterpret_cast<float4*>(dst)[1] = make_float4(o[4], o[5], o[6], o[7]);
+        }
+    }
+}
+
 // codes uint8 [rows, cols] -> packed [rows, pitch]: one thread per packed byte, tail fields zero
 __global__ __launch_bounds__(256) void lowbit_pack_kernel(const uint8_t* __restrict__ codes, uint8_t* __restrict__ packed, int64_t rows,
                                                           int64_t cols, int bits, int lsb_first) {
@@ -456,6 +497,22 @@ TPQ_EXPORT int tpq_lowbit_dequantize(const uint8_t* packed, int bits, int lsb_fi
     if (N == 0 || K == 0) return TPQ_OK;
     TPQ_REQUIRE(packed && scales_and_zeros && out, TPQ_ERR_INVALID_VALUE, "lowbit dequantize: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (K % 8 == 0 && group % 8 == 0 && aligned(packed, 8) && aligned(scales_and_zeros, 8) && aligned(out, 16)) {
+        const int64_t vblocks = (N * (K / 8) + 255) / 256;
+        const unsigned vgrid = static_cast<unsigned>(vblocks > (1 << 22) ? (1 << 22) : vblocks);
+        switch (dtype) {
+            case TPQ_DTYPE_F32:
+                lowbit_dequantize_vec_kernel<TPQ_DTYPE_F32><<<vgrid, 256, 0, s>>>(packed, scales_and_zeros, static_cast<float*>(out), N, K, group, bits, lsb_first);
+                break;
+            case TPQ_DTYPE_F16:
+                lowbit_dequantize_vec_kernel<TPQ_DTYPE_F16><<<vgrid, 256, 0, s>>>(packed, scales_and_zeros, static_cast<uint16_t*>(out), N, K, group, bits, lsb_first);
+                break;
+            default:
+                lowbit_dequantize_vec_kernel<TPQ_DTYPE_BF16><<<vgrid, 256, 0, s>>>(packed, scales_and_zeros, static_cast<uint16_t*>(out), N, K, group, bits, lsb_first);
+                break;
+        }
+        return check_launch("tpq_lowbit_dequantize");
+    }
     const int64_t blocks = (N * K + 255) / 256;
     const unsigned grid = static_cast<unsigned>(blocks > (1 << 20) ? (1 << 20) : blocks);
     switch (dtype) {

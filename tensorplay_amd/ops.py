@@ -229,16 +229,21 @@ def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.T
 
 
 # Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM; below, the library's own
-# kernels read the packed weight (decode kernels up to 112 rows, a tiled kernel above).  Measured (fp16, us, tiled kernel
-# against the dense route): K = 4096, N = 11008: 62 / 89 at 256 rows, 72 / 99 at 512, 141 / 131 at 1024; K = N = 8192:
-# 121 / 141 at 512, 140 / 190 at 1024, 300 / 262 at 2048; K = N = 4096: 42 / 43 at 256, 63 / 45 at 384;
-# K = 11008, N = 4096: 100 / 95 at 256.
-# bfloat16 pays ten vector operations per pair of weights for the dense weight's two roundings (fp16: three packed
-# ones), so the tiled kernel hands over earlier: K = 4096, N = 11008: 69 / 89 at 256 rows, 101 / 89 at 384.
+# kernels read the packed weight (decode kernels up to 112 rows, a tiled kernel above).  Measured (us, packed-weight
+# kernels against the dense route, whose dequantize pass takes 21 us in float16 and 25 us in bfloat16 at K = 4096,
+# N = 11008).  float16: K = 4096, N = 11008: 53 / 64 at 256 rows, 69 / 66 at 384, 73 / 75 at 512, 139 / 87 at 768;
+# K = N = 8192: 71 / 99 at 256, 115 / 92 at 384; K = N = 4096: 36 / 36 at 256, 60 / 38 at 384; K = 11008, N = 4096:
+# 50 / 49 at 64, 74 / 60 at 96, 85 / 64 at 256; K = 8192, N = 28672: 282 / 341 at 512, 414 / 457 at 768, 533 / 510 at 1024.
+# bfloat16 pays ten vector operations per pair of weights for the dense weight's two roundings in the tiled kernel
+# (float16: three packed ones), so it hands over earlier: K = 4096, N = 11008: 41 / 52 at 96, 54 / 55 at 128, 73 / 60
+# at 192; K = N = 8192: 62 / 67 at 96, 99 / 72 at 128; K = 11008, N = 4096: 48 / 51 at 64, 72 / 63 at 96; K = 8192,
+# N = 28672: 275 / 291 at 256, 336 / 349 at 512, 484 / 441 at 768.
 INT4_PREFILL_ROWS = 256
-INT4_PREFILL_ROWS_WIDE = 768  # N >= 8192
-INT4_PREFILL_ROWS_BF16 = 128
-INT4_PREFILL_ROWS_BF16_WIDE = 256
+INT4_PREFILL_ROWS_WIDE = 512       # N >= 10240
+INT4_PREFILL_ROWS_VERY_WIDE = 768  # N >= 16384
+INT4_PREFILL_ROWS_DEEP = 64        # K >= 2 N: few output tiles, a long k range
+INT4_PREFILL_ROWS_BF16 = 112
+INT4_PREFILL_ROWS_BF16_VERY_WIDE = 512
 # float32 activations have no matrix-core decode kernel: the per-row kernel costs about 16 us a row at K = 4096,
 # N = 11008 (71 us at 4 rows, 253 us at 16), the dense float32 route 95 us at 16 rows and 134 us at 64.
 INT4_PREFILL_ROWS_F32 = 4
@@ -285,10 +290,12 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     sz = qScaleAndZeros.to(self.dtype).contiguous()
     if self.dtype == torch.float32:
         prefill_rows = INT4_PREFILL_ROWS_F32
+    elif k >= 2 * n:
+        prefill_rows = INT4_PREFILL_ROWS_DEEP
     elif self.dtype == torch.bfloat16:
-        prefill_rows = INT4_PREFILL_ROWS_BF16_WIDE if n >= 8192 else INT4_PREFILL_ROWS_BF16
+        prefill_rows = INT4_PREFILL_ROWS_BF16_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS_BF16
     else:
-        prefill_rows = INT4_PREFILL_ROWS_WIDE if n >= 8192 else INT4_PREFILL_ROWS
+        prefill_rows = INT4_PREFILL_ROWS_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS_WIDE if n >= 10240 else INT4_PREFILL_ROWS
     if m > prefill_rows and inner == 2:
         # Many rows: what the reference does for every shape (QuantGemmKernels.cu:1296-1341) - dequantise
         # the weight to a dense matrix of the activation dtype, then one plain library GEMM.  The decode
@@ -540,7 +547,11 @@ def dequantize_affine(input, block_size, scales: torch.Tensor, zero_points: Opti
 
 # ---- packed n-bit weight-only linear (int2 / intx / binary modules) ------------------------------
 
-LOWBIT_PREFILL_ROWS = 64  # above this many activation rows the weight is dequantised once for the library GEMM
+# above this many activation rows the weight is dequantised once for the library GEMM (measured, 2 bits, float16, us,
+# decode kernel / dense route: K = 4096, N = 11008: 35 / 51 at 32 rows, 52 / 52 at 48, 68 / 53 at 64; K = N = 8192:
+# 66 / 71 at 48, 87 / 72 at 64; K = N = 4096: 23 / 36 at 48, 29 / 37 at 64)
+LOWBIT_PREFILL_ROWS = 48
+LOWBIT_PREFILL_ROWS_SMALL = 64  # N K <= 2^24
 LOWBIT_PREFILL_ROWS_F32 = 40  # float32 activations (per-row kernel): 144 / 165 us at 32 rows, 278 / 192 us at 64 (K = 4096, N = 11008)
 
 
@@ -619,7 +630,7 @@ def _lowbit_mm(input: torch.Tensor, packed: torch.Tensor, bits: int, columns: in
     x = input.contiguous()
     m = x.shape[0]
     b = None if bias is None else bias.to(torch.float32).contiguous()
-    if m > (LOWBIT_PREFILL_ROWS_F32 if x.dtype == torch.float32 else LOWBIT_PREFILL_ROWS):
+    if m > (LOWBIT_PREFILL_ROWS_F32 if x.dtype == torch.float32 else LOWBIT_PREFILL_ROWS_SMALL if n * columns <= (1 << 24) else LOWBIT_PREFILL_ROWS):
         dense = _lowbit_dequantize(w, bits, columns, sz, x.dtype, lsb_first)
         out = torch.matmul(x, dense.t())
         return out if b is None else out + b.to(out.dtype)

@@ -192,7 +192,7 @@ def test_cpu_layout_equals_torch_cpu_pack(ops):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
-@pytest.mark.parametrize("N,K,group", [(64, 256, 128), (40, 96, 32), (136, 1024, 64), (8, 70, 32)])
+@pytest.mark.parametrize("N,K,group", [(64, 256, 128), (40, 96, 32), (136, 1024, 64), (8, 70, 32), (264, 4096, 128), (16, 2080, 32)])
 def test_dequantize_bit_exact(ops, dtype, N, K, group):
     """Dense weight from the packed layout: the reference's dequantize kernel, bit for bit."""
     rng = np.random.default_rng(N + K + group)
@@ -203,6 +203,22 @@ def test_dequantize_bit_exact(ops, dtype, N, K, group):
     packed = oracle.int4_pack_tc(codes, 2)
     got = ops._int4_dequantize(dev(packed), 2, packed.shape[0] * 8, K, group, dev(szb, dtype))
     want = oracle.int4_dequantize_tc(packed, szb, dtype, K, group)
+    np.testing.assert_array_equal(host(got), want)
+
+
+def test_dequantize_bf16_non_finite_scale(ops):
+    """An infinite scale gives +-inf and, for code 8, NaN: the dense bf16 weight carries the same bit patterns as the
+    scalar conversion of the oracle (NaN = 0x7FC0)."""
+    rng = np.random.default_rng(77)
+    N, K, group = 16, 256, 128
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    codes[3, :16] = np.arange(16)
+    sz[0, 3, 0] = np.inf
+    sz[1, 5, 1] = np.nan
+    szb = cast_bits(sz, "bf16")
+    packed = oracle.int4_pack_tc(codes, 2)
+    got = ops._int4_dequantize(dev(packed), 2, N, K, group, dev(szb, "bf16"))
+    want = oracle.int4_dequantize_tc(packed, szb, "bf16", K, group)
     np.testing.assert_array_equal(host(got), want)
 
 

@@ -191,11 +191,29 @@ def test_gpu_dequantize_bit_exact_and_many_rows(bits):
     np.testing.assert_array_equal(dense.cpu().numpy(), dense_weight(codes, sz, group))
     dense16 = ops._lowbit_dequantize(packed, bits, K, torch.from_numpy(sz).to(DEV), torch.float16)
     np.testing.assert_array_equal(dense16.cpu().numpy(), dense_weight(codes, sz, group).astype(np.float16))
-    M = ops.LOWBIT_PREFILL_ROWS + 5   # dequantise + library GEMM
+    M = ops.LOWBIT_PREFILL_ROWS_SMALL + 5   # dequantise + library GEMM
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32))
     got = ops._lowbit_mm(x.to(DEV), packed, bits, K, torch.from_numpy(sz).to(DEV))
     want = x.double().numpy() @ dense_weight(codes, sz, group).astype(np.float64).T
     assert rel_err(got.cpu().numpy(), want) < 1e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("lsb_first", [False, True])
+@pytest.mark.parametrize("bits", range(1, 9))
+@pytest.mark.parametrize("N,K,group", [(24, 1024, 64), (7, 2056, 8), (5, 132, 66)])
+def test_gpu_dequantize_vector_and_plain_kernels(bits, lsb_first, N, K, group):
+    """Dense weight in float32 / float16 / bfloat16, bit for bit: rows taken eight k per thread (K and group
+    multiples of 8, several groups and threads per row) and the per-element kernel (K = 132)."""
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(bits * 7 + K + int(lsb_first))
+    codes, sz = make_case(rng, bits, N, K, group)
+    packed = torch.from_numpy(oracle.lowbit_pack(codes, bits, lsb_first)).to(DEV)
+    want = torch.from_numpy(dense_weight(codes, sz, group))
+    szd = torch.from_numpy(sz).to(DEV)
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        got = ops._lowbit_dequantize(packed, bits, K, szd, dtype, lsb_first)
+        assert torch.equal(got.cpu(), want.to(dtype)), (bits, lsb_first, dtype)
 
 
 @pytest.mark.gpu
