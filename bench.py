@@ -67,6 +67,17 @@ def time_region(fn, stream_sync, reps):
     return start.elapsed_time(stop) / reps
 
 
+def steady(fn, stream_sync, reps=1, warm_ms=30.0, batches=7):
+    """fn() repeated for at least `warm_ms` of wall time (after host-side set-up the chip needs about 20 ms of
+    work to reach its sustained clocks), then the median over `batches` timed regions of `reps` calls; ms per call."""
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < warm_ms:
+        for _ in range(reps):
+            fn()
+        stream_sync()
+    return sorted(time_region(fn, stream_sync, reps) for _ in range(batches))[batches // 2]
+
+
 def graph_of(fn):
     """Record fn() (which only enqueues kernels on the current stream) into a HIP graph."""
     import torch
@@ -243,8 +254,7 @@ def decoder_layer_share(dev, rng_seed=5):
     for key, g in (("layer_decode_b8_kv2048_us", g_layer), ("layer_int4_linears_us", g_lin),
                    ("layer_decode_fused_mlp_us", g_layer_f), ("layer_int4_linears_fused_us", g_lin_f)):
         g.replay(); torch.cuda.synchronize()
-        ts = [time_region(g.replay, torch.cuda.synchronize, 1) / reps for _ in range(5)]
-        res[key] = sorted(ts)[2] * 1e3
+        res[key] = steady(g.replay, torch.cuda.synchronize) / reps * 1e3
     res["layer_int4_linear_share"] = res["layer_int4_linears_us"] / res["layer_decode_b8_kv2048_us"]
     lin_bytes = sum(n * k // 2 + (k // 128) * n * 4 + 2 * B * k + 2 * B * n for n, k in shapes.values())
     res["layer_int4_linears_GBs"] = lin_bytes / (res["layer_int4_linears_us"] * 1e-6) / 1e9
@@ -357,7 +367,7 @@ def main() -> int:
         # cache-resident variant: one copy, weights stay in the last-level cache
         gc = graph_of(lambda: [gemv(0) for _ in range(500)])
         gc.replay(); sync()
-        ms = time_region(gc.replay, sync, 1) / 500
+        ms = steady(gc.replay, sync) / 500
         extras["int4_gemv_cache_resident_us"] = ms * 1e3
         extras["int4_gemv_cache_resident_GBs"] = GEMV_BYTES / (ms * 1e-3) / 1e9
         # batched decode M = 4, 16, 32 (decode kernels) and 256 rows (tiled kernel), rotating weights
@@ -372,7 +382,7 @@ def main() -> int:
             n_b = 260 if mb <= 32 else 64
             gb = graph_of(lambda: [gemv_b(i) for i in range(n_b)])
             gb.replay(); sync()
-            ms = time_region(gb.replay, sync, 1) / n_b
+            ms = steady(gb.replay, sync) / n_b
             if mb >= 128:
                 extras[f"int4_gemm_M{mb}_us"] = ms * 1e3
                 extras[f"int4_gemm_M{mb}_TFLOPs"] = 2.0 * mb * N * K / (ms * 1e-3) / 1e12
@@ -395,7 +405,7 @@ def main() -> int:
 
             g8 = graph_of(lambda: [i8mm(i) for i in range(140)])
             g8.replay(); sync()
-            ms = time_region(g8.replay, sync, 1) / 140
+            ms = steady(g8.replay, sync) / 140
             extras[f"int8pack_M{mb}_us"] = ms * 1e3
             extras[f"int8pack_M{mb}_GBs"] = (N * K + 4 * N + 2 * mb * K + 2 * mb * N) / (ms * 1e-3) / 1e9
         del w8s
@@ -417,7 +427,7 @@ def main() -> int:
 
             gl = graph_of(lambda: [lbmm(i) for i in range(2 * n_copies)])
             gl.replay(); sync()
-            ms = time_region(gl.replay, sync, 1) / (2 * n_copies)
+            ms = steady(gl.replay, sync) / (2 * n_copies)
             extras[f"lowbit{bits}_M1_us"] = ms * 1e3
             extras[f"lowbit{bits}_M1_GBs"] = (N * row_bytes + 8 * G * N + 2 * K + 2 * N) / (ms * 1e-3) / 1e9
             del wl
@@ -438,9 +448,9 @@ def main() -> int:
             lib.tpq_int8_mm_dequant(a_q.data_ptr(), w_q.data_ptr(), a_s.data_ptr(), w_s.data_ptr(), None,
                                     out8.data_ptr(), _lib.BF16, M8, N8, K8, cur())
 
-        for _ in range(5):
-            gemm8()
-        ms = time_region(gemm8, sync, 50)
+        # warm-up of at least 30 ms, then the median of 7 batches of 50 launches (the first batches after the
+        # host-side set-up above run 10..30 % slower)
+        ms = steady(gemm8, sync, 50)
         tops = 2.0 * M8 * N8 * K8 / (ms * 1e-3) / 1e12
         extras["int8_gemm_2048x4096x4096_us"] = ms * 1e3
         extras["int8_gemm_TOPS"] = tops
@@ -449,9 +459,7 @@ def main() -> int:
         # writes raw int32 sums, without the dequant epilogue that the kernel above includes
         try:
             w_qt = w_q.t()
-            for _ in range(5):
-                torch._int_mm(a_q, w_qt)
-            ms_lib = time_region(lambda: torch._int_mm(a_q, w_qt), sync, 50)
+            ms_lib = steady(lambda: torch._int_mm(a_q, w_qt), sync, 50)
             extras["int8_gemm_vendor_int_mm_us"] = ms_lib * 1e3
             extras["int8_gemm_vendor_int_mm_TOPS"] = 2.0 * M8 * N8 * K8 / (ms_lib * 1e-3) / 1e12
         except Exception as exc:  # the library may lack the shape: a comparison figure only
@@ -477,7 +485,7 @@ def main() -> int:
             gemm_small(0); sync()
             gs8 = graph_of(lambda: [gemm_small(i) for i in range(120)])
             gs8.replay(); sync()
-            ms = time_region(gs8.replay, sync, 1) / 120
+            ms = steady(gs8.replay, sync) / 120
             extras[f"int8_gemm_{m_small}x4096x4096_us"] = ms * 1e3
             extras[f"int8_gemm_{m_small}x4096x4096_weight_GBs"] = N8 * K8 / (ms * 1e-3) / 1e9
             extras[f"int8_gemm_{m_small}_rows_equal_big_gemm"] = bool(torch.equal(out_small, out8[:m_small]))
@@ -493,7 +501,7 @@ def main() -> int:
 
         for _ in range(5):
             quant()
-        ms = time_region(quant, sync, 100)
+        ms = steady(quant, sync, 100)
         extras["quantize_2048x4096_bf16_us"] = ms * 1e3
         extras["quantize_GBs"] = (3 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
 
@@ -511,7 +519,7 @@ def main() -> int:
 
         for _ in range(5):
             affine_rows()
-        ms = time_region(affine_rows, sync, 100)
+        ms = steady(affine_rows, sync, 100)
         extras["quantize_affine_2048x4096_rows_int8_us"] = ms * 1e3
         extras["quantize_affine_rows_GBs"] = (5 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
         wf = torch.from_numpy(rng.normal(0, 0.02, (4096, 4096)).astype(np.float32)).to(dev)
@@ -534,7 +542,7 @@ def main() -> int:
         for fn, key in ((affine_q4, "quantize_affine_4096x4096_g128_u4"), (affine_dq4, "dequantize_affine_4096x4096_g128_u4")):
             for _ in range(5):
                 fn()
-            ms = time_region(fn, sync, 100)
+            ms = steady(fn, sync, 100)
             extras[key + "_us"] = ms * 1e3
             extras[key + "_GBs"] = (4.5 * 4096 * 4096 + 8 * gs.numel()) / (ms * 1e-3) / 1e9
 
@@ -552,7 +560,7 @@ def main() -> int:
 
             gt = graph_of(lambda: [tmm() for _ in range(200)])
             gt.replay(); sync()
-            ms = time_region(gt.replay, sync, 1) / 200
+            ms = steady(gt.replay, sync) / 200
             key = f"ternary_M{mt}_{kt}x{nt}"
             extras[key + "_us"] = ms * 1e3
             if mt <= 8:
