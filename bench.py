@@ -207,13 +207,12 @@ def decoder_layer_share(dev, rng_seed=5):
     from tensorplay_amd import ops as tops
 
     def layer_fused(L, x):
-        """The same layer with the two fusions around the MLP matmuls: residual add in the epilogue of the
-        o and down projections, gate and up in one launch with the SwiGLU epilogue."""
+        """The same layer with q, k and v in one launch and the two fusions around the MLP matmuls: residual add
+        in the epilogue of the o and down projections, gate and up in one launch with the SwiGLU epilogue."""
         xf = x.view(B, d)
         xn = F.rms_norm(xf, (d,), n1, 1e-5)
-        q = L["q"](xn).view(B, 1, H, D).transpose(1, 2)
-        k = L["k"](xn).view(B, 1, H, D).transpose(1, 2)
-        v = L["v"](xn).view(B, 1, H, D).transpose(1, 2)
+        q, k, v = tops.int4pack_mm_multi(xn, [L[n].weight for n in "qkv"], 128, [L[n].scales_and_zeros for n in "qkv"])
+        q, k, v = (t.view(B, 1, H, D).transpose(1, 2) for t in (q, k, v))
         q, k = rope(q), rope(k)
         kc[:, :, T:T + 1] = k
         vc[:, :, T:T + 1] = v
@@ -227,8 +226,7 @@ def decoder_layer_share(dev, rng_seed=5):
     res_d = torch.randn(B, d, device=dev, generator=gen).half()
 
     def linears_fused(L):
-        for name in ("q", "k", "v"):
-            L[name](xin[name])
+        tops.int4pack_mm_multi(xin["q"].view(B, d), [L[n].weight for n in "qkv"], 128, [L[n].scales_and_zeros for n in "qkv"])
         tops.int4pack_mm_add(xin["o"].view(B, d), L["o"].weight, 128, L["o"].scales_and_zeros, res_d)
         tops.int4pack_mm_swiglu(xin["gate"].view(B, d), L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros,
                                 L["up"].scales_and_zeros)
@@ -258,6 +256,7 @@ def decoder_layer_share(dev, rng_seed=5):
     res["layer_int4_linear_share"] = res["layer_int4_linears_us"] / res["layer_decode_b8_kv2048_us"]
     lin_bytes = sum(n * k // 2 + (k // 128) * n * 4 + 2 * B * k + 2 * B * n for n, k in shapes.values())
     res["layer_int4_linears_GBs"] = lin_bytes / (res["layer_int4_linears_us"] * 1e-6) / 1e9
+    res["layer_int4_linears_fused_GBs"] = lin_bytes / (res["layer_int4_linears_fused_us"] * 1e-6) / 1e9
     return res
 
 

@@ -187,6 +187,20 @@ int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K, const int
                        const void* sz_gate, const void* sz_up, void* out, void* stream);
 
 /*
+ * `count` (1..4) int4 weights applied to the same activations in one launch per 16 rows:
+ * out[w] = T(x . W[w]^T), out[w]: [M, N[w]] of dtype, for w < count.  Same kernel, same shapes
+ * (float16 / bfloat16, innerKTiles = 2, group 128, K % 128 == 0, else TPQ_ERR_UNSUPPORTED) and same
+ * result as `count` calls of tpq_int4_mm at up to 16 rows per call.  packed, N, scales_and_zeros and
+ * out are host arrays of `count` entries (device pointers / widths).  It stands for the three
+ * _weight_int4pack_mm calls on one input that compute q, k and v in the reference's decoder layer
+ * (benchmark/bench_llama_e2e.py:128-130): at 4096 x 4096 a launch costs more than the transfer of
+ * its weight, so one launch for the three takes about half the time of three.
+ */
+int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count,
+                      const int32_t* const* packed, int inner_k_tiles, const int64_t* N, int64_t group,
+                      const void* const* scales_and_zeros, void* const* out, void* stream);
+
+/*
  * Dense weight [N, K] of `dtype` from the packed device layout: W = T(code - 8) * scale + zero, the
  * product and the sum each rounded to T.  The reference runs this before its library GEMM
  * (int4_tc_dequantize_kernel, p10/src/backend/cuda/QuantGemmKernels.cu:1170-1202, 1296-1341); the

@@ -80,11 +80,12 @@ __device__ __forceinline__ uint16_t swiglu_of(float gate_sum, float up_sum) {
 // QuantGemmKernels.cu:1170-1202), three packed operations per pair.  bf16 (no packed bf16 arithmetic): one fp32
 // fma per code and one rounding to bf16, five operations per pair.
 // MB = blocks of 16 activation rows per launch (1 or 2): the unpacked weights of a step feed MB column blocks.
+// block: index of the workgroup among those of this weight (the grid index when a launch serves one weight).
 template <int DT, int NB, int WAVES, bool PAIR = false, int GKT = 4, int MB = 1>
-__global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
+__device__ __forceinline__ void int4_mfma_body(
     const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
     uint16_t* __restrict__ y, int M, int N, int K, int group_shift, const uint4* __restrict__ packed_b,
-    const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual) {
+    const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual, int block) {
     static_assert(!PAIR || NB == 2, "a pair is two blocks");
     static_assert(GKT == 4 || !PAIR, "in-register dequantization is not built for the pair");
     static_assert(MB == 1 || !PAIR, "the pair takes 16 rows");
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int k_super = K / 32, steps = K / 128, n_tiles = N / 8;
-    const int n0 = blockIdx.x * (PAIR ? 16 : 16 * NB);
+    const int n0 = block * (PAIR ? 16 : 16 * NB);
 
     // per-lane bases
     const uint4* w_base[NB];
@@ -327,6 +328,48 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
                 make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
         }
     }
+}
+
+template <int DT, int NB, int WAVES, bool PAIR = false, int GKT = 4, int MB = 1>
+__global__ __launch_bounds__(WAVES * kWave) void int4_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
+    uint16_t* __restrict__ y, int M, int N, int K, int group_shift, const uint4* __restrict__ packed_b,
+    const uint32_t* __restrict__ sz_b, const uint16_t* __restrict__ residual) {
+    int4_mfma_body<DT, NB, WAVES, PAIR, GKT, MB>(x, packed, sz, y, M, N, K, group_shift, packed_b, sz_b, residual,
+                                                 static_cast<int>(blockIdx.x));
+}
+
+// Several weights that share the activations (the q, k and v projections of a decoder layer) in one launch: the
+// workgroups of weight w are blocks first[w] .. first[w + 1] - 1 of the grid.  One launch instead of `count` saves
+// the launch gap and the ramp of every launch after the first: 4096 x 4096 weights are 8.4 MB each, of whose 5 us
+// per launch at most 1.5 us is transfer time.
+constexpr int kMultiMax = 4;
+struct Int4MultiSet {
+    const uint4* packed[kMultiMax];
+    const uint32_t* sz[kMultiMax];
+    uint16_t* y[kMultiMax];
+    int N[kMultiMax];
+    int first[kMultiMax + 1];
+    int count;
+};
+
+template <int DT, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void int4_mfma_multi_kernel(const uint16_t* __restrict__ x, Int4MultiSet set, int M,
+                                                                       int K, int group_shift) {
+    const int block = static_cast<int>(blockIdx.x);
+    int w = 0;
+#pragma unroll
+    for (int i = 1; i < kMultiMax; ++i)
+        if (i < set.count && block >= set.first[i]) w = i;
+    // selected with wave-uniform compares: the struct stays in scalar registers
+    const uint4* packed = set.packed[0];
+    const uint32_t* sz = set.sz[0];
+    uint16_t* y = set.y[0];
+    int N = set.N[0], first = set.first[0];
+#pragma unroll
+    for (int i = 1; i < kMultiMax; ++i)
+        if (w == i) { packed = set.packed[i]; sz = set.sz[i]; y = set.y[i]; N = set.N[i]; first = set.first[i]; }
+    int4_mfma_body<DT, NB, WAVES>(x, packed, sz, y, M, N, K, group_shift, nullptr, nullptr, nullptr, block - first);
 }
 
 }  // namespace

@@ -497,6 +497,41 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
     return TPQ_OK;
 }
 
+// Several weights, one launch per slab of 16 rows (see int4_mfma_multi_kernel).  The workgroup shape follows the
+// rule of launch_mfma_rows for the sum of the widths: that is the width the chip sees.
+template <int DT>
+int launch_multi(const void* x, int64_t M, int count, const int32_t* const* packed, const int64_t* N, const void* const* sz,
+                 void* const* y, int K, int group, hipStream_t s) {
+    int64_t n_total = 0;
+    for (int w = 0; w < count; ++w) n_total += N[w];
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        const bool wide = n_total >= 10240 && n_total <= 28672 && rows <= 12;
+        const int nb = n_total > 5120 ? (n_total < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
+        const int waves = n_total < 10240 || wide ? 8 : 4;
+        Int4MultiSet set{};
+        set.count = count;
+        int blocks = 0;
+        for (int w = 0; w < count; ++w) {
+            set.packed[w] = reinterpret_cast<const uint4*>(packed[w]);
+            set.sz[w] = static_cast<const uint32_t*>(sz[w]);
+            set.y[w] = static_cast<uint16_t*>(y[w]) + m0 * N[w];
+            set.N[w] = static_cast<int>(N[w]);
+            set.first[w] = blocks;
+            blocks += static_cast<int>((N[w] + 16 * nb - 1) / (16 * nb));
+        }
+        set.first[count] = blocks;
+        const auto* xp = static_cast<const uint16_t*>(x) + m0 * K;
+        const int shift = group == 128 ? 0 : 1;
+#define TPQ_MULTI(NBV, WV) int4_mfma_multi_kernel<DT, NBV, WV><<<dim3(blocks), dim3(WV * kWave), 0, s>>>(xp, set, rows, K, shift)
+        if (waves == 8) { if (nb == 1) TPQ_MULTI(1, 8); else if (nb == 2) TPQ_MULTI(2, 8); else TPQ_MULTI(4, 8); }
+        else { if (nb == 2) TPQ_MULTI(2, 4); else TPQ_MULTI(4, 4); }
+#undef TPQ_MULTI
+        if (int rc = check_launch("tpq_int4_mm_multi")) return rc;
+    }
+    return TPQ_OK;
+}
+
 template <int DT>
 int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* sz, void* y, int N,
                   int K, int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
@@ -808,4 +843,30 @@ TPQ_EXPORT int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K
     if (dtype == TPQ_DTYPE_F16)
         return launch_fused<TPQ_DTYPE_F16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s);
     return launch_fused<TPQ_DTYPE_BF16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s);
+}
+
+TPQ_EXPORT int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count, const int32_t* const* packed,
+                                 int inner_k_tiles, const int64_t* N, int64_t group, const void* const* scales_and_zeros,
+                                 void* const* out, void* stream) {
+    TPQ_REQUIRE(count >= 1 && count <= kMultiMax, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: 1 to %d weights per call", kMultiMax);
+    TPQ_REQUIRE(packed && N && scales_and_zeros && out, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: null pointer");
+    int64_t n_total = 0;
+    for (int w = 0; w < count; ++w) {
+        if (int rc = check_fused("tpq_int4_mm_multi", dtype, M, K, inner_k_tiles, N[w], group)) return rc;
+        n_total += N[w];
+    }
+    TPQ_REQUIRE(n_total <= 0x7FFFFFF8, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: dimension too large");
+    if (M == 0 || n_total == 0) return TPQ_OK;
+    TPQ_REQUIRE(K > 0, TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_multi: K = 0 is not built");
+    TPQ_REQUIRE(x && aligned(x, 16), TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: null or unaligned activations");
+    for (int w = 0; w < count; ++w) {
+        if (N[w] == 0) continue;
+        TPQ_REQUIRE(packed[w] && scales_and_zeros[w] && out[w], TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: null pointer");
+        TPQ_REQUIRE(aligned(packed[w], 16) && aligned(scales_and_zeros[w], 16) && aligned(out[w], 8), TPQ_ERR_UNSUPPORTED,
+                    "tpq_int4_mm_multi: unaligned operand");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == TPQ_DTYPE_F16)
+        return launch_multi<TPQ_DTYPE_F16>(x, M, count, packed, N, scales_and_zeros, out, (int)K, (int)group, s);
+    return launch_multi<TPQ_DTYPE_BF16>(x, M, count, packed, N, scales_and_zeros, out, (int)K, (int)group, s);
 }

@@ -8,6 +8,7 @@ Signatures: ``config/native_functions.yaml:5338-5350, 7987-7993`` of the referen
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -674,6 +675,40 @@ def int4pack_mm_add(input: torch.Tensor, mat2: torch.Tensor, qGroupSize: int, qS
         return r + _weight_int4pack_mm(x, w, qGroupSize, sz)
     _check(status)
     return out
+
+
+def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zeros) -> list:
+    """``[_weight_int4pack_mm(input, w, qGroupSize, sz) for w, sz in zip(mats, scales_and_zeros)]`` with one launch
+    per 16 rows for up to four weights (q, k, v of a decoder layer).  Shapes the fused kernel does not take, and more
+    than four weights, run the separate op."""
+    mats, scales_and_zeros = list(mats), list(scales_and_zeros)
+    if len(mats) != len(scales_and_zeros) or not mats:
+        raise ValueError("int4pack_mm_multi: one qScaleAndZeros per packed weight, at least one weight")
+    ops = [_fused_int4_operands(input, w, qGroupSize, sz, "int4pack_mm_multi") for w, sz in zip(mats, scales_and_zeros)]
+    x = ops[0][0]
+    m, k = x.shape
+
+    def separate():
+        return [_weight_int4pack_mm(x, w, qGroupSize, sz) for _, w, sz, _, _ in ops]
+
+    if len(ops) > 4 or len({inner for _, _, _, inner, _ in ops}) != 1 or x.dtype == torch.float32:
+        return separate()
+    outs = [torch.empty((m, n), dtype=x.dtype, device=x.device) for _, _, _, _, n in ops]
+    if m == 0:
+        return outs
+    count = len(ops)
+    packed = (ctypes.c_void_p * count)(*[_ptr(w) for _, w, _, _, _ in ops])
+    szs = (ctypes.c_void_p * count)(*[_ptr(sz) for _, _, sz, _, _ in ops])
+    ys = (ctypes.c_void_p * count)(*[_ptr(o) for o in outs])
+    widths = (ctypes.c_int64 * count)(*[n for _, _, _, _, n in ops])
+    with torch.cuda.device(x.device):
+        status = _lib.load().tpq_int4_mm_multi(_ptr(x), _DT[x.dtype], m, k, count, ctypes.cast(packed, ctypes.c_void_p), ops[0][3],
+                                               ctypes.cast(widths, ctypes.c_void_p), qGroupSize, ctypes.cast(szs, ctypes.c_void_p),
+                                               ctypes.cast(ys, ctypes.c_void_p), _stream(x))
+    if status == _lib.TPQ_ERR_UNSUPPORTED:
+        return separate()
+    _check(status)
+    return outs
 
 
 def int4pack_mm_swiglu(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, qGroupSize: int,

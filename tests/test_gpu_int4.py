@@ -287,6 +287,46 @@ def test_mm_swiglu_against_oracle(ops, tdt, tol, M, N, K):
     assert_close_norm(got.float().cpu().numpy(), want, 2 * tol)
 
 
+@pytest.mark.parametrize("tdt,tol", [(torch.float16, 1e-3), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("M,K,widths", [(1, 256, (64,)), (8, 512, (136, 136, 136)), (16, 1024, (1024, 256, 256)),
+                                        (19, 384, (48, 8, 200, 16)), (8, 4096, (4096, 4096, 4096)), (4, 4096, (11008, 11008))])
+def test_mm_multi_equals_separate_products(ops, tdt, tol, M, K, widths):
+    """Several weights on one input in one launch: every output against the separate op (the same kernel; the order
+    in which the wavefronts' partial sums are added may differ with the workgroup shape) and against the oracle."""
+    rng = np.random.default_rng(M * 31 + K + len(widths))
+    tag = "f16" if tdt == torch.float16 else "bf16"
+    cases = [_fused_case(rng, M, n, K, tdt) for n in widths]
+    x = cases[0][2].to(DEV)
+    packed = [ops._convert_weight_to_int4pack(torch.from_numpy(c).to(DEV), 2) for c, _, _ in cases]
+    szs = [sz.to(DEV) for _, sz, _ in cases]
+    got = ops.int4pack_mm_multi(x, packed, 128, szs)
+    assert len(got) == len(widths)
+    for (codes, sz, _), p, szd, y, n in zip(cases, packed, szs, got, widths):
+        assert tuple(y.shape) == (M, n) and y.dtype == tdt
+        assert_close_norm(y.float().cpu().numpy(), ops._weight_int4pack_mm(x, p, 128, szd).float().cpu().numpy(), tol)
+        if K <= 1024:
+            want = oracle.to_f32(oracle.int4_mm_tc(host(x), tag, oracle.int4_pack_tc(codes, 2), host(sz), 128), tag)
+            assert_close_norm(y.float().cpu().numpy(), want, 2 * tol)
+
+
+def test_mm_multi_other_shapes_and_errors(ops):
+    rng = np.random.default_rng(6)
+    codes = rng.integers(0, 16, (32, 128)).astype(np.int32)
+    packed = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(DEV), 2)
+    sz = torch.rand(4, 32, 2, device=DEV).half() * 0.01   # groups of 32: the separate op runs
+    x = torch.randn(3, 128, device=DEV).half()
+    outs = ops.int4pack_mm_multi(x, [packed, packed], 32, [sz, sz])
+    assert torch.equal(outs[0], ops._weight_int4pack_mm(x, packed, 32, sz)) and torch.equal(outs[0], outs[1])
+    sz128 = torch.rand(1, 32, 2, device=DEV).half() * 0.01
+    five = ops.int4pack_mm_multi(x, [packed] * 5, 128, [sz128] * 5)   # more than four weights: separate ops
+    assert len(five) == 5 and torch.equal(five[0], five[4])
+    assert ops.int4pack_mm_multi(x[:0], [packed], 128, [sz128])[0].shape == (0, 32)
+    with pytest.raises(ValueError):
+        ops.int4pack_mm_multi(x, [packed, packed], 128, [sz128])
+    with pytest.raises(ValueError):
+        ops.int4pack_mm_multi(x, [], 128, [])
+
+
 def test_fused_entry_points_fall_back_for_other_shapes(ops):
     rng = np.random.default_rng(5)
     codes = rng.integers(0, 16, (32, 128)).astype(np.int32)
