@@ -161,6 +161,91 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
     }
 }
 
+// One activation row (fp16 / bf16, K % 16 == 0, K <= 65536): the weight rows are contiguous, so a wavefront reads a
+// row's bytes directly: lane l owns the 16 k of chunk 64 t + l of its pass (a pass = four such turns = 4096 k), one
+// 16-byte load per turn and channel, 1 KB contiguous per wavefront and load, and the 32 bytes of activations that go
+// with them, shared by the wavefront's four channels.  Every load of a wavefront is issued before the first use, so
+// the whole weight is in flight within the first microsecond, as in the int4 kernel for one row.  A workgroup of
+// 4, 8 or 16 wavefronts = channel groups x passes (the fewer, the more workgroups: small weights need them to fill the chip); the lanes' sums meet by a butterfly, the passes' through LDS.
+// fp16: bytes -> fp16 pairs as in the kernel above, v_dot2_f32_f16; bf16: both operands widened to fp32, fma.
+constexpr int kRowChannels = 4, kRowTurns = 4;
+
+template <int DT, int kRowWaves>
+__global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const uint16_t* __restrict__ x, const int8_t* __restrict__ w,
+                                                                        const float* __restrict__ scale, uint16_t* __restrict__ y,
+                                                                        int N, int K, int passes, int groups) {
+    __shared__ float red[kRowWaves][kRowChannels];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = wave / passes, pass = wave - g * passes;
+    const int n0 = (blockIdx.x * groups + g) * kRowChannels;
+    const bool active = g < groups && n0 < N;
+    float acc[kRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) {
+        const int chunks = K >> 4;
+        uint4 wv[kRowChannels][kRowTurns];
+        uint4 xv[kRowTurns][2];
+        bool live[kRowTurns];
+#pragma unroll
+        for (int t = 0; t < kRowTurns; ++t) {
+            const int chunk = (pass * kRowTurns + t) * kWave + lane;
+            live[t] = chunk < chunks;
+            const int cl = live[t] ? chunk : chunks - 1;  // past the end: a valid chunk, multiplied by zeros
+#pragma unroll
+            for (int c = 0; c < kRowChannels; ++c) {
+                const int n = n0 + c < N ? n0 + c : N - 1;
+                wv[c][t] = nt_load(reinterpret_cast<const uint4*>(w + static_cast<size_t>(n) * K) + cl);
+            }
+            const uint4* xp = reinterpret_cast<const uint4*>(x) + 2 * cl;
+            xv[t][0] = live[t] ? xp[0] : make_uint4(0, 0, 0, 0);
+            xv[t][1] = live[t] ? xp[1] : make_uint4(0, 0, 0, 0);
+        }
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+        uint32_t magic;  // exponent bytes, kept in a VGPR behind an opaque move
+        asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(0x64646464u));
+#pragma unroll
+        for (int t = 0; t < kRowTurns; ++t) {
+            const uint32_t xw[8] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w, xv[t][1].x, xv[t][1].y, xv[t][1].z, xv[t][1].w};
+#pragma unroll
+            for (int c = 0; c < kRowChannels; ++c) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {  // dword j: k = 4 j .. 4 j + 3 of the chunk
+                    const uint32_t word = dword_at(wv[c][t], j);
+                    if constexpr (DT == TPQ_DTYPE_F16) {
+                        const uint32_t u = word ^ 0x80808080u;
+                        const uint32_t lo = __builtin_amdgcn_perm(magic, u, 0x04010400u);  // (1152 + b0, 1152 + b1)
+                        const uint32_t hi = __builtin_amdgcn_perm(magic, u, 0x04030402u);  // (1152 + b2, 1152 + b3)
+                        acc[c] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xw[2 * j]), __builtin_bit_cast(h2, lo) - bias, acc[c], false);
+                        acc[c] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xw[2 * j + 1]), __builtin_bit_cast(h2, hi) - bias, acc[c], false);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t xp2 = xw[2 * j + (e >> 1)];
+                            const float xf = __builtin_bit_cast(float, (e & 1) ? (xp2 & 0xFFFF0000u) : (xp2 << 16));
+                            acc[c] = __builtin_fmaf(xf, static_cast<float>(static_cast<int8_t>(word >> (8 * e))), acc[c]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < kRowChannels; ++c) acc[c] = wave_sum(acc[c]);
+    }
+    if (lane < kRowChannels) red[wave][lane] = lane == 0 ? acc[0] : lane == 1 ? acc[1] : lane == 2 ? acc[2] : acc[3];
+    __syncthreads();
+    const int tid = threadIdx.x;
+    if (tid < groups * kRowChannels) {  // thread = (group, channel): the passes in order
+        const int gg = tid / kRowChannels, c = tid - gg * kRowChannels;
+        const int n = (blockIdx.x * groups + gg) * kRowChannels + c;
+        if (n < N) {
+            float sum = 0.0f;
+            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][c];
+            y[n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
+        }
+    }
+}
+
 // Any floating activation dtype, K % 8 == 0, 16-byte aligned rows: a wavefront owns four consecutive output
 // channels and a slab of up to four activation rows; a lane takes eight consecutive k per turn (8 bytes of
 // each weight row, 16 or 32 bytes of each activation row), fp32 fma, one wavefront reduction at the end.
@@ -317,6 +402,29 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
     if (M == 0 || N == 0 || K == 0) return TPQ_OK;  // the reference returns an uninitialised [B, N] here
     TPQ_REQUIRE(x && w && scales && out, TPQ_ERR_INVALID_VALUE, "_weight_int8pack_mm(): null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // One row: the row kernel, at every shape (measured against the matrix-core kernel below, us: 4096 x 4096 5.8 / 6.4,
+    // 11008 -> 4096 10.8 / 14.3, 4096 -> 11008 10.6 / 12.9, 8192 x 8192 13.8 / 18.5, 8192 -> 28672 40.1 / 53.7, 28672 -> 8192
+    // 39.7 / 54.4, 2560 -> 6912 6.2 / 7.8).  Workgroup size by the size of the weight: small weights need many
+    // workgroups to fill the chip (4096 x 4096: 5.8 us with 4 wavefronts, 8.9 with 16), the largest stream best with 8
+    // (8192 -> 28672: 40.1 us = 5.9 TB/s; 42.0 with 4, 45.1 with 16).  TPQ_INT8PACK_ROW=0 / 1 pins the kernel and
+    // TPQ_INT8PACK_ROW_WAVES the workgroup size for comparison runs.
+    static const int forced_row = [] { const char* e = std::getenv("TPQ_INT8PACK_ROW"); return e ? std::atoi(e) : -1; }();
+    static const int forced_row_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_ROW_WAVES"); return e ? std::atoi(e) : 0; }();
+    if (M == 1 && dtype != TPQ_DTYPE_F32 && K % 16 == 0 && K <= 65536 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16) && forced_row != 0) {
+        const int passes = static_cast<int>((K + 4095) / 4096);
+        int waves = N * K >= (int64_t{1} << 27) ? 8 : N * K >= (int64_t{1} << 26) ? 16 : 4;
+        if (forced_row_waves == 4 || forced_row_waves == 8 || forced_row_waves == 16) waves = forced_row_waves;
+        while (waves < passes) waves *= 2;  // a workgroup holds all passes of its channels
+        const int groups = waves / passes;
+        const dim3 grid(static_cast<unsigned>((N + groups * kRowChannels - 1) / (groups * kRowChannels)));
+        const auto* xp = static_cast<const uint16_t*>(x);
+        auto* yp = static_cast<uint16_t*>(out);
+#define TPQ_I8ROW(DTV, WV) int8pack_row_kernel<DTV, WV><<<grid, WV * kWave, 0, s>>>(xp, w, scales, yp, (int)N, (int)K, passes, groups)
+        if (dtype == TPQ_DTYPE_F16) { if (waves == 4) TPQ_I8ROW(TPQ_DTYPE_F16, 4); else if (waves == 8) TPQ_I8ROW(TPQ_DTYPE_F16, 8); else TPQ_I8ROW(TPQ_DTYPE_F16, 16); }
+        else { if (waves == 4) TPQ_I8ROW(TPQ_DTYPE_BF16, 4); else if (waves == 8) TPQ_I8ROW(TPQ_DTYPE_BF16, 8); else TPQ_I8ROW(TPQ_DTYPE_BF16, 16); }
+#undef TPQ_I8ROW
+        return check_launch("_weight_int8pack_mm (row)");
+    }
     if (dtype != TPQ_DTYPE_F32 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
         static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT8PACK_NB"); return e ? std::atoi(e) : 0; }();
         static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_WAVES"); return e ? std::atoi(e) : 0; }();

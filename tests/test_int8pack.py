@@ -32,7 +32,10 @@ def test_oracle_literal_and_closed_form():
 
 CASES = [(1, 4096, 512), (4, 1024, 136), (16, 256, 40), (17, 384, 72), (2, 100, 9), (8, 16, 3), (33, 128, 24), (1, 11008, 256),
          # every shape of workgroup of the decode kernel: 16 / 32 channels, 16 / 32 rows per pass, ragged N
-         (32, 256, 8200), (64, 128, 50), (9, 128, 16390), (3, 256, 16400), (24, 384, 10250), (40, 128, 10240)]
+         (32, 256, 8200), (64, 128, 50), (9, 128, 16390), (3, 256, 16400), (24, 384, 10250), (40, 128, 10240),
+         # one row through the row kernel: a last turn that is partly past K, several passes per channel, ragged N,
+         # the three workgroup sizes (by N K), K of 16 only
+         (1, 4112, 10), (1, 16, 7), (1, 28672, 130), (1, 8192, 8200), (1, 4096, 32772), (1, 65536, 12), (1, 48, 1)]
 
 
 @pytest.mark.gpu
