@@ -424,6 +424,140 @@ int launch_generic(const void* x, const uint8_t* packed, const float* sz, const 
     return check_launch("tpq_lowbit_mm (generic)");
 }
 
+// One activation row (fp16 / bf16), 1, 2 or 4 bits: the packed rows are contiguous, so a wavefront reads them
+// directly, as the one-row int8 weight-only kernel does.  A pass is 4096 k: lane l owns 64 of them, as TURNS
+// segments of CPL codes (one 16-byte load each; 8 bytes at one bit), and the 128 bytes of activations that go with
+// them, shared by the wavefront's four channels.  Every load is issued before the first use.  A field position p of
+// the four bytes of a word is cut out with one shift and one mask, each byte converted with v_cvt_f32_ubyte, one fp32
+// fma per code; per segment and channel  y += scale (sum code x - zero sum x), a segment lying inside one group.
+// Workgroup = channel groups x passes; the lanes' sums meet by a butterfly, the passes' through LDS.
+constexpr int kLbRowChannels = 4;
+
+template <int DT, int BITS, bool LSB, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed,
+                                                                  const float* __restrict__ sz, const float* __restrict__ bias,
+                                                                  uint16_t* __restrict__ y, int N, int K, int group, int passes, int groups) {
+    constexpr int kPerByte = 8 / BITS;
+    constexpr int kLoadBytes = BITS == 1 ? 8 : 16;
+    constexpr int kCpl = kLoadBytes * kPerByte;  // codes per load: 64, 64, 32
+    constexpr int kTurns = 64 / kCpl;            // 1, 1, 2
+    constexpr int kWords = kLoadBytes / 4;
+    constexpr uint32_t kMask = ((1u << BITS) - 1u) * 0x01010101u;
+    __shared__ float red[WAVES][kLbRowChannels];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = wave / passes, pass = wave - g * passes;
+    const int n0 = (blockIdx.x * groups + g) * kLbRowChannels;
+    const bool active = g < groups && n0 < N;
+    float acc[kLbRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) {
+        const size_t pitch = static_cast<size_t>(K) / kPerByte;
+        uint32_t wv[kLbRowChannels][kTurns][kWords];
+        float2 p[kLbRowChannels][kTurns];
+        uint4 xv[kTurns][kCpl / 8];
+        bool live[kTurns];
+#pragma unroll
+        for (int t = 0; t < kTurns; ++t) {
+            const int k0 = ((pass * kTurns + t) * kWave + lane) * kCpl;
+            live[t] = k0 < K;
+            const int kl = live[t] ? k0 : 0;  // past the end: a valid segment, multiplied by zeros
+#pragma unroll
+            for (int c = 0; c < kLbRowChannels; ++c) {
+                const int n = n0 + c < N ? n0 + c : N - 1;
+                const uint8_t* src = packed + static_cast<size_t>(n) * pitch + kl / kPerByte;
+                if constexpr (kLoadBytes == 16) {
+                    const uint4 q = nt_load(reinterpret_cast<const uint4*>(src));
+                    wv[c][t][0] = q.x; wv[c][t][1] = q.y; wv[c][t][2] = q.z; wv[c][t][3] = q.w;
+                } else {
+                    const uint2 q = nt_load(reinterpret_cast<const uint2*>(src));
+                    wv[c][t][0] = q.x; wv[c][t][1] = q.y;
+                }
+                p[c][t] = *reinterpret_cast<const float2*>(sz + (static_cast<size_t>(kl / group) * N + n) * 2);
+            }
+            const uint4* xp = reinterpret_cast<const uint4*>(x + kl);
+#pragma unroll
+            for (int e = 0; e < kCpl / 8; ++e) xv[t][e] = live[t] ? xp[e] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < kTurns; ++t) {
+            float s[kLbRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float sx = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWords; ++w)
+#pragma unroll
+                for (int pos = 0; pos < kPerByte; ++pos) {  // field position counted from the low end of a byte
+                    uint32_t f[kLbRowChannels];
+#pragma unroll
+                    for (int c = 0; c < kLbRowChannels; ++c) f[c] = (wv[c][t][w] >> (pos * BITS)) & kMask;
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        // code index inside the segment: byte 4 w + b, field pos from the low end
+                        const int e = (4 * w + b) * kPerByte + (LSB ? pos : kPerByte - 1 - pos);
+                        const uint4& xq = xv[t][e >> 3];
+                        const uint32_t pair = ((e >> 1) & 3) == 0 ? xq.x : ((e >> 1) & 3) == 1 ? xq.y : ((e >> 1) & 3) == 2 ? xq.z : xq.w;
+                        const float xf = Elem<DT>::load(static_cast<uint16_t>((e & 1) ? pair >> 16 : pair & 0xFFFFu));
+                        sx += xf;
+#pragma unroll
+                        for (int c = 0; c < kLbRowChannels; ++c) {
+                            const float cf = static_cast<float>((f[c] >> (8 * b)) & 0xFFu);  // becomes v_cvt_f32_ubyte<b>
+                            s[c] = __builtin_fmaf(cf, xf, s[c]);
+                        }
+                    }
+                }
+#pragma unroll
+            for (int c = 0; c < kLbRowChannels; ++c) acc[c] = __builtin_fmaf(p[c][t].x, s[c] - p[c][t].y * sx, acc[c]);
+        }
+#pragma unroll
+        for (int c = 0; c < kLbRowChannels; ++c) acc[c] = wave_sum(acc[c]);
+    }
+    if (lane < kLbRowChannels) red[wave][lane] = lane == 0 ? acc[0] : lane == 1 ? acc[1] : lane == 2 ? acc[2] : acc[3];
+    __syncthreads();
+    const int tid = threadIdx.x;
+    if (tid < groups * kLbRowChannels) {  // thread = (group, channel): the passes in order
+        const int gg = tid / kLbRowChannels, c = tid - gg * kLbRowChannels;
+        const int n = (blockIdx.x * groups + gg) * kLbRowChannels + c;
+        if (n < N) {
+            float sum = 0.0f;
+            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][c];
+            if (bias != nullptr) sum += bias[n];
+            y[n] = Elem<DT>::store(sum);
+        }
+    }
+}
+
+// false if the shape is not one the row kernel takes
+template <int DT>
+bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t N, int64_t K,
+                       int64_t group, int bits, int lsb_first, bool forced, hipStream_t s, int* rc) {
+    if (bits != 1 && bits != 2 && bits != 4) return false;
+    const int cpl = bits == 4 ? 32 : 64;
+    if (K <= 0 || K % cpl != 0 || group % cpl != 0 || K > 65536 || N > 0x7FFFFFF0) return false;
+    // Measured against the matrix-core kernel (us, 1 / 2 / 4 bits): 4096 -> 11008: 8.8 / 9.3 / 9.3 against 9.8 / 10.1 / 10.4;
+    // 8192 x 8192: 11.3 / 11.7 / 12.1 against 12.7 / 13.2 / 15.4; 8192 -> 28672: 32.2 / 33.8 / 40.3 against 37.7 / 40.1 / 45.2.
+    // Smaller weights (4096 x 4096: 5.5 / 5.8 / 5.4 against 4.8 / 5.1 / 5.2) and rows of more than 16384 k (28672 -> 8192
+    // at 2 bits: 45.8 against 39.8) stay on that kernel unless forced: at 2.75 vector instructions per code this
+    // kernel is bound by instruction issue, not by the stream.
+    if (!forced && (N * K < (int64_t{1} << 25) || K > 16384 || N < K)) return false;  // 11008 -> 4096 at 2 bits: 10.3 against 9.1
+    if (!aligned(x, 16) || !aligned(packed, 16) || !aligned(sz, 8) || !aligned(out, 2)) return false;
+    const int passes = static_cast<int>((K + 4095) / 4096);
+    // small weights need many workgroups to fill the chip: 4 wavefronts; 16 from 64 MB of packed bytes and for long rows
+    const int waves = (N * (K / (8 / bits)) >= (int64_t{1} << 26) || passes > 4) ? 16 : 4;
+    const int groups = waves / passes;
+    const dim3 grid(static_cast<unsigned>((N + groups * kLbRowChannels - 1) / (groups * kLbRowChannels)));
+    const auto* xp = static_cast<const uint16_t*>(x);
+    auto* yp = static_cast<uint16_t*>(out);
+    const int n = static_cast<int>(N), k = static_cast<int>(K), gr = static_cast<int>(group);
+#define TPQ_LBROW(B, L, W) lowbit_row_kernel<DT, B, L, W><<<grid, W * kWave, 0, s>>>(xp, packed, sz, bias, yp, n, k, gr, passes, groups)
+#define TPQ_LBROW_W(B, L) do { if (waves == 4) TPQ_LBROW(B, L, 4); else TPQ_LBROW(B, L, 16); } while (0)
+#define TPQ_LBROW_L(B) do { if (lsb_first) TPQ_LBROW_W(B, true); else TPQ_LBROW_W(B, false); } while (0)
+    if (bits == 1) TPQ_LBROW_L(1); else if (bits == 2) TPQ_LBROW_L(2); else TPQ_LBROW_L(4);
+#undef TPQ_LBROW_L
+#undef TPQ_LBROW_W
+#undef TPQ_LBROW
+    *rc = check_launch("tpq_lowbit_mm (row)");
+    return true;
+}
+
 int check_lowbit(const char* op, int bits, int lsb_first, int64_t N, int64_t K, int64_t group) {
     TPQ_REQUIRE(bits >= 1 && bits <= 8, TPQ_ERR_INVALID_VALUE, "%s: bits must be in [1, 8], got %d", op, bits);
     TPQ_REQUIRE(lsb_first == 0 || lsb_first == 1, TPQ_ERR_INVALID_VALUE, "%s: lsb_first must be 0 or 1", op);
@@ -462,6 +596,14 @@ TPQ_EXPORT int tpq_lowbit_mm(const void* x, int dtype, int64_t M, int64_t K, con
     }
     const bool fast = dtype != TPQ_DTYPE_F32 && K > 0 && group_shift >= 0 && K % step_k == 0 && N % 4 == 0 && K <= 0x7FFFFF80 &&
                       N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(packed, 16) && aligned(scales_and_zeros, 16) && aligned(out, 8);
+    const char* row_env = M == 1 ? std::getenv("TPQ_LOWBIT_ROW") : nullptr;  // read per call: tests switch it
+    const int forced_row = row_env ? std::atoi(row_env) : -1;
+    if (M == 1 && dtype != TPQ_DTYPE_F32 && forced_row != 0) {  // TPQ_LOWBIT_ROW=0 / 1: never / wherever the shape allows, for comparison runs and tests
+        int rc = TPQ_OK;
+        if (dtype == TPQ_DTYPE_F16 ? launch_lowbit_row<TPQ_DTYPE_F16>(x, packed, scales_and_zeros, bias, out, N, K, group, bits, lsb_first, forced_row == 1, s, &rc)
+                                   : launch_lowbit_row<TPQ_DTYPE_BF16>(x, packed, scales_and_zeros, bias, out, N, K, group, bits, lsb_first, forced_row == 1, s, &rc))
+            return rc;
+    }
     if (fast) {
 #define TPQ_LB_CASE(BITS)                                                                                                      \
     case BITS:                                                                                                                 \

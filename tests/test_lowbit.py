@@ -165,6 +165,46 @@ def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits,lsb", [(1, False), (1, True), (2, False), (2, True), (4, False), (4, True)])
+@pytest.mark.parametrize("N,K,group", [(10, 4096, 128), (7, 8192, 64), (130, 4160, 32), (5, 20480, 1024), (1, 64, 64), (36, 11008, 128)])
+@pytest.mark.parametrize("tdt,tag,tol", [(torch.float16, "f16", 1e-3), (torch.bfloat16, "bf16", 8e-3)])
+def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatch):
+    """One activation row on the kernel that streams the packed rows: several passes per channel, a last segment
+    past K, ragged N, both bit orders, both workgroup sizes (by K), groups of one segment and of many, with a bias.
+    The kernel is the default only for large weights; TPQ_LOWBIT_ROW=1 selects it wherever the shape allows."""
+    from tensorplay_amd import ops
+    monkeypatch.setenv("TPQ_LOWBIT_ROW", "1")
+    if group % (32 if bits == 4 else 64):
+        pytest.skip("the groups of this case are shorter than a lane's segment: other kernel, covered elsewhere")
+    rng = np.random.default_rng(bits * 17 + K + N)
+    codes, sz = make_case(rng, bits, N, K, group)
+    x16 = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(tdt)
+    bias = rng.standard_normal(N).astype(np.float32) if N % 2 else None
+    packed = oracle.lowbit_pack(codes, bits, lsb_first=lsb)
+    want = oracle.lowbit_mm(x16.view(torch.int16).numpy().view(np.uint16), tag, packed, bits, sz, K, group, bias=bias,
+                            lsb_first=lsb, want_f64=True)[1]
+    got = ops._lowbit_mm(x16.to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV),
+                         None if bias is None else torch.from_numpy(bias).to(DEV), lsb_first=lsb)
+    assert got.shape == (1, N)
+    assert rel_err(got.float().cpu().numpy(), want) < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_gpu_mm_one_row_default_route_large_weight(bits):
+    """A weight large enough for the row kernel to be the default choice (N K >= 2^25, N >= K, K <= 16384)."""
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(90 + bits)
+    N, K, group = 8198, 4160, 32 if bits == 4 else 64
+    codes, sz = make_case(rng, bits, N, K, group)
+    x16 = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).half()
+    packed = oracle.lowbit_pack(codes, bits)
+    want = x16.double().numpy() @ dense_weight(codes, sz, group).astype(np.float64).T
+    got = ops._lowbit_mm(x16.to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV))
+    assert rel_err(got.float().cpu().numpy(), want) < 1e-3
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tdtype", [torch.bfloat16, torch.float16])
 def test_gpu_mm_other_routes(tdtype):
     """bf16 activations, and N % 4 != 0 / groups that the decode kernel does not take: plain kernel."""
