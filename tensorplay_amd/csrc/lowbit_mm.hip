@@ -427,9 +427,8 @@ int launch_generic(const void* x, const uint8_t* packed, const float* sz, const 
 // One activation row (fp16 / bf16), 1, 2 or 4 bits: the packed rows are contiguous, so a wavefront reads them
 // directly, as the one-row int8 weight-only kernel does.  A pass is 4096 k: lane l owns 64 of them, as TURNS
 // segments of CPL codes (one 16-byte load each; 8 bytes at one bit), and the 128 bytes of activations that go with
-// them, shared by the wavefront's four channels.  Every load is issued before the first use.  A field position p of
-// the four bytes of a word is cut out with one shift and one mask, each byte converted with v_cvt_f32_ubyte, one fp32
-// fma per code; per segment and channel  y += scale (sum code x - zero sum x), a segment lying inside one group.
+// them, shared by the wavefront's four channels.  Every load is issued before the first use.  Per segment and channel
+// y += scale (sum code x - zero sum x), a segment lying inside one group; three vector instructions per pair of codes.
 // Workgroup = channel groups x passes; the lanes' sums meet by a butterfly, the passes' through LDS.
 constexpr int kLbRowChannels = 4;
 
@@ -442,7 +441,6 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
     constexpr int kCpl = kLoadBytes * kPerByte;  // codes per load: 64, 64, 32
     constexpr int kTurns = 64 / kCpl;            // 1, 1, 2
     constexpr int kWords = kLoadBytes / 4;
-    constexpr uint32_t kMask = ((1u << BITS) - 1u) * 0x01010101u;
     __shared__ float red[WAVES][kLbRowChannels];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -478,34 +476,50 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
 #pragma unroll
             for (int e = 0; e < kCpl / 8; ++e) xv[t][e] = live[t] ? xp[e] : make_uint4(0, 0, 0, 0);
         }
+        // Codes become 16-bit floats in place.  A field of BITS bits moved to the top of the mantissa of each half
+        // of the word (one shift), masked and given the exponent whose lowest field bit weighs one (one v_and_or_b32)
+        // is the pair (2^BITS + code, 2^BITS + code') of the two halves' codes at that position; one v_dot2 multiplies
+        // it with the matching pair of activations, and the constant is removed with the segment's sum of activations,
+        // which the zero point needs anyway:  y += scale (dot - (2^BITS + zero) sum x).
+        using L = Lane16<DT>;
+        constexpr int kMant = DT == TPQ_DTYPE_F16 ? 10 : 7, kExpBias = DT == TPQ_DTYPE_F16 ? 15 : 127;
+        constexpr uint32_t kMagic = (static_cast<uint32_t>(kExpBias + BITS) << kMant) * 0x00010001u;
+        constexpr uint32_t kFieldMask = (((1u << BITS) - 1u) << (kMant - BITS)) * 0x00010001u;
+        constexpr int kFieldsPerHalf = 16 / BITS;
+        uint32_t magic;  // kept in a VGPR behind an opaque move: v_and_or_b32 takes one literal only
+        asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(kMagic));
 #pragma unroll
         for (int t = 0; t < kTurns; ++t) {
-            float s[kLbRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+            // activations: the natural pairs (k, k + 1) for the sum, and for every (word, position) the pair that
+            // sits under the two halves of the word: codes e and e + 2 kPerByte of the segment
+            auto half_of = [&](int e) -> uint32_t {
+                const uint4& xq = xv[t][e >> 3];
+                const uint32_t pair = ((e >> 1) & 3) == 0 ? xq.x : ((e >> 1) & 3) == 1 ? xq.y : ((e >> 1) & 3) == 2 ? xq.z : xq.w;
+                return (e & 1) ? pair >> 16 : pair & 0xFFFFu;
+            };
             float sx = 0.0f;
+#pragma unroll
+            for (int e = 0; e < kCpl; e += 2) sx = L::dot(half_of(e) | (half_of(e + 1) << 16), L::kOnes, sx);
+            float s[kLbRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int w = 0; w < kWords; ++w)
 #pragma unroll
-                for (int pos = 0; pos < kPerByte; ++pos) {  // field position counted from the low end of a byte
-                    uint32_t f[kLbRowChannels];
+                for (int fp = 0; fp < kFieldsPerHalf; ++fp) {  // field position inside a 16-bit half, from its low end
+                    const int byte = 4 * w + fp / kPerByte, pos = fp % kPerByte;
+                    const int e = byte * kPerByte + (LSB ? pos : kPerByte - 1 - pos);
+                    const uint32_t xpair = half_of(e) | (half_of(e + 2 * kPerByte) << 16);
+                    constexpr int kTop = kMant - BITS;
+                    const int shift = kTop - fp * BITS;  // to the top of the mantissa
 #pragma unroll
-                    for (int c = 0; c < kLbRowChannels; ++c) f[c] = (wv[c][t][w] >> (pos * BITS)) & kMask;
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        // code index inside the segment: byte 4 w + b, field pos from the low end
-                        const int e = (4 * w + b) * kPerByte + (LSB ? pos : kPerByte - 1 - pos);
-                        const uint4& xq = xv[t][e >> 3];
-                        const uint32_t pair = ((e >> 1) & 3) == 0 ? xq.x : ((e >> 1) & 3) == 1 ? xq.y : ((e >> 1) & 3) == 2 ? xq.z : xq.w;
-                        const float xf = Elem<DT>::load(static_cast<uint16_t>((e & 1) ? pair >> 16 : pair & 0xFFFFu));
-                        sx += xf;
-#pragma unroll
-                        for (int c = 0; c < kLbRowChannels; ++c) {
-                            const float cf = static_cast<float>((f[c] >> (8 * b)) & 0xFFu);  // becomes v_cvt_f32_ubyte<b>
-                            s[c] = __builtin_fmaf(cf, xf, s[c]);
-                        }
+                    for (int c = 0; c < kLbRowChannels; ++c) {
+                        const uint32_t word = wv[c][t][w];
+                        const uint32_t moved = shift >= 0 ? word << shift : word >> -shift;
+                        s[c] = L::dot(xpair, (moved & kFieldMask) | magic, s[c]);
                     }
                 }
 #pragma unroll
-            for (int c = 0; c < kLbRowChannels; ++c) acc[c] = __builtin_fmaf(p[c][t].x, s[c] - p[c][t].y * sx, acc[c]);
+            for (int c = 0; c < kLbRowChannels; ++c)
+                acc[c] = __builtin_fmaf(p[c][t].x, s[c] - (static_cast<float>(1 << BITS) + p[c][t].y) * sx, acc[c]);
         }
 #pragma unroll
         for (int c = 0; c < kLbRowChannels; ++c) acc[c] = wave_sum(acc[c]);
@@ -532,12 +546,10 @@ bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, co
     if (bits != 1 && bits != 2 && bits != 4) return false;
     const int cpl = bits == 4 ? 32 : 64;
     if (K <= 0 || K % cpl != 0 || group % cpl != 0 || K > 65536 || N > 0x7FFFFFF0) return false;
-    // Measured against the matrix-core kernel (us, 1 / 2 / 4 bits): 4096 -> 11008: 8.8 / 9.3 / 9.3 against 9.8 / 10.1 / 10.4;
-    // 8192 x 8192: 11.3 / 11.7 / 12.1 against 12.7 / 13.2 / 15.4; 8192 -> 28672: 32.2 / 33.8 / 40.3 against 37.7 / 40.1 / 45.2.
-    // Smaller weights (4096 x 4096: 5.5 / 5.8 / 5.4 against 4.8 / 5.1 / 5.2) and rows of more than 16384 k (28672 -> 8192
-    // at 2 bits: 45.8 against 39.8) stay on that kernel unless forced: at 2.75 vector instructions per code this
-    // kernel is bound by instruction issue, not by the stream.
-    if (!forced && (N * K < (int64_t{1} << 25) || K > 16384 || N < K)) return false;  // 11008 -> 4096 at 2 bits: 10.3 against 9.1
+    // Measured against the matrix-core kernel (us, 1 / 2 / 4 bits): 4096 -> 11008: 7.5 / 8.2 / 8.0 against 9.8 / 10.1 / 10.4;
+    // 8192 x 8192: 9.6 / 10.7 / 10.9 against 12.7 / 13.2 / 15.4; 8192 -> 28672: 26.4 / 29.8 / 35.7 against 37.7 / 40.1 / 45.2;
+    // 4096 x 4096: 4.8 / 5.0 / 4.7 against 4.8 / 5.1 / 5.2; 28672 -> 8192: 35.3 / 41.7 / 39.2 against 39.3 / 39.8 / 46.7.
+    (void)forced;
     if (!aligned(x, 16) || !aligned(packed, 16) || !aligned(sz, 8) || !aligned(out, 2)) return false;
     const int passes = static_cast<int>((K + 4095) / 4096);
     // small weights need many workgroups to fill the chip: 4 wavefronts; 16 from 64 MB of packed bytes and for long rows

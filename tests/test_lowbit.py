@@ -171,7 +171,7 @@ def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
 def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatch):
     """One activation row on the kernel that streams the packed rows: several passes per channel, a last segment
     past K, ragged N, both bit orders, both workgroup sizes (by K), groups of one segment and of many, with a bias.
-    The kernel is the default only for large weights; TPQ_LOWBIT_ROW=1 selects it wherever the shape allows."""
+    TPQ_LOWBIT_ROW=1 pins the kernel (it is also the default for these shapes)."""
     from tensorplay_amd import ops
     monkeypatch.setenv("TPQ_LOWBIT_ROW", "1")
     if group % (32 if bits == 4 else 64):
@@ -192,7 +192,7 @@ def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatc
 @pytest.mark.gpu
 @pytest.mark.parametrize("bits", [1, 2, 4])
 def test_gpu_mm_one_row_default_route_large_weight(bits):
-    """A weight large enough for the row kernel to be the default choice (N K >= 2^25, N >= K, K <= 16384)."""
+    """A model-sized weight with a ragged N and a last segment past K, on the default route."""
     from tensorplay_amd import ops
     rng = np.random.default_rng(90 + bits)
     N, K, group = 8198, 4160, 32 if bits == 4 else 64
