@@ -424,7 +424,7 @@ int launch_generic(const void* x, const uint8_t* packed, const float* sz, const 
     return check_launch("tpq_lowbit_mm (generic)");
 }
 
-// One activation row (fp16 / bf16), 1, 2 or 4 bits: the packed rows are contiguous, so a wavefront reads them
+// One activation row (fp16 / bf16), 1, 2, 4 or (fp16) 8 bits: the packed rows are contiguous, so a wavefront reads them
 // directly, as the one-row int8 weight-only kernel does.  A pass is 4096 k: lane l owns 64 of them, as TURNS
 // segments of CPL codes (one 16-byte load each; 8 bytes at one bit), and the 128 bytes of activations that go with
 // them, shared by the wavefront's four channels.  Every load is issued before the first use.  Per segment and channel
@@ -438,8 +438,8 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
                                                                   uint16_t* __restrict__ y, int N, int K, int group, int passes, int groups) {
     constexpr int kPerByte = 8 / BITS;
     constexpr int kLoadBytes = BITS == 1 ? 8 : 16;
-    constexpr int kCpl = kLoadBytes * kPerByte;  // codes per load: 64, 64, 32
-    constexpr int kTurns = 64 / kCpl;            // 1, 1, 2
+    constexpr int kCpl = kLoadBytes * kPerByte;  // codes per load: 64, 64, 32, 16 (1, 2, 4, 8 bits)
+    constexpr int kTurns = 64 / kCpl;            // 1, 1, 2, 4
     constexpr int kWords = kLoadBytes / 4;
     __shared__ float red[WAVES][kLbRowChannels];
     const int lane = threadIdx.x & (kWave - 1);
@@ -543,8 +543,10 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
 template <int DT>
 bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t N, int64_t K,
                        int64_t group, int bits, int lsb_first, bool forced, hipStream_t s, int* rc) {
-    if (bits != 1 && bits != 2 && bits != 4) return false;
-    const int cpl = bits == 4 ? 32 : 64;
+    // 8 bits: fp16 only (a byte does not fit the 7 mantissa bits of bfloat16), workgroups of four or eight wavefronts
+    // (four turns of loads per pass: 16 wavefronts would leave 128 registers per lane, too few), so K <= 32768
+    if (bits != 1 && bits != 2 && bits != 4 && !(bits == 8 && DT == TPQ_DTYPE_F16)) return false;
+    const int cpl = bits == 8 ? 16 : bits == 4 ? 32 : 64;
     if (K <= 0 || K % cpl != 0 || group % cpl != 0 || K > 65536 || N > 0x7FFFFFF0) return false;
     // Measured against the matrix-core kernel (us, 1 / 2 / 4 bits): 4096 -> 11008: 7.5 / 8.2 / 8.0 against 9.8 / 10.1 / 10.4;
     // 8192 x 8192: 9.6 / 10.7 / 10.9 against 12.7 / 13.2 / 15.4; 8192 -> 28672: 26.4 / 29.8 / 35.7 against 37.7 / 40.1 / 45.2;
@@ -553,7 +555,9 @@ bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, co
     if (!aligned(x, 16) || !aligned(packed, 16) || !aligned(sz, 8) || !aligned(out, 2)) return false;
     const int passes = static_cast<int>((K + 4095) / 4096);
     // small weights need many workgroups to fill the chip: 4 wavefronts; 16 from 64 MB of packed bytes and for long rows
-    const int waves = (N * (K / (8 / bits)) >= (int64_t{1} << 26) || passes > 4) ? 16 : 4;
+    int waves = (N * (K / (8 / bits)) >= (int64_t{1} << 26) || passes > 4) ? 16 : 4;
+    if (bits == 8 && waves == 16) waves = 8;  // 8 bits: at most eight wavefronts (256 registers per lane)
+    if (waves < passes) return false;
     const int groups = waves / passes;
     const dim3 grid(static_cast<unsigned>((N + groups * kLbRowChannels - 1) / (groups * kLbRowChannels)));
     const auto* xp = static_cast<const uint16_t*>(x);
@@ -562,7 +566,8 @@ bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, co
 #define TPQ_LBROW(B, L, W) lowbit_row_kernel<DT, B, L, W><<<grid, W * kWave, 0, s>>>(xp, packed, sz, bias, yp, n, k, gr, passes, groups)
 #define TPQ_LBROW_W(B, L) do { if (waves == 4) TPQ_LBROW(B, L, 4); else TPQ_LBROW(B, L, 16); } while (0)
 #define TPQ_LBROW_L(B) do { if (lsb_first) TPQ_LBROW_W(B, true); else TPQ_LBROW_W(B, false); } while (0)
-    if (bits == 1) TPQ_LBROW_L(1); else if (bits == 2) TPQ_LBROW_L(2); else TPQ_LBROW_L(4);
+    if (bits == 1) TPQ_LBROW_L(1); else if (bits == 2) TPQ_LBROW_L(2); else if (bits == 4) TPQ_LBROW_L(4);
+    else if constexpr (DT == TPQ_DTYPE_F16) { if (waves == 4) TPQ_LBROW(8, true, 4); else TPQ_LBROW(8, true, 8); }  // one code per byte: the bit order does not matter
 #undef TPQ_LBROW_L
 #undef TPQ_LBROW_W
 #undef TPQ_LBROW

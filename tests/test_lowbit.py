@@ -165,7 +165,7 @@ def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("bits,lsb", [(1, False), (1, True), (2, False), (2, True), (4, False), (4, True)])
+@pytest.mark.parametrize("bits,lsb", [(1, False), (1, True), (2, False), (2, True), (4, False), (4, True), (8, False)])
 @pytest.mark.parametrize("N,K,group", [(10, 4096, 128), (7, 8192, 64), (130, 4160, 32), (5, 20480, 1024), (1, 64, 64), (36, 11008, 128)])
 @pytest.mark.parametrize("tdt,tag,tol", [(torch.float16, "f16", 1e-3), (torch.bfloat16, "bf16", 8e-3)])
 def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatch):
@@ -174,7 +174,7 @@ def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatc
     TPQ_LOWBIT_ROW=1 pins the kernel (it is also the default for these shapes)."""
     from tensorplay_amd import ops
     monkeypatch.setenv("TPQ_LOWBIT_ROW", "1")
-    if group % (32 if bits == 4 else 64):
+    if group % {1: 64, 2: 64, 4: 32, 8: 16}[bits]:
         pytest.skip("the groups of this case are shorter than a lane's segment: other kernel, covered elsewhere")
     rng = np.random.default_rng(bits * 17 + K + N)
     codes, sz = make_case(rng, bits, N, K, group)
