@@ -406,14 +406,15 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     // Channels per workgroup (16 nb) and wavefronts per workgroup, from a sweep over model shapes
     // (K 4096..28672, 2..16 rows).  Every workgroup reads all of x from cache, so many rows want wide
     // workgroups, but only when N still yields enough of them to fill the chip:
-    //   N = 4096:  16 ch x 8 waves always (8 rows: 5.3 us against 6.0 for 32 ch, 8.5 for 64 ch)
-    //   N = 6144, 8192:  32 ch x 8 waves (8192 x 8192, 8 rows: 9.8 us against 13.4 for 16 ch, 14.6 for 64 ch)
+    //   N <= 4096:  16 ch x 8 waves always (8 rows: 5.3 us against 6.0 for 32 ch, 8.5 for 64 ch)
+    //   N = 4097 .. 10239:  32 ch x 8 waves (8192 x 8192, 8 rows: 9.8 us against 13.4 for 16 ch, 14.6 for 64 ch; N = 5120,
+    //                320 workgroups of 16 ch on 256 compute units: 13824 -> 5120 at 8 rows 14.2 us against 21.1, 5120 x 5120 7.4 against 9.9)
     //   N = 10240 .. 28672:  64 ch x 8 waves up to 12 rows (4096 -> 11008: 8.0 / 8.1 / 8.4 / 9.0 us at 2 / 4 / 8 / 12
     //                rows against 8.4 / 8.5 / 9.0 / 9.3 for the next best; 8192 -> 28672, 8 rows: 27.4 against 30.4),
     //                64 ch x 4 waves above (16 rows: 9.7 us against 12.3 for 32 ch)
     //   N > 28672:   32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (4096 -> 32000, 4 rows: 16.2 against 16.6)
     const bool wide = N >= 10240 && N <= 28672 && rows <= 12;
-    int nb = N > 5120 ? (N < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
+    int nb = N > 4096 ? (N < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
     if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
     int waves = N < 10240 || wide ? 8 : 4;
     if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
@@ -507,7 +508,7 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
         const bool wide = n_total >= 10240 && n_total <= 28672 && rows <= 12;
-        const int nb = n_total > 5120 ? (n_total < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
+        const int nb = n_total > 4096 ? (n_total < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
         const int waves = n_total < 10240 || wide ? 8 : 4;
         Int4MultiSet set{};
         set.count = count;

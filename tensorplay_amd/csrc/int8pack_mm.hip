@@ -434,9 +434,10 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
             const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
             const int rows = left < 16 * mb ? left : 16 * mb;
             // Workgroup shape from a sweep over model shapes (K, N = 1024..28672; 1, 8, 16 rows): 16 channels x 8
-            // wavefronts (4096 x 4096, one row: 6.4 us; 2 wavefronts 9.5); 32 channels where N gives whole rounds of
-            // workgroups and from 8 rows on at N >= 16384 (28672 -> 8192, 16 rows: 72 us against 88).
-            const bool wide = (N >= 8192 && N < 10240) || (N >= 16384 && rows >= 8);
+            // wavefronts (4096 x 4096, one row: 6.4 us; 2 wavefronts 9.5); 32 channels for N = 4097 .. 10239, where 16-channel
+            // workgroups would outnumber the compute units by less than two (13824 -> 5120, 8 rows: 28.6 us against 34.6;
+            // 4096 -> 6144, 16 rows: 12.6 against 14.8), and from 8 rows on at N >= 16384 (28672 -> 8192, 16 rows: 72 us against 88).
+            const bool wide = (N > 4096 && N < 10240) || (N >= 16384 && rows >= 8);
             const int nb = forced_nb ? forced_nb : (wide ? 2 : 1);
             const int waves = forced_waves ? forced_waves : (N >= 16384 && !wide ? 4 : 8);
             const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
