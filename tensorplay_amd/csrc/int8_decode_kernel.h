@@ -109,6 +109,108 @@ __global__ __launch_bounds__(WAVES * kWave) void int8_decode_kernel(const int8_t
     }
 }
 
+// One to four activation rows: the weight rows are contiguous, so a wavefront reads them directly.  Lane l owns the
+// 16 k of chunk 64 t + l of its pass (a pass = four such turns = 4096 k): one 16-byte load per turn and channel (1 KB
+// contiguous per wavefront and load) and the 16 bytes of every activation row that go with them, shared by the
+// wavefront's four channels; v_dot4_i32_i8 multiplies.  Every load is issued before the first use, so the whole
+// weight is requested within the first microsecond.  Workgroup = channel groups x passes; the lanes' sums meet by a
+// butterfly, the passes' through LDS; integer sums, so the result does not depend on any of this.
+constexpr int kI8RowChannels = 4, kI8RowTurns = 4;
+
+template <int ROWS, int WAVES, class Epilogue>
+__global__ __launch_bounds__(WAVES * kWave) void int8_row_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ w, int N, int K,
+                                                                int passes, int groups, Epilogue ep) {
+    __shared__ int red[WAVES][kI8RowChannels * ROWS];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = wave / passes, pass = wave - g * passes;
+    const int n0 = (blockIdx.x * groups + g) * kI8RowChannels;
+    const bool active = g < groups && n0 < N;
+    int acc[kI8RowChannels][ROWS];
+#pragma unroll
+    for (int c = 0; c < kI8RowChannels; ++c)
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) acc[c][r] = 0;
+    if (active) {
+        const int chunks = K >> 4;
+        uint4 wv[kI8RowChannels][kI8RowTurns];
+        uint4 xv[ROWS][kI8RowTurns];
+#pragma unroll
+        for (int t = 0; t < kI8RowTurns; ++t) {
+            const int chunk = (pass * kI8RowTurns + t) * kWave + lane;
+            const bool live = chunk < chunks;
+            const int cl = live ? chunk : chunks - 1;  // past the end: a valid chunk, multiplied by zeros
+#pragma unroll
+            for (int c = 0; c < kI8RowChannels; ++c) {
+                const int n = n0 + c < N ? n0 + c : N - 1;
+                wv[c][t] = nt_load(reinterpret_cast<const uint4*>(w + static_cast<size_t>(n) * K) + cl);
+            }
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+                xv[r][t] = live ? reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * K)[cl] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < kI8RowTurns; ++t)
+#pragma unroll
+            for (int c = 0; c < kI8RowChannels; ++c)
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    int a = acc[c][r];
+                    a = __builtin_amdgcn_sdot4(static_cast<int>(xv[r][t].x), static_cast<int>(wv[c][t].x), a, false);
+                    a = __builtin_amdgcn_sdot4(static_cast<int>(xv[r][t].y), static_cast<int>(wv[c][t].y), a, false);
+                    a = __builtin_amdgcn_sdot4(static_cast<int>(xv[r][t].z), static_cast<int>(wv[c][t].z), a, false);
+                    a = __builtin_amdgcn_sdot4(static_cast<int>(xv[r][t].w), static_cast<int>(wv[c][t].w), a, false);
+                    acc[c][r] = a;
+                }
+#pragma unroll
+        for (int c = 0; c < kI8RowChannels; ++c)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[c][r] = wave_sum(acc[c][r]);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int c = 0; c < kI8RowChannels; ++c)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) red[wave][c * ROWS + r] = acc[c][r];
+    }
+    __syncthreads();
+    const int tid = threadIdx.x;
+    if (tid < groups * kI8RowChannels * ROWS) {  // thread = (group, channel, row)
+        const int gg = tid / (kI8RowChannels * ROWS), rem = tid - gg * (kI8RowChannels * ROWS);
+        const int c = rem / ROWS, r = rem - c * ROWS;
+        const int n = (blockIdx.x * groups + gg) * kI8RowChannels + c;
+        if (n < N) {
+            int sum = 0;
+            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][rem];
+            ep.store(static_cast<int64_t>(r) * N + n, r, n, sum);
+        }
+    }
+}
+
+// false if the row kernel does not take the shape (rows of more than 32768 k)
+template <class Epilogue>
+bool launch_int8_rows(const int8_t* a, const int8_t* w, int rows, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
+    const int passes = static_cast<int>((K + 4095) / 4096);
+    // small weights need many workgroups to fill the chip: 4 wavefronts; the largest stream best with 8
+    int waves = N * K >= (int64_t{1} << 27) ? 8 : 4;
+    while (waves < passes) waves *= 2;
+    if (waves > 8) return false;
+    const int groups = waves / passes;
+    const dim3 grid(static_cast<unsigned>((N + groups * kI8RowChannels - 1) / (groups * kI8RowChannels)));
+    const int n = static_cast<int>(N), k = static_cast<int>(K);
+#define TPQ_I8ROW(R, WV) int8_row_kernel<R, WV, Epilogue><<<grid, WV * kWave, 0, s>>>(a, w, n, k, passes, groups, ep)
+#define TPQ_I8ROW_W(R) do { if (waves == 4) TPQ_I8ROW(R, 4); else TPQ_I8ROW(R, 8); } while (0)
+    switch (rows) {
+        case 1: TPQ_I8ROW_W(1); break;
+        case 2: TPQ_I8ROW_W(2); break;
+        case 3: TPQ_I8ROW_W(3); break;
+        default: TPQ_I8ROW_W(4); break;
+    }
+#undef TPQ_I8ROW_W
+#undef TPQ_I8ROW
+    return true;
+}
+
 inline bool int8_decode_ok(const void* a, const void* w, int64_t M, int64_t N, int64_t K) {
     return M >= 1 && K >= 128 && K % 128 == 0 && aligned(a, 16) && aligned(w, 16) && N <= 0x7FFFFFF0 && K <= 0x7FFFFF80;
 }
@@ -119,6 +221,14 @@ int launch_int8_decode(const int8_t* a, const int8_t* w, int64_t M, int64_t N, i
     static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT8_DECODE_NB"); return e ? std::atoi(e) : 0; }();
     static const int forced_mb = [] { const char* e = std::getenv("TPQ_INT8_DECODE_MB"); return e ? std::atoi(e) : 0; }();
     static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT8_DECODE_WAVES"); return e ? std::atoi(e) : 0; }();
+    // One or two rows: the row kernel.  Measured against the matrix-core kernel below (us, one row): 4096 x 4096 5.3 / 5.6,
+    // 11008 -> 4096 9.8 / 13.6, 4096 -> 11008 10.0 / 12.6, 8192 x 8192 13.5 / 16.2, 8192 -> 28672 38.1 / 46.2, 28672 -> 8192
+    // 36.9 / 51.2 (6.4 TB/s); two rows: 10.5 / 13.4, 10.4 / 11.4, 14.5 / 16.3, 38.8 / 47.1, 38.3 / 52.6.  At four rows
+    // the two are even (4096 x 4096: 6.8 / 5.9; 8192 x 8192: 15.8 / 17.4; 8192 -> 28672: 53.6 / 50.5) and the matrix-core
+    // kernel stays.  TPQ_INT8_ROW=0 / 1: never / up to four rows, for comparison runs and tests.
+    const char* row_env = M <= 4 ? std::getenv("TPQ_INT8_ROW") : nullptr;
+    const int row_limit = row_env ? (row_env[0] == '0' ? 0 : 4) : 2;
+    if (M <= row_limit && launch_int8_rows(a, w, static_cast<int>(M), N, K, ep, s)) return check_launch("int8 row gemm");
     const int steps = static_cast<int>(K / 128);
     const int n = static_cast<int>(N), k = static_cast<int>(K);
     for (int64_t m0 = 0; m0 < M;) {

@@ -27,7 +27,10 @@ SHAPES = [(5, 7, 3), (1, 1, 1), (64, 12, 32), (16, 1024, 1024), (64, 128, 32), (
           (1, 128, 40), (17, 256, 24), (48, 384, 72), (33, 4096, 100), (7, 11008, 64),
           (64, 256, 6150), (49, 128, 8200), (8, 384, 16400), (31, 256, 6144), (16, 128, 9000), (64, 512, 17),
           # tiled kernel with the k range in slices (few tiles, long K), ragged last slice
-          (130, 1024, 200), (300, 2048, 136), (65, 1152, 64), (257, 1280, 100), (33, 1024, 10248)]
+          (130, 1024, 200), (300, 2048, 136), (65, 1152, 64), (257, 1280, 100), (33, 1024, 10248),
+          # one or two rows on the row kernel: a last chunk past K, several passes per channel, ragged N, the long rows
+          # that fall back to the matrix-core kernel (more than 32768 k), and 3 / 4 rows (that kernel by default)
+          (2, 4224, 10), (1, 20480, 13), (2, 32768, 9), (1, 36864, 8), (2, 4096, 8200), (1, 8192, 16390), (3, 4096, 50), (4, 256, 7)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -126,6 +129,26 @@ def test_fused_dequant_bit_exact(ops, out_dtype, shape, with_bias):
     want = oracle.int8_mm_rescale(acc, xs, ws, bias=bias, out_dtype=out_dtype)
     got = ops.int8_mm_dequant(dev(xq), dev(wq), dev(xs), dev(ws), None if bias is None else dev(bias), TORCH_DT[out_dtype])
     np.testing.assert_array_equal(host(got), want)
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("K,N", [(4224, 50), (12288, 7), (256, 4100)])
+def test_row_kernel_one_to_four_rows(ops, M, K, N, monkeypatch):
+    """The kernel that streams the weight rows, for 1..4 activation rows (3 and 4 are not its default): raw sums exact,
+    fused dequant equal to the oracle bit for bit in float32 and bfloat16, with a bias."""
+    monkeypatch.setenv("TPQ_INT8_ROW", "1")
+    rng = np.random.default_rng(M * 5 + K + N)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    w = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    bias = rng.normal(0, 0.01, N).astype(np.float32)
+    xq, xs = oracle.quantize_int8_rowwise(x)
+    wq, ws = oracle.quantize_int8_rowwise(w)
+    acc = xq.astype(np.int32) @ wq.astype(np.int32).T
+    np.testing.assert_array_equal(host(ops._int_mm(dev(xq), dev(wq).t())), acc)
+    for out_dtype, tdt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        want = oracle.int8_mm_rescale(acc, xs, ws, bias=bias, out_dtype=out_dtype)
+        got = ops.int8_mm_dequant(dev(xq), dev(wq), dev(xs), dev(ws), dev(bias), tdt)
+        np.testing.assert_array_equal(host(got), want)
 
 
 def test_dynamic_int8_linear_config1_end_to_end(ops):
