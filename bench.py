@@ -468,10 +468,10 @@ def main() -> int:
         fused_chk = ((acc_chk.float() * a_s[:64, None]) * w_s[None, :]).bfloat16()
         extras["int8_gemm_rows_checked_equal"] = bool(torch.equal(fused_chk, out8[:64]))
 
-        # the same product for decode batches and short prompts (16 / 128 rows): the decode kernel, and the tiled
+        # the same product for decode batches and short prompts (1 / 16 / 128 rows): the row kernel, the decode kernel, and the tiled
         # kernel with its k range in slices (workspace entry point), weights rotating through 30 copies (0.5 GB)
         w_rot = [w_q.clone() for _ in range(30)]
-        for m_small in (16, 128):
+        for m_small in (1, 16, 128):
             a_small, s_small = a_q[:m_small].contiguous(), a_s[:m_small].contiguous()
             out_small = torch.empty((m_small, N8), dtype=torch.bfloat16, device=dev)
             ws_bytes = int(lib.tpq_int8_mm_workspace_bytes(m_small, N8, K8))
