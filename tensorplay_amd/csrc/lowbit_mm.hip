@@ -430,12 +430,15 @@ int launch_generic(const void* x, const uint8_t* packed, const float* sz, const 
 // them, shared by the wavefront's four channels.  Every load is issued before the first use.  Per segment and channel
 // y += scale (sum code x - zero sum x), a segment lying inside one group; three vector instructions per pair of codes.
 // Workgroup = channel groups x passes; the lanes' sums meet by a butterfly, the passes' through LDS.
-constexpr int kLbRowChannels = 4;
+// CH channels per wavefront share a lane's 128 bytes of activations: 8 for large weights at 1 and 2 bits, where the
+// activations re-read per wavefront would otherwise outweigh the packed bytes (8192 -> 28672 at 1 bit: 26.4 -> 21.9 us);
+// 4 for small weights, which need the wavefronts (4096 x 4096 at 1 bit: 4.8 us against 6.0 with 8).
 
-template <int DT, int BITS, bool LSB, int WAVES>
+template <int DT, int BITS, bool LSB, int WAVES, int CH>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed,
                                                                   const float* __restrict__ sz, const float* __restrict__ bias,
                                                                   uint16_t* __restrict__ y, int N, int K, int group, int passes, int groups) {
+    constexpr int kLbRowChannels = CH;
     constexpr int kPerByte = 8 / BITS;
     constexpr int kLoadBytes = BITS == 1 ? 8 : 16;
     constexpr int kCpl = kLoadBytes * kPerByte;  // codes per load: 64, 64, 32, 16 (1, 2, 4, 8 bits)
@@ -447,7 +450,9 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
     const int g = wave / passes, pass = wave - g * passes;
     const int n0 = (blockIdx.x * groups + g) * kLbRowChannels;
     const bool active = g < groups && n0 < N;
-    float acc[kLbRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float acc[kLbRowChannels];
+#pragma unroll
+    for (int c = 0; c < kLbRowChannels; ++c) acc[c] = 0.0f;
     if (active) {
         const size_t pitch = static_cast<size_t>(K) / kPerByte;
         uint32_t wv[kLbRowChannels][kTurns][kWords];
@@ -500,7 +505,9 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
             float sx = 0.0f;
 #pragma unroll
             for (int e = 0; e < kCpl; e += 2) sx = L::dot(half_of(e) | (half_of(e + 1) << 16), L::kOnes, sx);
-            float s[kLbRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float s[kLbRowChannels];
+#pragma unroll
+            for (int c = 0; c < kLbRowChannels; ++c) s[c] = 0.0f;
 #pragma unroll
             for (int w = 0; w < kWords; ++w)
 #pragma unroll
@@ -524,7 +531,10 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
 #pragma unroll
         for (int c = 0; c < kLbRowChannels; ++c) acc[c] = wave_sum(acc[c]);
     }
-    if (lane < kLbRowChannels) red[wave][lane] = lane == 0 ? acc[0] : lane == 1 ? acc[1] : lane == 2 ? acc[2] : acc[3];
+    if (lane == 0) {
+#pragma unroll
+        for (int c = 0; c < kLbRowChannels; ++c) red[wave][c] = acc[c];
+    }
     __syncthreads();
     const int tid = threadIdx.x;
     if (tid < groups * kLbRowChannels) {  // thread = (group, channel): the passes in order
@@ -558,12 +568,13 @@ bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, co
     int waves = (N * (K / (8 / bits)) >= (int64_t{1} << 26) || passes > 4) ? 16 : 4;
     if (bits == 8 && waves == 16) waves = 8;  // 8 bits: at most eight wavefronts (256 registers per lane)
     if (waves < passes) return false;
-    const int groups = waves / passes;
-    const dim3 grid(static_cast<unsigned>((N + groups * kLbRowChannels - 1) / (groups * kLbRowChannels)));
+    const int groups = waves / passes, channels = (bits <= 2 && N * K >= (int64_t{1} << 26)) ? 8 : 4;
+    const dim3 grid(static_cast<unsigned>((N + groups * channels - 1) / (groups * channels)));
     const auto* xp = static_cast<const uint16_t*>(x);
     auto* yp = static_cast<uint16_t*>(out);
     const int n = static_cast<int>(N), k = static_cast<int>(K), gr = static_cast<int>(group);
-#define TPQ_LBROW(B, L, W) lowbit_row_kernel<DT, B, L, W><<<grid, W * kWave, 0, s>>>(xp, packed, sz, bias, yp, n, k, gr, passes, groups)
+#define TPQ_LBROW_C(B, L, W, C) lowbit_row_kernel<DT, B, L, W, C><<<grid, W * kWave, 0, s>>>(xp, packed, sz, bias, yp, n, k, gr, passes, groups)
+#define TPQ_LBROW(B, L, W) do { if (B <= 2 && channels == 8) TPQ_LBROW_C(B, L, W, (B <= 2 ? 8 : 4)); else TPQ_LBROW_C(B, L, W, 4); } while (0)
 #define TPQ_LBROW_W(B, L) do { if (waves == 4) TPQ_LBROW(B, L, 4); else TPQ_LBROW(B, L, 16); } while (0)
 #define TPQ_LBROW_L(B) do { if (lsb_first) TPQ_LBROW_W(B, true); else TPQ_LBROW_W(B, false); } while (0)
     if (bits == 1) TPQ_LBROW_L(1); else if (bits == 2) TPQ_LBROW_L(2); else if (bits == 4) TPQ_LBROW_L(4);
@@ -571,6 +582,7 @@ bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, co
 #undef TPQ_LBROW_L
 #undef TPQ_LBROW_W
 #undef TPQ_LBROW
+#undef TPQ_LBROW_C
     *rc = check_launch("tpq_lowbit_mm (row)");
     return true;
 }

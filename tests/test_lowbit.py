@@ -190,12 +190,13 @@ def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatc
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("bits", [1, 2, 4])
-def test_gpu_mm_one_row_default_route_large_weight(bits):
-    """A model-sized weight with a ragged N and a last segment past K, on the default route."""
+@pytest.mark.parametrize("bits,N,K", [(1, 8198, 4160), (2, 8198, 4160), (4, 8198, 4160), (1, 8198, 8192), (2, 4100, 16448)])
+def test_gpu_mm_one_row_default_route_large_weight(bits, N, K):
+    """Model-sized weights with a ragged N and a last segment past K, on the default route: four channels per wavefront,
+    and eight for 1 and 2 bits from 2^26 codes on (the last two shapes)."""
     from tensorplay_amd import ops
     rng = np.random.default_rng(90 + bits)
-    N, K, group = 8198, 4160, 32 if bits == 4 else 64
+    group = 32 if bits == 4 else 64
     codes, sz = make_case(rng, bits, N, K, group)
     x16 = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).half()
     packed = oracle.lowbit_pack(codes, bits)
