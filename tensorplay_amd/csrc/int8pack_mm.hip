@@ -161,7 +161,8 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
     }
 }
 
-// One activation row (fp16 / bf16, K % 16 == 0, K <= 65536): the weight rows are contiguous, so a wavefront reads a
+// One or two activation rows (fp16 / bf16, K % 16 == 0, K <= 65536; two rows: K <= 32768, at most eight wavefronts):
+// the weight rows are contiguous, so a wavefront reads a
 // row's bytes directly: lane l owns the 16 k of chunk 64 t + l of its pass (a pass = four such turns = 4096 k), one
 // 16-byte load per turn and channel, 1 KB contiguous per wavefront and load, and the 32 bytes of activations that go
 // with them, shared by the wavefront's four channels.  Every load of a wavefront is issued before the first use, so
@@ -170,21 +171,25 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
 // fp16: bytes -> fp16 pairs as in the kernel above, v_dot2_f32_f16; bf16: both operands widened to fp32, fma.
 constexpr int kRowChannels = 4, kRowTurns = 4;
 
-template <int DT, int kRowWaves>
+template <int DT, int kRowWaves, int ROWS>
 __global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const uint16_t* __restrict__ x, const int8_t* __restrict__ w,
                                                                         const float* __restrict__ scale, uint16_t* __restrict__ y,
                                                                         int N, int K, int passes, int groups) {
-    __shared__ float red[kRowWaves][kRowChannels];
+    __shared__ float red[kRowWaves][kRowChannels * ROWS];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = wave / passes, pass = wave - g * passes;
     const int n0 = (blockIdx.x * groups + g) * kRowChannels;
     const bool active = g < groups && n0 < N;
-    float acc[kRowChannels] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float acc[kRowChannels][ROWS];
+#pragma unroll
+    for (int c = 0; c < kRowChannels; ++c)
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) acc[c][r] = 0.0f;
     if (active) {
         const int chunks = K >> 4;
         uint4 wv[kRowChannels][kRowTurns];
-        uint4 xv[kRowTurns][2];
+        uint4 xv[ROWS][kRowTurns][2];
         bool live[kRowTurns];
 #pragma unroll
         for (int t = 0; t < kRowTurns; ++t) {
@@ -196,9 +201,12 @@ __global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const u
                 const int n = n0 + c < N ? n0 + c : N - 1;
                 wv[c][t] = nt_load(reinterpret_cast<const uint4*>(w + static_cast<size_t>(n) * K) + cl);
             }
-            const uint4* xp = reinterpret_cast<const uint4*>(x) + 2 * cl;
-            xv[t][0] = live[t] ? xp[0] : make_uint4(0, 0, 0, 0);
-            xv[t][1] = live[t] ? xp[1] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const uint4* xp = reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * K) + 2 * cl;
+                xv[r][t][0] = live[t] ? xp[0] : make_uint4(0, 0, 0, 0);
+                xv[r][t][1] = live[t] ? xp[1] : make_uint4(0, 0, 0, 0);
+            }
         }
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         const h2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
@@ -206,7 +214,6 @@ __global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const u
         asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(0x64646464u));
 #pragma unroll
         for (int t = 0; t < kRowTurns; ++t) {
-            const uint32_t xw[8] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w, xv[t][1].x, xv[t][1].y, xv[t][1].z, xv[t][1].w};
 #pragma unroll
             for (int c = 0; c < kRowChannels; ++c) {
 #pragma unroll
@@ -214,34 +221,52 @@ __global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const u
                     const uint32_t word = dword_at(wv[c][t], j);
                     if constexpr (DT == TPQ_DTYPE_F16) {
                         const uint32_t u = word ^ 0x80808080u;
-                        const uint32_t lo = __builtin_amdgcn_perm(magic, u, 0x04010400u);  // (1152 + b0, 1152 + b1)
-                        const uint32_t hi = __builtin_amdgcn_perm(magic, u, 0x04030402u);  // (1152 + b2, 1152 + b3)
-                        acc[c] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xw[2 * j]), __builtin_bit_cast(h2, lo) - bias, acc[c], false);
-                        acc[c] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, xw[2 * j + 1]), __builtin_bit_cast(h2, hi) - bias, acc[c], false);
+                        const h2 lo = __builtin_bit_cast(h2, __builtin_amdgcn_perm(magic, u, 0x04010400u)) - bias;  // (b0, b1)
+                        const h2 hi = __builtin_bit_cast(h2, __builtin_amdgcn_perm(magic, u, 0x04030402u)) - bias;  // (b2, b3)
+#pragma unroll
+                        for (int r = 0; r < ROWS; ++r) {
+                            const uint4& xq = xv[r][t][j >> 1];
+                            const uint32_t x0 = (j & 1) ? xq.z : xq.x, x1 = (j & 1) ? xq.w : xq.y;
+                            acc[c][r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, x0), lo, acc[c][r], false);
+                            acc[c][r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, x1), hi, acc[c][r], false);
+                        }
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const uint32_t xp2 = xw[2 * j + (e >> 1)];
-                            const float xf = __builtin_bit_cast(float, (e & 1) ? (xp2 & 0xFFFF0000u) : (xp2 << 16));
-                            acc[c] = __builtin_fmaf(xf, static_cast<float>(static_cast<int8_t>(word >> (8 * e))), acc[c]);
+                            const float wf = static_cast<float>(static_cast<int8_t>(word >> (8 * e)));
+#pragma unroll
+                            for (int r = 0; r < ROWS; ++r) {
+                                const uint4& xq = xv[r][t][j >> 1];
+                                const uint32_t xp2 = (j & 1) ? ((e >> 1) ? xq.w : xq.z) : ((e >> 1) ? xq.y : xq.x);
+                                const float xf = __builtin_bit_cast(float, (e & 1) ? (xp2 & 0xFFFF0000u) : (xp2 << 16));
+                                acc[c][r] = __builtin_fmaf(xf, wf, acc[c][r]);
+                            }
                         }
                     }
                 }
             }
         }
 #pragma unroll
-        for (int c = 0; c < kRowChannels; ++c) acc[c] = wave_sum(acc[c]);
+        for (int c = 0; c < kRowChannels; ++c)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[c][r] = wave_sum(acc[c][r]);
     }
-    if (lane < kRowChannels) red[wave][lane] = lane == 0 ? acc[0] : lane == 1 ? acc[1] : lane == 2 ? acc[2] : acc[3];
+    if (lane == 0) {
+#pragma unroll
+        for (int c = 0; c < kRowChannels; ++c)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) red[wave][c * ROWS + r] = acc[c][r];
+    }
     __syncthreads();
     const int tid = threadIdx.x;
-    if (tid < groups * kRowChannels) {  // thread = (group, channel): the passes in order
-        const int gg = tid / kRowChannels, c = tid - gg * kRowChannels;
+    if (tid < groups * kRowChannels * ROWS) {  // thread = (group, channel, row): the passes in order
+        const int gg = tid / (kRowChannels * ROWS), rem = tid - gg * (kRowChannels * ROWS);
+        const int c = rem / ROWS, r = rem - c * ROWS;
         const int n = (blockIdx.x * groups + gg) * kRowChannels + c;
         if (n < N) {
             float sum = 0.0f;
-            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][c];
-            y[n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
+            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][rem];
+            y[static_cast<size_t>(r) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
         }
     }
 }
@@ -410,19 +435,22 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
     // TPQ_INT8PACK_ROW_WAVES the workgroup size for comparison runs.
     static const int forced_row = [] { const char* e = std::getenv("TPQ_INT8PACK_ROW"); return e ? std::atoi(e) : -1; }();
     static const int forced_row_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_ROW_WAVES"); return e ? std::atoi(e) : 0; }();
-    if (M == 1 && dtype != TPQ_DTYPE_F32 && K % 16 == 0 && K <= 65536 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16) && forced_row != 0) {
+    if (M <= 2 && dtype != TPQ_DTYPE_F32 && K % 16 == 0 && K <= (M == 1 ? 65536 : 32768) && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16) && forced_row != 0) {
         const int passes = static_cast<int>((K + 4095) / 4096);
         int waves = N * K >= (int64_t{1} << 27) ? 8 : N * K >= (int64_t{1} << 26) ? 16 : 4;
         if (forced_row_waves == 4 || forced_row_waves == 8 || forced_row_waves == 16) waves = forced_row_waves;
+        if (M == 2 && waves == 16) waves = 8;  // two rows: 64 more registers of activations per lane
         while (waves < passes) waves *= 2;  // a workgroup holds all passes of its channels
         const int groups = waves / passes;
         const dim3 grid(static_cast<unsigned>((N + groups * kRowChannels - 1) / (groups * kRowChannels)));
         const auto* xp = static_cast<const uint16_t*>(x);
         auto* yp = static_cast<uint16_t*>(out);
-#define TPQ_I8ROW(DTV, WV) int8pack_row_kernel<DTV, WV><<<grid, WV * kWave, 0, s>>>(xp, w, scales, yp, (int)N, (int)K, passes, groups)
+#define TPQ_I8ROW_R(DTV, WV, RV) int8pack_row_kernel<DTV, WV, RV><<<grid, WV * kWave, 0, s>>>(xp, w, scales, yp, (int)N, (int)K, passes, groups)
+#define TPQ_I8ROW(DTV, WV) do { if (M == 1) TPQ_I8ROW_R(DTV, WV, 1); else if (WV <= 8) TPQ_I8ROW_R(DTV, WV, (WV <= 8 ? 2 : 1)); } while (0)
         if (dtype == TPQ_DTYPE_F16) { if (waves == 4) TPQ_I8ROW(TPQ_DTYPE_F16, 4); else if (waves == 8) TPQ_I8ROW(TPQ_DTYPE_F16, 8); else TPQ_I8ROW(TPQ_DTYPE_F16, 16); }
         else { if (waves == 4) TPQ_I8ROW(TPQ_DTYPE_BF16, 4); else if (waves == 8) TPQ_I8ROW(TPQ_DTYPE_BF16, 8); else TPQ_I8ROW(TPQ_DTYPE_BF16, 16); }
 #undef TPQ_I8ROW
+#undef TPQ_I8ROW_R
         return check_launch("_weight_int8pack_mm (row)");
     }
     if (dtype != TPQ_DTYPE_F32 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {

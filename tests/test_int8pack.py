@@ -35,7 +35,9 @@ CASES = [(1, 4096, 512), (4, 1024, 136), (16, 256, 40), (17, 384, 72), (2, 100, 
          (32, 256, 8200), (64, 128, 50), (9, 128, 16390), (3, 256, 16400), (24, 384, 10250), (40, 128, 10240),
          # one row through the row kernel: a last turn that is partly past K, several passes per channel, ragged N,
          # the three workgroup sizes (by N K), K of 16 only
-         (1, 4112, 10), (1, 16, 7), (1, 28672, 130), (1, 8192, 8200), (1, 4096, 32772), (1, 65536, 12), (1, 48, 1)]
+         (1, 4112, 10), (1, 16, 7), (1, 28672, 130), (1, 8192, 8200), (1, 4096, 32772), (1, 65536, 12), (1, 48, 1),
+         # two rows on the same kernel (K up to 32768; longer rows take the matrix-core kernel)
+         (2, 4112, 10), (2, 32, 5), (2, 28672, 130), (2, 8192, 8200), (2, 4096, 32772), (2, 36864, 12)]
 
 
 @pytest.mark.gpu
