@@ -106,6 +106,22 @@ int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const float* row_sc
                            void* stream);
 
 /*
+ * tpq_int8_mm_dequant_ws without the workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The slice matrices live in a buffer built into the library, tpq_int8_mm_noalloc_max_bytes()
+ * (16 MiB) per GPU, held until the process ends; the call allocates and frees nothing.  A shape whose slices
+ * need more (tpq_int8_mm_workspace_bytes(M, N, K) above the maximum, e.g. 512 x 4096 x 4096) is rejected with
+ * TPQ_ERR_INVALID_VALUE and belongs to tpq_int8_mm_dequant_ws;
+ * a shape that uses no workspace runs as tpq_int8_mm_dequant.  Same result bits as tpq_int8_mm_dequant(_ws).
+ * All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (two streams, two
+ * threads) race; order them on one stream or with events.
+ */
+int64_t tpq_int8_mm_noalloc_max_bytes(void);
+int tpq_int8_mm_dequant_noalloc(const int8_t* a, const int8_t* w, const float* row_scale,
+                                const float* col_scale, const float* bias, void* out, int out_dtype,
+                                int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
  * int32 codes [N,K] in 0..15 -> int32 [ceil(N/8)][ceil(K/(16 I))][32][I/2],
  * the packed layout of the reference's device op (I = inner_k_tiles in {2,4,8}).
  * Replaces _convert_weight_to_int4pack: config/native_functions.yaml:7991,

@@ -27,6 +27,8 @@ SIGNATURES = {
     "tpq_int8_mm_workspace_bytes": [_i64, _i64, _i64],
     "tpq_int_mm_ws": [_ptr, _int, _ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr],
     "tpq_int8_mm_dequant_ws": [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _i64, _ptr],
+    "tpq_int8_mm_noalloc_max_bytes": [],
+    "tpq_int8_mm_dequant_noalloc": [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _ptr],
     "tpq_int4_pack": [_ptr, _i64, _i64, _int, _ptr, _ptr],
     "tpq_int4_mm": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr],
     "tpq_int4_mm_ws": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, ctypes.c_size_t, _ptr],

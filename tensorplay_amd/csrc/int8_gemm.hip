@@ -144,6 +144,29 @@ int launch_generic(const void* a, int a_unsigned, const int8_t* b, int64_t sbk, 
     return check_launch("_int_mm generic");
 }
 
+// Scratch of the allocation-free entry point: one copy per GPU, held until the process ends.
+constexpr int64_t kNoAllocScratchBytes = int64_t{16} << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+// Device address of this GPU's copy of `scratch`.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: each GPU has its own copy at its own address, looked up once per device.
+int noalloc_scratch(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void*> per_device[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(TPQ_ERR_RUNTIME, "int8_mm_dequant_noalloc: no current device");
+    TPQ_REQUIRE(dev >= 0 && dev < kMaxDevices, TPQ_ERR_RUNTIME, "int8_mm_dequant_noalloc: device id %d out of range", dev);
+    void* p = per_device[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(TPQ_ERR_RUNTIME, "int8_mm_dequant_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        per_device[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return TPQ_OK;
+}
+
 }  // namespace
 }  // namespace tpq
 
@@ -239,4 +262,21 @@ TPQ_EXPORT int tpq_int_mm_ws(const void* a, int a_unsigned, const int8_t* b, int
     const int64_t blocks = (M * N / 4 + 255) / 256;
     int32_sum_slices_kernel<<<static_cast<unsigned>(blocks > 4096 ? 4096 : blocks), 256, 0, s>>>(partial, slices, c, M * N);
     return check_launch("_int_mm (sum of slices)");
+}
+
+TPQ_EXPORT int64_t tpq_int8_mm_noalloc_max_bytes(void) { return kNoAllocScratchBytes; }
+
+TPQ_EXPORT int tpq_int8_mm_dequant_noalloc(const int8_t* a, const int8_t* w, const float* row_scale, const float* col_scale,
+                                           const float* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                           void* stream) {
+    const int64_t need = tpq_int8_mm_workspace_bytes(M, N, K);
+    TPQ_REQUIRE(need <= kNoAllocScratchBytes, TPQ_ERR_INVALID_VALUE,
+                "int8_mm_dequant_noalloc: %lld x %lld x %lld needs %lld bytes of scratch, the built-in buffer holds %lld",
+                static_cast<long long>(M), static_cast<long long>(N), static_cast<long long>(K), static_cast<long long>(need),
+                static_cast<long long>(kNoAllocScratchBytes));
+    if (need == 0) return tpq_int8_mm_dequant(a, w, row_scale, col_scale, bias, out, out_dtype, M, N, K, stream);
+    void* ws = nullptr;
+    if (int rc = noalloc_scratch(&ws)) return rc;
+    // every slice matrix is written in full before the finishing kernel reads it: nothing to clear between calls
+    return tpq_int8_mm_dequant_ws(a, w, row_scale, col_scale, bias, out, out_dtype, M, N, K, ws, kNoAllocScratchBytes, stream);
 }
