@@ -41,6 +41,15 @@ int tpq_abi_version(void);
 const char* tpq_last_error(void);
 
 /*
+ * Which kernel serves a call is a function of the call's arguments alone; the library never reads the environment.
+ * Two routes can be pinned for comparison runs and tests (no counterpart in the reference; results are bit-identical
+ * on either side of both): "int8_row" (0: the int8 row-streaming kernel never runs, 1: it takes up to four
+ * activation rows instead of two) and "lowbit_row" (0: the packed n-bit row kernel never runs, 1: it runs wherever
+ * the shape allows).  value -1 restores the default rule.  Process-wide, atomic.
+ */
+int tpq_set_kernel_override(const char* route, int value);
+
+/*
  * Fused row-wise signed quantizer.
  *   absmax = max_k |x[m,k]|; scale = max(absmax, eps) / divisor;
  *   code = clamp(rint(x / scale), qmin, qmax)   (sign_mode: x >= 0 ? qmax : qmin)

@@ -829,7 +829,8 @@ ORC_API void orc_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, i
  * _binary_mm (binary.py:88-95) is the case bits = 1, lsb_first, one group, scale' = 2 scale, zero = 0.5:
  * (bit - 0.5) * 2 s = (2 bit - 1) * s exactly.
  * Pinned by: numpy float64 x @ dq.T with dq from the closed form on independently unpacked codes; the
- * reference test's own check (test_int2_binary_modules.py:69-89, 140-155) restated in numpy.
+ * reference test's own check (test_int2_binary_modules.py:69-89, 140-155) restated in numpy; at 8 bits the
+ * reference's unpack -> int8 -> float chain written out in numpy on bytes of 128 and more.
  */
 ORC_API void orc_lowbit_mm(const void* x, int dtype, const uint8_t* packed, int bits, int lsb_first, const float* sz,
                            const float* bias, int64_t M, int64_t N, int64_t K, int64_t group, void* out, double* y64,
@@ -843,7 +844,9 @@ ORC_API void orc_lowbit_mm(const void* x, int dtype, const uint8_t* packed, int 
             for (int64_t k = 0; k < K; ++k) {
                 const int code = (packed[n * pitch + k / per_byte] >> lowbit_shift((int)(k % per_byte), bits, lsb_first)) & ((1 << bits) - 1);
                 const float* p = sz + ((k / group) * N + n) * 2;
-                const float dq = ((float)code - p[1]) * p[0];
+                /* unpack_intx ends in codes.to(int8) (intx_weight_only.py:80) and _dequantize_intx converts that int8
+                 * to float (:119): at 8 bits a byte of 128 or more counts as byte - 256 */
+                const float dq = ((float)(bits == 8 ? (int)(int8_t)code : code) - p[1]) * p[0];
                 if (dense && m == 0) dense[n * K + k] = dq;
                 if (M > 0) {
                     const float xv = load_as_f32(x, dtype, m * K + k);

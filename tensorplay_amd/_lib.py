@@ -20,6 +20,7 @@ _i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_
 # name -> argument types, in the order of include/tpq.h
 SIGNATURES = {
     "tpq_abi_version": [],
+    "tpq_set_kernel_override": [ctypes.c_char_p, _int],
     "tpq_quantize_rowwise": [_ptr, _int, _i64, _i64, _f32, _f32, _int, _int, _int, _ptr, _ptr, _ptr],
     "tpq_int_mm": [_ptr, _int, _ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr],
     "tpq_int8_mm_rescale": [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr],

@@ -72,7 +72,8 @@ class WeightOnlyBinaryLinear(nn.Module):
         if linear.bias is not None and linear.bias.dim() != 1:
             raise ValueError("binary weight-only requires a 1-D bias or no bias")
         w = linear.weight.detach()
-        sign_bits, scale = _quantize_binary_weight(w.float())
+        sign_bits, scale = _quantize_binary_weight(w)  # in the weight's own dtype, as the reference does (:151)
+        scale = scale.float()
         mod = cls(linear.in_features, linear.out_features, bias=linear.bias is not None, cache_unpacked=cache_unpacked,
                   device=w.device)
         mod.weight = pack_binary(sign_bits)

@@ -52,7 +52,12 @@ def bitnet_linear_packed(input: torch.Tensor, packed: torch.Tensor, scale: Union
 
 
 class BitNetPacked2bitLinear(nn.Module):
-    """Inference module over a 2-bit packed ternary weight (reference _BitNetPacked2bitLinear :528-547)."""
+    """Inference module over a 2-bit packed ternary weight (reference _BitNetPacked2bitLinear :528-547).
+
+    State: ``int_data`` (uint8 [N, ceil(K/4)]) and ``scale`` (0-dim, the weight's dtype), the two inner tensors the
+    reference's packed weight subclass flattens to (``BitNetPacked2bitLinearWeight.__tensor_flatten__``, :478-486),
+    plus ``bias``.  load_state_dict also takes ``weight`` holding such a subclass instance (anything with
+    ``int_data`` and ``scale`` attributes) or a dict of the two, which is what a reference model's ``weight`` entry is."""
 
     def __init__(self, packed: torch.Tensor, scale: Union[torch.Tensor, float], in_features: int,
                  bias: Optional[torch.Tensor] = None, eps: float = 1e-5):
@@ -61,11 +66,36 @@ class BitNetPacked2bitLinear(nn.Module):
         self.out_features = packed.shape[0]
         self.eps = eps
         self.register_buffer("int_data", packed)
-        self.scale = float(scale)
+        scale_t = scale.detach().reshape(()) if isinstance(scale, torch.Tensor) else torch.tensor(float(scale), dtype=torch.float32)
+        self.register_buffer("scale", scale_t.to(packed.device))
+        self._scale_value = float(scale_t)   # host copy: the kernel takes the scale by value, no sync per forward
         if bias is not None:
             self.register_buffer("bias", bias)
         else:
             self.bias = None
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        wkey = prefix + "weight"
+        if wkey in state_dict:   # the reference's flattened subclass: weight -> (int_data, scale)
+            w = state_dict[wkey]
+            inner = w if isinstance(w, dict) else {"int_data": getattr(w, "int_data", None), "scale": getattr(w, "scale", None)}
+            if isinstance(inner.get("int_data"), torch.Tensor) and isinstance(inner.get("scale"), torch.Tensor):
+                state_dict = {k: v for k, v in state_dict.items() if k != wkey}
+                state_dict[prefix + "int_data"] = inner["int_data"]
+                state_dict[prefix + "scale"] = inner["scale"].reshape(())
+            else:
+                error_msgs.append(f"{wkey}: expected a packed BitNet weight with int_data and scale")
+        skey = prefix + "scale"
+        if isinstance(state_dict.get(skey), torch.Tensor) and state_dict[skey].numel() == 1:
+            state_dict = dict(state_dict)
+            state_dict[skey] = state_dict[skey].reshape(())
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+        self._scale_value = float(self.scale)
+
+    def _apply(self, fn, recurse=True):
+        super()._apply(fn, recurse)
+        self._scale_value = float(self.scale)   # a dtype change rounds the scale
+        return self
 
     @classmethod
     def from_float(cls, linear: nn.Linear, eps: float = 1e-5) -> "BitNetPacked2bitLinear":
@@ -74,4 +104,4 @@ class BitNetPacked2bitLinear(nn.Module):
         return cls(pack_ternary(codes), scale, linear.in_features, bias, eps)
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return bitnet_linear_packed(input, self.int_data, self.scale, self.in_features, self.bias, self.eps)
+        return bitnet_linear_packed(input, self.int_data, self._scale_value, self.in_features, self.bias, self.eps)

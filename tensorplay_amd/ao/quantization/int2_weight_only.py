@@ -86,7 +86,9 @@ class WeightOnlyInt2Linear(nn.Module):
         if linear.bias is not None and linear.bias.dim() != 1:
             raise ValueError("int2 weight-only requires a 1-D bias or no bias")
         w = linear.weight.detach()
-        packed, scale_zero = _pack_int2_weight(w.float(), groupsize)
+        # quantized in the weight's own dtype, as the reference does (:207); the kernel reads float32 parameters
+        packed, scale_zero = _pack_int2_weight(w, groupsize)
+        scale_zero = scale_zero.float()
         mod = cls(linear.in_features, linear.out_features, groupsize=groupsize, bias=linear.bias is not None,
                   cache_unpacked=cache_unpacked, device=w.device)
         mod.weight = packed

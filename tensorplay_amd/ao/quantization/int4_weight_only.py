@@ -88,6 +88,33 @@ class WeightOnlyInt4Linear(nn.Module):
             out = out + self.bias
         return out
 
+    # Layout of a CPU-packed ``weight`` met in a state_dict: (columns per block, half-split nibbles).  The reference's
+    # CPU pack depends on the ISA tier it was compiled for (p10/src/backend/cpu/QuantizedElementwiseKernels.cpp:19,
+    # 370-390): (64, True) AVX-512 (also what torch's CPU pack writes on such a host), (32, True) AVX2, (32, False)
+    # the plain tier.  A state_dict does not say which; set this before load_state_dict for another tier.
+    cpu_pack_layout = (64, True)
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        """Accepts the module's own buffers (device layout int32 [N/8, K/32, 32, 1]) and the buffers a CPU model of the
+        reference saves (reference :150-154, 180-181): ``weight`` uint8 [N, K/2] in the CPU layout, which the device
+        op rejects (p10/src/backend/cuda/QuantGemmKernels.cu:1216-1220) and which is converted here on the GPU, and
+        ``scales_and_zeros`` [K/g, N, 2] of any float dtype (float32 placeholders included), cast to the module's."""
+        key = prefix + "weight"
+        w = state_dict.get(key)
+        if isinstance(w, torch.Tensor) and w.dtype == torch.uint8 and w.dim() == 2:
+            if tuple(w.shape) != (self.out_features, self.in_features // 2):
+                error_msgs.append(f"{key}: CPU-layout int4 weight must be [{self.out_features}, {self.in_features // 2}], "
+                                  f"got {list(w.shape)}")
+            elif self.out_features % 16 != 0:
+                error_msgs.append(f"{key}: the CPU layout needs out_features % 16 == 0")
+            elif not self.weight.is_cuda:
+                error_msgs.append(f"{key}: move the module to the GPU before loading a CPU-layout weight (the converter is a GPU kernel)")
+            else:
+                block_cols, half_split = self.cpu_pack_layout
+                state_dict = dict(state_dict)
+                state_dict[key] = ops.int4pack_cpu_to_device(w.to(self.weight.device), block_cols=block_cols, half_split=half_split)
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+
     @classmethod
     def from_float(cls, linear: nn.Linear, groupsize: int = 128) -> "WeightOnlyInt4Linear":
         if linear.bias is not None and linear.bias.dim() != 1:

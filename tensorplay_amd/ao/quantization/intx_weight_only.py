@@ -105,7 +105,9 @@ class WeightOnlyIntxLinear(nn.Module):
         if linear.bias is not None and linear.bias.dim() != 1:
             raise ValueError("intx weight-only requires a 1-D bias or no bias")
         w = linear.weight.detach()
-        codes, scale, zero = _quantize_intx_groupwise(w.float(), groupsize, bits)
+        # quantized in the weight's own dtype, as the reference does (:204-206); the kernel reads float32 parameters
+        codes, scale, zero = _quantize_intx_groupwise(w, groupsize, bits)
+        scale, zero = scale.float(), zero.float()
         mod = cls(linear.in_features, linear.out_features, bits=bits, groupsize=groupsize, bias=linear.bias is not None,
                   cache_unpacked=cache_unpacked, device=w.device)
         mod.weight = pack_intx(codes, bits)

@@ -44,14 +44,16 @@ def hipcc() -> str:
     return exe
 
 
-def build_library(verbose: bool = False, jobs: int = 5) -> str:
+def build_library(verbose: bool = False, jobs: int = 5, tuning: bool = False) -> str:
+    """tuning=True compiles the sweep knobs in (-DTPQ_TUNING: TPQ_* environment variables pick kernels and workgroup
+    shapes); the library that ships is built without it and never reads the environment."""
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     cc = hipcc()
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        cmd = [cc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [cc, *HIPCC_FLAGS, *(["-DTPQ_TUNING"] if tuning else []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -75,4 +77,4 @@ def build_library(verbose: bool = False, jobs: int = 5) -> str:
 
 
 if __name__ == "__main__":
-    print(build_library(verbose="-v" in sys.argv))
+    print(build_library(verbose="-v" in sys.argv, tuning="--tuning" in sys.argv))

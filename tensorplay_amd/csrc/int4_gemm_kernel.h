@@ -250,9 +250,9 @@ int launch_int4_gemm_shape(const void* x, const int32_t* packed, const void* sz,
 
 template <int DT>
 int launch_int4_gemm(const void* x, const int32_t* packed, const void* sz, void* y, int64_t M, int64_t N, int64_t K, int group, hipStream_t s) {
-    static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT4_GEMM_NB"); return e ? std::atoi(e) : 0; }();
-    static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT4_GEMM_WAVES"); return e ? std::atoi(e) : 0; }();
-    static const int forced_rsplit = [] { const char* e = std::getenv("TPQ_INT4_GEMM_RSPLIT"); return e ? std::atoi(e) : 0; }();
+    static const int forced_nb = [] { const char* e = tuning_env("TPQ_INT4_GEMM_NB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_waves = [] { const char* e = tuning_env("TPQ_INT4_GEMM_WAVES"); return e ? std::atoi(e) : 0; }();
+    static const int forced_rsplit = [] { const char* e = tuning_env("TPQ_INT4_GEMM_RSPLIT"); return e ? std::atoi(e) : 0; }();
     // Eight wavefronts per workgroup.  Few workgroups (up to 256 rows): two groups of four share the channels and split
     // the rows, 64 channels per workgroup while that gives at most one workgroup per compute unit, else 128; more rows:
     // 256 channels, which halves the LDS reads per product.  Measured (us, fp16): 4096 -> 11008: 128 rows 37.5 (42.2

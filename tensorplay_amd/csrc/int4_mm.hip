@@ -302,8 +302,8 @@ inline DecodePlan plan_decode(int N, int K, int mrows, size_t workspace_bytes) {
     const int n_chunks = K / 128;
     const int col_groups = (N + kWave - 1) / kWave;
     DecodePlan plan{kDecodeWaves, 1};
-    const char* env_wpb = std::getenv("TPQ_INT4_WPB");
-    const char* env_ks = std::getenv("TPQ_INT4_KS");
+    const char* env_wpb = tuning_env("TPQ_INT4_WPB");
+    const char* env_ks = tuning_env("TPQ_INT4_KS");
     int wpb = 0, ks = 0;
     if (workspace_bytes > kCounterBytes && col_groups <= kCounterSlots) {
         const size_t per_slice = static_cast<size_t>(mrows) * N * sizeof(float);
@@ -363,7 +363,7 @@ bool launch_stream(const void* x, const int32_t* packed, const void* sz, void* y
                    hipStream_t s, int* rc) {
     // Measured on MI355X at M=1, K=4096, N=11008 the column-per-lane kernel is the faster of the
     // two (7.1 us against 8.3 us); the streaming kernel is kept selectable for comparison runs.
-    const char* force = std::getenv("TPQ_INT4_KERNEL");
+    const char* force = tuning_env("TPQ_INT4_KERNEL");
     if (!(force && force[0] == 's')) return false;  // TPQ_INT4_KERNEL=stream opts in
     const int k_super = K / 32, n_tiles = N / 8;
     int tiles_per_block = (n_tiles + compute_units() - 1) / compute_units();
@@ -397,7 +397,7 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     const bool deq = (group == 32 || group == 64) && residual == nullptr;  // dequantized in registers
     if ((group != 128 && group != 256 && !deq) || !aligned(sz, 16) || !aligned(y, 8)) return false;
     if (residual != nullptr && !aligned(residual, 8)) return false;
-    const char* force = std::getenv("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
+    const char* force = tuning_env("TPQ_INT4_KERNEL");  // "mfma" / "decode" pin the choice for comparison runs
     if (force && force[0] == 'd' && residual == nullptr) return false;
     // One row: the column-per-lane kernel wins only where N is wide enough to fill the chip with its
     // 64-column workgroups (measured: N = 11008, K = 4096: 7.1 us against 8.5 us here; N = 4096,
@@ -415,9 +415,9 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     //   N > 28672:   32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (4096 -> 32000, 4 rows: 16.2 against 16.6)
     const bool wide = N >= 10240 && N <= 28672 && rows <= 12;
     int nb = N > 4096 ? (N < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
-    if (const char* env = std::getenv("TPQ_INT4_NB")) nb = std::atoi(env);
+    if (const char* env = tuning_env("TPQ_INT4_NB")) nb = std::atoi(env);
     int waves = N < 10240 || wide ? 8 : 4;
-    if (const char* env = std::getenv("TPQ_INT4_WAVES")) waves = std::atoi(env);
+    if (const char* env = tuning_env("TPQ_INT4_WAVES")) waves = std::atoi(env);
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
     const auto* sp = static_cast<const uint32_t*>(sz);
@@ -477,7 +477,7 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
         char* ys = static_cast<char*>(y) + m0 * row_y;
         int rc = TPQ_OK;
         if (packed_b != nullptr) {
-            static const int pair_waves = [] { const char* e = std::getenv("TPQ_INT4_PAIR_WAVES"); return e ? std::atoi(e) : 4; }();
+            static const int pair_waves = [] { const char* e = tuning_env("TPQ_INT4_PAIR_WAVES"); return e ? std::atoi(e) : 4; }();
             const auto* xp = reinterpret_cast<const uint16_t*>(xs);
             const auto* pa = reinterpret_cast<const uint4*>(packed);
             const auto* pb = reinterpret_cast<const uint4*>(packed_b);
@@ -539,10 +539,10 @@ int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* s
     // Many rows: the tiled kernel, the packed weight read once per 128 rows.  Measured against the 32-row slabs below
     // (us, fp16): K = 4096, N = 11008: 43 / 55 at 128 rows, 62 / 107 at 256, 258 / 821 at 2048; K = N = 8192:
     // 77 / 81 at 128, 82 / 157 at 256; at 96 rows the slabs still win (42 against 43, 63 against 77).
-    static const int64_t gemm_rows = [] { const char* e = std::getenv("TPQ_INT4_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{113}; }();
+    static const int64_t gemm_rows = [] { const char* e = tuning_env("TPQ_INT4_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{113}; }();
     if (M >= gemm_rows && int4_gemm_ok(x, packed, sz, y, M, N, K, group)) return launch_int4_gemm<DT>(x, packed, sz, y, M, N, K, group, s);
     {   // slabs of 32 rows (16 with groups of 32 / 64) on the matrix cores where the shape allows
-        static const int slab_rows = [] { const char* e = std::getenv("TPQ_INT4_SLAB_ROWS"); return e ? std::atoi(e) : 32; }();
+        static const int slab_rows = [] { const char* e = tuning_env("TPQ_INT4_SLAB_ROWS"); return e ? std::atoi(e) : 32; }();
         const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;
         const int slab = (group == 32 || group == 64) ? 16 : slab_rows;
         int64_t m0 = 0;

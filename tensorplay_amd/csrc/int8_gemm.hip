@@ -26,7 +26,7 @@ EpilogueDequant<DT> rebase_rows(const EpilogueDequant<DT>& ep, int64_t m0, int64
 
 // Up to this many rows the decode kernel streams the weight once per 32 rows.
 inline int int8_decode_rows(int64_t N) {
-    static const int forced = [] { const char* e = std::getenv("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
+    static const int forced = [] { const char* e = tuning_env("TPQ_INT8_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
     return forced >= 0 ? forced : (N >= 10240 ? 32 : 64);
 }
 
@@ -34,7 +34,7 @@ inline int int8_decode_rows(int64_t N) {
 // With a workspace at hand the decode kernel keeps only what it does in one pass (32 rows): two passes cost more
 // than the sliced kernel (K = N = 8192, 48 rows: 41 us against 28).
 inline int int8_slices(const void* a, const void* w, int64_t M, int64_t N, int64_t K) {
-    const char* force = std::getenv("TPQ_INT8_KERNEL");
+    const char* force = tuning_env("TPQ_INT8_KERNEL");
     if (K <= 0 || !mfma_path_ok(a, w, M, N, K) || (force && force[0] == 'r')) return 1;
     const int decode_rows = int8_decode_rows(N) < 32 ? int8_decode_rows(N) : 32;
     if (M <= decode_rows && int8_decode_ok(a, w, M, N, K)) return 1;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void int32_sum_slices_kernel(const int32_t* __
 
 template <class Epilogue>
 int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
-    const char* force = std::getenv("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
+    const char* force = tuning_env("TPQ_INT8_KERNEL");  // "reg" keeps the register-staged kernel
     // a few rows: stream the weight once per 32 rows through the decode kernel.  K = N = 4096: 16 rows 6.9 us,
     // 32 rows 9.1 us, 64 rows 17.8 us, against 27.5 us for the tiled kernels below at any of these row counts
     // (28672 -> 8192: 61 / 69 / 138 us against 182 us; 4096 -> 11008: 15 / 21 / 41 us against 31 / 31 / 32 us)

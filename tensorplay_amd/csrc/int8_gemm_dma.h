@@ -533,7 +533,7 @@ int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int
 // TPQ_INT8_KSPLIT=1 selects the four-wavefront variant for comparison runs.
 template <class Tile>
 int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
-    const char* env = std::getenv("TPQ_INT8_KSPLIT");
+    const char* env = tuning_env("TPQ_INT8_KSPLIT");
     if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s, slices);
     return launch_dma_split<2>(a, w, M, N, K, tile, s, slices);
 }
@@ -543,11 +543,11 @@ int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K
 // own; a second kernel adds them.  How many slices: enough workgroups for the chip, at least four stages each
 // and none empty; 1 = not worth it.
 inline int dma_slices(int64_t M, int64_t N, int64_t K) {
-    static const int forced = [] { const char* e = std::getenv("TPQ_INT8_SLICES"); return e ? std::atoi(e) : 0; }();
+    static const int forced = [] { const char* e = tuning_env("TPQ_INT8_SLICES"); return e ? std::atoi(e) : 0; }();
     if (M < 1 || K % kDmaRowBytes != 0) return 1;
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128), nk = K / kDmaRowBytes;
-    static const int min_stages = [] { const char* e = std::getenv("TPQ_INT8_SLICE_STAGES"); return e ? std::atoi(e) : 4; }();
-    static const int target = [] { const char* e = std::getenv("TPQ_INT8_SLICE_TARGET"); return e ? std::atoi(e) : 256; }();
+    static const int min_stages = [] { const char* e = tuning_env("TPQ_INT8_SLICE_STAGES"); return e ? std::atoi(e) : 4; }();
+    static const int target = [] { const char* e = tuning_env("TPQ_INT8_SLICE_TARGET"); return e ? std::atoi(e) : 256; }();
     int64_t slices = forced ? forced : target / tiles;
     if (slices > nk / min_stages) slices = nk / min_stages;
     if (slices < 2) return 1;

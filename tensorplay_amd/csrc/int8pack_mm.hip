@@ -433,8 +433,8 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
     // workgroups to fill the chip (4096 x 4096: 5.8 us with 4 wavefronts, 8.9 with 16), the largest stream best with 8
     // (8192 -> 28672: 40.1 us = 5.9 TB/s; 42.0 with 4, 45.1 with 16).  TPQ_INT8PACK_ROW=0 / 1 pins the kernel and
     // TPQ_INT8PACK_ROW_WAVES the workgroup size for comparison runs.
-    static const int forced_row = [] { const char* e = std::getenv("TPQ_INT8PACK_ROW"); return e ? std::atoi(e) : -1; }();
-    static const int forced_row_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_ROW_WAVES"); return e ? std::atoi(e) : 0; }();
+    static const int forced_row = [] { const char* e = tuning_env("TPQ_INT8PACK_ROW"); return e ? std::atoi(e) : -1; }();
+    static const int forced_row_waves = [] { const char* e = tuning_env("TPQ_INT8PACK_ROW_WAVES"); return e ? std::atoi(e) : 0; }();
     if (M <= 2 && dtype != TPQ_DTYPE_F32 && K % 16 == 0 && K <= (M == 1 ? 65536 : 32768) && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16) && forced_row != 0) {
         const int passes = static_cast<int>((K + 4095) / 4096);
         int waves = N * K >= (int64_t{1} << 27) ? 8 : N * K >= (int64_t{1} << 26) ? 16 : 4;
@@ -454,9 +454,9 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
         return check_launch("_weight_int8pack_mm (row)");
     }
     if (dtype != TPQ_DTYPE_F32 && K % 128 == 0 && K <= 0x7FFFFF80 && N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(w, 16)) {
-        static const int forced_nb = [] { const char* e = std::getenv("TPQ_INT8PACK_NB"); return e ? std::atoi(e) : 0; }();
-        static const int forced_waves = [] { const char* e = std::getenv("TPQ_INT8PACK_WAVES"); return e ? std::atoi(e) : 0; }();
-        static const int forced_mb = [] { const char* e = std::getenv("TPQ_INT8PACK_MB"); return e ? std::atoi(e) : 0; }();
+        static const int forced_nb = [] { const char* e = tuning_env("TPQ_INT8PACK_NB"); return e ? std::atoi(e) : 0; }();
+        static const int forced_waves = [] { const char* e = tuning_env("TPQ_INT8PACK_WAVES"); return e ? std::atoi(e) : 0; }();
+        static const int forced_mb = [] { const char* e = tuning_env("TPQ_INT8PACK_MB"); return e ? std::atoi(e) : 0; }();
         for (int64_t m0 = 0; m0 < M;) {
             const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
             const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);

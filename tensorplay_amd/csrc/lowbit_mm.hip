@@ -60,6 +60,12 @@ struct Fields {
 
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 
+// 8-bit codes are signed in the reference: unpack_intx ends in codes.to(int8) and _dequantize_intx converts that int8
+// to float (tensorplay/ao/quantization/intx_weight_only.py:62-80, 110-124), so a byte of 128 or more counts as
+// byte - 256.  The matrix-core and row kernels keep their unsigned field arithmetic: byte ^ 0x80 = value + 128, so
+// the packed words are flipped after the load and 128 is added to the zero point.
+constexpr uint32_t kSignFlip = 0x80808080u;
+
 // x: [M][K] fp16 or bf16; packed: [N][K / per_byte]; sz: [K / group][N][2] fp32; steps = K / kStepK; a group
 // is kStepK << group_shift k.  N % 4 == 0.
 // bf16 has seven mantissa bits, too few for the exponent trick: there a code is cut out of its dword,
@@ -107,6 +113,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
         if constexpr (F::kBytes == 16) st.w = nt_load(reinterpret_cast<const uint4*>(src));
         if constexpr (F::kBytes == 8) { const uint2 t = nt_load(reinterpret_cast<const uint2*>(src)); st.w = make_uint4(t.x, t.y, 0, 0); }
         if constexpr (F::kBytes == 4) st.w = make_uint4(nt_load(reinterpret_cast<const uint32_t*>(src)), 0, 0, 0);
+        if constexpr (BITS == 8) st.w = make_uint4(st.w.x ^ kSignFlip, st.w.y ^ kSignFlip, st.w.z ^ kSignFlip, st.w.w ^ kSignFlip);
         const uint4* prm = reinterpret_cast<const uint4*>(sz_base + static_cast<size_t>(s >> group_shift) * N * 2);
         st.p[0] = prm[0];
         st.p[1] = prm[1];
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
         for (int v = 0; v < 4; ++v) {
             const uint4& pv = st.p[v >> 1];
             const float scale = __builtin_bit_cast(float, (v & 1) ? pv.z : pv.x);
-            const float zero = __builtin_bit_cast(float, (v & 1) ? pv.w : pv.y);
+            const float zero = __builtin_bit_cast(float, (v & 1) ? pv.w : pv.y) + (BITS == 8 ? 128.0f : 0.0f);
             yacc[v] = __builtin_fmaf(scale, (d[v] - corr) - zero * sx, yacc[v]);
         }
     };
@@ -202,6 +209,13 @@ __device__ __forceinline__ int code_at(const uint8_t* row, int64_t k, int bits, 
     return (row[k / per_byte] >> shift) & ((1 << bits) - 1);
 }
 
+// Value of a code as the reference dequantizes it: unpack_intx ends in codes.to(int8) and _dequantize_intx converts
+// that int8 to float (tensorplay/ao/quantization/intx_weight_only.py:62-80, 110-124), so at 8 bits a byte of 128 or
+// more counts as byte - 256; narrower fields never reach the sign bit.
+__device__ __forceinline__ float code_value(uint32_t code, int bits) {
+    return bits == 8 ? static_cast<float>(static_cast<int>(static_cast<int8_t>(code))) : static_cast<float>(code);
+}
+
 // Any floating activation dtype and bit width, K % 8 == 0, group % 8 == 0, aligned rows: a wavefront owns
 // four consecutive output channels and a slab of up to four activation rows; a lane takes eight consecutive k
 // per turn (1 to 8 bytes of each weight row), forms (code - zero) * scale in fp32 as the reference does, fp32
@@ -246,7 +260,7 @@ __global__ __launch_bounds__(256) void lowbit_vector_kernel(
             for (int e = 0; e < 8; ++e) {
                 const int i = e & (per_byte - 1);  // per_byte is 1, 2, 4 or 8
                 const int shift = 8 * (e >> pb_shift) + (lsb_first ? i * bits : 8 - (i + 1) * bits);
-                const float wv = (static_cast<float>(static_cast<uint32_t>(raw >> shift) & field) - p.y) * p.x;
+                const float wv = (code_value(static_cast<uint32_t>(raw >> shift) & field, bits) - p.y) * p.x;
 #pragma unroll
                 for (int r = 0; r < kVecRows; ++r)
                     if (r < rows) acc[c][r] = __builtin_fmaf(wv, xv[r][e], acc[c][r]);
@@ -281,7 +295,7 @@ __global__ __launch_bounds__(256) void lowbit_generic_kernel(
     for (int b = 0; b < 8; ++b) acc[b] = 0.0f;
     for (int64_t k = threadIdx.x; k < K; k += 256) {
         const float* p = sz + ((k / group) * N + n) * 2;
-        const float wv = (static_cast<float>(code_at(wr, k, bits, per_byte, lsb_first)) - p[1]) * p[0];
+        const float wv = (code_value(code_at(wr, k, bits, per_byte, lsb_first), bits) - p[1]) * p[0];
 #pragma unroll
         for (int b = 0; b < 8; ++b)
             if (b < rows) acc[b] = __builtin_fmaf(wv, Elem<DT>::load(x[(m0 + b) * K + k]), acc[b]);
@@ -312,7 +326,7 @@ __global__ __launch_bounds__(256) void lowbit_dequantize_kernel(const uint8_t* _
          idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
         const int64_t n = idx / K, k = idx - n * K;
         const float* p = sz + ((k / group) * N + n) * 2;
-        out[idx] = Elem<DT>::store((static_cast<float>(code_at(packed + n * pitch, k, bits, per_byte, lsb_first != 0)) - p[1]) * p[0]);
+        out[idx] = Elem<DT>::store((code_value(code_at(packed + n * pitch, k, bits, per_byte, lsb_first != 0), bits) - p[1]) * p[0]);
     }
 }
 
@@ -344,7 +358,7 @@ __global__ __launch_bounds__(256) void lowbit_dequantize_vec_kernel(const uint8_
             const int field = i & (per_byte - 1);
             const int shift = 8 * (i >> pb_shift) + (lsb_first ? field * bits : 8 - (field + 1) * bits);
             const uint32_t code = static_cast<uint32_t>(v >> shift) & mask;
-            o[i] = Elem<DT>::store((static_cast<float>(code) - p.y) * p.x);
+            o[i] = Elem<DT>::store((code_value(code, bits) - p.y) * p.x);
         }
         S* dst = out + n * K + k0;
         if constexpr (sizeof(S) == 2) {
@@ -389,7 +403,7 @@ template <int DT, int BITS, bool LSB>
 int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t M, int64_t N,
                 int64_t K, int group_shift, hipStream_t s) {
     // wavefronts per 16-channel workgroup: each takes every WAVES-th step, two in flight
-    static const int forced = [] { const char* e = getenv("TPQ_LOWBIT_WAVES"); return e ? atoi(e) : 0; }();
+    static const int forced = [] { const char* e = tuning_env("TPQ_LOWBIT_WAVES"); return e ? atoi(e) : 0; }();
     const int64_t steps = K / Fields<BITS, LSB>::kStepK;
     // measured at 4096 -> 11008, one row, 2 bits: 4 waves 11.1 us, 8 waves 10.4 - 11.0 us, 16 waves 14.3 us
     const int waves = forced ? forced : steps >= 16 ? 8 : 4;
@@ -476,6 +490,11 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
                     wv[c][t][0] = q.x; wv[c][t][1] = q.y;
                 }
                 p[c][t] = *reinterpret_cast<const float2*>(sz + (static_cast<size_t>(kl / group) * N + n) * 2);
+                if constexpr (BITS == 8) {  // signed bytes: value + 128 in the fields, 128 more in the zero point
+#pragma unroll
+                    for (int w = 0; w < kWords; ++w) wv[c][t][w] ^= kSignFlip;
+                    p[c][t].y += 128.0f;
+                }
             }
             const uint4* xp = reinterpret_cast<const uint4*>(x + kl);
 #pragma unroll
@@ -625,9 +644,8 @@ TPQ_EXPORT int tpq_lowbit_mm(const void* x, int dtype, int64_t M, int64_t K, con
     }
     const bool fast = dtype != TPQ_DTYPE_F32 && K > 0 && group_shift >= 0 && K % step_k == 0 && N % 4 == 0 && K <= 0x7FFFFF80 &&
                       N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(packed, 16) && aligned(scales_and_zeros, 16) && aligned(out, 8);
-    const char* row_env = M == 1 ? std::getenv("TPQ_LOWBIT_ROW") : nullptr;  // read per call: tests switch it
-    const int forced_row = row_env ? std::atoi(row_env) : -1;
-    if (M == 1 && dtype != TPQ_DTYPE_F32 && forced_row != 0) {  // TPQ_LOWBIT_ROW=0 / 1: never / wherever the shape allows, for comparison runs and tests
+    const int forced_row = g_override_lowbit_row.load(std::memory_order_relaxed);
+    if (M == 1 && dtype != TPQ_DTYPE_F32 && forced_row != 0) {  // tpq_set_kernel_override("lowbit_row", 0 / 1): never / wherever the shape allows
         int rc = TPQ_OK;
         if (dtype == TPQ_DTYPE_F16 ? launch_lowbit_row<TPQ_DTYPE_F16>(x, packed, scales_and_zeros, bias, out, N, K, group, bits, lsb_first, forced_row == 1, s, &rc)
                                    : launch_lowbit_row<TPQ_DTYPE_BF16>(x, packed, scales_and_zeros, bias, out, N, K, group, bits, lsb_first, forced_row == 1, s, &rc))

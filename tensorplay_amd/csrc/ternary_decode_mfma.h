@@ -148,9 +148,9 @@ inline bool ternary_decode_mfma_ok(const void* x, const void* packed, int64_t M,
 // slabs of 32 rows (16 for what is left)
 template <class Epilogue>
 int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N, int64_t K, Epilogue ep, hipStream_t s) {
-    static const int forced_nb = [] { const char* e = std::getenv("TPQ_TERNARY_NB"); return e ? std::atoi(e) : 0; }();
-    static const int forced_mb = [] { const char* e = std::getenv("TPQ_TERNARY_MB"); return e ? std::atoi(e) : 0; }();
-    static const int forced_waves = [] { const char* e = std::getenv("TPQ_TERNARY_WAVES"); return e ? std::atoi(e) : 0; }();
+    static const int forced_nb = [] { const char* e = tuning_env("TPQ_TERNARY_NB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_mb = [] { const char* e = tuning_env("TPQ_TERNARY_MB"); return e ? std::atoi(e) : 0; }();
+    static const int forced_waves = [] { const char* e = tuning_env("TPQ_TERNARY_WAVES"); return e ? std::atoi(e) : 0; }();
     // Workgroup shape from a sweep over model shapes (K 2560..28672, 1..16 rows), about 2000..4000 wavefronts in all:
     //   N < 8192: 16 channels x 8 wavefronts (4096 x 4096, 8 rows: 5.0 us; 32 channels: 6.6)
     //   N < 10240: 32 x 8 (8192 x 28672 -> 8192, 16 rows: 26.4 us; 16 channels: 36.3)

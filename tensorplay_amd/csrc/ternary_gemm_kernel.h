@@ -152,7 +152,7 @@ int launch_ternary_gemm_m128(const int8_t* x, const uint8_t* packed, int64_t M, 
     // 4096 x 4096 12.3 against 14.2) and when 128-row tiles would occupy at most half of the 256 compute units
     // (4096 x 4096 at 128 rows: 13.8 us against 15.7; 2560 -> 6912, 216 tiles: 14.7 against 13.1, stays on 128)
     const int64_t tiles128 = ((N + kTgN - 1) / kTgN) * ((M + 127) / 128);
-    static const int forced = [] { const char* e = getenv("TPQ_TERNARY_BM"); return e ? atoi(e) : 0; }();
+    static const int forced = [] { const char* e = tuning_env("TPQ_TERNARY_BM"); return e ? atoi(e) : 0; }();
     const bool small = forced ? forced == 64 : (M <= 64 || tiles128 <= 128);
     return small ? launch_ternary_gemm_tile<64>(x, packed, M, N, K, ep, s) : launch_ternary_gemm_tile<128>(x, packed, M, N, K, ep, s);
 }

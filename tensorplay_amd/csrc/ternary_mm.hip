@@ -123,16 +123,16 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
     // the tile kernel below takes over where it is faster and its shape conditions hold
     // Measured at 2560 -> 6912 / 6912 -> 2560 (216 / 80 tiles of 32 channels): the decode kernel takes 7, 7.5, 9.4, 11.4 us
     // for 1..4 rows and twice that for 5..8, the tile kernel 9.3 / 18.3 us for any row count up to 128.
-    static const int forced_decode_rows = [] { const char* e = std::getenv("TPQ_TERNARY_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
+    static const int forced_decode_rows = [] { const char* e = tuning_env("TPQ_TERNARY_DECODE_ROWS"); return e ? std::atoi(e) : -1; }();
     // ... and stays ahead of the 256 x 128-tile kernel at every larger row count tried (512 rows: 30 / 33 us against
     // 54 / 103 us; 2048 rows: 100 / 85 us against 111 / 112 us), so there is no upper limit by default.
-    static const int64_t gemm_rows = [] { const char* e = std::getenv("TPQ_TERNARY_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{1} << 40; }();
+    static const int64_t gemm_rows = [] { const char* e = tuning_env("TPQ_TERNARY_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{1} << 40; }();
     const int decode_rows = forced_decode_rows >= 0 ? forced_decode_rows : ((N + kTgN - 1) / kTgN >= 128 ? 3 : 6);
     // Up to 32 rows, in slabs of 16: the weight streamed once per slab through the matrix cores.  Measured against the
     // kernels below over K, N = 1024..28672: one row 4.3..19.8 us (the dot-product kernel 4.7..19.2), 16 rows
     // 5.2..29.6 us (the tile kernel 9.3..75 us for any row count up to 128; two slabs stay below it, three do not).
-    static const int mfma_min = [] { const char* e = std::getenv("TPQ_TERNARY_MFMA_MIN"); return e ? std::atoi(e) : 1; }();
-    static const int mfma_rows = [] { const char* e = std::getenv("TPQ_TERNARY_MFMA_ROWS"); return e ? std::atoi(e) : 32; }();
+    static const int mfma_min = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_MIN"); return e ? std::atoi(e) : 1; }();
+    static const int mfma_rows = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_ROWS"); return e ? std::atoi(e) : 32; }();
     if (forced_decode_rows < 0 && M >= mfma_min && M <= mfma_rows && ternary_decode_mfma_ok(x, packed, M, N, K))
         return launch_ternary_decode_mfma(x, packed, M, N, K, ep, s);
     const bool gemm_ok = sizes_ok && M <= gemm_rows && K % kTgStage == 0 && aligned(x, 16) && aligned(packed, 4);

@@ -8,6 +8,8 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 
 #include "../../include/tpq.h"
 
@@ -43,6 +45,22 @@ inline int ensure_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint
     done.fetch_or(bit, std::memory_order_release);
     return TPQ_OK;
 }
+
+// Sweep knobs.  Environment variables named TPQ_* select kernels and workgroup shapes only in a build made with
+// -DTPQ_TUNING (sweeps, comparison runs).  The shipped library never reads the environment: which kernel runs is a
+// function of the arguments alone, and no entry point depends on getenv (not safe against a concurrent setenv).
+inline const char* tuning_env(const char* name) {
+#ifdef TPQ_TUNING
+    return std::getenv(name);
+#else
+    (void)name;
+    return nullptr;
+#endif
+}
+
+// The two routes that tests pin explicitly (tpq_set_kernel_override): -1 = the default rule.
+extern std::atomic<int> g_override_int8_row;    // 0 never / 1 up to four rows on the int8 row kernel
+extern std::atomic<int> g_override_lowbit_row;  // 0 never / 1 wherever the shape allows, the packed n-bit row kernel
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 

@@ -217,6 +217,20 @@ using namespace tpq;
 
 TPQ_EXPORT int tpq_abi_version(void) { return 1; }
 
+namespace tpq {
+std::atomic<int> g_override_int8_row{-1};
+std::atomic<int> g_override_lowbit_row{-1};
+}  // namespace tpq
+
+TPQ_EXPORT int tpq_set_kernel_override(const char* route, int value) {
+    TPQ_REQUIRE(route != nullptr, TPQ_ERR_INVALID_VALUE, "tpq_set_kernel_override: null route name");
+    TPQ_REQUIRE(value >= -1 && value <= 1, TPQ_ERR_INVALID_VALUE, "tpq_set_kernel_override: value must be -1, 0 or 1");
+    if (std::strcmp(route, "int8_row") == 0) tpq::g_override_int8_row.store(value, std::memory_order_relaxed);
+    else if (std::strcmp(route, "lowbit_row") == 0) tpq::g_override_lowbit_row.store(value, std::memory_order_relaxed);
+    else return tpq::fail(TPQ_ERR_INVALID_VALUE, "tpq_set_kernel_override: unknown route '%s'", route);
+    return TPQ_OK;
+}
+
 TPQ_EXPORT const char* tpq_last_error(void) { return error_buffer(); }
 
 TPQ_EXPORT int tpq_int8_mm_rescale(const int32_t* acc, const float* row_scale,

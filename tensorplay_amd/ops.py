@@ -644,15 +644,29 @@ def _lowbit_mm(input: torch.Tensor, packed: torch.Tensor, bits: int, columns: in
 
 # ---- fusions around the int4 decode matmul (MLP of a decoder layer) -------------------------------
 
-def _fused_int4_operands(x, packed, group, sz, what):
+def _fused_int4_check(x, packed, group, sz, what):
+    """Shape, layout and extent checks of one (activations, packed weight, scales) triple; host only."""
     if packed.dtype != torch.int32 or packed.dim() != 4 or packed.size(2) != 32:
         raise TypeError(f"{what}: packed weight must be 4-D int32 in the tensor-core B layout")
     if x.dim() != 2 or x.dtype not in _DT:
         raise ValueError(f"{what}: expected 2-D float activations [m,k]")
-    _require_device(x, what)
-    inner, n = packed.size(3) * 2, packed.size(0) * 8
-    if tuple(sz.shape) != ((x.shape[1] + group - 1) // group, n, 2):
+    if group not in (32, 64, 128):
+        raise ValueError(f"{what}: qGroupSize must be 32, 64 or 128")
+    inner, n, k = packed.size(3) * 2, packed.size(0) * 8, x.shape[1]
+    if inner not in (2, 4, 8):
+        raise ValueError(f"{what}: packed weight layout is invalid")
+    # the kernels only receive pointers: a packed weight that covers fewer k than the activations would be read
+    # past its end, so the extent is checked here, as _weight_int4pack_mm does
+    if packed.size(1) != (k + inner * 16 - 1) // (inner * 16):
+        raise ValueError(f"{what}: K dimension does not match packed B")
+    if sz.dim() != 3 or tuple(sz.shape) != ((k + group - 1) // group, n, 2):
         raise ValueError(f"{what}: qScaleAndZeros must be [K/group, N, 2]")
+    return inner, n
+
+
+def _fused_int4_operands(x, packed, group, sz, what):
+    inner, n = _fused_int4_check(x, packed, group, sz, what)
+    _require_device(x, what)
     return x.contiguous(), packed.contiguous(), sz.to(x.dtype).contiguous(), inner, n
 
 
@@ -684,6 +698,8 @@ def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zer
     mats, scales_and_zeros = list(mats), list(scales_and_zeros)
     if len(mats) != len(scales_and_zeros) or not mats:
         raise ValueError("int4pack_mm_multi: one qScaleAndZeros per packed weight, at least one weight")
+    for w, sz in zip(mats, scales_and_zeros):
+        _fused_int4_check(input, w, qGroupSize, sz, "int4pack_mm_multi")
     ops = [_fused_int4_operands(input, w, qGroupSize, sz, "int4pack_mm_multi") for w, sz in zip(mats, scales_and_zeros)]
     x = ops[0][0]
     m, k = x.shape
@@ -716,6 +732,8 @@ def int4pack_mm_swiglu(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor
     """``silu_mul(_weight_int4pack_mm(input, gate, ...), _weight_int4pack_mm(input, up, ...))`` in one launch
     (the reference's ``silu_mul``: gate * sigmoid(gate) * up in float32, rounded once).  Shapes the fused kernel
     does not take run the separate ops."""
+    _fused_int4_check(input, gate, qGroupSize, gate_scale_and_zeros, "int4pack_mm_swiglu")
+    _fused_int4_check(input, up, qGroupSize, up_scale_and_zeros, "int4pack_mm_swiglu")
     x, wg, szg, inner, n = _fused_int4_operands(input, gate, qGroupSize, gate_scale_and_zeros, "int4pack_mm_swiglu")
     _, wu, szu, inner_u, n_u = _fused_int4_operands(input, up, qGroupSize, up_scale_and_zeros, "int4pack_mm_swiglu")
     if (inner_u, n_u) != (inner, n) or wu.shape != wg.shape:

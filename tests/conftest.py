@@ -28,3 +28,20 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def kernel_override():
+    """Pins one of the library's two selectable routes for the duration of a test: kernel_override("int8_row", 1)."""
+    from tensorplay_amd import _lib
+
+    lib = _lib.load()
+    touched = []
+
+    def pin(route: str, value: int) -> None:
+        assert lib.tpq_set_kernel_override(route.encode(), value) == 0, _lib.last_error()
+        touched.append(route)
+
+    yield pin
+    for route in touched:
+        lib.tpq_set_kernel_override(route.encode(), -1)

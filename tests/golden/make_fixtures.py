@@ -93,9 +93,9 @@ for K in (3, 31, 32, 65):
     v[f"packed_K{K}_acc"] = (xcodes.astype(np.int64) @ wcodes.astype(np.int64).T).astype(np.int32)
 
 # ---- int8 weight-only matmul: the literal example of test/test_mps.py:1052-1061 and a seeded case --
-a_lit = np.array([[1., 2., 3., 4.], [-1., 0.5, 2., -3.]], np.float32)
-w_lit = np.array([[1, -2, 3, 4], [0, 5, -6, 7], [8, -9, 10, -11]], np.int8)
-s_lit = np.array([0.5, 0.25, 2.0], np.float32)
+a_lit = np.array([[0.5, -1.0, 2.0, 0.25], [1.0, 0.5, -0.5, 2.0]], np.float32)
+w_lit = np.array([[1, -2, 0, 1], [0, 1, -1, 2], [2, 0, 1, -1]], np.int8)
+s_lit = np.array([0.5, 1.0, 2.0], np.float32)
 v.update(int8pack_lit_a=a_lit, int8pack_lit_w=w_lit, int8pack_lit_s=s_lit,
          int8pack_lit_y=((a_lit @ w_lit.astype(np.float32).T) * s_lit).astype(np.float32))
 rng = np.random.default_rng(901)

@@ -77,3 +77,33 @@ def test_no_cpu_fallback():
         m(torch.zeros(1, 256, dtype=torch.float16))
     with pytest.raises((RuntimeError, ValueError, TypeError)):
         WeightOnlyInt4Linear.from_float(nn.Linear(256, 64, bias=False))
+
+
+def test_fused_int4_ops_check_the_packed_extent_on_the_host():
+    """add / swiglu / multi validate layout, K extent and group size before any launch: the kernels only receive
+    pointers, so a packed weight that covers fewer k than the activations must never reach them.  CPU tensors
+    are enough: every check below fires before the device check."""
+    from tensorplay_amd import ops
+
+    x = torch.zeros(2, 256, dtype=torch.float16)
+    good = torch.zeros(4, 8, 32, 1, dtype=torch.int32)       # N = 32, K = 256
+    narrow = torch.zeros(4, 4, 32, 1, dtype=torch.int32)     # covers K = 128 only
+    sz = torch.zeros(2, 32, 2, dtype=torch.float16)
+    res = torch.zeros(2, 32, dtype=torch.float16)
+    for call in (lambda w, s, g: ops.int4pack_mm_add(x, w, g, s, res),
+                 lambda w, s, g: ops.int4pack_mm_swiglu(x, w, good, g, s, sz),
+                 lambda w, s, g: ops.int4pack_mm_swiglu(x, good, w, g, sz, s),    # the up weight is checked too
+                 lambda w, s, g: ops.int4pack_mm_multi(x, [good, w], g, [sz, s])):
+        with pytest.raises(ValueError, match="K dimension does not match"):
+            call(narrow, sz, 128)
+        with pytest.raises(ValueError, match="qGroupSize"):
+            call(good, sz, 96)
+        with pytest.raises(ValueError, match="qScaleAndZeros"):
+            call(good, torch.zeros(1, 32, 2, dtype=torch.float16), 128)
+        with pytest.raises(ValueError, match="layout is invalid"):
+            call(torch.zeros(4, 1, 32, 8, dtype=torch.int32), sz, 128)   # innerKTiles = 16
+        with pytest.raises(TypeError):
+            call(torch.zeros(4, 8, 16, 1, dtype=torch.int32), sz, 128)
+    # with consistent operands the only thing left to fail on the host is the missing GPU
+    with pytest.raises(RuntimeError):
+        ops.int4pack_mm_add(x, good, 128, sz, res)

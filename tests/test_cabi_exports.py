@@ -79,3 +79,20 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     run = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert run.returncode == 2 and "ONE GPU" in run.stderr
+
+
+def test_dispatch_does_not_depend_on_the_environment():
+    """The shipped library imports no getenv: which kernel runs is a function of the arguments.  The two selectable
+    routes go through tpq_set_kernel_override, which validates its arguments on the host."""
+    import subprocess
+    from tensorplay_amd import _lib
+
+    lib = _lib.load()
+    syms = subprocess.run(["nm", "-D", "--undefined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    assert "getenv" not in syms, "the library was built with -DTPQ_TUNING (sweep knobs compiled in)"
+    assert lib.tpq_set_kernel_override(b"int8_row", 1) == 0 and lib.tpq_set_kernel_override(b"int8_row", -1) == 0
+    assert lib.tpq_set_kernel_override(b"lowbit_row", 0) == 0 and lib.tpq_set_kernel_override(b"lowbit_row", -1) == 0
+    assert lib.tpq_set_kernel_override(b"no_such_route", 1) == _lib.TPQ_ERR_INVALID_VALUE
+    assert "unknown route" in _lib.last_error()
+    assert lib.tpq_set_kernel_override(b"int8_row", 5) == _lib.TPQ_ERR_INVALID_VALUE
+    assert lib.tpq_set_kernel_override(None, 0) == _lib.TPQ_ERR_INVALID_VALUE

@@ -202,3 +202,97 @@ def test_lowbit_quantize_kernels_match_reference_formulas():
     codes_b, scales_b = ops._quantize_binary_rowwise(w, 1e-8)
     assert bool((codes_b == torch.where(w >= 0, 1, -1).to(torch.int8)).all())
     assert float((scales_b.unsqueeze(-1) - w.abs().amax(dim=-1, keepdim=True)).abs().max()) < 1e-6
+
+
+# ---- on-disk format: state_dict of the packed modules ------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype,tag", [(torch.float16, "f16"), (torch.bfloat16, "bf16")])
+def test_int4_linear_loads_a_cpu_saved_state_dict(dtype, tag, tmp_path):
+    """A checkpoint written by a CPU model of the reference holds `weight` in the CPU layout (uint8 [N, K/2]) and
+    float32 `scales_and_zeros` (int4_weight_only.py:150-154, 180-181).  The writer here is PyTorch's own CPU pack, which
+    the reference's CPU pack equals byte for byte (test_native_operator_families.py:587-589); the file goes through
+    torch.save / torch.load; the loaded module must compute what the oracle computes from the same codes."""
+    q = _ao()
+    rng = np.random.default_rng(150)
+    N, K, g, M = 272, 512, 128, 5
+    codes = rng.integers(0, 16, (N, K)).astype(np.int32)
+    sz32 = np.stack([rng.uniform(0.002, 0.01, (K // g, N)), rng.normal(0, 0.02, (K // g, N))], -1).astype(np.float32)
+    bias = rng.normal(0, 0.01, N).astype(np.float32)
+    cpu_packed = torch._convert_weight_to_int4pack_for_cpu(torch.from_numpy(codes), 2)
+    assert cpu_packed.dtype == torch.uint8 and tuple(cpu_packed.shape) == (N, K // 2)
+    path = tmp_path / "cpu_int4.pt"
+    torch.save({"weight": cpu_packed, "scales_and_zeros": torch.from_numpy(sz32), "bias": torch.from_numpy(bias)}, path)
+
+    mod = q.WeightOnlyInt4Linear(K, N, groupsize=g, bias=True, device=DEV, dtype=dtype)
+    result = mod.load_state_dict(torch.load(path, weights_only=True))
+    assert not result.missing_keys and not result.unexpected_keys
+    assert mod.weight.dtype == torch.int32 and tuple(mod.weight.shape) == (N // 8, K // 32, 32, 1)
+    np.testing.assert_array_equal(host(mod.weight), oracle.int4_pack_tc(codes, 2))      # the converter, bit for bit
+    szb = cast_bits(sz32, tag)
+    np.testing.assert_array_equal(host(mod.scales_and_zeros), szb)                      # cast to the module dtype
+    x = torch.from_numpy(rng.normal(0, 1, (M, K)).astype(np.float32)).to(DEV, dtype)
+    _, y64 = oracle.int4_mm_tc(bits_of(x.cpu()), tag, oracle.int4_pack_tc(codes, 2), szb, g, round_w=False, want_f64=True)
+    bias_t = torch.from_numpy(bias).to(dtype).double().numpy()
+    assert_close_norm(mod(x).float().cpu().numpy(), y64 + bias_t[None, :], 2e-3 if tag == "f16" else 1e-2, "loaded int4 linear")
+
+    # the module's own state_dict (device layout) round-trips through a file as well
+    path2 = tmp_path / "device_int4.pt"
+    torch.save(mod.state_dict(), path2)
+    again = q.WeightOnlyInt4Linear(K, N, groupsize=g, bias=True, device=DEV, dtype=dtype)
+    again.load_state_dict(torch.load(path2, weights_only=True))
+    assert torch.equal(again(x), mod(x))
+
+    # the other ISA tiers of the CPU pack, written by the library's own CPU-layout kernel
+    from tensorplay_amd import ops
+    for cols, split in ((32, True), (32, False)):
+        other = q.WeightOnlyInt4Linear(K, N, groupsize=g, bias=True, device=DEV, dtype=dtype)
+        other.cpu_pack_layout = (cols, split)
+        w = ops._convert_weight_to_int4pack_for_cpu(dev(codes), 2, block_cols=cols, half_split=split).cpu()
+        other.load_state_dict({"weight": w, "scales_and_zeros": torch.from_numpy(sz32), "bias": torch.from_numpy(bias)})
+        assert torch.equal(other.weight, mod.weight)
+
+    # errors: wrong extent, and a module still on the CPU
+    with pytest.raises(RuntimeError, match="CPU-layout int4 weight must be"):
+        mod.load_state_dict({"weight": cpu_packed[:, :-2].contiguous(), "scales_and_zeros": torch.from_numpy(sz32),
+                             "bias": torch.from_numpy(bias)})
+    with pytest.raises(RuntimeError, match="move the module to the GPU"):
+        q.WeightOnlyInt4Linear(K, N, groupsize=g, bias=True).load_state_dict(
+            {"weight": cpu_packed, "scales_and_zeros": torch.from_numpy(sz32), "bias": torch.from_numpy(bias)})
+
+
+def test_bitnet_packed_linear_state_dict(tmp_path):
+    """`int_data` + `scale` are the on-disk form of the packed BitNet weight (the inner tensors of the reference's
+    subclass, bitnet.py:478-486): save, load into a fresh module, and the reference-style `weight` entry."""
+    from types import SimpleNamespace
+    q = _ao()
+    rng = np.random.default_rng(611)
+    M, K, N = 6, 256, 72
+    w = rng.normal(0, 0.05, (N, K)).astype(np.float32)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    lin = nn.Linear(K, N, bias=True).to(DEV)
+    with torch.no_grad():
+        lin.weight.copy_(dev(w))
+    mod = q.BitNetPacked2bitLinear.from_float(lin)
+    sd = mod.state_dict()
+    assert set(sd) == {"int_data", "scale", "bias"} and sd["int_data"].dtype == torch.uint8 and sd["scale"].dim() == 0
+    ocodes, oscale = oracle.quantize_bitnet_weight(w)
+    np.testing.assert_array_equal(host(sd["int_data"]), oracle.pack_ternary(ocodes))
+    path = tmp_path / "bitnet.pt"
+    torch.save(sd, path)
+
+    fresh = q.BitNetPacked2bitLinear(torch.zeros(N, K // 4, dtype=torch.uint8, device=DEV), 1.0, K,
+                                     bias=torch.zeros(N, device=DEV))
+    fresh.load_state_dict(torch.load(path, weights_only=True))
+    y = fresh(dev(x))
+    assert torch.equal(y, mod(dev(x)))
+    xq, xs = oracle.quantize_int8_rowwise(x, "f32", 1e-5)
+    want, _ = oracle.ternary_mm(xq, xs, oracle.pack_ternary(ocodes), float(sd["scale"]), K, bias=lin.bias.detach().cpu().numpy())
+    np.testing.assert_array_equal(host(y), want)
+
+    # a reference model's state_dict holds the subclass under `weight`; its inner tensors are int_data and scale
+    ref_style = {"weight": SimpleNamespace(int_data=sd["int_data"].cpu(), scale=sd["scale"].cpu().reshape(1)), "bias": sd["bias"].cpu()}
+    other = q.BitNetPacked2bitLinear(torch.zeros(N, K // 4, dtype=torch.uint8, device=DEV), 1.0, K, bias=torch.zeros(N, device=DEV))
+    other.load_state_dict(ref_style)
+    assert torch.equal(other(dev(x)), y)
+    with pytest.raises(RuntimeError, match="int_data and scale"):
+        other.load_state_dict({"weight": torch.zeros(3), "bias": sd["bias"]})

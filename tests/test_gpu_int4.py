@@ -247,6 +247,14 @@ def _fused_case(rng, M, N, K, tdt):
     return codes, torch.from_numpy(sz).to(tdt), x
 
 
+def _tile_subset(rng, n_tiles, count):
+    """Indices of up to `count` packed tiles (8 channels each), sorted, always with the first and the last."""
+    if n_tiles <= count:
+        return np.arange(n_tiles)
+    inner = rng.choice(np.arange(1, n_tiles - 1), size=count - 2, replace=False)
+    return np.sort(np.concatenate([[0, n_tiles - 1], inner]))
+
+
 @pytest.mark.parametrize("tdt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 4096, 1024), (19, 48, 384)])
 def test_mm_add_equals_the_two_ops(ops, tdt, M, N, K):
@@ -304,9 +312,11 @@ def test_mm_multi_equals_separate_products(ops, tdt, tol, M, K, widths):
     for (codes, sz, _), p, szd, y, n in zip(cases, packed, szs, got, widths):
         assert tuple(y.shape) == (M, n) and y.dtype == tdt
         assert_close_norm(y.float().cpu().numpy(), ops._weight_int4pack_mm(x, p, 128, szd).float().cpu().numpy(), tol)
-        if K <= 1024:
-            want = oracle.to_f32(oracle.int4_mm_tc(host(x), tag, oracle.int4_pack_tc(codes, 2), host(sz), 128), tag)
-            assert_close_norm(y.float().cpu().numpy(), want, 2 * tol)
+        # against the oracle on a subset of the output channels (whole packed tiles of 8, first and last included)
+        tiles = _tile_subset(rng, n // 8, 32)
+        cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+        want = oracle.to_f32(oracle.int4_mm_tc(host(x), tag, oracle.int4_pack_tc(codes[cols], 2), host(sz)[:, cols], 128), tag)
+        assert_close_norm(y.float().cpu().numpy()[:, cols], want, 2 * tol)
 
 
 def test_mm_multi_other_shapes_and_errors(ops):
@@ -338,3 +348,89 @@ def test_fused_entry_points_fall_back_for_other_shapes(ops):
     out = ops.int4pack_mm_swiglu(x, packed, packed, 32, sz, sz)
     g = ops._weight_int4pack_mm(x, packed, 32, sz).float()
     assert torch.equal(out, (g * torch.sigmoid(g) * g).half())
+
+
+# ---- the decoder layer of the benchmark configuration: seven int4 linears at batch 8 -----------------------------------
+
+class _LayerWeight:
+    """One int4 g=128 weight of the layer on the device, plus what the oracle needs for a subset of its channels."""
+
+    def __init__(self, ops, rng, n, k):
+        w = rng.normal(0, 0.02, (n, k)).astype(np.float32)
+        self.codes, sz = asym_quant(w, 128)
+        self.sz_bits = cast_bits(sz, "f16")                       # [K/128, N, 2] fp16 bits
+        self.packed = ops._convert_weight_to_int4pack(dev(self.codes), 2)
+        self.sz = dev(self.sz_bits, "f16")
+        self.n, self.k = n, k
+        tiles = _tile_subset(rng, n // 8, 48)                     # 384 channels: the oracle takes well under a second
+        self.cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+
+    def oracle_products(self, x_bits):
+        """(device formulation rounded to fp16 as float32, exact fp64 sums) on the channel subset."""
+        packed = oracle.int4_pack_tc(self.codes[self.cols], 2)
+        sz = np.ascontiguousarray(self.sz_bits[:, self.cols])
+        ref = oracle.to_f32(oracle.int4_mm_tc(x_bits, "f16", packed, sz, 128, round_w=True), "f16")
+        _, y64 = oracle.int4_mm_tc(x_bits, "f16", packed, sz, 128, round_w=False, want_f64=True)
+        return ref, y64
+
+
+def _check_product(got, weight, x_bits, what):
+    ref, y64 = weight.oracle_products(x_bits)
+    sub = got.float().cpu().numpy()[:, weight.cols]
+    assert_close_norm(sub, ref, 1e-2, f"{what} vs reference formulation")
+    assert rel_err(sub, y64) < 1e-3, f"{what} vs fp64 sums: {rel_err(sub, y64):.2e}"
+
+
+def test_decoder_layer_linears_batch8_against_oracle(ops):
+    """Llama-style layer, d = 4096, MLP 11008, batch 8, fp16, all seven linears int4 in groups of 128
+    (the reference's layer: benchmark/bench_llama_e2e.py:107-144), each through the entry point the layer uses:
+    q, k, v in one launch, o and down with the residual added in the epilogue, gate and up with the SwiGLU epilogue,
+    and each also through the plain op.  Checked against the oracle on 384 channels per weight: 1e-2 against the
+    reference's device formulation, 1e-3 against the fp64 sums."""
+    d, inter, M = 4096, 11008, 8
+    rng = np.random.default_rng(505)
+    print("config 5: building seven int4 weights", flush=True)
+    wq, wk, wv, wo = (_LayerWeight(ops, rng, d, d) for _ in range(4))
+    wg, wu = _LayerWeight(ops, rng, inter, d), _LayerWeight(ops, rng, inter, d)
+    wd = _LayerWeight(ops, rng, d, inter)
+    xb = cast_bits(rng.normal(0, 1, (M, d)).astype(np.float32), "f16")       # normed hidden state
+    hb = cast_bits(rng.normal(0, 0.3, (M, inter)).astype(np.float32), "f16")  # MLP activations
+    rb = cast_bits(rng.normal(0, 1, (M, d)).astype(np.float32), "f16")       # residual stream
+    x, h, res = dev(xb, "f16"), dev(hb, "f16"), dev(rb, "f16")
+
+    # q, k, v: one launch
+    print("config 5: q, k, v (int4pack_mm_multi)", flush=True)
+    qkv = ops.int4pack_mm_multi(x, [wq.packed, wk.packed, wv.packed], 128, [wq.sz, wk.sz, wv.sz])
+    for name, w, y in zip("qkv", (wq, wk, wv), qkv):
+        assert tuple(y.shape) == (M, d) and y.dtype == torch.float16
+        _check_product(y, w, xb, name)
+        _check_product(ops._weight_int4pack_mm(x, w.packed, 128, w.sz), w, xb, name + " (plain op)")
+
+    # o and down: residual added in the epilogue, out = T(T(x.W^T) + residual)
+    for name, w, inp, inp_bits in (("o", wo, x, xb), ("down", wd, h, hb)):
+        print(f"config 5: {name} (int4pack_mm_add, K = {w.k})", flush=True)
+        plain = ops._weight_int4pack_mm(inp, w.packed, 128, w.sz)
+        _check_product(plain, w, inp_bits, name + " (plain op)")
+        got = ops.int4pack_mm_add(inp, w.packed, 128, w.sz, res)
+        ref, y64 = w.oracle_products(inp_bits)
+        r32 = oracle.to_f32(rb, "f16")[:, w.cols]
+        want = oracle.to_f32(cast_bits(ref + r32, "f16"), "f16")              # both roundings of the separate ops
+        sub = got.float().cpu().numpy()[:, w.cols]
+        assert_close_norm(sub, want, 1e-2, f"{name} + residual vs reference formulation")
+        assert rel_err(sub, y64 + r32) < 1e-3, f"{name} + residual vs fp64"
+        assert torch.equal(got, (plain + res)), f"{name}: fused epilogue differs from the separate add"
+
+    # gate, up: one launch, silu_mul epilogue
+    print("config 5: gate, up (int4pack_mm_swiglu)", flush=True)
+    got = ops.int4pack_mm_swiglu(x, wg.packed, wu.packed, 128, wg.sz, wu.sz)
+    assert tuple(got.shape) == (M, inter)
+    cols = wu.cols = wg.cols   # same channels of both weights
+    g_ref, g64 = wg.oracle_products(xb)
+    u_ref, u64 = wu.oracle_products(xb)
+    want = g_ref * (1.0 / (1.0 + np.exp(-g_ref.astype(np.float64)))) * u_ref   # silu_mul of the two rounded products
+    exact = g64 * (1.0 / (1.0 + np.exp(-g64))) * u64
+    sub = got.float().cpu().numpy()[:, cols]
+    assert_close_norm(sub, want, 1e-2, "swiglu vs reference formulation")
+    assert rel_err(sub, exact) < 2e-3, f"swiglu vs fp64: {rel_err(sub, exact):.2e}"  # two fp16 roundings feed a product
+    _check_product(ops._weight_int4pack_mm(x, wg.packed, 128, wg.sz), wg, xb, "gate (plain op)")
+    _check_product(ops._weight_int4pack_mm(x, wu.packed, 128, wu.sz), wu, xb, "up (plain op)")

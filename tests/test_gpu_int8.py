@@ -133,10 +133,10 @@ def test_fused_dequant_bit_exact(ops, out_dtype, shape, with_bias):
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4])
 @pytest.mark.parametrize("K,N", [(4224, 50), (12288, 7), (256, 4100)])
-def test_row_kernel_one_to_four_rows(ops, M, K, N, monkeypatch):
+def test_row_kernel_one_to_four_rows(ops, M, K, N, kernel_override):
     """The kernel that streams the weight rows, for 1..4 activation rows (3 and 4 are not its default): raw sums exact,
     fused dequant equal to the oracle bit for bit in float32 and bfloat16, with a bias."""
-    monkeypatch.setenv("TPQ_INT8_ROW", "1")
+    kernel_override("int8_row", 1)
     rng = np.random.default_rng(M * 5 + K + N)
     x = rng.normal(0, 1, (M, K)).astype(np.float32)
     w = rng.normal(0, 0.02, (N, K)).astype(np.float32)

@@ -35,11 +35,13 @@ def ref_pack_binary(codes):
     return sum(((x[:, i::8] & 1) << i) for i in range(8)).astype(np.uint8)
 
 
-def dense_weight(codes, sz, group):
-    """(code - zero) * scale in float32 with sz [G, N, 2]."""
+def dense_weight(codes, sz, group, bits=None):
+    """(code - zero) * scale in float32 with sz [G, N, 2].  The reference's chain is unpack -> .to(int8) -> .to(float32)
+    (intx_weight_only.py:80, 119): at 8 bits the uint8 code is reinterpreted as int8 first (128 -> -128)."""
     s = np.repeat(sz[:, :, 0].T, group, axis=1)
     z = np.repeat(sz[:, :, 1].T, group, axis=1)
-    return ((codes.astype(np.float32) - z) * s).astype(np.float32)
+    c = codes.astype(np.uint8).view(np.int8) if bits == 8 else codes
+    return ((c.astype(np.float32) - z) * s).astype(np.float32)
 
 
 def make_case(rng, bits, N, K, group):
@@ -86,11 +88,31 @@ def test_oracle_mm_matches_float64_product(bits):
     bias = rng.standard_normal(N).astype(np.float32)
     out, y64, dense = oracle.lowbit_mm(x, "f32", ref_pack_msb_first(codes, bits), bits, sz, K, group, bias=bias,
                                        want_f64=True, want_dense=True)
-    dq = dense_weight(codes, sz, group)
+    dq = dense_weight(codes, sz, group, bits)
     np.testing.assert_array_equal(dense, dq)
     want = x.astype(np.float64) @ dq.astype(np.float64).T + bias
     np.testing.assert_allclose(y64, want, rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-5)
+
+
+def test_oracle_eight_bit_codes_are_signed_like_the_reference():
+    """bits = 8: unpack_intx returns codes.to(int8) and _dequantize_intx converts that to float, so bytes of 128 and
+    more dequantize as (byte - 256 - zero) * scale.  Hand-computed: bytes 0, 127, 128, 200, 255 with zero 3, scale 0.5."""
+    packed = np.array([[0, 127, 128, 200, 255, 1, 2, 3]], np.uint8)   # bits = 8: the packed bytes are the codes
+    sz = np.array([[[0.5, 3.0]]], np.float32)
+    x = np.eye(8, dtype=np.float32)
+    out, dense = oracle.lowbit_mm(x, "f32", packed, 8, sz, 8, 8, want_dense=True)
+    want = np.array([[-1.5, 62.0, -65.5, -29.5, -2.0, -1.0, -0.5, 0.0]], np.float32)
+    np.testing.assert_array_equal(dense, want)
+    np.testing.assert_array_equal(out, want.T)
+    # and through the numpy restatement of the reference's chain on random bytes
+    rng = np.random.default_rng(8)
+    codes, sz = make_case(rng, 8, 6, 32, 16)
+    assert (codes >= 128).any()
+    dense = oracle.lowbit_mm(None, "f32", ref_pack_msb_first(codes, 8), 8, sz, 32, 16, want_dense=True)[1]
+    unpacked_int8 = codes.astype(np.uint8).astype(np.int8)            # unpack_intx(...): uint8 fields, then .to(int8)
+    s, z = np.repeat(sz[:, :, 0].T, 16, axis=1), np.repeat(sz[:, :, 1].T, 16, axis=1)
+    np.testing.assert_array_equal(dense, (unpacked_int8.astype(np.float32) - z) * s)
 
 
 def test_oracle_binary_is_the_sign_times_scale():
@@ -168,12 +190,12 @@ def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
 @pytest.mark.parametrize("bits,lsb", [(1, False), (1, True), (2, False), (2, True), (4, False), (4, True), (8, False)])
 @pytest.mark.parametrize("N,K,group", [(10, 4096, 128), (7, 8192, 64), (130, 4160, 32), (5, 20480, 1024), (1, 64, 64), (36, 11008, 128)])
 @pytest.mark.parametrize("tdt,tag,tol", [(torch.float16, "f16", 1e-3), (torch.bfloat16, "bf16", 8e-3)])
-def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, monkeypatch):
+def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, kernel_override):
     """One activation row on the kernel that streams the packed rows: several passes per channel, a last segment
     past K, ragged N, both bit orders, both workgroup sizes (by K), groups of one segment and of many, with a bias.
-    TPQ_LOWBIT_ROW=1 pins the kernel (it is also the default for these shapes)."""
+    kernel_override("lowbit_row", 1) pins the kernel (it is also the default for these shapes)."""
     from tensorplay_amd import ops
-    monkeypatch.setenv("TPQ_LOWBIT_ROW", "1")
+    kernel_override("lowbit_row", 1)
     if group % {1: 64, 2: 64, 4: 32, 8: 16}[bits]:
         pytest.skip("the groups of this case are shorter than a lane's segment: other kernel, covered elsewhere")
     rng = np.random.default_rng(bits * 17 + K + N)
@@ -200,7 +222,7 @@ def test_gpu_mm_one_row_default_route_large_weight(bits, N, K):
     codes, sz = make_case(rng, bits, N, K, group)
     x16 = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).half()
     packed = oracle.lowbit_pack(codes, bits)
-    want = x16.double().numpy() @ dense_weight(codes, sz, group).astype(np.float64).T
+    want = x16.double().numpy() @ dense_weight(codes, sz, group, bits).astype(np.float64).T
     got = ops._lowbit_mm(x16.to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV))
     assert rel_err(got.float().cpu().numpy(), want) < 1e-3
 
@@ -229,13 +251,13 @@ def test_gpu_dequantize_bit_exact_and_many_rows(bits):
     codes, sz = make_case(rng, bits, N, K, group)
     packed = torch.from_numpy(oracle.lowbit_pack(codes, bits)).to(DEV)
     dense = ops._lowbit_dequantize(packed, bits, K, torch.from_numpy(sz).to(DEV), torch.float32)
-    np.testing.assert_array_equal(dense.cpu().numpy(), dense_weight(codes, sz, group))
+    np.testing.assert_array_equal(dense.cpu().numpy(), dense_weight(codes, sz, group, bits))
     dense16 = ops._lowbit_dequantize(packed, bits, K, torch.from_numpy(sz).to(DEV), torch.float16)
-    np.testing.assert_array_equal(dense16.cpu().numpy(), dense_weight(codes, sz, group).astype(np.float16))
+    np.testing.assert_array_equal(dense16.cpu().numpy(), dense_weight(codes, sz, group, bits).astype(np.float16))
     M = ops.LOWBIT_PREFILL_ROWS_SMALL + 5   # dequantise + library GEMM
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32))
     got = ops._lowbit_mm(x.to(DEV), packed, bits, K, torch.from_numpy(sz).to(DEV))
-    want = x.double().numpy() @ dense_weight(codes, sz, group).astype(np.float64).T
+    want = x.double().numpy() @ dense_weight(codes, sz, group, bits).astype(np.float64).T
     assert rel_err(got.cpu().numpy(), want) < 1e-5
 
 
@@ -250,7 +272,7 @@ def test_gpu_dequantize_vector_and_plain_kernels(bits, lsb_first, N, K, group):
     rng = np.random.default_rng(bits * 7 + K + int(lsb_first))
     codes, sz = make_case(rng, bits, N, K, group)
     packed = torch.from_numpy(oracle.lowbit_pack(codes, bits, lsb_first)).to(DEV)
-    want = torch.from_numpy(dense_weight(codes, sz, group))
+    want = torch.from_numpy(dense_weight(codes, sz, group, bits))
     szd = torch.from_numpy(sz).to(DEV)
     for dtype in (torch.float32, torch.float16, torch.bfloat16):
         got = ops._lowbit_dequantize(packed, bits, K, szd, dtype, lsb_first)
@@ -284,7 +306,7 @@ def test_gpu_modules_follow_the_reference_tests():
         modx = q.WeightOnlyIntxLinear.from_float(nn.Linear(16, 32, bias=True).to(DEV), bits=bits, groupsize=8)
         s = modx.scales_and_zeros[..., 0].t().contiguous().repeat_interleave(8, dim=-1)
         z = modx.scales_and_zeros[..., 1].t().contiguous().repeat_interleave(8, dim=-1)
-        codes = q.unpack_intx(modx.weight, bits, 16).view(torch.uint8).float()
+        codes = q.unpack_intx(modx.weight, bits, 16).float()   # int8, as the reference dequantizes it (8 bits wrap)
         torch.testing.assert_close(modx(x), x @ ((codes - z) * s).T + modx.bias, atol=1e-5, rtol=1e-5)
 
     model = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Linear(32, 8)).to(DEV)
@@ -314,3 +336,39 @@ def test_gpu_full_size_int2_decode_linearity():
     rows = slice(5000, 5064)
     want = oracle.lowbit_mm(xa.view(torch.int16).numpy().view(np.uint16), "f16", packed[rows], 2, sz[:, rows], K, group, want_f64=True)[1]
     assert rel_err(ya[:, rows].cpu().numpy(), want) < 1e-3
+
+
+@pytest.mark.gpu
+def test_gpu_from_float_quantizes_in_the_weight_dtype():
+    """from_float of the int2 / intx / binary modules quantizes the weight in its own dtype, as the reference does
+    (int2_weight_only.py:207, intx_weight_only.py:204-206, binary.py:151): for a float16 weight the division and the
+    rounding happen in float16, which picks other codes at ties than a float32 evaluation would.  The stored
+    parameters are the float16 values widened to float32."""
+    import torch.nn as nn
+    from tensorplay_amd.ao import quantization as q
+    torch.manual_seed(3)
+    lin = nn.Linear(64, 24, bias=False).to(DEV).half()
+    w = lin.weight.detach()
+
+    wg = w.reshape(24, 2, 32)
+    # intx, 3 bits: the reference's formulas (intx_weight_only.py:97-107) in float16
+    lo, hi = wg.min(-1).values, wg.max(-1).values
+    scale = ((hi - lo) / 7.0).clamp(min=1e-8)
+    zero = (-lo / scale).round().clamp(0, 7)
+    codes = ((wg - lo.unsqueeze(-1)) / scale.unsqueeze(-1)).round().clamp(0, 7).to(torch.uint8).reshape(24, 64)
+    mod = q.WeightOnlyIntxLinear.from_float(lin, bits=3, groupsize=32)
+    assert torch.equal(q.unpack_intx(mod.weight, 3, 64).view(torch.uint8), codes)
+    assert mod.scales_and_zeros.dtype == torch.float32
+    assert torch.equal(mod.scales_and_zeros[..., 0].t(), scale.float()) and torch.equal(mod.scales_and_zeros[..., 1].t(), zero.float())
+
+    # int2 (int2_weight_only.py:52-60) in float16
+    s2 = (wg.abs().amax(-1) / 2.0).clamp(min=1e-8)
+    c2 = ((wg / s2.unsqueeze(-1)).round() + 2.0).clamp(0, 3).to(torch.uint8).reshape(24, 64)
+    mod2 = q.WeightOnlyInt2Linear.from_float(lin, groupsize=32)
+    assert torch.equal(q.unpack_int2(mod2.weight, 64), c2)
+    assert torch.equal(mod2.scales_and_zeros[..., 0].t(), s2.float())
+
+    # binary (binary.py:36-47): per-row mean of |w| in float16
+    modb = q.WeightOnlyBinaryLinear.from_float(lin)
+    assert torch.equal(modb.scale, w.abs().mean(dim=-1, keepdim=True).clamp(min=1e-8).float())
+    assert torch.equal(q.unpack_binary(modb.weight, 64), (w >= 0).to(torch.uint8))
