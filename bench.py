@@ -33,10 +33,20 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 M, K, N, GROUP = 1, 4096, 11008, 128
 GEMV_BYTES = N * K // 2 + (K // GROUP) * N * 4 + 2 * M * K + 2 * M * N   # 23,983,616
-# HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
-# by what the same counter reads for a 256 MiB device copy (--calibrate-copy): 11770.35 KiB x 1.99973
-# fetched + 21.50 KiB x 1.0 written.  Summary: profiles/int4_decode_gemv_M1_K4096_N11008.md
-MEASURED_TRAFFIC_BYTES = 24_120_100
+GEMV_PROFILE = os.path.join(ROOT, "profiles", "int4_decode_gemv_M1_K4096_N11008.md")
+
+
+def measured_traffic_bytes():
+    """HBM bytes per launch of the GEMV kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
+    what the same counter reads for a 256 MiB device copy, --calibrate-copy).  The figure lives in the committed profile
+    summary, on a line `traffic_bytes_per_launch: <bytes> (commit <hash>)`; None when that file or line is missing."""
+    import re
+
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", open(GEMV_PROFILE).read(), flags=re.M)
+    except OSError:
+        return None
+    return int(m.group(1)) if m else None
 
 
 def asym_quant_int4(w, group):
@@ -89,36 +99,85 @@ def graph_of(fn):
     return g
 
 
-def cpu_baseline(x16, codes, sz16, want, budget_s=12.0):
-    """The CPU oracle's port of the reference's CPU int4 kernel (AVX-512 layout, 4-row x 64-column
-    tasks spread over threads), timed on the host on the full M=1 workload."""
+def host_description():
+    """What the CPU baseline ran on: logical CPUs the OS reports, CPUs this process may use, physical cores, model name
+    and the ISA tier that decides the reference's CPU int4 layout (64-column blocks on AVX-512, 32 on AVX2 / plain)."""
+    info = {"os_cpu_count": os.cpu_count()}
+    try:
+        info["usable_cpus"] = len(os.sched_getaffinity(0))
+    except AttributeError:
+        info["usable_cpus"] = os.cpu_count()
+    model, flags, cores = None, set(), set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name" and model is None:
+                model = val
+            elif key == "flags" and not flags:
+                flags = set(val.split())
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif not key and phys is not None and core is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    info["cpu_model"] = model
+    info["physical_cores"] = len(cores) or None
+    info["isa_tier"] = "avx512" if "avx512f" in flags else "avx2" if "avx2" in flags else "default"
+    return info
+
+
+def cpu_baseline(x16, codes, sz16, want, budget_s=8.0):
+    """The CPU oracle's port of the reference's CPU int4 kernel (AVX-512 layout, 4-row x 64-column tasks spread over
+    threads), timed on the host on the full M=1 workload at two thread counts: every CPU this process may use (the
+    box gives a one-GPU job a share of the host, so that is capped at 16) and 4, the default of the reference's own
+    benchmark (benchmark/bench_quantized_native.py:181).  The timed library is the oracle's source compiled with
+    -march=native on this host; if that build fails the portable AVX2 build is timed and the record says so."""
+    import tempfile
+
     import numpy as np
 
     import oracle
 
-    threads = max(1, min(16, os.cpu_count() or 1))
+    host = host_description()
+    native, build = None, "gcc -O3 -march=native"
+    try:
+        native = oracle.build_native(tempfile.mkdtemp(prefix="tpq_oracle_"))
+    except Exception as exc:  # no compiler on the host: the library that travelled with the repository
+        build = f"portable build (-mavx2 -mfma); native build failed: {str(exc)[:80]}"
     packed = oracle.int4_pack_cpu(codes, 64, True)
-    out = np.zeros((M, N), np.uint16)
     blocks = N // 64
-    per = (blocks + threads - 1) // threads
-    spans = [(b, min(b + per, blocks)) for b in range(0, blocks, per)]
-    pool = ThreadPoolExecutor(max_workers=threads)
 
-    def call():
-        list(pool.map(lambda sp: oracle.int4_mm_cpu_blocked(x16, "f16", packed, sz16, GROUP, sp, out), spans))
+    def timed(threads, budget):
+        out = np.zeros((M, N), np.uint16)
+        per = (blocks + threads - 1) // threads
+        spans = [(b, min(b + per, blocks)) for b in range(0, blocks, per)]
+        pool = ThreadPoolExecutor(max_workers=threads)
 
-    call()
-    err = float(np.abs(oracle.to_f32(out, "f16") - want).max() / np.abs(want).max())
-    t0 = time.perf_counter()
-    calls = 0
-    while True:
+        def call():
+            list(pool.map(lambda sp: oracle.int4_mm_cpu_blocked(x16, "f16", packed, sz16, GROUP, sp, out, library=native), spans))
+
         call()
-        calls += 1
-        dt = time.perf_counter() - t0
-        if dt > budget_s or calls >= 2000:
-            break
-    pool.shutdown()
-    per_call = dt / calls
+        err = float(np.abs(oracle.to_f32(out, "f16") - want).max() / np.abs(want).max())
+        t0 = time.perf_counter()
+        calls = 0
+        while True:
+            call()
+            calls += 1
+            dt = time.perf_counter() - t0
+            if dt > budget or calls >= 2000:
+                break
+        pool.shutdown()
+        return dt / calls, calls, err
+
+    all_threads = max(1, min(16, host["usable_cpus"] or 1))
+    per_call, calls, err = timed(all_threads, budget_s)
+    per_call4, calls4, _ = timed(min(4, all_threads), budget_s / 2)
     # the library twin the reference benchmarks its CPU op against (test_native_operator_families.py:579-599):
     # PyTorch's own CPU int4 kernel on the same codes, default thread count, a few seconds
     twin = None
@@ -142,10 +201,15 @@ def cpu_baseline(x16, codes, sz16, want, budget_s=12.0):
         "torch_cpu_twin": twin,
         "value": round(GEMV_BYTES / per_call / 1e9, 3),
         "unit": "GB/s",
-        "cores": threads,
+        "cores": all_threads,
         "kind": "port",
         "sample": f"{calls} calls of the full M=1 K=4096 N=11008 GEMV ({per_call * 1e6:.0f} us/call), "
                   f"oracle port of the reference CPU int4 kernel; max rel diff vs GPU {err:.2e}",
+        "four_threads": {"value": round(GEMV_BYTES / per_call4 / 1e9, 3), "unit": "GB/s", "cores": min(4, all_threads),
+                         "sample": f"{calls4} calls ({per_call4 * 1e6:.0f} us/call)"},
+        "host": host,
+        "build": build,
+        "layout": "64-column blocks, half-split nibbles (the reference's AVX-512 tier)",
     }
 
 
@@ -344,9 +408,38 @@ def main() -> int:
     gbs = GEMV_BYTES / (ms_per_step * 1e-3) / 1e9
 
     extras = {"gemv_max_rel_err_vs_fp64": gpu_err, "graph_wall_ms_per_step": wall_ms / steps}
+    roofline_int8 = None
     if not args.no_extras:  # the same graph seven more times: median step time
         reps = sorted(time_region(g.replay, sync, 1) / steps for _ in range(7))
         extras["int4_gemv_us_median_of_7_replays"] = reps[3] * 1e3
+    if not args.no_extras:
+        # The ceiling this kernel is held against: a pure read of the same number of bytes (packed weight + scales and
+        # zeros, 23,953,408 B, rotating through the same number of copies so that it comes from HBM), with every compute
+        # unit busy, 1 KB contiguous per wavefront load and all of it requested early; the best of a few shapes of
+        # that read.  And an empty kernel of the same grid: what a launch costs inside a graph when it moves nothing.
+        probe_bytes = (N * K // 2 + (K // GROUP) * N * 4) // 1024 * 1024
+        probe_bufs = [torch.empty(probe_bytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
+        sink = torch.zeros(256, dtype=torch.uint8, device=dev)
+        best = None
+        for wg, waves, loads, contiguous in ((256, 8, 4, 0), (256, 8, 12, 0), (256, 16, 8, 1), (512, 4, 12, 0)):
+            def read(i, wg=wg, waves=waves, loads=loads, contiguous=contiguous):
+                lib.tpq_probe_read(probe_bufs[i % copies].data_ptr(), probe_bytes, wg, waves, loads, contiguous, sink.data_ptr(), cur())
+
+            gp = graph_of(lambda: [read(i) for i in range(10 * copies)])
+            gp.replay(); sync()
+            us = steady(gp.replay, sync) / (10 * copies) * 1e3
+            if best is None or us < best[0]:
+                best = (us, f"{wg} workgroups x {waves} wavefronts, {loads} KB in flight each, {'contiguous runs' if contiguous else 'interleaved'}")
+            del gp
+        ge = graph_of(lambda: [lib.tpq_probe_read(None, 0, 256, 8, 4, 0, sink.data_ptr(), cur()) for _ in range(640)])
+        ge.replay(); sync()
+        extras["empty_kernel_in_graph_us"] = steady(ge.replay, sync) / 640 * 1e3
+        extras["int4_gemv_read_ceiling_us"] = best[0]
+        extras["int4_gemv_read_ceiling_GBs"] = probe_bytes / (best[0] * 1e-6) / 1e9
+        extras["int4_gemv_read_ceiling_pattern"] = best[1]
+        extras["int4_gemv_frac_of_read_ceiling"] = best[0] / extras["int4_gemv_us_median_of_7_replays"]
+        del probe_bufs, ge
+        torch.cuda.empty_cache()
     if args.calibrate_copy:
         src_c = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst_c = torch.empty_like(src_c)
@@ -454,6 +547,11 @@ def main() -> int:
         extras["int8_gemm_2048x4096x4096_us"] = ms * 1e3
         extras["int8_gemm_TOPS"] = tops
         extras["int8_gemm_frac_of_mfma_peak"] = tops / INT8_PEAK_TOPS
+        roofline_int8 = {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
+                         "kernel": "int8_gemm_dma_kernel<bf16 dequant epilogue> (tpq_int8_mm_dequant)",
+                         "algorithmic_ops_per_launch": 2 * M8 * N8 * K8, "avg_launch_us": ms * 1e3,
+                         "workload": "int8 x int8 prefill GEMM M=2048 K=4096 N=4096, fused per-row x per-channel dequant, bf16 out (BASELINE configs[2])"}
         # the vendor library's int8 GEMM on the same operands (torch._int_mm -> hipBLASLt), for scale: it
         # writes raw int32 sums, without the dequant epilogue that the kernel above includes
         try:
@@ -563,7 +661,21 @@ def main() -> int:
             key = f"ternary_M{mt}_{kt}x{nt}"
             extras[key + "_us"] = ms * 1e3
             if mt <= 8:
-                extras[key + "_GBs_cache_resident"] = (nt * kt // 4 + mt * kt + 4 * mt + 2 * mt * nt) / (ms * 1e-3) / 1e9
+                t_bytes = nt * kt // 4 + mt * kt + 4 * mt + 2 * mt * nt
+                extras[key + "_GBs_cache_resident"] = t_bytes / (ms * 1e-3) / 1e9
+                if mt == 1:  # the same call on 160 rotating copies of the packed weight (0.7 GB): streamed from HBM
+                    pks = [pk] + [pk.clone() for _ in range(159)]
+
+                    def tmm_rot(i, pks=pks, xq_t=xq_t, rs_t=rs_t, yt=yt, mt=mt, kt=kt, nt=nt):
+                        lib.tpq_ternary_mm(xq_t.data_ptr(), rs_t.data_ptr(), pks[i % 160].data_ptr(), 0.0173, None, mt, nt, kt,
+                                           yt.data_ptr(), _lib.F16, None, cur())
+
+                    gr = graph_of(lambda: [tmm_rot(i) for i in range(480)])
+                    gr.replay(); sync()
+                    ms_rot = steady(gr.replay, sync) / 480
+                    extras[key + "_hbm_rotated_us"] = ms_rot * 1e3
+                    extras[key + "_GBs_hbm_rotated"] = t_bytes / (ms_rot * 1e-3) / 1e9
+                    del pks, gr
             else:
                 extras[key + "_TOPS"] = 2.0 * mt * nt * kt / (ms * 1e-3) / 1e12
 
@@ -596,11 +708,12 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "traffic": measured_traffic_bytes(),
             "kernel": "int4_decode_kernel<f16, M=1, g=128>",
             "algorithmic_bytes_per_launch": GEMV_BYTES,
             "avg_launch_us": ms_per_step * 1e3,
         },
+        "roofline_int8": roofline_int8,
         "cpu_baseline": None,
         "extras": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in extras.items()},
     }

@@ -42,10 +42,11 @@ const char* tpq_last_error(void);
 
 /*
  * Which kernel serves a call is a function of the call's arguments alone; the library never reads the environment.
- * Two routes can be pinned for comparison runs and tests (no counterpart in the reference; results are bit-identical
- * on either side of both): "int8_row" (0: the int8 row-streaming kernel never runs, 1: it takes up to four
- * activation rows instead of two) and "lowbit_row" (0: the packed n-bit row kernel never runs, 1: it runs wherever
- * the shape allows).  value -1 restores the default rule.  Process-wide, atomic.
+ * Three routes can be pinned for comparison runs and tests (no counterpart in the reference): "int8_row" (0: the
+ * int8 row-streaming kernel never runs, 1: it takes up to four activation rows instead of two; integer sums, so the
+ * results are bit-identical either way), "lowbit_row" (0: the packed n-bit row kernel never runs, 1: it runs wherever
+ * the shape allows) and "int4_row" (the same for the int4 one-row kernel that deals whole tiles of eight channels to the
+ * compute units).  value -1 restores the default rule.  Process-wide, atomic.
  */
 int tpq_set_kernel_override(const char* route, int value);
 
@@ -338,6 +339,16 @@ int tpq_lowbit_pack(const uint8_t* codes, int bits, int lsb_first, int64_t rows,
                     uint8_t* packed, void* stream);
 int tpq_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, int64_t rows, int64_t cols,
                       uint8_t* codes, void* stream);
+
+/*
+ * Measurement probe, no counterpart in the reference: reads `bytes` (a multiple of 1024) of device memory and does
+ * nothing else, with `workgroups` x `waves` wavefronts that each keep `loads_in_flight` (2, 4, 8, 12, 16 or 24) 1 KB
+ * loads outstanding; `contiguous` = 1 gives every wavefront one contiguous run, 0 interleaves the wavefronts
+ * kilobyte by kilobyte.  bytes = 0 launches an empty kernel of the same grid.  `sink`: 256 bytes that are practically
+ * never written.  The benchmark uses it as the ceiling a bandwidth-bound kernel of the same footprint is held against.
+ */
+int tpq_probe_read(const void* src, int64_t bytes, int workgroups, int waves, int loads_in_flight, int contiguous,
+                   void* sink, void* stream);
 
 #ifdef __cplusplus
 }

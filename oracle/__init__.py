@@ -32,6 +32,18 @@ def build(force: bool = False) -> str:
     return _LIB_PATH
 
 
+def build_native(directory: str) -> ctypes.CDLL:
+    """The same source compiled with ``-march=native`` into `directory`, loaded and returned: the benchmark's CPU
+    baseline is timed with the host's full ISA (the library that travels with the repository is built for AVX2 so that
+    it runs on any host).  Raises if the compiler is missing or fails."""
+    out = os.path.join(directory, "liboracle_native.so")
+    flags = ["-O3", "-fPIC", "-std=c11", "-ffp-contract=off", "-fno-fast-math", "-fno-math-errno", "-fvisibility=hidden",
+             "-march=native"]
+    subprocess.run([os.environ.get("CC", "gcc"), *flags, "-shared", "-o", out, os.path.join(_HERE, "tpq_oracle.c"), "-lm"],
+                   check=True, capture_output=True)
+    return ctypes.CDLL(out)
+
+
 _lib = None
 
 
@@ -165,9 +177,9 @@ def int4_mm_cpu(x, dtype, packed, params, group, columns=64, half_split=True, ro
     return out
 
 
-def int4_mm_cpu_blocked(x, dtype, packed, params, group, blocks=None, out=None):
+def int4_mm_cpu_blocked(x, dtype, packed, params, group, blocks=None, out=None, library=None):
     """Vectorisable twin of int4_mm_cpu (64-column AVX-512 layout); `blocks` = (begin, end)
-    column blocks to compute, so that threads can split the work."""
+    column blocks to compute, so that threads can split the work; `library`: a build_native() library."""
     x = _c(x, storage(dtype))
     packed = _c(packed, np.uint8)
     params = _c(params, storage(dtype))
@@ -177,7 +189,7 @@ def int4_mm_cpu_blocked(x, dtype, packed, params, group, blocks=None, out=None):
     b0, b1 = (0, n // 64) if blocks is None else blocks
     if out is None:
         out = np.zeros((m, n), storage(dtype))
-    lib().orc_int4_mm_cpu_blocked(_p(x), _DT[dtype], _p(packed), _p(params), _p(out), ctypes.c_int64(m),
+    (library or lib()).orc_int4_mm_cpu_blocked(_p(x), _DT[dtype], _p(packed), _p(params), _p(out), ctypes.c_int64(m),
                                   ctypes.c_int64(n), ctypes.c_int64(k), ctypes.c_int64(group),
                                   ctypes.c_int64(b0), ctypes.c_int64(b1))
     return out

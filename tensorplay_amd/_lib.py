@@ -50,6 +50,7 @@ SIGNATURES = {
     "tpq_lowbit_dequantize": [_ptr, _int, _int, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],
     "tpq_lowbit_pack": [_ptr, _int, _int, _i64, _i64, _ptr, _ptr],
     "tpq_lowbit_unpack": [_ptr, _int, _int, _i64, _i64, _ptr, _ptr],
+    "tpq_probe_read": [_ptr, _i64, _int, _int, _int, _int, _ptr, _ptr],
     "tpq_dequantize_affine": [_ptr, _int, _int, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr],
 }
 

@@ -39,6 +39,7 @@
 #include "int4_lane.h"
 #include "int4_mfma_kernel.h"
 #include "int4_gemm_kernel.h"
+#include "int4_row_kernel.h"
 
 namespace tpq {
 namespace {
@@ -322,6 +323,7 @@ inline DecodePlan plan_decode(int N, int K, int mrows, size_t workspace_bytes) {
         if (ks > 64) ks = 64;
     }
     if (ks >= 2 && (wpb == 1 || wpb == 2 || wpb == 4 || wpb == 8 || wpb == 16)) plan = DecodePlan{wpb, ks};
+    if (const char* e = tuning_env("TPQ_INT4_WPB1")) plan = DecodePlan{std::atoi(e), 1};  // wavefronts per workgroup without slices (sweeps)
     return plan;
 }
 
@@ -533,9 +535,49 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
     return TPQ_OK;
 }
 
+// One activation row on the kernel that deals whole tiles of eight channels round-robin to one workgroup per compute
+// unit (int4_row_kernel.h); false if the shape does not fit it.
+template <int DT>
+bool launch_row(const void* x, const int32_t* packed, const void* sz, void* y, int N, int K, int group, hipStream_t s, int* rc) {
+    const char* force = tuning_env("TPQ_INT4_KERNEL");  // "row" pins it, any other value excludes it (sweeps)
+    const int pinned = g_override_int4_row.load(std::memory_order_relaxed);
+    if ((force && force[0] != 'r') || pinned == 0) return false;
+    if (K % 256 != 0 || K > 12288 || N % 8 != 0) return false;  // three 1 KB blocks per wavefront and tile at most (registers)
+    int cus = compute_units() / 32 * 32;
+    if (cus < 32) cus = 32;
+    const int n_tiles = N / 8;
+    const int blocks = K / 256;
+    const int seg = (blocks + kRowWaves - 1) / kRowWaves;
+    const int waves = (blocks + seg - 1) / seg;  // <= 16; the last one may own a segment past K (zero activations)
+    const int rounds = seg == 1 ? 6 : seg == 2 ? 3 : 2;
+    // Where it wins (measured, one row, fp16, us: this kernel / matrix-core kernel / column-per-lane kernel):
+    // 11008 -> 4096: 7.0 / 8.7 / 12.1;  5120 x 5120: 5.9 / 6.8 / 7.1.  Not for K <= 4096 (4096 -> 11008: 7.2 / 8.1 / 6.8;
+    // 4096 x 4096: 6.0 / 4.7 / 5.8), not when the tiles need a second batch of rounds (4096 -> 14336: 10.1 / 8.6 / 7.7;
+    // 8192 x 8192: 10.6 / 9.3 / 10.9), and a workgroup wants at least two tiles.
+    const bool wins = K > 4096 && n_tiles >= 2 * cus && n_tiles <= rounds * cus;
+    if (!(force || pinned == 1) && !wins) return false;
+    const int shift = group == 32 ? 0 : group == 64 ? 1 : group == 128 ? 2 : 3;
+    const dim3 grid(cus), block(waves * kWave);
+    const auto* xp = static_cast<const uint16_t*>(x);
+    const auto* pp = reinterpret_cast<const uint4*>(packed);
+    const auto* sp = static_cast<const uint32_t*>(sz);
+    auto* yp = static_cast<uint16_t*>(y);
+    switch (seg) {
+        case 1: int4_row_kernel<DT, 1, 1, 6><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
+        case 2: int4_row_kernel<DT, 1, 2, 3><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
+        default: int4_row_kernel<DT, 1, 3, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
+    }
+    *rc = check_launch("tpq_int4_mm (row)");
+    return true;
+}
+
 template <int DT>
 int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* sz, void* y, int N,
                   int K, int group, void* workspace, size_t workspace_bytes, hipStream_t s) {
+    if (M == 1) {
+        int rc;
+        if (launch_row<DT>(x, packed, sz, y, N, K, group, s, &rc)) return rc;
+    }
     // Many rows: the tiled kernel, the packed weight read once per 128 rows.  Measured against the 32-row slabs below
     // (us, fp16): K = 4096, N = 11008: 43 / 55 at 128 rows, 62 / 107 at 256, 258 / 821 at 2048; K = N = 8192:
     // 77 / 81 at 128, 82 / 157 at 256; at 96 rows the slabs still win (42 against 43, 63 against 77).

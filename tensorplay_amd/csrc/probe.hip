@@ -1,0 +1,70 @@
+// Measurement probe: a pure read of a device buffer, the ceiling that the bandwidth-bound decode kernels are held
+// against.  It does no arithmetic on what it reads beyond an exclusive-or that keeps the loads alive.
+//
+// Pattern: every wavefront load is 1 KB contiguous (16 bytes per lane); a wavefront issues all its loads of a round
+// before it looks at the first one, so the whole buffer is requested within the first microsecond when
+// workgroups x wavefronts x loads x 1 KB covers it.  Blocks of 1 KB are dealt to the wavefronts either interleaved
+// (wavefront w takes blocks w, w + W, w + 2 W, ...: neighbouring wavefronts read neighbouring kilobytes) or as one
+// contiguous run per wavefront.
+#include "tpq_common.h"
+
+namespace tpq {
+namespace {
+
+template <int LOADS>
+__global__ __launch_bounds__(1024) void read_probe_kernel(const uint4* __restrict__ src, int64_t blocks, int contiguous,
+                                                          uint32_t* __restrict__ sink) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t waves_per_group = blockDim.x / kWave;
+    const int64_t wave = blockIdx.x * waves_per_group + (threadIdx.x >> 6);
+    const int64_t total_waves = gridDim.x * waves_per_group;
+    const int64_t per_wave = (blocks + total_waves - 1) / total_waves;
+    uint32_t acc = 0;
+    for (int64_t r = 0; r < per_wave; r += LOADS) {
+        uint4 v[LOADS];
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            int64_t b = contiguous ? wave * per_wave + r + i : (r + i) * total_waves + wave;
+            const bool live = r + i < per_wave && b < blocks;
+            b = live ? b : 0;  // past the end: a valid block, not counted
+            v[i] = nt_load(src + b * kWave + lane);
+            if (!live) v[i] = make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    }
+    if (acc == 0x9E3779B9u && sink != nullptr) sink[wave & 63] = acc;  // practically never: keeps the loads alive
+}
+
+__global__ void empty_probe_kernel() {}
+
+}  // namespace
+}  // namespace tpq
+
+using namespace tpq;
+
+TPQ_EXPORT int tpq_probe_read(const void* src, int64_t bytes, int workgroups, int waves, int loads_in_flight, int contiguous,
+                              void* sink, void* stream) {
+    TPQ_REQUIRE(bytes >= 0 && bytes % 1024 == 0, TPQ_ERR_INVALID_VALUE, "probe_read: bytes must be a multiple of 1024");
+    TPQ_REQUIRE(workgroups >= 1 && waves >= 1 && waves <= 16, TPQ_ERR_INVALID_VALUE, "probe_read: 1..16 wavefronts per workgroup");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (bytes == 0) {  // the cost of a launch alone
+        empty_probe_kernel<<<workgroups, waves * kWave, 0, s>>>();
+        return check_launch("probe_read (empty)");
+    }
+    TPQ_REQUIRE(src && aligned(src, 16), TPQ_ERR_INVALID_VALUE, "probe_read: source must be 16-byte aligned");
+    const int64_t blocks = bytes / 1024;
+    const uint4* p = static_cast<const uint4*>(src);
+    uint32_t* out = static_cast<uint32_t*>(sink);
+    const dim3 grid(static_cast<unsigned>(workgroups)), block(static_cast<unsigned>(waves * kWave));
+    switch (loads_in_flight) {
+        case 2: read_probe_kernel<2><<<grid, block, 0, s>>>(p, blocks, contiguous, out); break;
+        case 4: read_probe_kernel<4><<<grid, block, 0, s>>>(p, blocks, contiguous, out); break;
+        case 8: read_probe_kernel<8><<<grid, block, 0, s>>>(p, blocks, contiguous, out); break;
+        case 12: read_probe_kernel<12><<<grid, block, 0, s>>>(p, blocks, contiguous, out); break;
+        case 16: read_probe_kernel<16><<<grid, block, 0, s>>>(p, blocks, contiguous, out); break;
+        case 24: read_probe_kernel<24><<<grid, block, 0, s>>>(p, blocks, contiguous, out); break;
+        default: return fail(TPQ_ERR_INVALID_VALUE, "probe_read: loads in flight must be 2, 4, 8, 12, 16 or 24");
+    }
+    return check_launch("probe_read");
+}

@@ -58,9 +58,10 @@ inline const char* tuning_env(const char* name) {
 #endif
 }
 
-// The two routes that tests pin explicitly (tpq_set_kernel_override): -1 = the default rule.
+// The routes that tests pin explicitly (tpq_set_kernel_override): -1 = the default rule.
 extern std::atomic<int> g_override_int8_row;    // 0 never / 1 up to four rows on the int8 row kernel
 extern std::atomic<int> g_override_lowbit_row;  // 0 never / 1 wherever the shape allows, the packed n-bit row kernel
+extern std::atomic<int> g_override_int4_row;    // 0 never / 1 wherever the shape allows, the int4 tile-streaming one-row kernel
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 

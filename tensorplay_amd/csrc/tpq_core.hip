@@ -220,6 +220,7 @@ TPQ_EXPORT int tpq_abi_version(void) { return 1; }
 namespace tpq {
 std::atomic<int> g_override_int8_row{-1};
 std::atomic<int> g_override_lowbit_row{-1};
+std::atomic<int> g_override_int4_row{-1};
 }  // namespace tpq
 
 TPQ_EXPORT int tpq_set_kernel_override(const char* route, int value) {
@@ -227,6 +228,7 @@ TPQ_EXPORT int tpq_set_kernel_override(const char* route, int value) {
     TPQ_REQUIRE(value >= -1 && value <= 1, TPQ_ERR_INVALID_VALUE, "tpq_set_kernel_override: value must be -1, 0 or 1");
     if (std::strcmp(route, "int8_row") == 0) tpq::g_override_int8_row.store(value, std::memory_order_relaxed);
     else if (std::strcmp(route, "lowbit_row") == 0) tpq::g_override_lowbit_row.store(value, std::memory_order_relaxed);
+    else if (std::strcmp(route, "int4_row") == 0) tpq::g_override_int4_row.store(value, std::memory_order_relaxed);
     else return tpq::fail(TPQ_ERR_INVALID_VALUE, "tpq_set_kernel_override: unknown route '%s'", route);
     return TPQ_OK;
 }

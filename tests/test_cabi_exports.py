@@ -92,6 +92,7 @@ def test_dispatch_does_not_depend_on_the_environment():
     assert "getenv" not in syms, "the library was built with -DTPQ_TUNING (sweep knobs compiled in)"
     assert lib.tpq_set_kernel_override(b"int8_row", 1) == 0 and lib.tpq_set_kernel_override(b"int8_row", -1) == 0
     assert lib.tpq_set_kernel_override(b"lowbit_row", 0) == 0 and lib.tpq_set_kernel_override(b"lowbit_row", -1) == 0
+    assert lib.tpq_set_kernel_override(b"int4_row", 1) == 0 and lib.tpq_set_kernel_override(b"int4_row", -1) == 0
     assert lib.tpq_set_kernel_override(b"no_such_route", 1) == _lib.TPQ_ERR_INVALID_VALUE
     assert "unknown route" in _lib.last_error()
     assert lib.tpq_set_kernel_override(b"int8_row", 5) == _lib.TPQ_ERR_INVALID_VALUE

@@ -434,3 +434,51 @@ def test_decoder_layer_linears_batch8_against_oracle(ops):
     assert rel_err(sub, exact) < 2e-3, f"swiglu vs fp64: {rel_err(sub, exact):.2e}"  # two fp16 roundings feed a product
     _check_product(ops._weight_int4pack_mm(x, wg.packed, 128, wg.sz), wg, xb, "gate (plain op)")
     _check_product(ops._weight_int4pack_mm(x, wu.packed, 128, wu.sz), wu, xb, "up (plain op)")
+
+
+# ---- one row on the kernel that deals whole tiles of eight channels to the compute units ---------------------------------
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("N,K,group", [
+    (4096, 256, 128),      # one block per tile: a single wavefront per workgroup
+    (2056, 2560, 128),     # ten wavefronts; fewer tiles than workgroups x 2, a last partial group of four tiles
+    (16400, 4096, 32),     # 16 wavefronts, nine rounds = two batches, groups of 32 (eight groups per block)
+    (4104, 5120, 64),      # two blocks per wavefront (ten wavefronts)
+    (2048, 11008, 128),    # three blocks per wavefront, 15 wavefronts, the last with a block past K
+    (520, 8192, 128),      # fewer tiles than workgroups: most workgroups idle
+])
+def test_mm_one_row_tile_streaming_kernel(ops, kernel_override, dtype, N, K, group):
+    """kernel_override("int4_row", 1) pins the one-row kernel for every shape it can take (its default shapes are few and
+    large): against the fp64 sums (1e-3 fp16, 1e-2 bf16), the reference's device formulation (1e-2), and the default route."""
+    rng = np.random.default_rng(N + K + group)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (1, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = oracle.int4_pack_tc(codes, 2)
+    args = (dev(xb, dtype), dev(packed), group, dev(szb, dtype))
+    default = ops._weight_int4pack_mm(*args).float().cpu().numpy()
+    kernel_override("int4_row", 1)
+    got = ops._weight_int4pack_mm(*args).float().cpu().numpy()
+    tiles = _tile_subset(rng, N // 8, 64)   # the oracle on 512 channels: first and last tile included
+    cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    sub_packed, sub_sz = oracle.int4_pack_tc(codes[cols], 2), np.ascontiguousarray(szb[:, cols])
+    ref_dev = oracle.to_f32(oracle.int4_mm_tc(xb, dtype, sub_packed, sub_sz, group, round_w=True), dtype)
+    _, y64 = oracle.int4_mm_tc(xb, dtype, sub_packed, sub_sz, group, round_w=False, want_f64=True)
+    assert_close_norm(got[:, cols], ref_dev, 1.5e-2 if dtype == "bf16" else 1e-2, "row kernel vs reference formulation")
+    assert rel_err(got[:, cols], y64) < (1e-3 if dtype == "f16" else 1e-2)
+    # every channel against the default route (another kernel, another order of the fp32 additions)
+    assert rel_err(got, default) < (2e-3 if dtype == "f16" else 1.6e-2)
+
+
+def test_mm_one_row_down_projection_default_route(ops):
+    """11008 -> 4096 at one row: the shape the tile-streaming kernel serves by default."""
+    rng = np.random.default_rng(77)
+    N, K = 4096, 11008
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), 128)
+    xb, szb = cast_bits(rng.normal(0, 1, (1, K)).astype(np.float32), "f16"), cast_bits(sz, "f16")
+    got = ops._weight_int4pack_mm(dev(xb, "f16"), dev(oracle.int4_pack_tc(codes, 2)), 128, dev(szb, "f16")).float().cpu().numpy()
+    tiles = _tile_subset(rng, N // 8, 48)
+    cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    _, y64 = oracle.int4_mm_tc(xb, "f16", oracle.int4_pack_tc(codes[cols], 2), np.ascontiguousarray(szb[:, cols]), 128,
+                               round_w=False, want_f64=True)
+    assert rel_err(got[:, cols], y64) < 1e-3
