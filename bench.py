@@ -421,7 +421,8 @@ def main() -> int:
         probe_bufs = [torch.empty(probe_bytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
         sink = torch.zeros(256, dtype=torch.uint8, device=dev)
         best = None
-        for wg, waves, loads, contiguous in ((256, 8, 4, 0), (256, 8, 12, 0), (256, 16, 8, 1), (512, 4, 12, 0)):
+        # (the last shape is the column-per-lane pattern of the decode kernel itself: `contiguous` = K / 128, one workgroup per 64 columns)
+        for wg, waves, loads, contiguous in ((256, 8, 4, 0), (256, 8, 12, 0), (256, 16, 8, 1), (512, 4, 12, 0), (1, 16, 8, K // 128)):
             def read(i, wg=wg, waves=waves, loads=loads, contiguous=contiguous):
                 lib.tpq_probe_read(probe_bufs[i % copies].data_ptr(), probe_bytes, wg, waves, loads, contiguous, sink.data_ptr(), cur())
 
@@ -429,7 +430,8 @@ def main() -> int:
             gp.replay(); sync()
             us = steady(gp.replay, sync) / (10 * copies) * 1e3
             if best is None or us < best[0]:
-                best = (us, f"{wg} workgroups x {waves} wavefronts, {loads} KB in flight each, {'contiguous runs' if contiguous else 'interleaved'}")
+                best = (us, f"column-per-lane pattern, one workgroup of {waves} wavefronts per 64 columns, all loads in flight" if contiguous >= 2 else
+                        f"{wg} workgroups x {waves} wavefronts, {loads} KB in flight each, {'contiguous runs' if contiguous else 'interleaved'}")
             del gp
         ge = graph_of(lambda: [lib.tpq_probe_read(None, 0, 256, 8, 4, 0, sink.data_ptr(), cur()) for _ in range(640)])
         ge.replay(); sync()

@@ -344,7 +344,9 @@ int tpq_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, int64_t ro
  * Measurement probe, no counterpart in the reference: reads `bytes` (a multiple of 1024) of device memory and does
  * nothing else, with `workgroups` x `waves` wavefronts that each keep `loads_in_flight` (2, 4, 8, 12, 16 or 24) 1 KB
  * loads outstanding; `contiguous` = 1 gives every wavefront one contiguous run, 0 interleaves the wavefronts
- * kilobyte by kilobyte.  bytes = 0 launches an empty kernel of the same grid.  `sink`: 256 bytes that are practically
+ * kilobyte by kilobyte; `contiguous` >= 2 selects the access pattern of the column-per-lane decode kernel for a packed
+ * int4 weight with K = 128 x contiguous (one workgroup per 64 columns, `workgroups` ignored, 16-byte loads that touch
+ * eight 128-byte lines per wavefront).  bytes = 0 launches an empty kernel of the same grid.  `sink`: 256 bytes that are practically
  * never written.  The benchmark uses it as the ceiling a bandwidth-bound kernel of the same footprint is held against.
  */
 int tpq_probe_read(const void* src, int64_t bytes, int workgroups, int waves, int loads_in_flight, int contiguous,

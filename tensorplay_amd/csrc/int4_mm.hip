@@ -62,7 +62,12 @@ struct Chunk {
 // partials in slice order (so the result does not depend on arrival order), stores y and puts
 // the counter back to zero.  Partials and counter move with agent-scope atomic accesses, which
 // are coherent across the chip's L2 slices.
-template <int DT, int MROWS, int GROUP_KT, int WPB>
+// CPW > 0: every wavefront owns exactly CPW chunks (K = 128 x WPB x CPW, one workgroup per column group) and the code
+// from the first load to the LDS exchange is free of branches: all loads are issued up front, the small ones first,
+// and the k-tiles are consumed one by one as they arrive.  With a loop and its bounds checks around the chunks
+// (CPW = 0) the compiler waits for every outstanding load before the first use, which leaves the whole
+// arithmetic of the wavefront (two chunks: about 400 vector instructions) behind the end of the stream.
+template <int DT, int MROWS, int GROUP_KT, int WPB, int CPW = 0>
 __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
     const uint32_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
     uint16_t* __restrict__ y, int N, int K, int k_super, float* ws_part, unsigned* ws_count) {
@@ -156,7 +161,28 @@ __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
         }
     };
 
-    const int slices = gridDim.y;
+    const int slices = CPW > 0 ? 1 : gridDim.y;
+    if constexpr (CPW > 0) {
+        Chunk<MROWS, kGroups> own[CPW];
+        // (scale, zero) words and this lane's activation word of every chunk first: loads return in issue order, and
+        // the sums of the activations are the first thing a chunk needs
+#pragma unroll
+        for (int u = 0; u < CPW; ++u) {
+            const int chunk = wave + u * WPB;
+#pragma unroll
+            for (int m = 0; m < MROWS; ++m) own[u].xw[m] = x[static_cast<size_t>(m) * words_per_row + chunk * 64 + lane];
+#pragma unroll
+            for (int g = 0; g < kGroups; ++g) own[u].p[g] = nt_load(szp + static_cast<size_t>(chunk * kGroups + g) * N);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < CPW; ++u)
+#pragma unroll
+            for (int i = 0; i < kChunkKT; ++i) own[u].q[i] = nt_load(wp + static_cast<size_t>((wave + u * WPB) * kChunkKT + i) * 8);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < CPW; ++u) consume(own[u], wave + u * WPB);
+    } else {
     const int stride = WPB * slices;                 // chunks between two turns of this wavefront
     const int first = blockIdx.y * WPB + wave;
     Chunk<MROWS, kGroups> ring[kRing];
@@ -171,6 +197,7 @@ __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
                 if (cu + kRing * stride < n_chunks) issue(ring[u], cu + kRing * stride);
             }
         }
+    }
     }
 
     // wavefronts of the workgroup meet in LDS
@@ -338,10 +365,20 @@ int launch_decode_rows(const void* x, const int32_t* packed, const void* sz, voi
     auto* yp = static_cast<uint16_t*>(y);
     auto* counters = static_cast<unsigned*>(workspace);
     auto* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kCounterBytes);
+    auto run = [&](auto gkt) {
+        constexpr int G = decltype(gkt)::value;
+        if (WPB == 16 && slices == 1 && !tuning_env("TPQ_DECODE_LOOP")) {  // the branch-free body where the chunks divide evenly
+            const int n_chunks = K / 128;
+            if (n_chunks == 16) { int4_decode_kernel<DT, MROWS, G, WPB, 1><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+            if (n_chunks == 32) { int4_decode_kernel<DT, MROWS, G, WPB, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+            if (n_chunks == 48 && MROWS == 1 && G == 4) { int4_decode_kernel<DT, MROWS, G, WPB, 3><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+        }
+        int4_decode_kernel<DT, MROWS, G, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters);
+    };
     switch (group) {
-        case 32: int4_decode_kernel<DT, MROWS, 1, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); break;
-        case 64: int4_decode_kernel<DT, MROWS, 2, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); break;
-        default: int4_decode_kernel<DT, MROWS, 4, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); break;
+        case 32: run(std::integral_constant<int, 1>{}); break;
+        case 64: run(std::integral_constant<int, 2>{}); break;
+        default: run(std::integral_constant<int, 4>{}); break;
     }
     return check_launch("tpq_int4_mm (decode)");
 }

@@ -36,6 +36,36 @@ __global__ __launch_bounds__(1024) void read_probe_kernel(const uint4* __restric
     if (acc == 0x9E3779B9u && sink != nullptr) sink[wave & 63] = acc;  // practically never: keeps the loads alive
 }
 
+// The access pattern of the column-per-lane decode kernel, without its arithmetic: workgroup = 64 columns = eight
+// tiles of the packed layout (k_super x 128 bytes each), 16 wavefronts, wavefront w reads the chunks (four k-tiles)
+// w, w + 16, ...; lane l = row l % 8 of tile l / 8, 16 bytes per k-tile: a wavefront load touches eight 128-byte
+// lines that lie k_super x 128 bytes apart.  All loads of a wavefront are issued before the first use.
+template <int CHUNKS>
+__global__ __launch_bounds__(1024) void read_probe_columns_kernel(const uint4* __restrict__ src, int n_tiles, int k_super,
+                                                                  uint32_t* __restrict__ sink) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    int tile = blockIdx.x * 8 + (lane >> 3);
+    tile = tile < n_tiles ? tile : n_tiles - 1;
+    const uint4* base = src + (static_cast<size_t>(tile) * k_super) * 8 + (lane & 7);
+    const int n_chunks = k_super / 4;
+    uint32_t acc = 0;
+    for (int c0 = wave; c0 < n_chunks; c0 += waves * CHUNKS) {
+        uint4 v[CHUNKS][4];
+#pragma unroll
+        for (int u = 0; u < CHUNKS; ++u) {
+            int c = c0 + u * waves;
+            c = c < n_chunks ? c : n_chunks - 1;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[u][i] = nt_load(base + static_cast<size_t>(c * 4 + i) * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < CHUNKS; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc ^= v[u][i].x ^ v[u][i].y ^ v[u][i].z ^ v[u][i].w;
+    }
+    if (acc == 0x9E3779B9u && sink != nullptr) sink[wave & 63] = acc;
+}
+
 __global__ void empty_probe_kernel() {}
 
 }  // namespace
@@ -53,6 +83,14 @@ TPQ_EXPORT int tpq_probe_read(const void* src, int64_t bytes, int workgroups, in
         return check_launch("probe_read (empty)");
     }
     TPQ_REQUIRE(src && aligned(src, 16), TPQ_ERR_INVALID_VALUE, "probe_read: source must be 16-byte aligned");
+    if (contiguous >= 2) {  // the column-per-lane pattern: `workgroups` is ignored, one per 64 columns; K = 128 x contiguous
+        const int k_super = contiguous * 4;  // contiguous = K / 128
+        const int n_tiles = static_cast<int>(bytes / (static_cast<int64_t>(k_super) * 128));
+        const dim3 g((n_tiles + 7) / 8), b(static_cast<unsigned>(waves * kWave));
+        if (loads_in_flight >= 8) read_probe_columns_kernel<2><<<g, b, 0, s>>>(static_cast<const uint4*>(src), n_tiles, k_super, static_cast<uint32_t*>(sink));
+        else read_probe_columns_kernel<1><<<g, b, 0, s>>>(static_cast<const uint4*>(src), n_tiles, k_super, static_cast<uint32_t*>(sink));
+        return check_launch("probe_read (columns)");
+    }
     const int64_t blocks = bytes / 1024;
     const uint4* p = static_cast<const uint4*>(src);
     uint32_t* out = static_cast<uint32_t*>(sink);
