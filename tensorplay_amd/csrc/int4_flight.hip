@@ -1,0 +1,139 @@
+// Launcher of the all-in-flight matrix-core int4 kernel: picks the workgroup width and the instantiation.
+#include "int4_flight.h"
+
+#include <cstdlib>
+
+#include "int4_mfma_flight_kernel.h"
+
+namespace tpq {
+namespace {
+
+inline int flight_compute_units() {
+    static std::atomic<int> cached{0};
+    int v = cached.load(std::memory_order_relaxed);
+    if (v == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        v = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
+        cached.store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
+
+template <int DT, int NB, int SPW, int XR, int MODE>
+int launch_as(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
+    constexpr size_t bytes = flight_lds_bytes<NB, SPW, XR>();
+    static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
+    static std::atomic<uint64_t> reserved{0};
+    const auto kernel = int4_mfma_flight_kernel<DT, NB, SPW, XR, MODE>;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), bytes, reserved, "tpq_int4_mm (mfma, all in flight)")) return rc;
+    constexpr int C = MODE == kFlightPair ? NB / 2 : NB;
+    kernel<<<dim3((blocks + C - 1) / C), dim3(kFlightWaves * kWave), bytes, s>>>(x, set, rows, K, shift, residual);
+    return check_launch("tpq_int4_mm (mfma, all in flight)");
+}
+
+// the row capacity: 4, 8 or 16 rows through LDS
+template <int DT, int NB, int SPW, int MODE>
+int launch_rows(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
+    if (rows <= 4) return launch_as<DT, NB, SPW, 4, MODE>(x, rows, set, blocks, K, shift, residual, s);
+    if (rows <= 8) return launch_as<DT, NB, SPW, 8, MODE>(x, rows, set, blocks, K, shift, residual, s);
+    if constexpr (flight_lds_bytes<NB, SPW, 16>() <= 160 * 1024 && SPW <= 4) {
+        return launch_as<DT, NB, SPW, 16, MODE>(x, rows, set, blocks, K, shift, residual, s);
+    } else {
+        return TPQ_ERR_UNSUPPORTED;  // not reached: flight_shape() excludes the case
+    }
+}
+
+// Workgroup width (blocks of 16 channels) for `blocks` blocks in all, or 0 when the kernel is not built for the case.
+// spw = steps per wavefront; the registers hold spw x width weight loads in flight, so long K means narrow workgroups.
+// Measured at K = 4096, fp16 (us, loop kernel / this kernel at widths 1, 2, 3, 4):
+//   N = 4096, 8 rows: 5.4 / 4.5 5.1 5.6 6.3     N = 8192, 8 rows: 6.4 / 7.6 5.7 6.1 6.9
+//   N = 11008, 8 rows: 8.4 / 10.5 9.2 6.7 7.4    N = 16384, 8 rows: 9.7 / 14.0 10.2 11.6 9.1
+//   N = 32000, 2 rows: 17.0 / 17.4 14.5 16.9 14.9;  8 rows: 17.9 / 25.8 18.1 17.0 15.4
+// One workgroup per compute unit and pass: the narrowest width that needs one pass.  Several passes pay off only with
+// two steps per wavefront or at most four rows (5120 -> 13824, 8 rows: 11.7 us against 10.5 for the loop kernel;
+// 8192 -> 10240: 16.2 against 13.2; at 2 rows 10.0 / 10.4 and 12.4 / 12.9): then the width with the fewest
+// passes x width, or 2 for few rows (their small LDS tiles let two workgroups share a compute unit).
+int flight_width(int blocks, int rows, int spw, bool pair) {
+    const int cus = flight_compute_units();
+    const int widest = pair ? 3 : spw <= 2 ? 4 : spw <= 4 ? 2 : 1;
+    for (int nb = 1; nb <= widest; ++nb)
+        if ((blocks + nb - 1) / nb <= cus) return nb;
+    if (spw > 2 && rows > 4) return 0;
+    if (rows <= 4 && widest >= 2 && !pair) return 2;
+    int best = widest, cost = 1 << 30;
+    for (int nb = widest; nb >= 1; --nb) {
+        const int c = ((blocks + nb - 1) / nb + cus - 1) / cus * nb;
+        if (c < cost) { cost = c; best = nb; }
+    }
+    return best;
+}
+
+template <int DT>
+bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group, bool pair, const void* residual, hipStream_t s, int* rc) {
+    if (rows < 2 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256)) return false;
+    const int steps = K / 128;
+    const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
+    if (steps < kFlightWaves || spw > 7 || spw == 5) return false;
+    // five and more steps per wavefront at more than eight rows: the tiles of 16 rows keep one step in LDS at a time and
+    // the registers fill up (11008 -> 4096 at 16 rows: 17.7 us against 14.0 for the loop kernel)
+    if (spw > 4 && rows > 8) return false;
+    if (wts.count < 1 || wts.count > kFlightMaxWeights || (pair && (wts.count != 2 || wts.N[0] != wts.N[1] || spw != 2))) return false;
+    // gate / up at more than eight rows: the tiles of 16 rows leave LDS for two blocks of each weight only, and the
+    // loop kernel is faster then (4096 -> 11008 at 12 rows: 15.9 us against 17.1)
+    if (pair && rows > 8) return false;
+    if (residual != nullptr && (wts.count != 1 || pair || !aligned(residual, 8))) return false;
+    FlightSet set{};
+    FlightWeight* const slots[kFlightMaxWeights] = {&set.w0, &set.w1, &set.w2, &set.w3};
+    set.count = pair ? 1 : wts.count;
+    int blocks = 0;
+    for (int w = 0; w < wts.count; ++w) {
+        if (wts.N[w] % 8 != 0 || !aligned(wts.sz[w], 4) || !aligned(wts.packed[w], 16) || !aligned(wts.y[pair ? 0 : w], 8)) return false;
+        slots[w]->packed = static_cast<const uint4*>(wts.packed[w]);
+        slots[w]->sz = static_cast<const uint32_t*>(wts.sz[w]);
+        slots[w]->y = static_cast<uint16_t*>(wts.y[pair ? 0 : w]);
+        slots[w]->N = wts.N[w];
+        slots[w]->first = pair ? 0 : blocks;
+        if (!pair || w == 0) blocks += (wts.N[w] + 15) / 16;
+    }
+    int nb = flight_width(blocks, rows, spw, pair);
+    if (const char* env = tuning_env("TPQ_INT4_FLIGHT")) nb = std::atoi(env);  // 0 switches the kernel off, 1..4 pin the width
+    if (nb <= 0) return false;
+    const auto* xp = static_cast<const uint16_t*>(x);
+    const auto* rp = static_cast<const uint16_t*>(residual);
+    const int shift = group == 128 ? 0 : 1;
+    int code = TPQ_ERR_UNSUPPORTED;
+    if (pair) {
+        if (nb >= 3 && rows <= 8) code = launch_rows<DT, 6, 2, kFlightPair>(xp, rows, set, blocks, K, shift, rp, s);
+        else if (nb >= 2) code = launch_rows<DT, 4, 2, kFlightPair>(xp, rows, set, blocks, K, shift, rp, s);
+        else code = launch_rows<DT, 2, 2, kFlightPair>(xp, rows, set, blocks, K, shift, rp, s);
+    } else {
+#define TPQ_FLIGHT(NBV, SPWV)                                                                                   \
+    code = wts.count == 1 ? launch_rows<DT, NBV, SPWV, kFlightOne>(xp, rows, set, blocks, K, shift, rp, s)    \
+                          : launch_rows<DT, NBV, SPWV, kFlightMany>(xp, rows, set, blocks, K, shift, rp, s)
+        switch (spw) {
+            case 1: case 2:
+                if (nb == 1) TPQ_FLIGHT(1, 2); else if (nb == 2) TPQ_FLIGHT(2, 2); else if (nb == 3) TPQ_FLIGHT(3, 2); else TPQ_FLIGHT(4, 2);
+                break;
+            case 3: if (nb == 1) TPQ_FLIGHT(1, 3); else TPQ_FLIGHT(2, 3); break;
+            case 4: if (nb == 1) TPQ_FLIGHT(1, 4); else TPQ_FLIGHT(2, 4); break;
+            case 6: TPQ_FLIGHT(1, 6); break;
+            case 7: TPQ_FLIGHT(1, 7); break;
+            default: return false;
+        }
+#undef TPQ_FLIGHT
+    }
+    *rc = code;
+    return true;
+}
+
+}  // namespace
+
+bool flight_launch(int dtype, const void* x, int rows, const FlightWeights& weights, int K, int group, bool pair,
+                   const void* residual, hipStream_t stream, int* rc) {
+    if (dtype == TPQ_DTYPE_F16) return launch<TPQ_DTYPE_F16>(x, rows, weights, K, group, pair, residual, stream, rc);
+    if (dtype == TPQ_DTYPE_BF16) return launch<TPQ_DTYPE_BF16>(x, rows, weights, K, group, pair, residual, stream, rc);
+    return false;
+}
+
+}  // namespace tpq

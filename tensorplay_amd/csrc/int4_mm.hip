@@ -36,6 +36,7 @@
 // (p10/src/backend/cpu/QuantizedElementwiseKernels.cpp:470-479).
 #include <cstdlib>
 
+#include "int4_flight.h"
 #include "int4_lane.h"
 #include "int4_mfma_kernel.h"
 #include "int4_gemm_kernel.h"
@@ -452,6 +453,11 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     //                rows against 8.4 / 8.5 / 9.0 / 9.3 for the next best; 8192 -> 28672, 8 rows: 27.4 against 30.4),
     //                64 ch x 4 waves above (16 rows: 9.7 us against 12.3 for 32 ch)
     //   N > 28672:   32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (4096 -> 32000, 4 rows: 16.2 against 16.6)
+    if (rows > 1 && !(force && force[0] == 'm')) {  // the all-in-flight form, where it is built
+        FlightWeights one{};
+        one.packed[0] = packed; one.sz[0] = sz; one.y[0] = y; one.N[0] = N; one.count = 1;
+        if (flight_launch(DT, x, rows, one, K, group, false, residual, s, rc)) return true;
+    }
     const bool wide = N >= 10240 && N <= 28672 && rows <= 12;
     int nb = N > 4096 ? (N < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
     if (const char* env = tuning_env("TPQ_INT4_NB")) nb = std::atoi(env);
@@ -516,6 +522,13 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
         char* ys = static_cast<char*>(y) + m0 * row_y;
         int rc = TPQ_OK;
         if (packed_b != nullptr) {
+            FlightWeights two{};
+            two.packed[0] = packed; two.packed[1] = packed_b; two.sz[0] = sz; two.sz[1] = sz_b; two.y[0] = ys; two.N[0] = two.N[1] = N;
+            two.count = 2;
+            if (flight_launch(DT, xs, rows, two, K, group, true, nullptr, s, &rc)) {
+                if (rc != TPQ_OK) return rc;
+                continue;
+            }
             static const int pair_waves = [] { const char* e = tuning_env("TPQ_INT4_PAIR_WAVES"); return e ? std::atoi(e) : 4; }();
             const auto* xp = reinterpret_cast<const uint16_t*>(xs);
             const auto* pa = reinterpret_cast<const uint4*>(packed);
@@ -546,6 +559,19 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
     for (int w = 0; w < count; ++w) n_total += N[w];
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
+        {
+            FlightWeights all{};
+            all.count = count;
+            for (int w = 0; w < count; ++w) {
+                all.packed[w] = packed[w]; all.sz[w] = sz[w]; all.N[w] = static_cast<int>(N[w]);
+                all.y[w] = static_cast<uint16_t*>(y[w]) + m0 * N[w];
+            }
+            int rc = TPQ_OK;
+            if (flight_launch(DT, static_cast<const uint16_t*>(x) + m0 * K, rows, all, K, group, false, nullptr, s, &rc)) {
+                if (rc != TPQ_OK) return rc;
+                continue;
+            }
+        }
         const bool wide = n_total >= 10240 && n_total <= 28672 && rows <= 12;
         const int nb = n_total > 4096 ? (n_total < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
         const int waves = n_total < 10240 || wide ? 8 : 4;

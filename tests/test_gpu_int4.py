@@ -245,6 +245,49 @@ def test_mm_many_rows_takes_the_dense_route(ops, dtype):
 
 # ---- fusions around the decode matmul --------------------------------------------------------------
 
+FLIGHT_CASES = [  # M, N, K, group: the all-in-flight matrix-core kernel (K >= 2048, 2..16 rows, groups of 128)
+    (2, 72, 2048, 128),      # 16 steps: one per wavefront, the second one dead; half a block at the end
+    (3, 200, 4096, 128),     # four rows through LDS
+    (5, 4104, 4096, 128),    # eight rows, 257 blocks: two per workgroup
+    (8, 11008, 4096, 128),   # the decode configuration: three blocks per workgroup
+    (4, 16392, 4096, 128),   # more blocks than four per compute unit cover in one pass
+    (9, 136, 4096, 128),     # 16 rows through LDS, one step resident at a time
+    (16, 264, 5120, 128),    # 40 steps: three per wavefront, the third dead for half of them
+    (4, 520, 6144, 128),     # 48 steps
+    (7, 136, 8192, 128),     # four steps per wavefront
+    (8, 4104, 11008, 128),   # 86 steps: six per wavefront, one block per workgroup
+    (13, 72, 11008, 128),
+    (6, 264, 14336, 128),    # seven steps per wavefront
+    (12, 264, 14336, 128),   # (that many steps at more than eight rows: the loop kernel)
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,group", FLIGHT_CASES)
+def test_mm_all_in_flight_kernel_matches_oracle(ops, dtype, M, N, K, group):
+    rng = np.random.default_rng(M * 977 + N * 13 + K + group)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(DEV), 2)
+    got32 = ops._weight_int4pack_mm(dev(xb, dtype), packed, group, dev(szb, dtype)).float().cpu().numpy()
+    assert got32.shape == (M, N)
+    # the oracle on whole packed tiles of eight channels, first and last included
+    tiles = _tile_subset(rng, N // 8, 40)
+    cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    sub = oracle.int4_pack_tc(codes[cols], 2)
+    ref_dev = oracle.to_f32(oracle.int4_mm_tc(xb, dtype, sub, szb[:, cols], group, round_w=True), dtype)
+    _, y64 = oracle.int4_mm_tc(xb, dtype, sub, szb[:, cols], group, round_w=False, want_f64=True)
+    assert_close_norm(got32[:, cols], ref_dev, 1.5e-2 if dtype == "bf16" else 1e-2, "vs reference formulation")
+    assert rel_err(got32[:, cols], y64) < {"f16": 1e-3, "bf16": 1e-2}[dtype]
+    # every channel: against the same kernel family at one row more or less is no check, so the rest of the columns
+    # are held against a float64 product of the dequantized weights
+    s64 = szb if dtype == "f32" else oracle.to_f32(szb, dtype)
+    wq = (codes - 8) * np.repeat(s64[:, :, 0].T, group, axis=1).astype(np.float64) + np.repeat(s64[:, :, 1].T, group, axis=1)
+    want = oracle.to_f32(xb, dtype).astype(np.float64) @ wq.T
+    assert rel_err(got32, want) < {"f16": 1e-3, "bf16": 1e-2}[dtype]
+
+
 def _fused_case(rng, M, N, K, tdt):
     codes = rng.integers(0, 16, (N, K)).astype(np.int32)
     sz = np.stack([rng.uniform(0.005, 0.02, (K // 128, N)), rng.uniform(-0.05, 0.05, (K // 128, N))], axis=-1).astype(np.float32)
@@ -261,7 +304,8 @@ def _tile_subset(rng, n_tiles, count):
 
 
 @pytest.mark.parametrize("tdt", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 4096, 1024), (19, 48, 384)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 4096, 1024), (19, 48, 384),
+                                   (8, 264, 4096), (3, 72, 11008), (12, 4104, 4096)])  # the all-in-flight kernel
 def test_mm_add_equals_the_two_ops(ops, tdt, M, N, K):
     """out = residual + x.W^T with both roundings of the separate ops: equal bit for bit whenever the matmul
     runs on the same kernel (rows > 1), within one rounding of it otherwise."""
@@ -278,7 +322,9 @@ def test_mm_add_equals_the_two_ops(ops, tdt, M, N, K):
 
 
 @pytest.mark.parametrize("tdt,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)])
-@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 1024, 1024), (19, 48, 384)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 1024, 1024), (19, 48, 384),
+                                   # the all-in-flight kernel: 4 / 8 / 16 rows through LDS, every width of workgroup, a partial block
+                                   (2, 72, 4096), (5, 136, 2048), (12, 200, 4096), (8, 4104, 4096), (7, 8200, 4096)])
 def test_mm_swiglu_against_oracle(ops, tdt, tol, M, N, K):
     """silu_mul(T(x.Wg^T), T(x.Wu^T)): the oracle's two device-layout products rounded to T, then
     gate * sigmoid(gate) * up in float32 (p10/src/backend/cpu/PointwiseKernels.cpp:1466-1478)."""
@@ -302,7 +348,9 @@ def test_mm_swiglu_against_oracle(ops, tdt, tol, M, N, K):
 
 @pytest.mark.parametrize("tdt,tol", [(torch.float16, 1e-3), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("M,K,widths", [(1, 256, (64,)), (8, 512, (136, 136, 136)), (16, 1024, (1024, 256, 256)),
-                                        (19, 384, (48, 8, 200, 16)), (8, 4096, (4096, 4096, 4096)), (4, 4096, (11008, 11008))])
+                                        (19, 384, (48, 8, 200, 16)), (8, 4096, (4096, 4096, 4096)), (4, 4096, (11008, 11008)),
+                                        # the all-in-flight kernel: blocks of different weights in one workgroup
+                                        (5, 4096, (72, 8, 200, 16)), (9, 11008, (136, 264)), (3, 8192, (4104, 24, 4096))])
 def test_mm_multi_equals_separate_products(ops, tdt, tol, M, K, widths):
     """Several weights on one input in one launch: every output against the separate op (the same kernel; the order
     in which the wavefronts' partial sums are added may differ with the workgroup shape) and against the oracle."""
