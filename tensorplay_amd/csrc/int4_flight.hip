@@ -54,12 +54,17 @@ int launch_rows(const uint16_t* x, int rows, const FlightSet& set, int blocks, i
 // two steps per wavefront or at most four rows (5120 -> 13824, 8 rows: 11.7 us against 10.5 for the loop kernel;
 // 8192 -> 10240: 16.2 against 13.2; at 2 rows 10.0 / 10.4 and 12.4 / 12.9): then the width with the fewest
 // passes x width, or 2 for few rows (their small LDS tiles let two workgroups share a compute unit).
-int flight_width(int blocks, int rows, int spw, bool pair) {
+int flight_width(int blocks, int rows, int spw, bool pair, bool one_weight) {
     const int cus = flight_compute_units();
     const int widest = pair ? 3 : spw <= 2 ? 4 : spw <= 4 ? 2 : 1;
+    // gate / up at one or two rows: one block of each (4096 -> 11008: 11.8 / 12.1 us against 12.5 / 12.5 for three)
+    if (pair && rows <= 2) return 1;
+    // One row of one weight: only narrow workgroups in one pass; wider weights belong to the column-per-lane kernel
+    // (4096 -> 4096: 3.9 us against 4.5; 4096 -> 6144: 5.0 / 5.5; 14336 -> 4096: 9.0 / 10.2; but 4096 -> 11008: 6.6 / 6.35).
+    const bool narrow_only = rows == 1 && one_weight;
     for (int nb = 1; nb <= widest; ++nb)
-        if ((blocks + nb - 1) / nb <= cus) return nb;
-    if (spw > 2 && rows > 4) return 0;
+        if ((blocks + nb - 1) / nb <= cus) return narrow_only && nb > 2 ? 0 : nb;
+    if (narrow_only || (spw > 2 && rows > 4)) return 0;
     if (rows <= 4 && widest >= 2 && !pair) return 2;
     int best = widest, cost = 1 << 30;
     for (int nb = widest; nb >= 1; --nb) {
@@ -71,7 +76,7 @@ int flight_width(int blocks, int rows, int spw, bool pair) {
 
 template <int DT>
 bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group, bool pair, const void* residual, hipStream_t s, int* rc) {
-    if (rows < 2 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256)) return false;
+    if (rows < 1 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256)) return false;
     const int steps = K / 128;
     const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
     if (steps < kFlightWaves || spw > 7 || spw == 5) return false;
@@ -96,7 +101,7 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
         slots[w]->first = pair ? 0 : blocks;
         if (!pair || w == 0) blocks += (wts.N[w] + 15) / 16;
     }
-    int nb = flight_width(blocks, rows, spw, pair);
+    int nb = flight_width(blocks, rows, spw, pair, wts.count == 1);
     if (const char* env = tuning_env("TPQ_INT4_FLIGHT")) nb = std::atoi(env);  // 0 switches the kernel off, 1..4 pin the width
     if (nb <= 0) return false;
     const auto* xp = static_cast<const uint16_t*>(x);

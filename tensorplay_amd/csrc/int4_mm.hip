@@ -453,7 +453,7 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
     //                rows against 8.4 / 8.5 / 9.0 / 9.3 for the next best; 8192 -> 28672, 8 rows: 27.4 against 30.4),
     //                64 ch x 4 waves above (16 rows: 9.7 us against 12.3 for 32 ch)
     //   N > 28672:   32 ch x 4 waves up to 4 rows, 64 ch x 4 waves above (4096 -> 32000, 4 rows: 16.2 against 16.6)
-    if (rows > 1 && !(force && force[0] == 'm')) {  // the all-in-flight form, where it is built
+    if (!(force && force[0] == 'm')) {  // the all-in-flight form, where it is built and wins
         FlightWeights one{};
         one.packed[0] = packed; one.sz[0] = sz; one.y[0] = y; one.N[0] = N; one.count = 1;
         if (flight_launch(DT, x, rows, one, K, group, false, residual, s, rc)) return true;
@@ -640,6 +640,12 @@ int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* s
     if (M == 1) {
         int rc;
         if (launch_row<DT>(x, packed, sz, y, N, K, group, s, &rc)) return rc;
+        const char* force = tuning_env("TPQ_INT4_KERNEL");
+        if (!force) {  // narrow weights: the all-in-flight matrix-core kernel
+            FlightWeights one{};
+            one.packed[0] = packed; one.sz[0] = sz; one.y[0] = y; one.N[0] = N; one.count = 1;
+            if (flight_launch(DT, x, 1, one, K, group, false, nullptr, s, &rc)) return rc;
+        }
     }
     // Many rows: the tiled kernel, the packed weight read once per 128 rows.  Measured against the 32-row slabs below
     // (us, fp16): K = 4096, N = 11008: 43 / 55 at 128 rows, 62 / 107 at 256, 258 / 821 at 2048; K = N = 8192:
