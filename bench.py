@@ -336,6 +336,9 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB device copy a few times: the known-size kernel that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--profile-rows", type=int, default=0, metavar="M",
+                    help="also launch the int4 product at M activation rows (same weights, rotating) 200 times, eagerly: "
+                         "the dispatches that the rocprofv3 summaries of the batched-decode kernels are collected on")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -442,6 +445,17 @@ def main() -> int:
         extras["int4_gemv_frac_of_read_ceiling"] = best[0] / extras["int4_gemv_us_median_of_7_replays"]
         del probe_bufs, ge
         torch.cuda.empty_cache()
+    if args.profile_rows > 0:
+        mb = args.profile_rows
+        xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
+        yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
+        for i in range(200):
+            rc = lib.tpq_int4_mm_ws(xb.data_ptr(), _lib.F16, mb, K, packs[i % copies].data_ptr(), 2, N, GROUP,
+                                    szs[i % copies].data_ptr(), yb.data_ptr(), ws.data_ptr(), ws.numel(), cur())
+            if rc:
+                raise RuntimeError(_lib.last_error())
+        sync()
+        extras["profile_rows"] = mb
     if args.calibrate_copy:
         src_c = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst_c = torch.empty_like(src_c)
