@@ -667,9 +667,13 @@ def main() -> int:
             xq_t, rs_t = ops._quantize_int8_rowwise(xt, 1e-5)
             yt = torch.empty((mt, nt), dtype=torch.float16, device=dev)
 
-            def tmm(xq_t=xq_t, rs_t=rs_t, pk=pk, yt=yt, mt=mt, kt=kt, nt=nt):
-                lib.tpq_ternary_mm(xq_t.data_ptr(), rs_t.data_ptr(), pk.data_ptr(), 0.0173, None, mt, nt, kt,
-                                   yt.data_ptr(), _lib.F16, None, cur())
+            # (the scratch matrix for the split-K partial sums, as the op wrapper passes it; 0 bytes for most shapes)
+            tws_bytes = int(lib.tpq_ternary_mm_workspace_bytes(mt, nt, kt))
+            tws = torch.empty(max(tws_bytes, 4) // 4, dtype=torch.int32, device=dev)
+
+            def tmm(xq_t=xq_t, rs_t=rs_t, pk=pk, yt=yt, mt=mt, kt=kt, nt=nt, tws=tws, tws_bytes=tws_bytes):
+                lib.tpq_ternary_mm_ws(xq_t.data_ptr(), rs_t.data_ptr(), pk.data_ptr(), 0.0173, None, mt, nt, kt,
+                                      yt.data_ptr(), _lib.F16, None, tws.data_ptr(), tws_bytes, cur())
 
             gt = graph_of(lambda: [tmm() for _ in range(200)])
             gt.replay(); sync()

@@ -193,6 +193,17 @@ int tpq_ternary_unpack(const uint8_t* packed, int64_t rows, int64_t cols, int8_t
 int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packed, float w_scale,
                    const float* bias, int64_t M, int64_t N, int64_t K, void* out, int out_dtype,
                    int32_t* acc_out, void* stream);
+/*
+ * The same product (same reference lines) with an optional device workspace.  From 33 rows on with
+ * K > 2560 the fastest kernel cuts K into splits whose exact int32 partial sums go to the workspace
+ * ([splits][M][N]) and are added by a second kernel: bit-identical results.  tpq_ternary_mm_workspace_bytes
+ * says how many bytes the shape can use (0: none needed); a NULL or smaller workspace runs
+ * tpq_ternary_mm's kernels.  Nothing has to be cleared between calls.
+ */
+int64_t tpq_ternary_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int tpq_ternary_mm_ws(const int8_t* x, const float* row_scale, const uint8_t* packed, float w_scale,
+                      const float* bias, int64_t M, int64_t N, int64_t K, void* out, int out_dtype,
+                      int32_t* acc_out, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * Two fusions around the decode matmul for the MLP of a decoder layer (float16 / bfloat16

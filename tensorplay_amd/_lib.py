@@ -37,6 +37,8 @@ SIGNATURES = {
     "tpq_ternary_pack": [_ptr, _i64, _i64, _ptr, _ptr],
     "tpq_ternary_unpack": [_ptr, _i64, _i64, _ptr, _ptr],
     "tpq_ternary_mm": [_ptr, _ptr, _ptr, _f32, _ptr, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],
+    "tpq_ternary_mm_workspace_bytes": [_i64, _i64, _i64],
+    "tpq_ternary_mm_ws": [_ptr, _ptr, _ptr, _f32, _ptr, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr, _i64, _ptr],
     "tpq_int4_mm_add": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, _ptr],
     "tpq_int4_mm_swiglu": [_ptr, _int, _i64, _i64, _ptr, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, _ptr],
     "tpq_int4_mm_multi": [_ptr, _int, _i64, _i64, _int, _ptr, _int, _ptr, _i64, _ptr, _ptr, _ptr],

@@ -67,6 +67,19 @@ struct EpilogueTernary {
             out[idx] = Elem<DT>::store(f);
         }
     }
+    // The same in two steps, for kernels that store many elements per lane: the scale and the bias are fetched
+    // first (a load after a store to `out` cannot be moved ahead of it by the compiler, so store() in a loop
+    // waits for memory once per element).
+    __device__ __forceinline__ float row_scale_of(int m) const { return out ? rs[m] : 0.0f; }
+    __device__ __forceinline__ float bias_of(int n) const { return out && bias ? bias[n] : 0.0f; }
+    __device__ __forceinline__ void store_scaled(int64_t idx, int v, float row_scale, float bias_n) const {
+        if (acc_out) acc_out[idx] = v;
+        if (out) {
+            float f = __fmul_rn(__fmul_rn(static_cast<float>(v), row_scale), w_scale);
+            if (bias) f = __fadd_rn(f, bias_n);
+            out[idx] = Elem<DT>::store(f);
+        }
+    }
 };
 
 // One packed byte holds four ternary codes, first code in bits 7..6

@@ -117,10 +117,19 @@ __global__ __launch_bounds__(kTgThreads) void ternary_gemm_m128_kernel(const int
             for (int v = 0; v < 16; ++v) acc[v] += part[((q * kMBlocks + mb) * 16 + v) * kWave + lane];
         // C fragment of a 32x32 block: lane holds column lane%32, rows 8*(v/4) + 4*(lane/32) + v%4
         const int n = n0 + frag_row;
+        if (n < N) {
+            float row_scale[16];  // fetched before the first store: a load behind a store to `out` has to wait for it
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int m = m0 + mb * 32 + 8 * (v >> 2) + 4 * frag_half + (v & 3);
-            if (m < M && n < N) ep.store(static_cast<int64_t>(m) * N + n, m, n, acc[v]);
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + mb * 32 + 8 * (v >> 2) + 4 * frag_half + (v & 3);
+                row_scale[v] = ep.row_scale_of(m < M ? m : M - 1);
+            }
+            const float bias_n = ep.bias_of(n);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + mb * 32 + 8 * (v >> 2) + 4 * frag_half + (v & 3);
+                if (m < M) ep.store_scaled(static_cast<int64_t>(m) * N + n, acc[v], row_scale[v], bias_n);
+            }
         }
     }
 }

@@ -27,6 +27,7 @@
 #include "int8_gemm_kernel.h"
 #include "ternary_gemm_kernel.h"
 #include "ternary_decode_mfma.h"
+#include "ternary_slab_kernel.h"
 
 namespace tpq {
 namespace {
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(256) void ternary_generic_kernel(const int8_t* __re
 
 template <class Epilogue>
 int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N, int64_t K,
-                   Epilogue ep, hipStream_t s) {
+                   Epilogue ep, hipStream_t s, void* workspace, int64_t workspace_bytes) {
     const bool sizes_ok = M <= 0x7FFFFFFF && N <= 0x7FFFFFFF && K <= 0x7FFFFFFF;
     // the tile kernel below takes over where it is faster and its shape conditions hold
     // Measured at 2560 -> 6912 / 6912 -> 2560 (216 / 80 tiles of 32 channels): the decode kernel takes 7, 7.5, 9.4, 11.4 us
@@ -135,6 +136,13 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
     static const int mfma_rows = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_ROWS"); return e ? std::atoi(e) : 32; }();
     if (forced_decode_rows < 0 && M >= mfma_min && M <= mfma_rows && ternary_decode_mfma_ok(x, packed, M, N, K))
         return launch_ternary_decode_mfma(x, packed, M, N, K, ep, s);
+    // 33 rows and more: the slab kernel (every load of a workgroup in flight at once); K beyond 2560 is split and
+    // needs the caller's workspace for the exact partial sums
+    if (forced_decode_rows < 0 && !tuning_env("TPQ_TERNARY_NO_SLAB") && aligned(x, 16) && aligned(packed, 16)) {
+        const int splits = ternary_slab_splits(M, N, K);
+        const bool room = splits == 1 || (workspace != nullptr && aligned(workspace, 16) && workspace_bytes >= static_cast<int64_t>(splits) * M * N * 4);
+        if (splits >= 1 && room) return launch_ternary_slab(x, packed, M, N, K, splits, static_cast<int32_t*>(workspace), ep, s);
+    }
     const bool gemm_ok = sizes_ok && M <= gemm_rows && K % kTgStage == 0 && aligned(x, 16) && aligned(packed, 4);
     if (sizes_ok && M <= 8 && (M <= decode_rows || !gemm_ok) && K % 64 == 0 && aligned(x, 16) && aligned(packed, 16)) {
         const int waves = static_cast<int>((N + kRowsPerWave - 1) / kRowsPerWave);
@@ -164,9 +172,21 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
 
 using namespace tpq;
 
+TPQ_EXPORT int64_t tpq_ternary_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int splits = M > 0 && N > 0 && K > 0 ? ternary_slab_splits(M, N, K) : 0;
+    return splits > 1 ? static_cast<int64_t>(splits) * M * N * 4 : 0;
+}
+
 TPQ_EXPORT int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uint8_t* packed,
                               float w_scale, const float* bias, int64_t M, int64_t N, int64_t K,
                               void* out, int out_dtype, int32_t* acc_out, void* stream) {
+    return tpq_ternary_mm_ws(x, row_scale, packed, w_scale, bias, M, N, K, out, out_dtype, acc_out, nullptr, 0, stream);
+}
+
+TPQ_EXPORT int tpq_ternary_mm_ws(const int8_t* x, const float* row_scale, const uint8_t* packed,
+                                 float w_scale, const float* bias, int64_t M, int64_t N, int64_t K,
+                                 void* out, int out_dtype, int32_t* acc_out, void* workspace, int64_t workspace_bytes,
+                                 void* stream) {
     TPQ_REQUIRE(M >= 0 && N >= 0 && K >= 0, TPQ_ERR_INVALID_VALUE, "bitnet_linear_packed: negative shape");
     TPQ_REQUIRE(out_dtype == TPQ_DTYPE_F32 || out_dtype == TPQ_DTYPE_F16 || out_dtype == TPQ_DTYPE_BF16,
                 TPQ_ERR_INVALID_TYPE, "bitnet_linear_packed: unsupported output dtype");
@@ -178,15 +198,15 @@ TPQ_EXPORT int tpq_ternary_mm(const int8_t* x, const float* row_scale, const uin
     switch (out_dtype) {
         case TPQ_DTYPE_F32: {
             const EpilogueTernary<TPQ_DTYPE_F32> ep{static_cast<float*>(out), acc_out, row_scale, bias, w_scale};
-            return launch_ternary(x, packed, M, N, K, ep, s);
+            return launch_ternary(x, packed, M, N, K, ep, s, workspace, workspace_bytes);
         }
         case TPQ_DTYPE_F16: {
             const EpilogueTernary<TPQ_DTYPE_F16> ep{static_cast<uint16_t*>(out), acc_out, row_scale, bias, w_scale};
-            return launch_ternary(x, packed, M, N, K, ep, s);
+            return launch_ternary(x, packed, M, N, K, ep, s, workspace, workspace_bytes);
         }
         default: {
             const EpilogueTernary<TPQ_DTYPE_BF16> ep{static_cast<uint16_t*>(out), acc_out, row_scale, bias, w_scale};
-            return launch_ternary(x, packed, M, N, K, ep, s);
+            return launch_ternary(x, packed, M, N, K, ep, s, workspace, workspace_bytes);
         }
     }
 }

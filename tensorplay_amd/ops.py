@@ -361,9 +361,14 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
         if rs.numel() != M:
             raise ValueError("ternary_mm: one row scale per activation row expected")
         b = None if bias is None else bias.contiguous().to(torch.float32)
+        lib = _lib.load()
         with torch.cuda.device(x.device):
-            _check(_lib.load().tpq_ternary_mm(_ptr(x), _ptr(rs), _ptr(p), float(w_scale), _ptr(b), M, N, K,
-                                              _ptr(out), _DT[out_dtype], _ptr(acc), _stream(x)))
+            # prefill chunks against a long K: the library cuts K into splits that meet in an int32 scratch matrix
+            # (same bits); it says for which shapes
+            scratch_bytes = int(lib.tpq_ternary_mm_workspace_bytes(M, N, K))
+            scratch = torch.empty(scratch_bytes // 4, dtype=torch.int32, device=x.device) if scratch_bytes else None
+            _check(lib.tpq_ternary_mm_ws(_ptr(x), _ptr(rs), _ptr(p), float(w_scale), _ptr(b), M, N, K,
+                                         _ptr(out), _DT[out_dtype], _ptr(acc), _ptr(scratch), scratch_bytes, _stream(x)))
     return (out, acc) if return_acc else out
 
 
