@@ -19,4 +19,9 @@ struct FlightWeights {
 bool flight_launch(int dtype, const void* x, int rows, const FlightWeights& weights, int K, int group, bool pair,
                    const void* residual, hipStream_t stream, int* rc);
 
+// The int8 weight-only product (w: [N][K] int8, scales: [N] float, y = (x . w^T) * scale) on the same structure
+// (int8pack_flight_kernel.h): 3..16 rows of 16-bit activations.  Returns false when the shape is not built.
+bool flight_launch_int8pack(int dtype, const void* x, int rows, const int8_t* w, const float* scales, void* y, int N, int K,
+                            hipStream_t stream, int* rc);
+
 }  // namespace tpq

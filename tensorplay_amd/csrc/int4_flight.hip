@@ -4,6 +4,7 @@
 #include <cstdlib>
 
 #include "int4_mfma_flight_kernel.h"
+#include "int8pack_flight_kernel.h"
 
 namespace tpq {
 namespace {
@@ -132,7 +133,74 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
     return true;
 }
 
+template <int DT, int NB, int SPW, int XR>
+int launch_int8_as(const uint16_t* x, int rows, const int8_t* w, const float* scales, uint16_t* y, int N, int K, hipStream_t s) {
+    constexpr size_t bytes = int8_flight_lds_bytes<NB, SPW, XR>();
+    static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
+    static std::atomic<uint64_t> reserved{0};
+    const auto kernel = int8pack_flight_kernel<DT, NB, SPW, XR>;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), bytes, reserved, "_weight_int8pack_mm (all in flight)")) return rc;
+    kernel<<<dim3((N + 16 * NB - 1) / (16 * NB)), dim3(kFlightWaves * kWave), bytes, s>>>(x, w, scales, y, rows, N, K);
+    return check_launch("_weight_int8pack_mm (all in flight)");
+}
+
+template <int DT, int NB, int SPW>
+int launch_int8_rows(const uint16_t* x, int rows, const int8_t* w, const float* scales, uint16_t* y, int N, int K, hipStream_t s) {
+    if (rows <= 4) return launch_int8_as<DT, NB, SPW, 4>(x, rows, w, scales, y, N, K, s);
+    if (rows <= 8) return launch_int8_as<DT, NB, SPW, 8>(x, rows, w, scales, y, N, K, s);
+    if constexpr (SPW <= 2) {
+        return launch_int8_as<DT, NB, SPW, 16>(x, rows, w, scales, y, N, K, s);
+    } else {
+        return TPQ_ERR_UNSUPPORTED;  // not reached
+    }
+}
+
+// Measured (fp16, us, loop kernel -> this one): 4096 -> 11008 at 3 / 8 / 16 rows 14.4 / 16.6 / 20.7 -> 11.5 / 12.1 / 13.1;
+// 4096 x 4096 at 8 rows 7.5 -> 6.4; 4096 -> 32000 at 8 rows 34.7 -> 28.5; 11008 -> 4096 at 8 rows 16.2 -> 14.2.
+template <int DT>
+bool launch_int8(const void* x, int rows, const int8_t* w, const float* scales, void* y, int N, int K, hipStream_t s, int* rc) {
+    if (rows < 1 || rows > 16 || K % 128 != 0 || !aligned(x, 16) || !aligned(w, 16)) return false;
+    const int steps = K / 128;
+    const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
+    // more than two steps per wavefront at more than eight rows: the loop kernel is as fast or faster (8192 x 8192 at 12 rows:
+    // 22.0 us against 19.5; 11008 -> 4096: 17.8 / 17.8)
+    if (steps < kFlightWaves || spw > 7 || spw == 5 || (spw > 2 && rows > 8)) return false;
+    const int blocks = (N + 15) / 16;
+    const int cus = flight_compute_units();
+    const int widest = spw <= 2 ? 4 : spw <= 4 ? 2 : 1;
+    int nb = 0;
+    for (int c = 1; c <= widest && nb == 0; ++c)
+        if ((blocks + c - 1) / c <= cus) nb = c;
+    if (nb == 0 && spw <= 2) nb = widest;  // several passes pay off with two steps per wavefront only (see flight_width)
+    if (const char* env = tuning_env("TPQ_INT8PACK_FLIGHT")) nb = std::atoi(env);  // 0 switches the kernel off, 1..4 pin the width
+    if (nb <= 0 || nb > widest) return false;
+    const auto* xp = static_cast<const uint16_t*>(x);
+    auto* yp = static_cast<uint16_t*>(y);
+    int code = TPQ_ERR_UNSUPPORTED;
+#define TPQ_FLIGHT8(NBV, SPWV) code = launch_int8_rows<DT, NBV, SPWV>(xp, rows, w, scales, yp, N, K, s)
+    switch (spw) {
+        case 1: case 2:
+            if (nb == 1) TPQ_FLIGHT8(1, 2); else if (nb == 2) TPQ_FLIGHT8(2, 2); else if (nb == 3) TPQ_FLIGHT8(3, 2); else TPQ_FLIGHT8(4, 2);
+            break;
+        case 3: if (nb == 1) TPQ_FLIGHT8(1, 3); else TPQ_FLIGHT8(2, 3); break;
+        case 4: if (nb == 1) TPQ_FLIGHT8(1, 4); else TPQ_FLIGHT8(2, 4); break;
+        case 6: TPQ_FLIGHT8(1, 6); break;
+        case 7: TPQ_FLIGHT8(1, 7); break;
+        default: return false;
+    }
+#undef TPQ_FLIGHT8
+    *rc = code;
+    return true;
+}
+
 }  // namespace
+
+bool flight_launch_int8pack(int dtype, const void* x, int rows, const int8_t* w, const float* scales, void* y, int N, int K,
+                            hipStream_t stream, int* rc) {
+    if (dtype == TPQ_DTYPE_F16) return launch_int8<TPQ_DTYPE_F16>(x, rows, w, scales, y, N, K, stream, rc);
+    if (dtype == TPQ_DTYPE_BF16) return launch_int8<TPQ_DTYPE_BF16>(x, rows, w, scales, y, N, K, stream, rc);
+    return false;
+}
 
 bool flight_launch(int dtype, const void* x, int rows, const FlightWeights& weights, int K, int group, bool pair,
                    const void* residual, hipStream_t stream, int* rc) {

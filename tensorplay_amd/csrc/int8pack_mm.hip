@@ -18,6 +18,7 @@
 // output channel and slab of up to 8 rows, block reduction.
 #include <cstdlib>
 
+#include "int4_flight.h"
 #include "int4_lane.h"
 
 namespace tpq {
@@ -459,6 +460,15 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
         static const int forced_mb = [] { const char* e = tuning_env("TPQ_INT8PACK_MB"); return e ? std::atoi(e) : 0; }();
         for (int64_t m0 = 0; m0 < M;) {
             const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
+            if (left <= 16 && N <= 0x7FFFFFF0 && K <= 0x7FFFFF80) {  // the all-in-flight form, where it is built
+                int rc = TPQ_OK;
+                if (flight_launch_int8pack(dtype, static_cast<const uint16_t*>(x) + m0 * K, left, w, scales, static_cast<uint16_t*>(out) + m0 * N,
+                                           static_cast<int>(N), static_cast<int>(K), s, &rc)) {
+                    if (rc != TPQ_OK) return rc;
+                    m0 += left;
+                    continue;
+                }
+            }
             const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
             const int rows = left < 16 * mb ? left : 16 * mb;
             // Workgroup shape from a sweep over model shapes (K, N = 1024..28672; 1, 8, 16 rows): 16 channels x 8

@@ -37,7 +37,11 @@ CASES = [(1, 4096, 512), (4, 1024, 136), (16, 256, 40), (17, 384, 72), (2, 100, 
          # the three workgroup sizes (by N K), K of 16 only
          (1, 4112, 10), (1, 16, 7), (1, 28672, 130), (1, 8192, 8200), (1, 4096, 32772), (1, 65536, 12), (1, 48, 1),
          # two rows on the same kernel (K up to 32768; longer rows take the matrix-core kernel)
-         (2, 4112, 10), (2, 32, 5), (2, 28672, 130), (2, 8192, 8200), (2, 4096, 32772), (2, 36864, 12)]
+         (2, 4112, 10), (2, 32, 5), (2, 28672, 130), (2, 8192, 8200), (2, 4096, 32772), (2, 36864, 12),
+         # the all-in-flight matrix-core kernel (3..16 rows, K = 2048..14336): 4 / 8 / 16 rows through LDS, every width of
+         # workgroup, a dead last step (K = 2048, 5120, 11008), ragged N, more workgroups than one pass
+         (3, 2048, 72), (5, 4096, 4104), (8, 4096, 11008), (4, 4096, 16392), (9, 4096, 136), (16, 5120, 264),
+         (7, 8192, 136), (8, 11008, 4104), (6, 14336, 264), (13, 11008, 72)]
 
 
 @pytest.mark.gpu
