@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "int8_gemm_kernel.h"
+#include "int8_flight_kernel.h"
 
 namespace tpq {
 namespace {
@@ -215,6 +216,57 @@ inline bool int8_decode_ok(const void* a, const void* w, int64_t M, int64_t N, i
     return M >= 1 && K >= 128 && K % 128 == 0 && aligned(a, 16) && aligned(w, 16) && N <= 0x7FFFFFF0 && K <= 0x7FFFFF80;
 }
 
+inline int i8_flight_compute_units() {
+    static std::atomic<int> cached{0};
+    int v = cached.load(std::memory_order_relaxed);
+    if (v == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        v = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
+        cached.store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
+
+template <int NB, int MB, int SPW, int XR, class Epilogue>
+int launch_int8_flight_as(const int8_t* x, const int8_t* w, int rows, int N, int K, const Epilogue& ep, hipStream_t s) {
+    constexpr size_t bytes = i8_flight_lds_bytes<NB, MB, XR>();
+    static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
+    static std::atomic<uint64_t> reserved{0};
+    const auto kernel = int8_flight_kernel<NB, MB, SPW, XR, Epilogue>;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), bytes, reserved, "int8 decode gemm (all in flight)")) return rc;
+    kernel<<<dim3((N + 16 * NB - 1) / (16 * NB)), dim3(kFlightWaves * kWave), bytes, s>>>(x, w, rows, N, K, ep);
+    return check_launch("int8 decode gemm (all in flight)");
+}
+
+// 3..32 rows on the all-in-flight kernel (int8_flight_kernel.h); false when the shape is not one of its cases
+template <class Epilogue>
+bool launch_int8_flight(const int8_t* x, const int8_t* w, int rows, int N, int K, const Epilogue& ep, hipStream_t s, int* rc) {
+    const int steps = K / 128;
+    const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
+    // Measured (us, bf16 out, loop kernel -> this one): 4096 x 4096 at 16 / 32 rows 7.2 / 9.9 -> 6.2 / 7.1; 4096 -> 11008 at 8 / 16 / 32
+    // rows 13.4 / 15.5 / 20.9 -> 11.4 / 11.9 / 18.0; 4096 -> 32000 at 16 rows 34.0 -> 29.0; 8192 x 8192 at 16 rows 18.3 -> 16.7.
+    // Not with one step per wavefront (2048 -> 4096 at 8 rows: 5.1 us against 4.7) and not beyond 16 rows at long K (even).
+    if (steps < 2 * kFlightWaves - 8 || spw > 4 || rows > 32 || (spw > 2 && rows > 16)) return false;
+    const int blocks = (N + 15) / 16, cus = i8_flight_compute_units();
+    const int widest = spw <= 2 ? (rows > 16 ? 2 : 4) : 2;
+    int nb = 0;
+    for (int c = 1; c <= widest && nb == 0; ++c)
+        if ((blocks + c - 1) / c <= cus) nb = c;
+    if (nb == 0 && spw <= 2) nb = widest;
+    if (const char* env = tuning_env("TPQ_INT8_FLIGHT")) nb = std::atoi(env);  // 0 switches the kernel off, 1..4 pin the width
+    if (nb <= 0 || nb > widest) return false;
+#define TPQ_I8F(NBV, MBV, SPWV, XRV) *rc = launch_int8_flight_as<NBV, MBV, SPWV, XRV, Epilogue>(x, w, rows, N, K, ep, s)
+#define TPQ_I8F_ROWS(NBV, SPWV) do { if (rows <= 8) TPQ_I8F(NBV, 1, SPWV, 8); else TPQ_I8F(NBV, 1, SPWV, 16); } while (0)
+    if (rows > 16) { if (nb == 1) TPQ_I8F(1, 2, 2, 32); else TPQ_I8F(2, 2, 2, 32); }
+    else if (spw <= 2) { if (nb == 1) TPQ_I8F_ROWS(1, 2); else if (nb == 2) TPQ_I8F_ROWS(2, 2); else if (nb == 3) TPQ_I8F_ROWS(3, 2); else TPQ_I8F_ROWS(4, 2); }
+    else if (spw == 3) { if (nb == 1) TPQ_I8F_ROWS(1, 3); else TPQ_I8F_ROWS(2, 3); }
+    else { if (nb == 1) TPQ_I8F_ROWS(1, 4); else TPQ_I8F_ROWS(2, 4); }
+#undef TPQ_I8F_ROWS
+#undef TPQ_I8F
+    return true;
+}
+
 // slabs of 32 rows (16 for what is left); the epilogue sees row indices of the whole problem through `rebase`
 template <class Epilogue, class Rebase>
 int launch_int8_decode(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Epilogue ep, Rebase rebase, hipStream_t s) {
@@ -233,6 +285,14 @@ int launch_int8_decode(const int8_t* a, const int8_t* w, int64_t M, int64_t N, i
     const int n = static_cast<int>(N), k = static_cast<int>(K);
     for (int64_t m0 = 0; m0 < M;) {
         const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
+        {
+            int rc = TPQ_OK;
+            if (launch_int8_flight(a + m0 * K, w, left, static_cast<int>(N), static_cast<int>(K), rebase(ep, m0), s, &rc)) {
+                if (rc != TPQ_OK) return rc;
+                m0 += left;
+                continue;
+            }
+        }
         const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
         const int rows = left < 16 * mb ? left : 16 * mb;
         // Workgroup shape from a sweep over model shapes (K, N = 1024..28672): 32 channels pay from 8 rows on where

@@ -36,6 +36,12 @@ __device__ __forceinline__ int swz(int row) { return (((row >> 1) ^ (row >> 3)) 
 struct EpilogueInt32 {
     int32_t* c;
     __device__ __forceinline__ void store(int64_t idx, int m, int n, int v) const { c[idx] = v; }
+    // `count` (1..4) consecutive channels n .. of row m
+    __device__ __forceinline__ void store_run(int64_t idx, int m, int n, const int (&v)[4], int count) const {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (e < count) c[idx + e] = v[e];
+    }
 };
 
 template <int DT>
@@ -48,6 +54,23 @@ struct EpilogueDequant {
         float f = __fmul_rn(__fmul_rn(static_cast<float>(v), rs[m]), cs[n]);
         if (bias) f = __fadd_rn(f, bias[n]);
         out[idx] = Elem<DT>::store(f);
+    }
+    // `count` (1..4) consecutive channels n .. of row m; every scale is fetched before the first store (a load behind a
+    // store to `out` cannot be moved ahead of it, so store() in a loop waits for memory once per element)
+    __device__ __forceinline__ void store_run(int64_t idx, int m, int n, const int (&v)[4], int count) const {
+        const float r = rs[m];
+        float c[4], b[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            c[e] = cs[e < count ? n + e : n];
+            b[e] = bias ? bias[e < count ? n + e : n] : 0.0f;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float f = __fmul_rn(__fmul_rn(static_cast<float>(v[e]), r), c[e]);
+            if (bias) f = __fadd_rn(f, b[e]);
+            if (e < count) out[idx + e] = Elem<DT>::store(f);
+        }
     }
 };
 

@@ -30,7 +30,11 @@ SHAPES = [(5, 7, 3), (1, 1, 1), (64, 12, 32), (16, 1024, 1024), (64, 128, 32), (
           (130, 1024, 200), (300, 2048, 136), (65, 1152, 64), (257, 1280, 100), (33, 1024, 10248),
           # one or two rows on the row kernel: a last chunk past K, several passes per channel, ragged N, the long rows
           # that fall back to the matrix-core kernel (more than 32768 k), and 3 / 4 rows (that kernel by default)
-          (2, 4224, 10), (1, 20480, 13), (2, 32768, 9), (1, 36864, 8), (2, 4096, 8200), (1, 8192, 16390), (3, 4096, 50), (4, 256, 7)]
+          (2, 4224, 10), (1, 20480, 13), (2, 32768, 9), (1, 36864, 8), (2, 4096, 8200), (1, 8192, 16390), (3, 4096, 50), (4, 256, 7),
+          # all-in-flight decode kernel (3..32 rows, K = 2048..8192): 8 / 16 / 32 rows through LDS, every width of
+          # workgroup, a dead last step (K = 2048, 5120), ragged N
+          (3, 2048, 72), (8, 4096, 4104), (16, 4096, 264), (12, 5120, 136), (24, 4096, 520), (32, 2048, 40), (9, 8192, 72),
+          (5, 4096, 16392)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -113,7 +117,9 @@ def test_rescale_bit_exact(ops):
 
 @pytest.mark.parametrize("out_dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("shape", [(16, 1024, 1024), (300, 208, 200), (5, 7, 3), (256, 512, 384), (40, 256, 36), (1, 4096, 64), (50, 256, 6160), (9, 128, 16390),
-                                   (130, 1024, 200), (300, 2048, 136), (65, 1152, 66), (257, 1280, 100)])
+                                   (130, 1024, 200), (300, 2048, 136), (65, 1152, 66), (257, 1280, 100),
+                                   # all-in-flight decode kernel: runs of four channels stored with the scales fetched first
+                                   (8, 4096, 264), (16, 2048, 4104), (27, 4096, 134), (5, 6144, 70)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_fused_dequant_bit_exact(ops, out_dtype, shape, with_bias):
     from gpu_util import TORCH_DT
