@@ -41,19 +41,32 @@ __device__ __forceinline__ int quantize_one(float v, float scale, const QParams&
 // absolute error is below 2^-14.  If q lies at least 2^-13 inside (c - 1/2, c + 1/2), so does the
 // correctly rounded quotient, and both round to c.  Otherwise (about one element in a few thousand;
 // also NaN and infinities) the element is redone with the IEEE division.
-__device__ __forceinline__ void quantize_eight(const float (&v)[kVec], float scale, float inv_scale, const QParams& p,
-                                               int (&code)[kVec]) {
+// The codes leave as two packed words.  v_cvt_pk_u8_f32 converts a float to an unsigned byte (saturating at 0 and
+// 255) and drops it into one byte of a register: the rounded quotient c is an integer already, so c + 128 converts
+// exactly, the upper clamp is the saturation when qmax = 127, and one xor takes the 128 off the four bytes again.
+// Four instructions per code less than clamp, convert, mask, shift, or.
+__device__ __forceinline__ void quantize_eight_packed(const float (&v)[kVec], float scale, float inv_scale, const QParams& p,
+                                                      uint32_t& lo, uint32_t& hi) {
     bool redo = false;
+    uint32_t word[2] = {0u, 0u};
+    const float qmin = static_cast<float>(p.qmin), qmax = static_cast<float>(p.qmax);
 #pragma unroll
     for (int i = 0; i < kVec; ++i) {
         const float q = v[i] * inv_scale;
         const float c = rintf(q);
         redo |= !(fabsf(q - c) <= 0.5f - 0x1p-13f);
-        code[i] = static_cast<int>(fminf(fmaxf(c, static_cast<float>(p.qmin)), static_cast<float>(p.qmax)));
+        const float biased = fminf(fmaxf(c, qmin), qmax) + 128.0f;  // 0 .. 255, an integer
+        word[i >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(biased, i & 3, word[i >> 2]);
     }
+    lo = word[0] ^ 0x80808080u;
+    hi = word[1] ^ 0x80808080u;
     if (redo) {
+        lo = hi = 0;
 #pragma unroll
-        for (int i = 0; i < kVec; ++i) code[i] = quantize_one(v[i], scale, p);
+        for (int i = 0; i < 4; ++i) {
+            lo |= (static_cast<uint32_t>(quantize_one(v[i], scale, p)) & 0xFFu) << (8 * i);
+            hi |= (static_cast<uint32_t>(quantize_one(v[i + 4], scale, p)) & 0xFFu) << (8 * i);
+        }
     }
 }
 
@@ -101,15 +114,18 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_cached(
 
     float v[CHUNKS][kVec];
     float absmax = 0.0f;
+    // No branch around the loads: at the join of a branch the compiler waits for every outstanding load, which made
+    // the chunks one round trip to memory each.  A chunk past the end re-reads the last chunk of the row: the same
+    // elements again do not change the maximum, and nothing is stored for it.
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * THREADS + threadIdx.x) * kVec;
-        if (k0 < K) {
-            load_chunk<DT>(xr + k0, v[c]);
-#pragma unroll
-            for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
-        }
+        load_chunk<DT>(xr + (k0 < K ? k0 : K - kVec), v[c]);
     }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
     absmax = block_max<THREADS>(absmax, smem);
     const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
     if (threadIdx.x == 0) scales[row] = scale;
@@ -122,18 +138,15 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_cached(
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * THREADS + threadIdx.x) * kVec;
         if (k0 < K) {
-            int code[kVec];
+            uint32_t lo = 0, hi = 0;
             if (shortcut) {
-                quantize_eight(v[c], scale, inv_scale, p, code);
+                quantize_eight_packed(v[c], scale, inv_scale, p, lo, hi);
             } else {
 #pragma unroll
-                for (int i = 0; i < kVec; ++i) code[i] = quantize_one(v[c][i], scale, p);
-            }
-            uint32_t lo = 0, hi = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                lo |= (static_cast<uint32_t>(code[i]) & 0xFFu) << (8 * i);
-                hi |= (static_cast<uint32_t>(code[i + 4]) & 0xFFu) << (8 * i);
+                for (int i = 0; i < 4; ++i) {
+                    lo |= (static_cast<uint32_t>(quantize_one(v[c][i], scale, p)) & 0xFFu) << (8 * i);
+                    hi |= (static_cast<uint32_t>(quantize_one(v[c][i + 4], scale, p)) & 0xFFu) << (8 * i);
+                }
             }
             *reinterpret_cast<uint2*>(cr + k0) = make_uint2(lo, hi);
         }
@@ -158,11 +171,13 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_subwave(
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * LANES + sub) * kVec;
-        if (live && k0 < K) {
-            load_chunk<DT>(xr + k0, v[c]);
+        load_chunk<DT>(xr + (k0 < K ? k0 : K - kVec), v[c]);  // branch-free: see quantize_rows_cached; dead rows read row 0
+    }
+    if (live) {
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
             for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
-        }
     }
 #pragma unroll
     for (int off = LANES / 2; off >= 1; off >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, off));
@@ -175,18 +190,15 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_subwave(
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * LANES + sub) * kVec;
         if (live && k0 < K) {
-            int code[kVec];
+            uint32_t lo = 0, hi = 0;
             if (shortcut) {
-                quantize_eight(v[c], scale, inv_scale, p, code);
+                quantize_eight_packed(v[c], scale, inv_scale, p, lo, hi);
             } else {
 #pragma unroll
-                for (int i = 0; i < kVec; ++i) code[i] = quantize_one(v[c][i], scale, p);
-            }
-            uint32_t lo = 0, hi = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                lo |= (static_cast<uint32_t>(code[i]) & 0xFFu) << (8 * i);
-                hi |= (static_cast<uint32_t>(code[i + 4]) & 0xFFu) << (8 * i);
+                for (int i = 0; i < 4; ++i) {
+                    lo |= (static_cast<uint32_t>(quantize_one(v[c][i], scale, p)) & 0xFFu) << (8 * i);
+                    hi |= (static_cast<uint32_t>(quantize_one(v[c][i + 4], scale, p)) & 0xFFu) << (8 * i);
+                }
             }
             *reinterpret_cast<uint2*>(cr + k0) = make_uint2(lo, hi);
         }
