@@ -286,6 +286,21 @@ def decoder_layer_share(dev, rng_seed=5):
         h = tops.int4pack_mm_swiglu(xn, L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros, L["up"].scales_and_zeros)
         return tops.int4pack_mm_add(h, L["down"].weight, 128, L["down"].scales_and_zeros, x1).view(B, 1, d)
 
+    def layer_fused_norm(L, x):
+        """layer_fused with the two RMS norms inside the launches that consume them (q, k, v; gate and up)."""
+        xf = x.view(B, d)
+        q, k, v = tops.int4pack_mm_multi(xf, [L[n].weight for n in "qkv"], 128, [L[n].scales_and_zeros for n in "qkv"],
+                                         norm_weight=n1, eps=1e-5)
+        q, k, v = (t.view(B, 1, H, D).transpose(1, 2) for t in (q, k, v))
+        q, k = rope(q), rope(k)
+        kc[:, :, T:T + 1] = k
+        vc[:, :, T:T + 1] = v
+        a = F.scaled_dot_product_attention(q, kc, vc).transpose(1, 2).reshape(B, H * D)
+        x1 = tops.int4pack_mm_add(a, L["o"].weight, 128, L["o"].scales_and_zeros, xf)
+        h = tops.int4pack_mm_swiglu(x1, L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros, L["up"].scales_and_zeros,
+                                    norm_weight=n2, eps=1e-5)
+        return tops.int4pack_mm_add(h, L["down"].weight, 128, L["down"].scales_and_zeros, x1).view(B, 1, d)
+
     xin = {n: torch.randn(B, 1, k, device=dev, generator=gen).half() for n, (_, k) in shapes.items()}
     res_d = torch.randn(B, d, device=dev, generator=gen).half()
 
@@ -294,6 +309,14 @@ def decoder_layer_share(dev, rng_seed=5):
         tops.int4pack_mm_add(xin["o"].view(B, d), L["o"].weight, 128, L["o"].scales_and_zeros, res_d)
         tops.int4pack_mm_swiglu(xin["gate"].view(B, d), L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros,
                                 L["up"].scales_and_zeros)
+        tops.int4pack_mm_add(xin["down"].view(B, inter), L["down"].weight, 128, L["down"].scales_and_zeros, res_d)
+
+    def linears_fused_norm(L):
+        tops.int4pack_mm_multi(xin["q"].view(B, d), [L[n].weight for n in "qkv"], 128, [L[n].scales_and_zeros for n in "qkv"],
+                               norm_weight=n1, eps=1e-5)
+        tops.int4pack_mm_add(xin["o"].view(B, d), L["o"].weight, 128, L["o"].scales_and_zeros, res_d)
+        tops.int4pack_mm_swiglu(xin["gate"].view(B, d), L["gate"].weight, L["up"].weight, 128, L["gate"].scales_and_zeros,
+                                L["up"].scales_and_zeros, norm_weight=n2, eps=1e-5)
         tops.int4pack_mm_add(xin["down"].view(B, inter), L["down"].weight, 128, L["down"].scales_and_zeros, res_d)
 
     def linears(L):
@@ -308,13 +331,20 @@ def decoder_layer_share(dev, rng_seed=5):
     torch.cuda.synchronize()
     fused_diff = float((out_f.float() - out.float()).abs().max() / out.float().abs().max())
     assert fused_diff < 2e-2, fused_diff
+    out_n = layer_fused_norm(layers[0], x0)
+    torch.cuda.synchronize()
+    norm_diff = float((out_n.float() - out.float()).abs().max() / out.float().abs().max())
+    assert norm_diff < 2e-2, norm_diff
     g_layer = graph_of(lambda: [layer(layers[i % copies], x0) for i in range(reps)])
     g_lin = graph_of(lambda: [linears(layers[i % copies]) for i in range(reps)])
     g_layer_f = graph_of(lambda: [layer_fused(layers[i % copies], x0) for i in range(reps)])
     g_lin_f = graph_of(lambda: [linears_fused(layers[i % copies]) for i in range(reps)])
-    res = {"layer_fused_vs_unfused_max_rel_diff": fused_diff}
+    g_layer_n = graph_of(lambda: [layer_fused_norm(layers[i % copies], x0) for i in range(reps)])
+    g_lin_n = graph_of(lambda: [linears_fused_norm(layers[i % copies]) for i in range(reps)])
+    res = {"layer_fused_vs_unfused_max_rel_diff": fused_diff, "layer_fused_norm_vs_unfused_max_rel_diff": norm_diff}
     for key, g in (("layer_decode_b8_kv2048_us", g_layer), ("layer_int4_linears_us", g_lin),
-                   ("layer_decode_fused_mlp_us", g_layer_f), ("layer_int4_linears_fused_us", g_lin_f)):
+                   ("layer_decode_fused_mlp_us", g_layer_f), ("layer_int4_linears_fused_us", g_lin_f),
+                   ("layer_decode_fused_mlp_norm_us", g_layer_n), ("layer_int4_linears_fused_norm_us", g_lin_n)):
         g.replay(); torch.cuda.synchronize()
         res[key] = steady(g.replay, torch.cuda.synchronize) / reps * 1e3
     res["layer_int4_linear_share"] = res["layer_int4_linears_us"] / res["layer_decode_b8_kv2048_us"]

@@ -238,6 +238,24 @@ int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count,
                       const void* const* scales_and_zeros, void* const* out, void* stream);
 
 /*
+ * The two entry points above with the RMS normalization of the activations in front, the norm -> projection
+ * pairs of a decoder layer (benchmark/bench_llama_e2e.py:126-128 q, k, v after n1; :143 gate and up after n2):
+ *   xn = rms_norm(x, norm_weight, eps) = T((float(x) * rsqrt(mean(float(x)^2) + eps)) * float(norm_weight)),
+ * computed in fp32 and rounded once to the activation dtype (tensorplay/nn/functional.py:2350-2372; native op
+ * rms_norm, config/native_functions.yaml:5962), then out = the product with xn as above.  norm_weight: [K] of
+ * dtype.  Built for K = 2048..4096 (every workgroup normalizes the rows for itself, no launch and no round trip
+ * of the activations through memory); other shapes return TPQ_ERR_UNSUPPORTED and the caller runs the norm and
+ * the plain entry point.
+ */
+int tpq_int4_mm_swiglu_norm(const void* x, int dtype, int64_t M, int64_t K, const void* norm_weight, float eps,
+                            const int32_t* packed_gate, const int32_t* packed_up, int inner_k_tiles,
+                            int64_t N, int64_t group, const void* sz_gate, const void* sz_up, void* out,
+                            void* stream);
+int tpq_int4_mm_multi_norm(const void* x, int dtype, int64_t M, int64_t K, const void* norm_weight, float eps,
+                           int count, const int32_t* const* packed, int inner_k_tiles, const int64_t* N,
+                           int64_t group, const void* const* scales_and_zeros, void* const* out, void* stream);
+
+/*
  * Dense weight [N, K] of `dtype` from the packed device layout: W = T(code - 8) * scale + zero, the
  * product and the sum each rounded to T.  The reference runs this before its library GEMM
  * (int4_tc_dequantize_kernel, p10/src/backend/cuda/QuantGemmKernels.cu:1170-1202, 1296-1341); the

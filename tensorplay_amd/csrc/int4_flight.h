@@ -11,6 +11,8 @@ struct FlightWeights {
     void* y[4];             // [rows][N]
     int N[4];
     int count;              // 1..4 weights; pair: 2 weights of the same N, one output y[0]
+    const void* norm_weight;  // not null: the activations are RMS-normalized first, weights [K] of the activation dtype
+    float norm_eps;
 };
 
 // 2..16 activation rows, 16-bit activations.  Returns false when the shape is not one of the built cases (nothing

@@ -21,12 +21,12 @@ inline int flight_compute_units() {
     return v;
 }
 
-template <int DT, int NB, int SPW, int XR, int MODE>
+template <int DT, int NB, int SPW, int XR, int MODE, bool NORM>
 int launch_as(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
     constexpr size_t bytes = flight_lds_bytes<NB, SPW, XR>();
     static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
     static std::atomic<uint64_t> reserved{0};
-    const auto kernel = int4_mfma_flight_kernel<DT, NB, SPW, XR, MODE>;
+    const auto kernel = int4_mfma_flight_kernel<DT, NB, SPW, XR, MODE, NORM>;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), bytes, reserved, "tpq_int4_mm (mfma, all in flight)")) return rc;
     constexpr int C = MODE == kFlightPair ? NB / 2 : NB;
     kernel<<<dim3((blocks + C - 1) / C), dim3(kFlightWaves * kWave), bytes, s>>>(x, set, rows, K, shift, residual);
@@ -36,10 +36,23 @@ int launch_as(const uint16_t* x, int rows, const FlightSet& set, int blocks, int
 // the row capacity: 4, 8 or 16 rows through LDS
 template <int DT, int NB, int SPW, int MODE>
 int launch_rows(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
-    if (rows <= 4) return launch_as<DT, NB, SPW, 4, MODE>(x, rows, set, blocks, K, shift, residual, s);
-    if (rows <= 8) return launch_as<DT, NB, SPW, 8, MODE>(x, rows, set, blocks, K, shift, residual, s);
+    if constexpr (SPW == 2 && MODE != kFlightOne) {  // the normalizing form: built for K = 2048..4096, pair and several weights
+        if (set.norm_weight != nullptr) {
+            if (rows <= 4) return launch_as<DT, NB, SPW, 4, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
+            if (rows <= 8) return launch_as<DT, NB, SPW, 8, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
+            if constexpr (flight_lds_bytes<NB, SPW, 16>() <= 160 * 1024) {
+                return launch_as<DT, NB, SPW, 16, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
+            } else {
+                return TPQ_ERR_UNSUPPORTED;
+            }
+        }
+    } else {
+        if (set.norm_weight != nullptr) return TPQ_ERR_UNSUPPORTED;  // not reached: launch() excludes the case
+    }
+    if (rows <= 4) return launch_as<DT, NB, SPW, 4, MODE, false>(x, rows, set, blocks, K, shift, residual, s);
+    if (rows <= 8) return launch_as<DT, NB, SPW, 8, MODE, false>(x, rows, set, blocks, K, shift, residual, s);
     if constexpr (flight_lds_bytes<NB, SPW, 16>() <= 160 * 1024 && SPW <= 4) {
-        return launch_as<DT, NB, SPW, 16, MODE>(x, rows, set, blocks, K, shift, residual, s);
+        return launch_as<DT, NB, SPW, 16, MODE, false>(x, rows, set, blocks, K, shift, residual, s);
     } else {
         return TPQ_ERR_UNSUPPORTED;  // not reached: flight_shape() excludes the case
     }
@@ -77,7 +90,9 @@ int flight_width(int blocks, int rows, int spw, bool pair, bool one_weight) {
 
 template <int DT>
 bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group, bool pair, const void* residual, hipStream_t s, int* rc) {
-    if (rows < 1 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256)) return false;
+    const bool norm = wts.norm_weight != nullptr;
+    if (norm && (!aligned(wts.norm_weight, 16) || K > 4096)) return false;  // two steps per wavefront
+    if (rows < 1 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256) || !aligned(x, 16)) return false;
     const int steps = K / 128;
     const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
     if (steps < kFlightWaves || spw > 7 || spw == 5) return false;
@@ -92,6 +107,9 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
     FlightSet set{};
     FlightWeight* const slots[kFlightMaxWeights] = {&set.w0, &set.w1, &set.w2, &set.w3};
     set.count = pair ? 1 : wts.count;
+    set.norm_weight = static_cast<const uint16_t*>(wts.norm_weight);
+    set.norm_eps = wts.norm_eps;
+    set.norm_inv_k = 1.0f / static_cast<float>(K);
     int blocks = 0;
     for (int w = 0; w < wts.count; ++w) {
         if (wts.N[w] % 8 != 0 || !aligned(wts.sz[w], 4) || !aligned(wts.packed[w], 16) || !aligned(wts.y[pair ? 0 : w], 8)) return false;
@@ -115,7 +133,7 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
         else code = launch_rows<DT, 2, 2, kFlightPair>(xp, rows, set, blocks, K, shift, rp, s);
     } else {
 #define TPQ_FLIGHT(NBV, SPWV)                                                                                   \
-    code = wts.count == 1 ? launch_rows<DT, NBV, SPWV, kFlightOne>(xp, rows, set, blocks, K, shift, rp, s)    \
+    code = wts.count == 1 && !norm ? launch_rows<DT, NBV, SPWV, kFlightOne>(xp, rows, set, blocks, K, shift, rp, s)    \
                           : launch_rows<DT, NBV, SPWV, kFlightMany>(xp, rows, set, blocks, K, shift, rp, s)
         switch (spw) {
             case 1: case 2:

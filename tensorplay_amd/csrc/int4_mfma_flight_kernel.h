@@ -27,6 +27,15 @@
 // A launch serves up to four weights that share the activations (the q, k and v projections of a decoder layer):
 // the blocks of 16 channels of all weights are numbered through, and a workgroup takes NB consecutive ones.
 // Pair mode: NB / 2 blocks of a gate weight and the same blocks of an up weight; the output is silu_mul(gate, up).
+// NORM: y = rms_norm(x, g, eps) . W^T, the norm -> projection pairs of a decoder layer
+// (benchmark/bench_llama_e2e.py:113-114, 126-128, 143), with rms_norm(x)[k] = (x[k] * rsqrt(mean(x^2) + eps)) * g[k]
+// (tensorplay/nn/functional.py:2350-2372).  The factor rsqrt(...) is one number per row, so it is taken out of the
+// sum: the activations are multiplied by g on their way into LDS (rounded to the activation dtype there, where the
+// reference rounds the normalized value: the same relative error), every wavefront adds the squares of its steps
+// (v_dot2 of the value with itself), and the finishing wavefront multiplies the row's sum by rsqrt(mean + eps) before
+// it rounds.  No barrier and no division in front of the products, no launch and no round trip of the activations
+// through memory for the norm; every workgroup does it for itself.  Results agree with the reference's two-step
+// formulation to the matmul's own tolerance, not bit for bit.
 #pragma once
 
 #include "int4_mfma_kernel.h"
@@ -51,6 +60,8 @@ struct FlightWeight {
 struct FlightSet {
     FlightWeight w0, w1, w2, w3;
     int count;
+    const uint16_t* norm_weight;  // NORM: [K] of the activation dtype
+    float norm_eps, norm_inv_k;   // eps and 1 / K
 };
 
 // Keeps the memory operations on either side in program order, for the compiler's code motion and for its
@@ -71,6 +82,9 @@ __device__ __forceinline__ GlobalWord opaque1(const void* p) {
     return (GlobalWord)p;
 }
 __device__ __forceinline__ uint4 as_uint4(word4_t v) { return make_uint4(v.x, v.y, v.z, v.w); }
+// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for every outstanding global load,
+// i.e. for the weights that are meant to stay in flight across it.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // steps of activations resident in LDS per wavefront at a time
 template <int XR>
@@ -80,13 +94,14 @@ template <int NB, int SPW, int XR>
 constexpr size_t flight_lds_bytes() {
     return static_cast<size_t>(kFlightWaves) * flight_resident_steps<XR>() * XR * kFlightRowStride  // activation tiles
          + static_cast<size_t>(kFlightWaves) * SPW * (NB > 4 ? 2 : 1) * kWave * 4                    // parameter words
-         + static_cast<size_t>(kFlightWaves) * NB * 4 * (4 * XR) * 4;                                // partial sums, live rows
+         + static_cast<size_t>(kFlightWaves) * NB * 4 * (4 * XR) * 4                                 // partial sums, live rows
+         + static_cast<size_t>(kFlightWaves) * XR * 4;                                               // NORM: sums of squares
 }
 
 // x: [M][K] 16-bit, M <= XR; weights as in FlightSet (packed: [N/8][K/32][8] x 16 bytes; sz: [K/group][N] words
 // (scale, zero)); K % 128 == 0, 16 <= K / 128 <= 16 SPW and K / 128 > 16 (SPW - 1); a group is 128 << group_shift k;
 // residual (one weight, may be null): [M][N], added to the rounded output.
-template <int DT, int NB, int SPW, int XR, int MODE>
+template <int DT, int NB, int SPW, int XR, int MODE, bool NORM = false>
 __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(const uint16_t* __restrict__ x, FlightSet set, int M,
                                                                               int K, int group_shift,
                                                                               const uint16_t* __restrict__ residual) {
@@ -209,6 +224,12 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
 #pragma unroll
         for (int j = 0; j < SPW; ++j) xg[j][t] = as_uint4(src[step_of[j] * 16]);
     }
+    uint4 gk[NORM ? SPW : 1];  // NORM: the norm weights of this lane's eight k per step
+    if constexpr (NORM) {
+        const GlobalWords4 src = opaque4(reinterpret_cast<const uint4*>(set.norm_weight) + i);
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) gk[j] = as_uint4(src[step_of[j] * 16]);
+    }
     order_fence();
     uint4 w[SPW][NB];
     {
@@ -246,6 +267,36 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
     for (int j = 0; j < SPW; ++j)
 #pragma unroll
         for (int h = 0; h < PW; ++h) my_par[(j * PW + h) * kWave + lane] = pw[j][h];
+
+    float* const ssq = red + kFlightWaves * NB * 4 * (4 * XR);  // [wave][XR], NORM only
+    if constexpr (NORM) {
+        // lane (i, q) holds eight k of row 4 t + q per step: squares added per row, the values multiplied by g in place
+        const bool last_counts = wave + (SPW - 1) * kFlightWaves < steps;
+#pragma unroll
+        for (int t = 0; t < XR / 4; ++t) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < SPW; ++j) {
+                const uint32_t gw[4] = {gk[j].x, gk[j].y, gk[j].z, gk[j].w};
+                uint32_t xw[4] = {xg[j][t].x, xg[j][t].y, xg[j][t].z, xg[j][t].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (j < SPW - 1 || last_counts) acc = L::dot(xw[e], xw[e], acc);  // a step past the end was read twice
+                    if constexpr (DT == TPQ_DTYPE_F16) {
+                        xw[e] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, xw[e]) * __builtin_bit_cast(half2_t, gw[e]));
+                    } else {
+                        const float lo = __fmul_rn(bf16_bits_to_f32(static_cast<uint16_t>(xw[e] & 0xFFFFu)), bf16_bits_to_f32(static_cast<uint16_t>(gw[e] & 0xFFFFu)));
+                        const float hi = __fmul_rn(bf16_bits_to_f32(static_cast<uint16_t>(xw[e] >> 16)), bf16_bits_to_f32(static_cast<uint16_t>(gw[e] >> 16)));
+                        xw[e] = static_cast<uint32_t>(f32_to_bf16_bits(lo)) | (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
+                    }
+                }
+                xg[j][t] = make_uint4(xw[0], xw[1], xw[2], xw[3]);
+            }
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+            if (i == 0) ssq[wave * XR + 4 * t + q] = acc;  // read behind the barrier at the end
+        }
+    }
 
     float yacc[NB][4];
 #pragma unroll
@@ -340,6 +391,16 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
 #pragma unroll
                 for (int ww = 0; ww < kFlightWaves; ++ww) sum[h][v] += red[((ww * NB + b + h * C) * 4 + v) * (4 * XR) + slot];
             }
+        if constexpr (NORM) {  // the row's factor rsqrt(mean(x^2) + eps)
+            float total = 0.0f;
+#pragma unroll
+            for (int ww = 0; ww < kFlightWaves; ++ww) total += ssq[ww * XR + i];
+            const float inv = __builtin_amdgcn_rsqf(__builtin_fmaf(total, set.norm_inv_k, set.norm_eps));
+#pragma unroll
+            for (int h = 0; h < (PAIR ? 2 : 1); ++h)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) sum[h][v] *= inv;
+        }
         uint16_t o[4];
         if constexpr (PAIR) {
 #pragma unroll

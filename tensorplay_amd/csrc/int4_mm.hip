@@ -514,7 +514,8 @@ bool launch_mfma_rows(const void* x, int rows, const int32_t* packed, const void
 // gate / up pair with the SwiGLU epilogue, and the plain product plus a residual: slabs of 16 rows
 template <int DT>
 int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz, const int32_t* packed_b, const void* sz_b,
-                 const void* residual, void* y, int N, int K, int group, hipStream_t s) {
+                 const void* residual, void* y, int N, int K, int group, hipStream_t s, const void* norm_weight = nullptr,
+                 float norm_eps = 0.0f) {
     const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
@@ -525,10 +526,13 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
             FlightWeights two{};
             two.packed[0] = packed; two.packed[1] = packed_b; two.sz[0] = sz; two.sz[1] = sz_b; two.y[0] = ys; two.N[0] = two.N[1] = N;
             two.count = 2;
+            two.norm_weight = norm_weight;
+            two.norm_eps = norm_eps;
             if (flight_launch(DT, xs, rows, two, K, group, true, nullptr, s, &rc)) {
                 if (rc != TPQ_OK) return rc;
                 continue;
             }
+            if (norm_weight != nullptr) return fail(TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_swiglu_norm: this shape is not built");
             static const int pair_waves = [] { const char* e = tuning_env("TPQ_INT4_PAIR_WAVES"); return e ? std::atoi(e) : 4; }();
             const auto* xp = reinterpret_cast<const uint16_t*>(xs);
             const auto* pa = reinterpret_cast<const uint4*>(packed);
@@ -554,7 +558,7 @@ int launch_fused(const void* x, int64_t M, const int32_t* packed, const void* sz
 // rule of launch_mfma_rows for the sum of the widths: that is the width the chip sees.
 template <int DT>
 int launch_multi(const void* x, int64_t M, int count, const int32_t* const* packed, const int64_t* N, const void* const* sz,
-                 void* const* y, int K, int group, hipStream_t s) {
+                 void* const* y, int K, int group, hipStream_t s, const void* norm_weight = nullptr, float norm_eps = 0.0f) {
     int64_t n_total = 0;
     for (int w = 0; w < count; ++w) n_total += N[w];
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
@@ -566,11 +570,14 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
                 all.packed[w] = packed[w]; all.sz[w] = sz[w]; all.N[w] = static_cast<int>(N[w]);
                 all.y[w] = static_cast<uint16_t*>(y[w]) + m0 * N[w];
             }
+            all.norm_weight = norm_weight;
+            all.norm_eps = norm_eps;
             int rc = TPQ_OK;
             if (flight_launch(DT, static_cast<const uint16_t*>(x) + m0 * K, rows, all, K, group, false, nullptr, s, &rc)) {
                 if (rc != TPQ_OK) return rc;
                 continue;
             }
+            if (norm_weight != nullptr) return fail(TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_multi_norm: this shape is not built");
         }
         const bool wide = n_total >= 10240 && n_total <= 28672 && rows <= 12;
         const int nb = n_total > 4096 ? (n_total < 10240 ? 2 : (rows > 4 || wide ? 4 : 2)) : 1;
@@ -941,9 +948,47 @@ TPQ_EXPORT int tpq_int4_mm_add(const void* x, int dtype, int64_t M, int64_t K, c
     return launch_fused<TPQ_DTYPE_BF16>(x, M, packed, scales_and_zeros, nullptr, nullptr, residual, out, (int)N, (int)K, (int)group, s);
 }
 
+namespace {
+int swiglu_entry(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed_gate, const int32_t* packed_up,
+                 int inner_k_tiles, int64_t N, int64_t group, const void* sz_gate, const void* sz_up, void* out, void* stream,
+                 const void* norm_weight, float norm_eps);
+int multi_entry(const void* x, int dtype, int64_t M, int64_t K, int count, const int32_t* const* packed, int inner_k_tiles,
+                const int64_t* N, int64_t group, const void* const* scales_and_zeros, void* const* out, void* stream,
+                const void* norm_weight, float norm_eps);
+}  // namespace
+
 TPQ_EXPORT int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed_gate,
                                   const int32_t* packed_up, int inner_k_tiles, int64_t N, int64_t group,
                                   const void* sz_gate, const void* sz_up, void* out, void* stream) {
+    return swiglu_entry(x, dtype, M, K, packed_gate, packed_up, inner_k_tiles, N, group, sz_gate, sz_up, out, stream, nullptr, 0.0f);
+}
+
+TPQ_EXPORT int tpq_int4_mm_swiglu_norm(const void* x, int dtype, int64_t M, int64_t K, const void* norm_weight, float eps,
+                                       const int32_t* packed_gate, const int32_t* packed_up, int inner_k_tiles, int64_t N,
+                                       int64_t group, const void* sz_gate, const void* sz_up, void* out, void* stream) {
+    TPQ_REQUIRE(norm_weight != nullptr && aligned(norm_weight, 16), TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_swiglu_norm: null or unaligned norm weight");
+    TPQ_REQUIRE(eps >= 0.0f, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_swiglu_norm: negative eps");
+    return swiglu_entry(x, dtype, M, K, packed_gate, packed_up, inner_k_tiles, N, group, sz_gate, sz_up, out, stream, norm_weight, eps);
+}
+
+TPQ_EXPORT int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count, const int32_t* const* packed,
+                                 int inner_k_tiles, const int64_t* N, int64_t group, const void* const* scales_and_zeros,
+                                 void* const* out, void* stream) {
+    return multi_entry(x, dtype, M, K, count, packed, inner_k_tiles, N, group, scales_and_zeros, out, stream, nullptr, 0.0f);
+}
+
+TPQ_EXPORT int tpq_int4_mm_multi_norm(const void* x, int dtype, int64_t M, int64_t K, const void* norm_weight, float eps, int count,
+                                      const int32_t* const* packed, int inner_k_tiles, const int64_t* N, int64_t group,
+                                      const void* const* scales_and_zeros, void* const* out, void* stream) {
+    TPQ_REQUIRE(norm_weight != nullptr && aligned(norm_weight, 16), TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi_norm: null or unaligned norm weight");
+    TPQ_REQUIRE(eps >= 0.0f, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi_norm: negative eps");
+    return multi_entry(x, dtype, M, K, count, packed, inner_k_tiles, N, group, scales_and_zeros, out, stream, norm_weight, eps);
+}
+
+namespace {
+int swiglu_entry(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed_gate, const int32_t* packed_up,
+                 int inner_k_tiles, int64_t N, int64_t group, const void* sz_gate, const void* sz_up, void* out, void* stream,
+                 const void* norm_weight, float norm_eps) {
     if (int rc = check_fused("tpq_int4_mm_swiglu", dtype, M, K, inner_k_tiles, N, group)) return rc;
     if (M == 0 || N == 0) return TPQ_OK;
     TPQ_REQUIRE(K > 0, TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_swiglu: K = 0 is not built");
@@ -953,13 +998,13 @@ TPQ_EXPORT int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K
                 TPQ_ERR_UNSUPPORTED, "tpq_int4_mm_swiglu: unaligned operand");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TPQ_DTYPE_F16)
-        return launch_fused<TPQ_DTYPE_F16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s);
-    return launch_fused<TPQ_DTYPE_BF16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s);
+        return launch_fused<TPQ_DTYPE_F16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s, norm_weight, norm_eps);
+    return launch_fused<TPQ_DTYPE_BF16>(x, M, packed_gate, sz_gate, packed_up, sz_up, nullptr, out, (int)N, (int)K, (int)group, s, norm_weight, norm_eps);
 }
 
-TPQ_EXPORT int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count, const int32_t* const* packed,
-                                 int inner_k_tiles, const int64_t* N, int64_t group, const void* const* scales_and_zeros,
-                                 void* const* out, void* stream) {
+int multi_entry(const void* x, int dtype, int64_t M, int64_t K, int count, const int32_t* const* packed, int inner_k_tiles,
+                const int64_t* N, int64_t group, const void* const* scales_and_zeros, void* const* out, void* stream,
+                const void* norm_weight, float norm_eps) {
     TPQ_REQUIRE(count >= 1 && count <= kMultiMax, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: 1 to %d weights per call", kMultiMax);
     TPQ_REQUIRE(packed && N && scales_and_zeros && out, TPQ_ERR_INVALID_VALUE, "tpq_int4_mm_multi: null pointer");
     int64_t n_total = 0;
@@ -979,6 +1024,7 @@ TPQ_EXPORT int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K,
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TPQ_DTYPE_F16)
-        return launch_multi<TPQ_DTYPE_F16>(x, M, count, packed, N, scales_and_zeros, out, (int)K, (int)group, s);
-    return launch_multi<TPQ_DTYPE_BF16>(x, M, count, packed, N, scales_and_zeros, out, (int)K, (int)group, s);
+        return launch_multi<TPQ_DTYPE_F16>(x, M, count, packed, N, scales_and_zeros, out, (int)K, (int)group, s, norm_weight, norm_eps);
+    return launch_multi<TPQ_DTYPE_BF16>(x, M, count, packed, N, scales_and_zeros, out, (int)K, (int)group, s, norm_weight, norm_eps);
 }
+}  // namespace

@@ -696,10 +696,29 @@ def int4pack_mm_add(input: torch.Tensor, mat2: torch.Tensor, qGroupSize: int, qS
     return out
 
 
-def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zeros) -> list:
+def rms_norm(input: torch.Tensor, weight: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+    """The reference's ``rms_norm`` over the last dimension (tensorplay/nn/functional.py:2350-2372): fp32 compute for
+    reduced dtypes, ``(x * rsqrt(mean(x^2) + eps)) * weight`` rounded once to the input dtype.  Plain tensor ops: it is
+    what the fused entry points below fall back to, not a kernel of this library."""
+    x = input.float()
+    out = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        out = out * weight.float()
+    return out.to(input.dtype)
+
+
+def _norm_operand(x: torch.Tensor, norm_weight: torch.Tensor, what: str) -> torch.Tensor:
+    if norm_weight.dim() != 1 or norm_weight.numel() != x.shape[1] or norm_weight.dtype != x.dtype or norm_weight.device != x.device:
+        raise ValueError(f"{what}: norm_weight must be [k] of the activation dtype, on the activations' device")
+    return norm_weight.contiguous()
+
+
+def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zeros, norm_weight: Optional[torch.Tensor] = None,
+                      eps: float = 1e-5) -> list:
     """``[_weight_int4pack_mm(input, w, qGroupSize, sz) for w, sz in zip(mats, scales_and_zeros)]`` with one launch
     per 16 rows for up to four weights (q, k, v of a decoder layer).  Shapes the fused kernel does not take, and more
-    than four weights, run the separate op."""
+    than four weights, run the separate op.  With ``norm_weight`` the products are taken of ``rms_norm(input,
+    norm_weight, eps)``, normalized inside the same launch where the kernel is built for it."""
     mats, scales_and_zeros = list(mats), list(scales_and_zeros)
     if len(mats) != len(scales_and_zeros) or not mats:
         raise ValueError("int4pack_mm_multi: one qScaleAndZeros per packed weight, at least one weight")
@@ -709,8 +728,11 @@ def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zer
     x = ops[0][0]
     m, k = x.shape
 
+    g = None if norm_weight is None else _norm_operand(x, norm_weight, "int4pack_mm_multi")
+
     def separate():
-        return [_weight_int4pack_mm(x, w, qGroupSize, sz) for _, w, sz, _, _ in ops]
+        xn = x if g is None else rms_norm(x, g, eps)
+        return [_weight_int4pack_mm(xn, w, qGroupSize, sz) for _, w, sz, _, _ in ops]
 
     if len(ops) > 4 or len({inner for _, _, _, inner, _ in ops}) != 1 or x.dtype == torch.float32:
         return separate()
@@ -723,9 +745,15 @@ def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zer
     ys = (ctypes.c_void_p * count)(*[_ptr(o) for o in outs])
     widths = (ctypes.c_int64 * count)(*[n for _, _, _, _, n in ops])
     with torch.cuda.device(x.device):
-        status = _lib.load().tpq_int4_mm_multi(_ptr(x), _DT[x.dtype], m, k, count, ctypes.cast(packed, ctypes.c_void_p), ops[0][3],
-                                               ctypes.cast(widths, ctypes.c_void_p), qGroupSize, ctypes.cast(szs, ctypes.c_void_p),
-                                               ctypes.cast(ys, ctypes.c_void_p), _stream(x))
+        if g is None:
+            status = _lib.load().tpq_int4_mm_multi(_ptr(x), _DT[x.dtype], m, k, count, ctypes.cast(packed, ctypes.c_void_p), ops[0][3],
+                                                   ctypes.cast(widths, ctypes.c_void_p), qGroupSize, ctypes.cast(szs, ctypes.c_void_p),
+                                                   ctypes.cast(ys, ctypes.c_void_p), _stream(x))
+        else:
+            status = _lib.load().tpq_int4_mm_multi_norm(_ptr(x), _DT[x.dtype], m, k, _ptr(g), float(eps), count,
+                                                        ctypes.cast(packed, ctypes.c_void_p), ops[0][3],
+                                                        ctypes.cast(widths, ctypes.c_void_p), qGroupSize,
+                                                        ctypes.cast(szs, ctypes.c_void_p), ctypes.cast(ys, ctypes.c_void_p), _stream(x))
     if status == _lib.TPQ_ERR_UNSUPPORTED:
         return separate()
     _check(status)
@@ -733,10 +761,12 @@ def int4pack_mm_multi(input: torch.Tensor, mats, qGroupSize: int, scales_and_zer
 
 
 def int4pack_mm_swiglu(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, qGroupSize: int,
-                       gate_scale_and_zeros: torch.Tensor, up_scale_and_zeros: torch.Tensor) -> torch.Tensor:
+                       gate_scale_and_zeros: torch.Tensor, up_scale_and_zeros: torch.Tensor,
+                       norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
     """``silu_mul(_weight_int4pack_mm(input, gate, ...), _weight_int4pack_mm(input, up, ...))`` in one launch
     (the reference's ``silu_mul``: gate * sigmoid(gate) * up in float32, rounded once).  Shapes the fused kernel
-    does not take run the separate ops."""
+    does not take run the separate ops.  With ``norm_weight`` the input is ``rms_norm(input, norm_weight, eps)``,
+    normalized inside the same launch where the kernel is built for it."""
     _fused_int4_check(input, gate, qGroupSize, gate_scale_and_zeros, "int4pack_mm_swiglu")
     _fused_int4_check(input, up, qGroupSize, up_scale_and_zeros, "int4pack_mm_swiglu")
     x, wg, szg, inner, n = _fused_int4_operands(input, gate, qGroupSize, gate_scale_and_zeros, "int4pack_mm_swiglu")
@@ -747,12 +777,18 @@ def int4pack_mm_swiglu(input: torch.Tensor, gate: torch.Tensor, up: torch.Tensor
     out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     if m == 0 or n == 0:
         return out
+    nw = None if norm_weight is None else _norm_operand(x, norm_weight, "int4pack_mm_swiglu")
     with torch.cuda.device(x.device):
-        status = _lib.load().tpq_int4_mm_swiglu(_ptr(x), _DT[x.dtype], m, k, _ptr(wg), _ptr(wu), inner, n, qGroupSize, _ptr(szg),
-                                                _ptr(szu), _ptr(out), _stream(x))
+        if nw is None:
+            status = _lib.load().tpq_int4_mm_swiglu(_ptr(x), _DT[x.dtype], m, k, _ptr(wg), _ptr(wu), inner, n, qGroupSize, _ptr(szg),
+                                                    _ptr(szu), _ptr(out), _stream(x))
+        else:
+            status = _lib.load().tpq_int4_mm_swiglu_norm(_ptr(x), _DT[x.dtype], m, k, _ptr(nw), float(eps), _ptr(wg), _ptr(wu), inner, n,
+                                                         qGroupSize, _ptr(szg), _ptr(szu), _ptr(out), _stream(x))
     if status == _lib.TPQ_ERR_UNSUPPORTED:
-        g = _weight_int4pack_mm(x, wg, qGroupSize, szg).float()
-        u = _weight_int4pack_mm(x, wu, qGroupSize, szu).float()
+        xn = x if nw is None else rms_norm(x, nw, eps)
+        g = _weight_int4pack_mm(xn, wg, qGroupSize, szg).float()
+        u = _weight_int4pack_mm(xn, wu, qGroupSize, szu).float()
         return (g * torch.sigmoid(g) * u).to(x.dtype)
     _check(status)
     return out

@@ -372,6 +372,63 @@ def test_mm_multi_equals_separate_products(ops, tdt, tol, M, K, widths):
         assert_close_norm(y.float().cpu().numpy()[:, cols], want, 2 * tol)
 
 
+def _rms_norm_bits(x_bits, g_bits, tag, eps):
+    """The reference's rms_norm in numpy float32 (tensorplay/nn/functional.py:2350-2372), rounded to the dtype."""
+    x = oracle.to_f32(x_bits, tag)
+    inv = (1.0 / np.sqrt((x * x).mean(-1, keepdims=True, dtype=np.float32) + np.float32(eps))).astype(np.float32)
+    return oracle.from_f32((x * inv) * oracle.to_f32(g_bits, tag), tag)
+
+
+@pytest.mark.parametrize("tdt,tol", [(torch.float16, 1e-3), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("M,K,widths", [(8, 4096, (4096, 4096, 4096)), (3, 2048, (72, 136)), (13, 4096, (264,)), (1, 4096, (520, 8)),
+                                        (20, 4096, (136, 136)), (4, 1024, (64, 64))])
+def test_mm_multi_with_rms_norm_against_oracle(ops, tdt, tol, M, K, widths):
+    """rms_norm -> several products in one launch (q, k, v after the first norm of a decoder layer): against the oracle's
+    product of the numpy-normalized activations, and against the unfused sequence on the device.  K = 1024 is a shape
+    the fused kernel is not built for: the wrapper normalizes with tensor ops."""
+    rng = np.random.default_rng(M * 17 + K + len(widths))
+    tag = "f16" if tdt == torch.float16 else "bf16"
+    cases = [_fused_case(rng, M, n, K, tdt) for n in widths]
+    x = (cases[0][2] * 3.0 + 0.5).to(tdt).to(DEV)    # not unit variance, not zero mean
+    g = torch.from_numpy(rng.uniform(0.5, 1.5, K).astype(np.float32)).to(tdt).to(DEV)
+    packed = [ops._convert_weight_to_int4pack(torch.from_numpy(c).to(DEV), 2) for c, _, _ in cases]
+    szs = [sz.to(DEV) for _, sz, _ in cases]
+    got = ops.int4pack_mm_multi(x, packed, 128, szs, norm_weight=g, eps=1e-5)
+    xn_dev = ops.rms_norm(x, g, 1e-5)
+    xn = _rms_norm_bits(host(x), host(g), tag, 1e-5)
+    # the normalized activations themselves: device composite against numpy, at most one rounding apart
+    assert_close_norm(xn_dev.float().cpu().numpy(), oracle.to_f32(xn, tag), 2.0 ** -10 if tag == "f16" else 2.0 ** -7)
+    for (codes, sz, _), p, szd, y, n in zip(cases, packed, szs, got, widths):
+        assert tuple(y.shape) == (M, n) and y.dtype == tdt
+        assert_close_norm(y.float().cpu().numpy(), ops._weight_int4pack_mm(xn_dev, p, 128, szd).float().cpu().numpy(), 2 * tol)
+        tiles = _tile_subset(rng, n // 8, 32)
+        cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+        want = oracle.to_f32(oracle.int4_mm_tc(xn, tag, oracle.int4_pack_tc(codes[cols], 2), host(sz)[:, cols], 128), tag)
+        assert_close_norm(y.float().cpu().numpy()[:, cols], want, 2 * tol)
+
+
+@pytest.mark.parametrize("tdt,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)])
+@pytest.mark.parametrize("M,N,K", [(8, 11008, 4096), (2, 72, 4096), (5, 136, 2048), (12, 200, 4096), (3, 64, 512)])
+def test_mm_swiglu_with_rms_norm_against_oracle(ops, tdt, tol, M, N, K):
+    """rms_norm -> gate / up -> silu_mul in one launch (the MLP front of a decoder layer)."""
+    rng = np.random.default_rng(M * 29 + N)
+    tag = "f16" if tdt == torch.float16 else "bf16"
+    cg, szg, x = _fused_case(rng, M, N, K, tdt)
+    cu, szu, _ = _fused_case(rng, M, N, K, tdt)
+    x = (x * 2.0 - 0.25).to(tdt).to(DEV)
+    g = torch.from_numpy(rng.uniform(0.5, 1.5, K).astype(np.float32)).to(tdt).to(DEV)
+    pg = ops._convert_weight_to_int4pack(torch.from_numpy(cg).to(DEV), 2)
+    pu = ops._convert_weight_to_int4pack(torch.from_numpy(cu).to(DEV), 2)
+    got = ops.int4pack_mm_swiglu(x, pg, pu, 128, szg.to(DEV), szu.to(DEV), norm_weight=g, eps=1e-5)
+    xn = _rms_norm_bits(host(x), host(g), tag, 1e-5)
+    tiles = _tile_subset(rng, N // 8, 32)
+    cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    og = oracle.to_f32(oracle.int4_mm_tc(xn, tag, oracle.int4_pack_tc(cg[cols], 2), host(szg)[:, cols], 128), tag)
+    ou = oracle.to_f32(oracle.int4_mm_tc(xn, tag, oracle.int4_pack_tc(cu[cols], 2), host(szu)[:, cols], 128), tag)
+    want = og * (1.0 / (1.0 + np.exp(-og))) * ou
+    assert_close_norm(got.float().cpu().numpy()[:, cols], want, 2 * tol)
+
+
 def test_mm_multi_other_shapes_and_errors(ops):
     rng = np.random.default_rng(6)
     codes = rng.integers(0, 16, (32, 128)).astype(np.int32)
