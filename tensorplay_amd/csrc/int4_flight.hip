@@ -36,7 +36,7 @@ int launch_as(const uint16_t* x, int rows, const FlightSet& set, int blocks, int
 // the row capacity: 4, 8 or 16 rows through LDS
 template <int DT, int NB, int SPW, int MODE>
 int launch_rows(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
-    if constexpr (SPW == 2 && MODE != kFlightOne) {  // the normalizing form: built for K = 2048..4096, pair and several weights
+    if constexpr (SPW <= 2 && MODE != kFlightOne) {  // the normalizing form: built for K = 2048..4096, pair and several weights
         if (set.norm_weight != nullptr) {
             if (rows <= 4) return launch_as<DT, NB, SPW, 4, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
             if (rows <= 8) return launch_as<DT, NB, SPW, 8, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
