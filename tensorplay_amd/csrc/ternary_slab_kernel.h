@@ -12,8 +12,9 @@
 //   * the activations go through LDS once: each 16-byte chunk is transposed as a 4 x 4 byte matrix on its way
 //     (the cheap expansion of a packed dword yields the codes of one field position of its four bytes, so the
 //     k order of the MFMA operands is field-major; see ternary_decode_mfma.h), a 64-byte segment becomes four
-//     16-byte MFMA operands (operand f = field f of its four chunks), kept in slot (8 unit + 4 half + f) ^ (row % 8)
-//     of the row: conflict-free reads;
+//     16-byte MFMA operands (operand f = field f of its four chunks), kept in slot (8 unit + 4 half + f) ^ (row % 16)
+//     of the row (rows are a multiple of 256 bytes apart): the 16 lanes that a 16-byte LDS read serves together
+//     hit 16 different bank groups;
 //   * one barrier, then wavefront (nb, kp) multiplies channel block nb with the units kp, kp + 4, ... :
 //     v_mfma_i32_32x32x32_i8, A = activations from LDS, B = weight fields masked out of the packed words in
 //     registers (5 instructions per 16 codes: the expansion is the vector ALU's whole load in this phase, and
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     // wavefront load is two runs of 512 contiguous bytes (eight cache lines; a 64-byte segment per lane made it 64
     // lines, and the texture path's line look-ups were the time of the whole kernel)
     uint4 xa[kSlabChunkRounds];
-    const int row_slots = 8 * U;
+    const int row_slots = 8 * (U + (U & 1));  // an even number of units per row: the swizzle below swaps neighbouring units
     const int x_row = tid >> 5, x_lane = tid & 31;
     {
         const int m = m0 + x_row < M ? m0 + x_row : M - 1;
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
 #pragma unroll
         for (int r = 0; r < kSlabChunkRounds; ++r) {
             const int cc = x_lane + 32 * r;  // chunk cc of the row: unit cc / 8, half (cc / 4) % 2, c = cc % 4
-            xa[r] = src[cc < row_slots ? cc : 0];
+            xa[r] = src[cc < 8 * U ? cc : 0];
         }
     }
     // weights: lane (n, half) of wavefront (nb, kp): row n0 + 32 nb + n, the 16 bytes (64 codes) of half `half` of the unit
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     TPQ_STAMP(1);
     // ---- activations into LDS, in MFMA operand order ------------------------------------------------------
     // chunk c of a segment, transposed, is dword c of each of the segment's four operands: operand f of segment
-    // (unit, half) sits in slot (8 unit + 4 half + f) ^ (row % 8) of the row.  The codes are multiplied as
+    // (unit, half) sits in slot (8 unit + 4 half + f) ^ (row % 16) of the row.  The codes are multiplied as
     // unsigned fields with the sign bit flipped (code = (field ^ 2) - 2), so the row sums of the activations
     // are needed once per row: every thread adds its chunks, the 32 threads of a row meet through the lanes.
     int* const row_sum = reinterpret_cast<int*>(slab_lds + lds_main_bytes);  // [32]
@@ -107,11 +108,11 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
 #pragma unroll
         for (int r = 0; r < kSlabChunkRounds; ++r) {
             const int cc = x_lane + 32 * r;
-            if (cc < row_slots) {
+            if (cc < 8 * U) {
                 const v4i t = transpose_4x4_bytes(xa[r]);
-                const int dst = (x_row * row_slots + ((cc & ~3) ^ (x_row & 7))) * 16 + (cc & 3) * 4;
+                const int dst = (x_row * row_slots + ((cc & ~3) ^ (x_row & 15))) * 16 + (cc & 3) * 4;
 #pragma unroll
-                for (int f = 0; f < 4; ++f) {  // f is xor-ed into the swizzled slot: row_slots is a multiple of 8
+                for (int f = 0; f < 4; ++f) {  // f is xor-ed into the swizzled slot: row_slots is a multiple of 16
                     *reinterpret_cast<int*>(slab_lds + (dst ^ (f * 16))) = t[f];
                     mine = __builtin_amdgcn_sdot4(t[f], 0x01010101, mine, false);
                 }
@@ -132,8 +133,9 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     v16i acc0, acc1, acc2, acc3;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = acc2[v] = acc3[v] = 0;
-    // A: lane (m, half) reads row m; operand f of unit u: slot (8 u + 4 half + f) ^ (m % 8) = 8 u + ((4 half + f) ^ (m % 8))
-    const unsigned char* a_row = slab_lds + static_cast<size_t>(wn) * row_slots * 16;
+    // A: lane (m, half) reads row m; operand f of unit u: slot (8 u + 4 half + f) ^ (m % 16) = 8 (u ^ (m / 8 % 2)) + ((4 half + f) ^ (m % 8));
+    // the units of a wavefront (kp, kp + 4, ...) have the parity of kp, so the swap of neighbours is one offset per lane
+    const unsigned char* a_row = slab_lds + static_cast<size_t>(wn) * row_slots * 16 + ((wn & 8) ? ((kp & 1) ? -128 : 128) : 0);
     int a_off[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) a_off[f] = ((4 * half + f) ^ (wn & 7)) * 16;
@@ -245,7 +247,7 @@ int launch_ternary_slab(const int8_t* x, const uint8_t* packed, int64_t M, int64
                         Epilogue ep, hipStream_t s) {
     const int units = static_cast<int>(K / 128);
     const int per_split = (units + splits - 1) / splits;
-    const size_t slab_bytes = static_cast<size_t>(kSlabRows) * per_split * 128;
+    const size_t slab_bytes = static_cast<size_t>(kSlabRows) * (per_split + (per_split & 1)) * 128;
     const size_t part_bytes = static_cast<size_t>(16) * 16 * kWave * sizeof(int);  // 64 KB
     const size_t main_bytes = slab_bytes > part_bytes ? slab_bytes : part_bytes;
     const size_t smem = main_bytes + kSlabRows * sizeof(int);
