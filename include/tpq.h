@@ -243,9 +243,12 @@ int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count,
  *   xn = rms_norm(x, norm_weight, eps) = T((float(x) * rsqrt(mean(float(x)^2) + eps)) * float(norm_weight)),
  * computed in fp32 and rounded once to the activation dtype (tensorplay/nn/functional.py:2350-2372; native op
  * rms_norm, config/native_functions.yaml:5962), then out = the product with xn as above.  norm_weight: [K] of
- * dtype.  Built for K = 2048..4096 (every workgroup normalizes the rows for itself, no launch and no round trip
- * of the activations through memory); other shapes return TPQ_ERR_UNSUPPORTED and the caller runs the norm and
- * the plain entry point.
+ * dtype.  The kernel takes the row factor rsqrt(mean + eps) out of the sum: it multiplies T(x * norm_weight) with
+ * the weights and scales the finished fp32 sums of a row, so no launch and no round trip of the activations through
+ * memory is spent on the norm; the result differs from the two-step formulation only in where the rounding to T
+ * falls and agrees with it to the tolerance of the product (1e-2 relative; 1e-3 against exact sums for float16).
+ * Built for K = 2048..8192 (the pair: 2049..4096) at up to 16 rows (the pair: 8); other shapes return
+ * TPQ_ERR_UNSUPPORTED and the caller runs the norm and the plain entry point.
  */
 int tpq_int4_mm_swiglu_norm(const void* x, int dtype, int64_t M, int64_t K, const void* norm_weight, float eps,
                             const int32_t* packed_gate, const int32_t* packed_up, int inner_k_tiles,

@@ -36,7 +36,7 @@ int launch_as(const uint16_t* x, int rows, const FlightSet& set, int blocks, int
 // the row capacity: 4, 8 or 16 rows through LDS
 template <int DT, int NB, int SPW, int MODE>
 int launch_rows(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
-    if constexpr (SPW <= 2 && MODE != kFlightOne) {  // the normalizing form: built for K = 2048..4096, pair and several weights
+    if constexpr (SPW <= 4 && MODE != kFlightOne) {  // the normalizing form: built for K = 2048..8192, pair and several weights
         if (set.norm_weight != nullptr) {
             if (rows <= 4) return launch_as<DT, NB, SPW, 4, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
             if (rows <= 8) return launch_as<DT, NB, SPW, 8, MODE, true>(x, rows, set, blocks, K, shift, residual, s);
@@ -91,7 +91,7 @@ int flight_width(int blocks, int rows, int spw, bool pair, bool one_weight) {
 template <int DT>
 bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group, bool pair, const void* residual, hipStream_t s, int* rc) {
     const bool norm = wts.norm_weight != nullptr;
-    if (norm && (!aligned(wts.norm_weight, 16) || K > 4096)) return false;  // two steps per wavefront
+    if (norm && (!aligned(wts.norm_weight, 16) || K > 8192)) return false;  // built for up to four steps per wavefront
     if (rows < 1 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256) || !aligned(x, 16)) return false;
     const int steps = K / 128;
     const int spw = (steps + kFlightWaves - 1) / kFlightWaves;

@@ -381,7 +381,8 @@ def _rms_norm_bits(x_bits, g_bits, tag, eps):
 
 @pytest.mark.parametrize("tdt,tol", [(torch.float16, 1e-3), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("M,K,widths", [(8, 4096, (4096, 4096, 4096)), (3, 2048, (72, 136)), (13, 4096, (264,)), (1, 4096, (520, 8)),
-                                        (20, 4096, (136, 136)), (4, 1024, (64, 64))])
+                                        (20, 4096, (136, 136)), (4, 1024, (64, 64)), (8, 8192, (1024, 136, 136)), (16, 5120, (264, 72)),
+                                        (2, 6144, (2048,))])
 def test_mm_multi_with_rms_norm_against_oracle(ops, tdt, tol, M, K, widths):
     """rms_norm -> several products in one launch (q, k, v after the first norm of a decoder layer): against the oracle's
     product of the numpy-normalized activations, and against the unfused sequence on the device.  K = 1024 is a shape
@@ -458,6 +459,32 @@ def test_fused_entry_points_fall_back_for_other_shapes(ops):
     out = ops.int4pack_mm_swiglu(x, packed, packed, 32, sz, sz)
     g = ops._weight_int4pack_mm(x, packed, 32, sz).float()
     assert torch.equal(out, (g * torch.sigmoid(g) * g).half())
+
+
+@pytest.mark.parametrize("K,taken", [(1024, False), (2048, True), (4096, True), (5120, True), (8192, True), (11008, False)])
+def test_norm_entry_point_takes_the_shapes_it_names(ops, K, taken):
+    """tpq_int4_mm_multi_norm through the C ABI: OK for K = 2048..8192, TPQ_ERR_UNSUPPORTED outside (the wrapper then runs
+    the norm and the plain entry), so the oracle comparisons above do exercise the fused kernel at those K."""
+    import ctypes
+    from tensorplay_amd import _lib
+    rng = np.random.default_rng(K)
+    n, m = 136, 5
+    codes = rng.integers(0, 16, (n, K)).astype(np.int32)
+    packed = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(DEV), 2)
+    sz = (torch.rand(K // 128, n, 2, device=DEV) * 0.01).half()
+    x = torch.randn(m, K, device=DEV).half()
+    g = torch.ones(K, device=DEV).half()
+    out = torch.empty(m, n, device=DEV).half()
+    ptrs = lambda t: (ctypes.c_void_p * 1)(t.data_ptr())
+    widths = (ctypes.c_int64 * 1)(n)
+    status = _lib.load().tpq_int4_mm_multi_norm(x.data_ptr(), 1, m, K, g.data_ptr(), 1e-5, 1, ctypes.cast(ptrs(packed), ctypes.c_void_p), 2,
+                                                ctypes.cast(widths, ctypes.c_void_p), 128, ctypes.cast(ptrs(sz), ctypes.c_void_p),
+                                                ctypes.cast(ptrs(out), ctypes.c_void_p), torch.cuda.current_stream().cuda_stream)
+    assert status == (0 if taken else _lib.TPQ_ERR_UNSUPPORTED)
+    if taken:
+        torch.cuda.synchronize()
+        want = ops._weight_int4pack_mm(ops.rms_norm(x, g, 1e-5), packed, 128, sz)
+        assert_close_norm(out.float().cpu().numpy(), want.float().cpu().numpy(), 2e-3)
 
 
 # ---- the decoder layer of the benchmark configuration: seven int4 linears at batch 8 -----------------------------------
