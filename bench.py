@@ -648,6 +648,20 @@ def main() -> int:
         extras["quantize_2048x4096_bf16_us"] = ms * 1e3
         extras["quantize_GBs"] = (3 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
 
+        # rms_norm of the same prefill block (the stand-alone op; at decode sizes the norm is folded into the int4 launches):
+        # 2*M*K read + 2*M*K written + 2*K bytes
+        gn = (torch.rand(K8, device=dev) + 0.5).to(torch.bfloat16)
+        yn = torch.empty_like(xa_d)
+
+        def norm():
+            lib.tpq_rms_norm(xa_d.data_ptr(), _lib.BF16, M8, K8, gn.data_ptr(), 1e-5, yn.data_ptr(), cur())
+
+        for _ in range(5):
+            norm()
+        ms = steady(norm, sync, 100)
+        extras["rms_norm_2048x4096_bf16_us"] = ms * 1e3
+        extras["rms_norm_GBs"] = (4 * M8 * K8 + 2 * K8) / (ms * 1e-3) / 1e9
+
         # block-wise affine quantizer: the same activations in f32, one block per row -> int8 (4 + 1 bytes per
         # element), and a 4096 x 4096 f32 weight in groups of 128 -> packed 4-bit (4 + 0.5) and back (0.5 + 4)
         import ctypes

@@ -259,6 +259,18 @@ int tpq_int4_mm_multi_norm(const void* x, int dtype, int64_t M, int64_t K, const
                            int64_t group, const void* const* scales_and_zeros, void* const* out, void* stream);
 
 /*
+ * rms_norm over the last dimension (native op rms_norm, config/native_functions.yaml:5962; CPU kernel
+ * p10/src/backend/cpu/NormalizationKernels.cpp:1355-1453; Python composite tensorplay/nn/functional.py:2350-2372):
+ *   out[m][k] = T((float(x[m][k]) * inv[m]) * float(weight[k])),  inv[m] = 1 / sqrt(mean_k(float(x[m][k])^2) + eps),
+ * all in fp32, one rounding to `dtype` (float32 / float16 / bfloat16).  x, out: [M, K] contiguous; weight: [K] of
+ * `dtype` or null (no scaling).  The sum of squares is added in a tree order, the reference's CPU kernel adds serially:
+ * results agree to an ulp of `dtype`, not bit for bit.  It is the stand-alone form of the norm that
+ * tpq_int4_mm_multi_norm / tpq_int4_mm_swiglu_norm fold into the matmul at decode sizes.
+ */
+int tpq_rms_norm(const void* x, int dtype, int64_t M, int64_t K, const void* weight, float eps, void* out,
+                 void* stream);
+
+/*
  * Dense weight [N, K] of `dtype` from the packed device layout: W = T(code - 8) * scale + zero, the
  * product and the sum each rounded to T.  The reference runs this before its library GEMM
  * (int4_tc_dequantize_kernel, p10/src/backend/cuda/QuantGemmKernels.cu:1170-1202, 1296-1341); the

@@ -325,6 +325,17 @@ def weight_int8pack_mm(x, dtype, w, scales, want_f64=False):
     return (out, y64) if want_f64 else out
 
 
+def rms_norm(x, dtype, weight=None, eps=1e-5, want_f64=False):
+    """rms_norm over the last dimension of a 2-D array of storage bits / float32; weight: [K] of the same type or None."""
+    x = _c(x, storage(dtype))
+    M, K = x.shape
+    weight = None if weight is None else _c(weight, storage(dtype))
+    out = np.zeros((M, K), storage(dtype))
+    y64 = np.zeros((M, K), np.float64) if want_f64 else None
+    lib().orc_rms_norm(_p(x), _DT[dtype], ctypes.c_int64(M), ctypes.c_int64(K), _p(weight), ctypes.c_float(eps), _p(out), _p(y64))
+    return (out, y64) if want_f64 else out
+
+
 AFFINE_STORAGE = {"qint8": (0, np.int8, 1), "quint8": (1, np.uint8, 1), "qint32": (2, np.int32, 1),
                   "quint4x2": (3, np.uint8, 2), "quint2x4": (4, np.uint8, 4), "quint1x8": (5, np.uint8, 8)}
 _AFFINE_BOUNDS = {"qint8": (-128, 127), "quint8": (0, 255), "qint32": (-2**31, 2**31 - 1),

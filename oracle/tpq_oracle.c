@@ -688,6 +688,45 @@ ORC_API void orc_weight_int8pack_mm(const void* x, int dtype, const int8_t* w, c
 }
 
 /* ------------------------------------------------------------------------ */
+/* rms_norm                                                                   */
+/* ------------------------------------------------------------------------ */
+
+/* rms_norm over the last dimension, rows of K: the CPU kernel of the reference
+ * (p10/src/backend/cpu/NormalizationKernels.cpp:1355-1453).  float32 rows
+ * (:1389-1396) and float16 / bfloat16 rows (:1424-1449) follow the same steps in
+ * float: acc += v * v serially, inv = 1 / sqrt(acc / K + eps), v = x * inv,
+ * v *= w, one rounding to the storage type.  weight may be NULL.  y64, when not
+ * NULL, receives the same formula evaluated in double on the same inputs (the
+ * composite of tensorplay/nn/functional.py:2350-2372 without its roundings).
+ * Pinned by: torch.nn.functional.rms_norm on the CPU (a library twin: float32
+ * within 2 ulp, 16-bit types within one rounding), the float64 closed form,
+ * exact invariance under scaling the row by a power of two at eps = 0, a
+ * constant row (x = c: out = sign(c) w up to rounding), zero rows (out = 0).
+ */
+ORC_API void orc_rms_norm(const void* x, int dtype, int64_t M, int64_t K, const void* weight, float eps,
+                          void* out, double* y64) {
+    for (int64_t m = 0; m < M; ++m) {
+        float acc = 0.0f;
+        double acc64 = 0.0;
+        for (int64_t k = 0; k < K; ++k) {
+            const float v = load_as_f32(x, dtype, m * K + k);
+            acc += v * v;
+            acc64 += (double)v * (double)v;
+        }
+        const float inv = 1.0f / sqrtf(acc / (float)K + eps);
+        const double inv64 = 1.0 / sqrt(acc64 / (double)K + (double)eps);
+        for (int64_t k = 0; k < K; ++k) {
+            const float xv = load_as_f32(x, dtype, m * K + k);
+            float v = xv * inv;
+            const float w = weight ? load_as_f32(weight, dtype, k) : 1.0f;
+            if (weight) v *= w;
+            store_from_f32(out, dtype, m * K + k, v);
+            if (y64) y64[m * K + k] = (double)xv * inv64 * (double)w;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* Block-wise affine quantizer                                               */
 /* ------------------------------------------------------------------------ */
 

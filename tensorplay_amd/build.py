@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libtpq_gfx950.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
-SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "probe.hip"]
+SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "rms_norm.hip", "probe.hip"]
 
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32.
 # -ffp-contract=off: fused multiply-adds only where the source asks for one,

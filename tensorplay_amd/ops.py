@@ -697,14 +697,31 @@ def int4pack_mm_add(input: torch.Tensor, mat2: torch.Tensor, qGroupSize: int, qS
 
 
 def rms_norm(input: torch.Tensor, weight: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
-    """The reference's ``rms_norm`` over the last dimension (tensorplay/nn/functional.py:2350-2372): fp32 compute for
-    reduced dtypes, ``(x * rsqrt(mean(x^2) + eps)) * weight`` rounded once to the input dtype.  Plain tensor ops: it is
-    what the fused entry points below fall back to, not a kernel of this library."""
-    x = input.float()
-    out = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    """The reference's ``rms_norm`` over the last dimension (native op ``rms_norm``, config/native_functions.yaml:5962;
+    tensorplay/nn/functional.py:2350-2372): fp32 compute, ``(x * (1 / sqrt(mean(x^2) + eps))) * weight`` rounded once
+    to the input dtype.  One launch; the fused entry points below fall back to it for the shapes they are not built for."""
+    _require_device(input, "rms_norm()")
+    if input.dim() < 1:
+        raise ValueError("rms_norm(): expected at least one dimension")
+    if input.dtype not in _DT:
+        raise TypeError(f"rms_norm(): unsupported dtype {input.dtype}")
+    k = input.shape[-1]
     if weight is not None:
-        out = out * weight.float()
-    return out.to(input.dtype)
+        _require_device(weight, "rms_norm()")
+        if weight.dim() != 1 or weight.numel() != k:
+            raise ValueError("rms_norm(): weight must have the size of the last dimension")
+        if weight.dtype != input.dtype:
+            weight = weight.to(input.dtype)
+        weight = weight.contiguous()
+    x = input.contiguous()
+    out = torch.empty_like(x)
+    m = x.numel() // k if k else 0
+    if m == 0 or k == 0:
+        return out
+    with torch.cuda.device(x.device):
+        _check(_lib.load().tpq_rms_norm(_ptr(x), _DT[x.dtype], m, k, _ptr(weight), float(eps),
+                                        _ptr(out), _stream(x)))
+    return out
 
 
 def _norm_operand(x: torch.Tensor, norm_weight: torch.Tensor, what: str) -> torch.Tensor:
