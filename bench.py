@@ -647,6 +647,20 @@ def main() -> int:
         ms = steady(quant, sync, 100)
         extras["quantize_2048x4096_bf16_us"] = ms * 1e3
         extras["quantize_GBs"] = (3 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
+        # the same with the input rotating through 24 copies (403 MB: beyond the 256 MB memory-side cache), i.e. read
+        # from HBM every time; the figure above re-reads one 16.8 MB input, as a quantizer behind the kernel that
+        # produced its input does
+        xa_rot = [xa_d] + [xa_d.clone() for _ in range(23)]
+        turn = [0]
+
+        def quant_rot():
+            turn[0] = (turn[0] + 1) % 24
+            lib.tpq_quantize_rowwise(xa_rot[turn[0]].data_ptr(), _lib.BF16, M8, K8, 1e-5, 127.0, -127, 127, 0, cq.data_ptr(),
+                                     sq.data_ptr(), cur())
+
+        ms = steady(quant_rot, sync, 96)
+        extras["quantize_2048x4096_bf16_hbm_rotated_us"] = ms * 1e3
+        extras["quantize_hbm_rotated_GBs"] = (3 * M8 * K8 + 4 * M8) / (ms * 1e-3) / 1e9
 
         # rms_norm of the same prefill block (the stand-alone op; at decode sizes the norm is folded into the int4 launches):
         # 2*M*K read + 2*M*K written + 2*K bytes
@@ -661,6 +675,15 @@ def main() -> int:
         ms = steady(norm, sync, 100)
         extras["rms_norm_2048x4096_bf16_us"] = ms * 1e3
         extras["rms_norm_GBs"] = (4 * M8 * K8 + 2 * K8) / (ms * 1e-3) / 1e9
+
+        def norm_rot():
+            turn[0] = (turn[0] + 1) % 24
+            lib.tpq_rms_norm(xa_rot[turn[0]].data_ptr(), _lib.BF16, M8, K8, gn.data_ptr(), 1e-5, yn.data_ptr(), cur())
+
+        ms = steady(norm_rot, sync, 96)
+        extras["rms_norm_2048x4096_bf16_hbm_rotated_us"] = ms * 1e3
+        extras["rms_norm_hbm_rotated_GBs"] = (4 * M8 * K8 + 2 * K8) / (ms * 1e-3) / 1e9
+        del xa_rot
 
         # block-wise affine quantizer: the same activations in f32, one block per row -> int8 (4 + 1 bytes per
         # element), and a 4096 x 4096 f32 weight in groups of 128 -> packed 4-bit (4 + 0.5) and back (0.5 + 4)
