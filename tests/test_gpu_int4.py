@@ -619,3 +619,36 @@ def test_mm_one_row_down_projection_default_route(ops):
     _, y64 = oracle.int4_mm_tc(xb, "f16", oracle.int4_pack_tc(codes[cols], 2), np.ascontiguousarray(szb[:, cols]), 128,
                                round_w=False, want_f64=True)
     assert rel_err(got[:, cols], y64) < 1e-3
+
+
+# ---- one row of a wide weight at lengths other than 2048 / 4096 / 6144: the looped form of the column-per-lane kernel ------
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("N,K", [
+    (10304, 2560),    # 20 chunks of 128 k: twelve of the 16 wavefronts take one, four take two
+    (10240, 5120),    # 40 chunks
+    (10248, 7168),    # 56 chunks; ragged last column group
+    (10240, 8192),    # 64 chunks: four per wavefront
+    (10240, 10240),   # five
+    (10312, 11008),   # 86 chunks
+    (10240, 14336),   # seven per wavefront
+])
+def test_mm_one_row_wide_weight_other_lengths(ops, dtype, N, K):
+    """Column-per-lane kernel (N >= 10240) at one row where K / 128 is not 16, 32 or 48: against the fp64 sums (1e-3 fp16,
+    1e-2 bf16) and the reference's device formulation (1e-2 / 1.5e-2) on a subset of whole tiles that contains the first
+    and the last, and every channel against the 2-row call's first row (the matrix-core kernel: another order of sums)."""
+    rng = np.random.default_rng(N + K)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), 128)
+    x = rng.normal(0, 1, (2, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = dev(oracle.int4_pack_tc(codes, 2))
+    got = ops._weight_int4pack_mm(dev(xb[:1], dtype), packed, 128, dev(szb, dtype)).float().cpu().numpy()
+    two = ops._weight_int4pack_mm(dev(xb, dtype), packed, 128, dev(szb, dtype)).float().cpu().numpy()
+    tiles = _tile_subset(rng, N // 8, 48)
+    cols = (tiles[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    sub_packed, sub_sz = oracle.int4_pack_tc(codes[cols], 2), np.ascontiguousarray(szb[:, cols])
+    ref_dev = oracle.to_f32(oracle.int4_mm_tc(xb[:1], dtype, sub_packed, sub_sz, 128, round_w=True), dtype)
+    _, y64 = oracle.int4_mm_tc(xb[:1], dtype, sub_packed, sub_sz, 128, round_w=False, want_f64=True)
+    assert_close_norm(got[:, cols], ref_dev, 1.5e-2 if dtype == "bf16" else 1e-2, "one row vs reference formulation")
+    assert rel_err(got[:, cols], y64) < (1e-3 if dtype == "f16" else 1e-2)
+    assert rel_err(got, two[:1]) < (2e-3 if dtype == "f16" else 1.6e-2)
