@@ -624,7 +624,17 @@ bool launch_row(const void* x, const int32_t* packed, const void* sz, void* y, i
     // 11008 -> 4096: 7.0 / 8.7 / 12.1;  5120 x 5120: 5.9 / 6.8 / 7.1.  Not for K <= 4096 (4096 -> 11008: 7.2 / 8.1 / 6.8;
     // 4096 x 4096: 6.0 / 4.7 / 5.8), not when the tiles need a second batch of rounds (4096 -> 14336: 10.1 / 8.6 / 7.7;
     // 8192 x 8192: 10.6 / 9.3 / 10.9), and a workgroup wants at least two tiles.
-    const bool wins = K > 4096 && n_tiles >= 2 * cus && n_tiles <= rounds * cus;
+    // Wide weights (several batches of rounds per workgroup): this kernel deals tiles evenly to one workgroup per compute
+    // unit, the column-per-lane kernel runs ceil(N / 64 / 256) rounds of workgroups and loses most where the last round
+    // is a small fraction.  Measured (us, this kernel / default): K = 8192: N = 10240 10.5 / 11.6, 16384 14.9 / 16.7,
+    // 20480 19.2 / 23.3, 28672 23.8 / 27.3 (14336: 14.5 / 14.7); K = 12288: N = 8192 11.6 / 12.8, 12288 15.9 / 17.1,
+    // 24576 28.4 / 33.1; last round at most 60 % full (N = 20480, 24576): K = 5120 14.2 / 15.3, 7168 17.7 / 19.8,
+    // 10240 22.1 / 25.7.  Elsewhere the default is as fast or faster (K = 5120, N = 14336: 11.1 / 9.1; K = 10240,
+    // N = 14336: 17.9 / 15.5).
+    const int column_groups = (N + kWave - 1) / kWave, last_round = column_groups % compute_units();
+    const bool short_last_round = column_groups > compute_units() && last_round > 0 && last_round * 10 <= compute_units() * 6;
+    const bool wide = K > 4096 && (short_last_round || (K >= 7680 && K < 10240 && N >= 10240) || (K >= 12288 && N >= 8192));
+    const bool wins = K > 4096 && ((n_tiles >= 2 * cus && n_tiles <= rounds * cus) || wide);
     if (!(force || pinned == 1) && !wins) return false;
     const int shift = group == 32 ? 0 : group == 64 ? 1 : group == 128 ? 2 : 3;
     const dim3 grid(cus), block(waves * kWave);
