@@ -632,9 +632,13 @@ def test_mm_one_row_down_projection_default_route(ops):
     (10240, 10240),   # five
     (10312, 11008),   # 86 chunks
     (10240, 14336),   # seven per wavefront
+    (20488, 8192),    # wide and ragged at K = 8192: the tile-streaming kernel in several batches, a last partial tile group
+    (8200, 12288),    # K = 12288: three blocks per wavefront
+    (20552, 5120),    # column groups whose last round is short: the tile-streaming kernel at K = 5120
 ])
 def test_mm_one_row_wide_weight_other_lengths(ops, dtype, N, K):
-    """Column-per-lane kernel (N >= 10240) at one row where K / 128 is not 16, 32 or 48: against the fp64 sums (1e-3 fp16,
+    """One row of a wide weight where K / 128 is not 16, 32 or 48 (the looped column-per-lane kernel, or the tile-streaming
+    kernel where the library prefers it): against the fp64 sums (1e-3 fp16,
     1e-2 bf16) and the reference's device formulation (1e-2 / 1.5e-2) on a subset of whole tiles that contains the first
     and the last, and every channel against the 2-row call's first row (the matrix-core kernel: another order of sums)."""
     rng = np.random.default_rng(N + K)
