@@ -68,7 +68,13 @@ struct Chunk {
 // and the k-tiles are consumed one by one as they arrive.  With a loop and its bounds checks around the chunks
 // (CPW = 0) the compiler waits for every outstanding load before the first use, which leaves the whole
 // arithmetic of the wavefront (two chunks: about 400 vector instructions) behind the end of the stream.
-template <int DT, int MROWS, int GROUP_KT, int WPB, int CPW = 0>
+// PAUSE > 0: the wavefront sleeps 64 x PAUSE clocks between the requests of its first chunk and those of the others.
+// The memory system takes a compute unit's requests at the rate it returns data, oldest wavefront first, so without the
+// pause wavefront 0 has asked for everything before wavefront 15 has asked for anything, the chunks of the last
+// wavefronts all arrive at the very end, and their arithmetic (a quarter of a SIMD's work) trails the stream.  With
+// it every wavefront's first chunk is asked for ahead of the second chunks and only half of that work is left at
+// the end.  Measured at 4096 -> 11008 (us): no pause 6.19; 12: 6.12; 16..24: 6.05..6.07; 32: 6.29; 40: 6.43.
+template <int DT, int MROWS, int GROUP_KT, int WPB, int CPW = 0, int PAUSE = 0>
 __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
     const uint32_t* __restrict__ x, const uint4* __restrict__ packed, const uint32_t* __restrict__ sz,
     uint16_t* __restrict__ y, int N, int K, int k_super, float* ws_part, unsigned* ws_count) {
@@ -177,9 +183,17 @@ __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < CPW; ++u)
+        for (int u = 0; u < CPW; ++u) {
 #pragma unroll
             for (int i = 0; i < kChunkKT; ++i) own[u].q[i] = nt_load(wp + static_cast<size_t>((wave + u * WPB) * kChunkKT + i) * 8);
+            if constexpr (PAUSE > 0) {
+                if (u == 0 && CPW > 1) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_sleep(PAUSE);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < CPW; ++u) consume(own[u], wave + u * WPB);
@@ -371,7 +385,14 @@ int launch_decode_rows(const void* x, const int32_t* packed, const void* sz, voi
         if (WPB == 16 && slices == 1 && !tuning_env("TPQ_DECODE_LOOP")) {  // the branch-free body where the chunks divide evenly
             const int n_chunks = K / 128;
             if (n_chunks == 16) { int4_decode_kernel<DT, MROWS, G, WPB, 1><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
-            if (n_chunks == 32) { int4_decode_kernel<DT, MROWS, G, WPB, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+            if (n_chunks == 32) {
+                if constexpr (MROWS == 1) {
+                    static const bool no_pause = tuning_env("TPQ_INT4_NO_PAUSE") != nullptr;
+                    if (!no_pause) { int4_decode_kernel<DT, MROWS, G, WPB, 2, 20><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+                }
+                int4_decode_kernel<DT, MROWS, G, WPB, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters);
+                return;
+            }
             if (n_chunks == 48 && MROWS == 1 && G == 4) { int4_decode_kernel<DT, MROWS, G, WPB, 3><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
         }
         int4_decode_kernel<DT, MROWS, G, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters);
