@@ -393,7 +393,12 @@ int launch_decode_rows(const void* x, const int32_t* packed, const void* sz, voi
                 int4_decode_kernel<DT, MROWS, G, WPB, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters);
                 return;
             }
-            if (n_chunks == 48 && MROWS == 1 && G == 4) { int4_decode_kernel<DT, MROWS, G, WPB, 3><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+            if (n_chunks == 48 && MROWS == 1 && G == 4) {
+                static const bool no_pause3 = tuning_env("TPQ_INT4_NO_PAUSE") != nullptr;
+                if (!no_pause3) { int4_decode_kernel<DT, MROWS, G, WPB, 3, 20><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters); return; }
+                int4_decode_kernel<DT, MROWS, G, WPB, 3><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters);
+                return;
+            }
         }
         int4_decode_kernel<DT, MROWS, G, WPB><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, k_super, partials, counters);
     };
