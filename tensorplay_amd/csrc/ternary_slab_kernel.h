@@ -7,20 +7,25 @@
 // U <= 20 units of 128 k:
 //
 //   * all 1024 threads request their share of the 32 x 128 U bytes of activations (16-byte chunks, a wavefront
-//     load = 1 KB contiguous) and their own packed weights (one 16-byte load = 64 codes per unit) up front,
-//     straight-line; nothing is waited for until everything has been asked for;
+//     load = 1 KB contiguous) and their own packed weights up front, straight-line; nothing is waited for until
+//     everything has been asked for.  The epilogue's row scales and bias are asked for first and parked in LDS;
 //   * the activations go through LDS once: each 16-byte chunk is transposed as a 4 x 4 byte matrix on its way
 //     (the cheap expansion of a packed dword yields the codes of one field position of its four bytes, so the
 //     k order of the MFMA operands is field-major; see ternary_decode_mfma.h), a 64-byte segment becomes four
 //     16-byte MFMA operands (operand f = field f of its four chunks), kept in slot (8 unit + 4 half + f) ^ (row % 16)
 //     of the row (rows are a multiple of 256 bytes apart): the 16 lanes that a 16-byte LDS read serves together
 //     hit 16 different bank groups;
-//   * one barrier, then wavefront (nb, kp) multiplies channel block nb with the units kp, kp + 4, ... :
-//     v_mfma_i32_32x32x32_i8, A = activations from LDS, B = weight fields masked out of the packed words in
-//     registers (5 instructions per 16 codes: the expansion is the vector ALU's whole load in this phase, and
-//     with 3 instructions per four codes it, not the matrix core, set the time), four MFMAs per unit;
+//   * one barrier, then wavefront (nb, kp) multiplies channel block nb with its units (slab_unit_of):
+//     v_mfma_i32_32x32x32_i8, A = activations from LDS, B = weight fields moved to the top of their bytes in
+//     registers, four MFMAs per unit;
 //   * the four k-parts meet in LDS (the slab's space, after a second barrier); every wavefront finishes and
 //     stores a quarter of its block.
+//
+// Where the time goes (clock stamps at 128 x 6912 x 2560, 216 workgroups): the requests of a workgroup are taken
+// at the rate data returns, and the last wavefront's activations are there after about half of the kernel; from then
+// on 16 wavefronts on four SIMDs pay four clocks of a SIMD per vector instruction and wavefront, so a hundred
+// instructions per wavefront are 1600 clocks: the expansion of the weights, the sums and the epilogue are
+// instruction issue, not memory (without the weight loads the phases behind the barrier take as long as with them).
 //
 // With more than one split of K the exact int32 sums of split z go to partial[z][M][N] and ternary_slab_finish_kernel
 // adds them and applies the epilogue; with one split the epilogue is applied here.
@@ -36,7 +41,7 @@ constexpr int kSlabUnitsPerWave = 5, kSlabKParts = 4, kSlabUnits = kSlabUnitsPer
 constexpr int kSlabChunkRounds = kSlabRows * kSlabUnits * 8 / kSlabThreads;                          // 5 chunks of 16 bytes per thread
 
 // x: [M][K] int8; packed: [N][K/4]; units_per_split units of 128 k per workgroup (<= kSlabUnits), split z takes the
-// units z units_per_split ...; lds_main_bytes: size of the slab / k-part area, the 32 row sums sit behind it;
+// units z units_per_split ...; lds_main_bytes: size of the slab / k-part area; 32 row scales and 128 bias values sit behind it;
 // grid: 8 m_tiles ceil(n_tiles splits / 8) workgroups (see the id mapping below); partial: [gridDim.z][M][N] int32 or null (one split: the epilogue stores)
 #ifdef TPQ_SLAB_STAMPS
 __device__ unsigned long long g_slab_stamps[16 * 16];
@@ -44,6 +49,13 @@ __device__ unsigned long long g_slab_stamps[16 * 16];
 #else
 #define TPQ_STAMP(I) do { } while (0)
 #endif
+
+// Unit j of k-part kp.  A row of packed weights holds four units per 128-byte cache line; a wavefront load takes 32
+// bytes of 32 rows, so the four units of a line go to one wavefront, which asks for them back to back: the line is
+// brought into the first-level cache once.  Dealt round-robin (unit kp + 4 j) every line was fetched by four
+// wavefronts at four different times, four times the traffic between the caches.  Units 16..19 go one to each k-part.
+__device__ __forceinline__ constexpr int slab_unit_of(int kp, int j) { return j < 4 ? 4 * kp + j : 16 + kp; }
+static_assert(kSlabUnitsPerWave == 5 && kSlabKParts == 4, "slab_unit_of deals 20 units");
 
 template <class Epilogue>
 __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t* __restrict__ x, const uint8_t* __restrict__ packed,
@@ -67,6 +79,13 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     const int U = units_total - unit0 < units_per_split ? units_total - unit0 : units_per_split;  // this workgroup's units, >= 1
 
     TPQ_STAMP(0);
+    // the epilogue's row scales and bias, asked for ahead of everything else and parked in LDS: fetched at the end they
+    // are a trip to memory that nothing covers
+    float scale_word = 0.0f;
+    if (partial == nullptr) {
+        if (tid < kSlabRows) scale_word = ep.row_scale_of(m0 + tid < M ? m0 + tid : M - 1);
+        else if (tid < kSlabRows + kSlabChannels) scale_word = ep.bias_of(n0 + tid - kSlabRows < N ? n0 + tid - kSlabRows : N - 1);
+    }
     // ---- requests ---------------------------------------------------------------------------------------------
     // activations: 16-byte chunks, 32 threads per row (thread t: row t / 32, chunks t % 32, t % 32 + 32, ...): a
     // wavefront load is two runs of 512 contiguous bytes (eight cache lines; a 64-byte segment per lane made it 64
@@ -83,93 +102,113 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
             xa[r] = src[cc < 8 * U ? cc : 0];
         }
     }
-    // weights: lane (n, half) of wavefront (nb, kp): row n0 + 32 nb + n, the 16 bytes (64 codes) of half `half` of the unit
+    // weights of wavefront (nb, kp).  The MFMA wants lane (n, half) to hold the 16 bytes (64 codes) of half `half` of
+    // a unit for row n0 + 32 nb + n: asked for like that, a wavefront load takes 32 bytes out of 32 cache lines.  The
+    // four units of the wavefront's own line are therefore fetched as two pairs of loads that take 64 bytes (two
+    // units) out of 16 lines each: load A rows 0..15, load B rows 16..31, the 16-lane groups of either holding the
+    // chunks (unit, half) of the run in the order (e, 0), (o, 0), (e, 1), (o, 1).  One v_permlane16_swap per register
+    // (group 1 of A against group 0 of B, group 3 against group 2) then leaves unit e in MFMA order in the one and
+    // unit o in the other.  The fifth unit (16 + kp) is asked for in MFMA order directly.
     const int wn = lane & 31, half = lane >> 5;
-    uint4 wq[kSlabUnitsPerWave];
+    uint4 wq[kSlabUnitsPerWave];  // pair 0: A, B; pair 1: A, B; the single unit
     {
-        const int n = n0 + 32 * nb + wn < N ? n0 + 32 * nb + wn : N - 1;
-        const uint4* src = reinterpret_cast<const uint4*>(packed + static_cast<size_t>(n) * (K >> 2) + (static_cast<size_t>(unit0) << 5)) + half;
+        const int n16 = lane & 15, group = lane >> 4;
+        const int odd = group & 1, run_half = group >> 1;  // the group's chunk: unit 2 pair + odd, half run_half
+        const int row_a = n0 + 32 * nb + n16 < N ? n0 + 32 * nb + n16 : N - 1;
+        const int row_b = n0 + 32 * nb + 16 + n16 < N ? n0 + 32 * nb + 16 + n16 : N - 1;
+        const size_t pitch = static_cast<size_t>(K >> 2);
+        const unsigned char* base = packed + (static_cast<size_t>(unit0) << 5) + run_half * 16;
 #pragma unroll
-        for (int j = 0; j < kSlabUnitsPerWave; ++j) {
-            const int u = kp + kSlabKParts * j;
-            wq[j] = nt_load(src + (u < U ? u : 0) * 2);  // a unit past the end re-reads unit 0 and is not multiplied
+        for (int pr = 0; pr < 2; ++pr) {
+            const int u = 4 * kp + 2 * pr + odd;
+            const int off = (u < U ? u : 0) * 32;  // a unit past the end re-reads unit 0 and is not multiplied
+            wq[2 * pr] = nt_load(reinterpret_cast<const uint4*>(base + row_a * pitch + off));
+            wq[2 * pr + 1] = nt_load(reinterpret_cast<const uint4*>(base + row_b * pitch + off));
         }
+        const int n = n0 + 32 * nb + wn < N ? n0 + 32 * nb + wn : N - 1;
+        const int u = 16 + kp;
+        wq[4] = nt_load(reinterpret_cast<const uint4*>(packed + n * pitch + (static_cast<size_t>(unit0) << 5)) + half + (u < U ? u : 0) * 2);
     }
 
     TPQ_STAMP(1);
     // ---- activations into LDS, in MFMA operand order ------------------------------------------------------
     // chunk c of a segment, transposed, is dword c of each of the segment's four operands: operand f of segment
-    // (unit, half) sits in slot (8 unit + 4 half + f) ^ (row % 16) of the row.  The codes are multiplied as
-    // unsigned fields with the sign bit flipped (code = (field ^ 2) - 2), so the row sums of the activations
-    // are needed once per row: every thread adds its chunks, the 32 threads of a row meet through the lanes.
-    int* const row_sum = reinterpret_cast<int*>(slab_lds + lds_main_bytes);  // [32]
-    {
-        int mine = 0;
+    // (unit, half) sits in slot (8 unit + 4 half + f) ^ (row % 16) of the row.
+    float* const scale_lds = reinterpret_cast<float*>(slab_lds + lds_main_bytes);  // [32] row scales, [128] bias (one split only)
+    if (partial == nullptr && tid < kSlabRows + kSlabChannels) scale_lds[tid] = scale_word;
 #pragma unroll
-        for (int r = 0; r < kSlabChunkRounds; ++r) {
-            const int cc = x_lane + 32 * r;
-            if (cc < 8 * U) {
-                const v4i t = transpose_4x4_bytes(xa[r]);
-                const int dst = (x_row * row_slots + ((cc & ~3) ^ (x_row & 15))) * 16 + (cc & 3) * 4;
+    for (int r = 0; r < kSlabChunkRounds; ++r) {
+        const int cc = x_lane + 32 * r;
+        if (cc < 8 * U) {
+            const v4i t = transpose_4x4_bytes(xa[r]);
+            const int dst = (x_row * row_slots + ((cc & ~3) ^ (x_row & 15))) * 16 + (cc & 3) * 4;
 #pragma unroll
-                for (int f = 0; f < 4; ++f) {  // f is xor-ed into the swizzled slot: row_slots is a multiple of 16
-                    *reinterpret_cast<int*>(slab_lds + (dst ^ (f * 16))) = t[f];
-                    mine = __builtin_amdgcn_sdot4(t[f], 0x01010101, mine, false);
-                }
-            }
+            for (int f = 0; f < 4; ++f)  // f is xor-ed into the swizzled slot: row_slots is a multiple of 16
+                *reinterpret_cast<int*>(slab_lds + (dst ^ (f * 16))) = t[f];
         }
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) mine += __shfl_xor(mine, off, kWave);
-        if (x_lane == 0) row_sum[x_row] = mine;
     }
     TPQ_STAMP(2);
     __syncthreads();
     TPQ_STAMP(3);
 
     // ---- wavefront (nb, kp): 32 rows x 32 channels over its units ------------------------------------------
-    // Field f of the sign-flipped word, left where it is: w & mask is the field times 16, 4, 1 (f = 1, 2, 3); the top
-    // field would overflow a signed byte there and is moved down one bit first (times 32).  One accumulator per
-    // field position, put together with exact shifts at the end: 5 instructions per 16 codes.
-    v16i acc0, acc1, acc2, acc3;
+    // A 2-bit field at the top of a byte is the code times 64 as a signed byte (0b11 -> -64, 0b10 -> -128: the
+    // reference's sign extension of the field, tensorplay/ao/quantization/bitnet.py:75-79), so field f of the four
+    // bytes of a word is (w << 2 f) & 0xC0C0C0C0: seven instructions per 16 codes, every field at the same weight, no
+    // offset to take out afterwards.  |sum| <= 2560 * 127 * 128 < 2^31.  Two accumulators, so that consecutive MFMAs
+    // do not wait for each other; the factor 64 is taken out of the finished sum with an exact shift.
+    v16i acc0, acc1;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = acc2[v] = acc3[v] = 0;
-    // A: lane (m, half) reads row m; operand f of unit u: slot (8 u + 4 half + f) ^ (m % 16) = 8 (u ^ (m / 8 % 2)) + ((4 half + f) ^ (m % 8));
-    // the units of a wavefront (kp, kp + 4, ...) have the parity of kp, so the swap of neighbours is one offset per lane
-    const unsigned char* a_row = slab_lds + static_cast<size_t>(wn) * row_slots * 16 + ((wn & 8) ? ((kp & 1) ? -128 : 128) : 0);
+    for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0;
+    // A: lane (m, half) reads row m; operand f of unit u: slot (8 u + 4 half + f) ^ (m % 16) = 8 (u ^ (m / 8 % 2)) + ((4 half + f) ^ (m % 8))
+    const unsigned char* a_row = slab_lds + static_cast<size_t>(wn) * row_slots * 16;
     int a_off[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) a_off[f] = ((4 * half + f) ^ (wn & 7)) * 16;
 #pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {  // loads A and B of a pair -> its even and its odd unit in MFMA order
+        uint32_t a[4] = {wq[2 * pr].x, wq[2 * pr].y, wq[2 * pr].z, wq[2 * pr].w};
+        uint32_t b[4] = {wq[2 * pr + 1].x, wq[2 * pr + 1].y, wq[2 * pr + 1].z, wq[2 * pr + 1].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const auto r = __builtin_amdgcn_permlane16_swap(a[d], b[d], false, false);
+            a[d] = r[0];
+            b[d] = r[1];
+        }
+        wq[2 * pr] = make_uint4(a[0], a[1], a[2], a[3]);
+        wq[2 * pr + 1] = make_uint4(b[0], b[1], b[2], b[3]);
+    }
+#pragma unroll
     for (int j = 0; j < kSlabUnitsPerWave; ++j) {
-        const int u = kp + kSlabKParts * j;
+        const int u = slab_unit_of(kp, j);
         if (u < U) {  // wave-uniform
-            const uint32_t w0 = wq[j].x ^ 0xAAAAAAAAu, w1 = wq[j].y ^ 0xAAAAAAAAu, w2 = wq[j].z ^ 0xAAAAAAAAu, w3 = wq[j].w ^ 0xAAAAAAAAu;
-            const unsigned char* a_unit = a_row + u * 128;
+            const uint32_t w0 = wq[j].x, w1 = wq[j].y, w2 = wq[j].z, w3 = wq[j].w;
+            const unsigned char* a_unit = a_row + (u ^ ((wn >> 3) & 1)) * 128;  // neighbouring units swapped for rows 8..15, 24..31
+            constexpr uint32_t kTop = 0xC0C0C0C0u;
             {
-                const v4i fb = {static_cast<int>((w0 >> 1) & 0x60606060u), static_cast<int>((w1 >> 1) & 0x60606060u),
-                                static_cast<int>((w2 >> 1) & 0x60606060u), static_cast<int>((w3 >> 1) & 0x60606060u)};
+                const v4i fb = {static_cast<int>(w0 & kTop), static_cast<int>(w1 & kTop), static_cast<int>(w2 & kTop), static_cast<int>(w3 & kTop)};
                 acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i*>(a_unit + a_off[0]), fb, acc0, 0, 0, 0);
             }
             {
-                const v4i fb = {static_cast<int>(w0 & 0x30303030u), static_cast<int>(w1 & 0x30303030u), static_cast<int>(w2 & 0x30303030u),
-                                static_cast<int>(w3 & 0x30303030u)};
+                const v4i fb = {static_cast<int>((w0 << 2) & kTop), static_cast<int>((w1 << 2) & kTop), static_cast<int>((w2 << 2) & kTop),
+                                static_cast<int>((w3 << 2) & kTop)};
                 acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i*>(a_unit + a_off[1]), fb, acc1, 0, 0, 0);
             }
             {
-                const v4i fb = {static_cast<int>(w0 & 0x0C0C0C0Cu), static_cast<int>(w1 & 0x0C0C0C0Cu), static_cast<int>(w2 & 0x0C0C0C0Cu),
-                                static_cast<int>(w3 & 0x0C0C0C0Cu)};
-                acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i*>(a_unit + a_off[2]), fb, acc2, 0, 0, 0);
+                const v4i fb = {static_cast<int>((w0 << 4) & kTop), static_cast<int>((w1 << 4) & kTop), static_cast<int>((w2 << 4) & kTop),
+                                static_cast<int>((w3 << 4) & kTop)};
+                acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i*>(a_unit + a_off[2]), fb, acc0, 0, 0, 0);
             }
             {
-                const v4i fb = {static_cast<int>(w0 & 0x03030303u), static_cast<int>(w1 & 0x03030303u), static_cast<int>(w2 & 0x03030303u),
-                                static_cast<int>(w3 & 0x03030303u)};
-                acc3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i*>(a_unit + a_off[3]), fb, acc3, 0, 0, 0);
+                const v4i fb = {static_cast<int>((w0 << 6) & kTop), static_cast<int>((w1 << 6) & kTop), static_cast<int>((w2 << 6) & kTop),
+                                static_cast<int>((w3 << 6) & kTop)};
+                acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i*>(a_unit + a_off[3]), fb, acc1, 0, 0, 0);
             }
         }
     }
     v16i acc;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = (acc0[v] >> 5) + (acc1[v] >> 4) + (acc2[v] >> 2) + acc3[v];  // exact: multiples of 32, 16, 4
+    for (int v = 0; v < 16; ++v) acc[v] = acc0[v] + acc1[v];  // 64 times the sum
 
     // ---- add the k-parts: every wavefront parks its sums in LDS and finishes a quarter of its block -------------
     TPQ_STAMP(4);
@@ -191,7 +230,7 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
             for (int p = 0; p < kSlabKParts; ++p) sum[i] += part[((p * 4 + nb) * 16 + 4 * kp + i) * kWave + lane];
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sum[i] -= 2 * row_sum[8 * kp + 4 * half + i];
+        for (int i = 0; i < 4; ++i) sum[i] >>= 6;  // exact: every term is a multiple of 64
         const int n = n0 + 32 * nb + wn;
         const int m_first = m0 + 8 * kp + 4 * half;
         if (n < N) {
@@ -201,10 +240,10 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
                 for (int i = 0; i < 4; ++i)
                     if (m_first + i < M) mine[static_cast<int64_t>(m_first + i) * N + n] = sum[i];
             } else {
-                float row_scale[4];  // all of them before the first store
+                float row_scale[4];  // fetched at the start of the kernel
 #pragma unroll
-                for (int i = 0; i < 4; ++i) row_scale[i] = ep.row_scale_of(m_first + i < M ? m_first + i : M - 1);
-                const float bias_n = ep.bias_of(n);
+                for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[8 * kp + 4 * half + i];
+                const float bias_n = scale_lds[kSlabRows + 32 * nb + wn];
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     if (m_first + i < M) ep.store_scaled(static_cast<int64_t>(m_first + i) * N + n, sum[i], row_scale[i], bias_n);
@@ -255,10 +294,10 @@ int launch_ternary_slab(const int8_t* x, const uint8_t* packed, int64_t M, int64
     const size_t slab_bytes = static_cast<size_t>(kSlabRows) * (per_split + (per_split & 1)) * 128;
     const size_t part_bytes = static_cast<size_t>(16) * 16 * kWave * sizeof(int);  // 64 KB
     const size_t main_bytes = slab_bytes > part_bytes ? slab_bytes : part_bytes;
-    const size_t smem = main_bytes + kSlabRows * sizeof(int);
+    const size_t smem = main_bytes + (kSlabRows + kSlabChannels) * sizeof(float);
     auto kernel = ternary_slab_kernel<Epilogue>;
     static std::atomic<uint64_t> configured{0};  // per instantiation
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<size_t>(kSlabRows) * kSlabUnits * 128 + kSlabRows * sizeof(int), configured, "ternary slab")) return rc;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<size_t>(kSlabRows) * kSlabUnits * 128 + (kSlabRows + kSlabChannels) * sizeof(float), configured, "ternary slab")) return rc;
     const int64_t n_tiles = (N + kSlabChannels - 1) / kSlabChannels, m_tiles = (M + kSlabRows - 1) / kSlabRows;
     const int64_t gx = 8 * m_tiles * ((n_tiles * splits + 7) / 8);
     TPQ_REQUIRE(gx <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "ternary slab: shape too large");
