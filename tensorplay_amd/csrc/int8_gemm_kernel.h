@@ -103,6 +103,39 @@ struct EpilogueTernary {
             out[idx] = Elem<DT>::store(f);
         }
     }
+    // Four consecutive columns of one row (idx = m N + n).  whole_and_aligned: all four exist and idx is a multiple of
+    // four with runs_aligned() true, so each destination takes one vector store.
+    __device__ __forceinline__ bool runs_aligned() const {
+        return (reinterpret_cast<uintptr_t>(out) & (4 * sizeof(typename Elem<DT>::storage) - 1)) == 0 && (reinterpret_cast<uintptr_t>(acc_out) & 15) == 0;
+    }
+    __device__ __forceinline__ void store_scaled_run(int64_t idx, const int (&v)[4], float row_scale, const float (&bias_n)[4], int count,
+                                                     bool whole_and_aligned) const {
+        if (acc_out) {
+            if (whole_and_aligned) {
+                *reinterpret_cast<int4*>(acc_out + idx) = make_int4(v[0], v[1], v[2], v[3]);
+            } else {
+                for (int e = 0; e < count; ++e) acc_out[idx + e] = v[e];
+            }
+        }
+        if (out) {
+            typename Elem<DT>::storage o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float f = __fmul_rn(__fmul_rn(static_cast<float>(v[e]), row_scale), w_scale);
+                if (bias) f = __fadd_rn(f, bias_n[e]);
+                o[e] = Elem<DT>::store(f);
+            }
+            if (whole_and_aligned) {
+                if constexpr (sizeof(typename Elem<DT>::storage) == 2) {
+                    *reinterpret_cast<uint2*>(out + idx) = make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
+                } else {
+                    *reinterpret_cast<float4*>(out + idx) = make_float4(o[0], o[1], o[2], o[3]);
+                }
+            } else {
+                for (int e = 0; e < count; ++e) out[idx + e] = o[e];
+            }
+        }
+    }
 };
 
 // One packed byte holds four ternary codes, first code in bits 7..6

@@ -18,8 +18,8 @@
 //   * one barrier, then wavefront (nb, kp) multiplies channel block nb with its units (slab_unit_of):
 //     v_mfma_i32_32x32x32_i8, A = activations from LDS, B = weight fields moved to the top of their bytes in
 //     registers, four MFMAs per unit;
-//   * the four k-parts meet in LDS (the slab's space, after a second barrier); every wavefront finishes and
-//     stores a quarter of its block.
+//   * the four k-parts meet in LDS (the slab's space, after a second barrier); every thread finishes and stores
+//     four consecutive columns of one row.
 //
 // Where the time goes (clock stamps at 128 x 6912 x 2560, 216 workgroups): the requests of a workgroup are taken
 // at the rate data returns, and the last wavefront's activations are there after about half of the kernel; from then
@@ -117,7 +117,8 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
         const int row_a = n0 + 32 * nb + n16 < N ? n0 + 32 * nb + n16 : N - 1;
         const int row_b = n0 + 32 * nb + 16 + n16 < N ? n0 + 32 * nb + 16 + n16 : N - 1;
         const size_t pitch = static_cast<size_t>(K >> 2);
-        const unsigned char* base = packed + (static_cast<size_t>(unit0) << 5) + run_half * 16;
+        const unsigned char* const wbase = packed;
+        const unsigned char* base = wbase + (static_cast<size_t>(unit0) << 5) + run_half * 16;
 #pragma unroll
         for (int pr = 0; pr < 2; ++pr) {
             const int u = 4 * kp + 2 * pr + odd;
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
         }
         const int n = n0 + 32 * nb + wn < N ? n0 + 32 * nb + wn : N - 1;
         const int u = 16 + kp;
-        wq[4] = nt_load(reinterpret_cast<const uint4*>(packed + n * pitch + (static_cast<size_t>(unit0) << 5)) + half + (u < U ? u : 0) * 2);
+        wq[4] = nt_load(reinterpret_cast<const uint4*>(wbase + n * pitch + (static_cast<size_t>(unit0) << 5) + 16 * half + (u < U ? u : 0) * 32));
     }
 
     TPQ_STAMP(1);
@@ -220,33 +221,34 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     __syncthreads();
     TPQ_STAMP(6);
     {
-        // C fragment of a 32 x 32 block: lane holds column lane % 32, rows 8 (v / 4) + 4 (lane / 32) + v % 4;
-        // wavefront (nb, kp) takes v = 4 kp .. 4 kp + 3: rows 8 kp + 4 (lane / 32) + 0..3
-        int sum[4];
+        // C fragment of a 32 x 32 block: register v of lane l is row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32.
+        // Thread -> (block, register v, lanes 4 c .. 4 c + 3): four consecutive columns of one row, one 16-byte read per
+        // k-part and one vector store
+        const int c = tid & 15, v = (tid >> 4) & 15, block = tid >> 8;
+        int sum[4] = {0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sum[i] = 0;
-#pragma unroll
-            for (int p = 0; p < kSlabKParts; ++p) sum[i] += part[((p * 4 + nb) * 16 + 4 * kp + i) * kWave + lane];
+        for (int p = 0; p < kSlabKParts; ++p) {
+            const int4 q = *reinterpret_cast<const int4*>(part + ((p * 4 + block) * 16 + v) * kWave + 4 * c);
+            sum[0] += q.x; sum[1] += q.y; sum[2] += q.z; sum[3] += q.w;
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sum[i] >>= 6;  // exact: every term is a multiple of 64
-        const int n = n0 + 32 * nb + wn;
-        const int m_first = m0 + 8 * kp + 4 * half;
-        if (n < N) {
+        for (int e = 0; e < 4; ++e) sum[e] >>= 6;  // exact: every term is a multiple of 64
+        const int row = 8 * (v >> 2) + 4 * (c >> 3) + (v & 3), col = 32 * block + ((4 * c) & 31);
+        const int m = m0 + row, n = n0 + col;
+        if (m < M && n < N) {
+            const int count = N - n < 4 ? N - n : 4;
+            const int64_t idx = static_cast<int64_t>(m) * N + n;
             if (partial) {
-                int32_t* const mine = partial + static_cast<size_t>(split) * M * N;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (m_first + i < M) mine[static_cast<int64_t>(m_first + i) * N + n] = sum[i];
+                int32_t* const mine = partial + static_cast<size_t>(split) * M * N;  // 16-byte aligned (launcher)
+                if (count == 4 && (N & 3) == 0 && ((static_cast<size_t>(split) * M * N) & 3) == 0) {
+                    *reinterpret_cast<int4*>(mine + idx) = make_int4(sum[0], sum[1], sum[2], sum[3]);
+                } else {
+                    for (int e = 0; e < count; ++e) mine[idx + e] = sum[e];
+                }
             } else {
-                float row_scale[4];  // fetched at the start of the kernel
-#pragma unroll
-                for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[8 * kp + 4 * half + i];
-                const float bias_n = scale_lds[kSlabRows + 32 * nb + wn];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (m_first + i < M) ep.store_scaled(static_cast<int64_t>(m_first + i) * N + n, sum[i], row_scale[i], bias_n);
+                const float4 b = *reinterpret_cast<const float4*>(scale_lds + kSlabRows + col);  // fetched at the start of the kernel
+                const float bias_n[4] = {b.x, b.y, b.z, b.w};
+                ep.store_scaled_run(idx, sum, scale_lds[row], bias_n, count, count == 4 && (N & 3) == 0 && ep.runs_aligned());
             }
         }
     }

@@ -107,3 +107,21 @@ def test_ternary_mm_arbitrary_bytes_and_extremes(ops):
     _, want_acc = oracle.ternary_mm(x128, np.ones(128, np.float32), packed, 1.0, K)
     _, acc = ops.ternary_mm(dev(x128), dev(np.ones(128, np.float32)), dev(packed), 1.0, K, return_acc=True)
     np.testing.assert_array_equal(host(acc), want_acc)
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 2560, 200), (40, 2560, 130), (64, 4096, 264), (96, 1152, 72)])
+def test_ternary_slab_arbitrary_bytes(ops, M, K, N):
+    """The slab kernel (33 rows and more) with any byte value in the packed weight (0b10 decodes to -2) and the
+    activations at the int8 extremes, one and two splits of K, channel counts that are and are not multiples of four:
+    exact accumulators, and the scaled output equal to the oracle's."""
+    rng = np.random.default_rng(M + K + N)
+    packed = rng.integers(0, 256, size=(N, K // 4)).astype(np.uint8)
+    x = np.where(rng.random((M, K)) < 0.5, -127, 127).astype(np.int8)
+    x[1::3] = rng.integers(-127, 128, size=x[1::3].shape).astype(np.int8)
+    rs = (rng.random(M) * 0.01 + 1e-3).astype(np.float32)
+    want, want_acc = oracle.ternary_mm(x, rs, packed, 0.03, K)
+    got, acc = ops.ternary_mm(dev(x), dev(rs), dev(packed), 0.03, K, return_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    np.testing.assert_array_equal(host(got), want)
+    got_only = ops.ternary_mm(dev(x), dev(rs), dev(packed), 0.03, K)
+    np.testing.assert_array_equal(host(got_only), want)
