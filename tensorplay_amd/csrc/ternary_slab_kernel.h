@@ -270,21 +270,22 @@ __global__ __launch_bounds__(256) void ternary_slab_finish_kernel(const int32_t*
 // Splits of K for the slab kernel (1: no workspace needed); 0 when the kernel does not take the shape.
 // It is built for one pass of workgroups over the chip: every 32 rows expand the packed weights again, which the
 // tile kernel of ternary_gemm_kernel.h does once per 128 (or 64) rows.  Measured (us, bf16 out, slab / tile kernel):
-//   2560 -> 6912: 8.7 / 9.6 at 64 rows, 9.4 / 11.3 at 128, 17.0 / 15.9 at 256
-//   6912 -> 2560 (three splits): 10.6 / 16.2 at 64, 12.6 / 16.8 at 128, 23.9 / 20.0 at 256
-//   4096 -> 4096 (two splits): 10.5 / 11.4 at 33, 11.1 / 11.7 at 64, 13.3 / 12.4 at 128; 5120 -> 5120: 11.4 / 13.2 at 33,
-//   11.9 / 13.4 at 64: with two splits the second kernel that adds them costs what the shorter chain saves once the
-//   row tiles fill the chip, so two splits are taken up to 64 rows only
+//   2560 -> 6912: 7.1 / 9.6 at 64 rows, 7.4 / 11.3 at 128, 17.0 / 15.9 at 256 (two passes of workgroups)
+//   6912 -> 2560 (three splits): 9.5 / 16.2 at 64, 10.8 / 16.8 at 128
+//   two splits: 4096 -> 4096 9.5 / 11.4 at 33 rows, 9.9 / 11.7 at 64, 11.4 / 11.8 at 128; 5120 -> 4096 11.6 / 13.5 at
+//   128; 4096 -> 2048 9.9 / 11.7 at 128; 3072 -> 4096 9.6 / 10.0 at 65 but 10.9 / 10.2 at 128: with two splits the second
+//   kernel that adds them costs what the shorter chain saves when the splits are short, so above 64 rows two
+//   splits are taken from K = 4096 on
 // Letting the splits meet inside the kernel (every workgroup leaves its sums with agent-scope stores and counts itself
 // in, the last one adds and finishes) was built and is slower than the second launch at three splits (6912 -> 2560:
-// 13.4 against 12.7 us at 128 rows, 11.6 against 10.1 at 33): store acknowledgement, counter and the reads of the
-// other sums are three trips to memory in a row, a launch and one trip are less.
+// 13.4 against 12.7 us at 128 rows, 11.6 against 10.1 at 33, with the kernel as it was then): store acknowledgement,
+// counter and the reads of the other sums are three trips to memory in a row, a launch and one trip are less.
 inline int ternary_slab_splits(int64_t M, int64_t N, int64_t K, int compute_units = 256) {
     if (M < 33 || K % 128 != 0 || K < 128 || M > 0x7FFFFFFF / 2 || N > 0x7FFFFFFF / 2 || K > 0x7FFFFFFF / 2) return 0;
     const int64_t units = K / 128;
     const int64_t splits = (units + kSlabUnits - 1) / kSlabUnits;
     const int64_t workgroups = ((M + kSlabRows - 1) / kSlabRows) * ((N + kSlabChannels - 1) / kSlabChannels) * splits;
-    if (workgroups > compute_units || (splits == 2 && M > 64) || splits > 8) return 0;
+    if (workgroups > compute_units || (splits == 2 && M > 64 && units < 32) || splits > 8) return 0;
     return static_cast<int>(splits);
 }
 

@@ -54,8 +54,9 @@ CASES = [(1, 2560, 6912), (1, 6912, 2560), (4, 2560, 256), (8, 128, 67), (5, 64,
          # slab kernel (33 rows and more, K % 128 == 0): one unit, ragged rows and channels, 21 units = two splits,
          # 40 units = two full splits, three splits with a short last one
          (33, 128, 8), (40, 384, 136), (129, 2688, 200), (128, 5120, 264), (70, 5248, 130),
-         # two splits are taken up to 64 rows: 21 units (a short second split), 32 units, 40 units
-         (40, 2688, 200), (64, 4096, 520), (33, 5120, 136)]
+         # two splits are taken up to 64 rows: 21 units (a short second split), 32 units, 40 units; above 64 rows from
+         # 32 units on (24 units at 97 rows go to the tile kernel)
+         (40, 2688, 200), (64, 4096, 520), (33, 5120, 136), (97, 4096, 520), (128, 4224, 136), (97, 3072, 264)]
 
 
 @pytest.mark.parametrize("M,K,N", CASES)
