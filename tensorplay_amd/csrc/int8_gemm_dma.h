@@ -50,6 +50,10 @@
 // LDS image of the output tile, which the workgroup then stores row by row, 16
 // bytes per lane.
 //
+// Second form of the main loop (KSPLIT = 0), used below 64 stages per workgroup: eight positions of 64 x 64, every
+// wavefront multiplies all four substeps of a stage with the fragments of all four in registers, the barrier in the
+// middle of the stage; no exchange of k-halves in the epilogue.
+//
 // Requires K % 128 == 0 and 16-byte aligned operands.  Edges in M and N are
 // handled by clamping source rows and masking the stores.
 #pragma once
@@ -115,16 +119,24 @@ struct TileDequant {
 constexpr int kDmaRowBytes = 128;  // bytes of k per stage: one cache line per row
 constexpr int kDmaStages = 3;
 
-// KSPLIT = 2: eight wavefronts as described above.  KSPLIT = 1: four wavefronts, each multiplying
-// all four substeps of a stage (no k-half exchange in the epilogue, one wavefront per SIMD).
+#ifdef TPQ_DMA_STAMPS
+__device__ unsigned long long g_dma_stamps[8 * 8];
+#define TPQ_DMA_STAMP(I) do { if (blockIdx.x == 9 && (threadIdx.x & 63) == 0) g_dma_stamps[(I) * 8 + (threadIdx.x >> 6)] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define TPQ_DMA_STAMP(I) do { } while (0)
+#endif
+
+// KSPLIT = 2: eight wavefronts as described above (four positions x two k-halves).  KSPLIT = 0: eight wavefronts,
+// eight positions of 64 x 64, no k split.  KSPLIT = 1: four wavefronts, each multiplying all four substeps of a
+// stage (no k-half exchange in the epilogue, one wavefront per SIMD).
 template <class Tile, int KSPLIT>
-__global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
+__global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(const int8_t* __restrict__ A,
                                                             const int8_t* __restrict__ W, int M, int N,
                                                             int K, Tile tile, int vector_stores, int slices) {
     using out_t = typename Tile::out_t;
-    constexpr int BM = 256, BN = 128, WM = 128, WN = 64, TM = 4, TN = 2;
+    constexpr int BM = 256, BN = 128, WM = KSPLIT == 0 ? 64 : 128, WN = 64, TM = WM / 32, TN = 2;
     constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;    // 48 KB
-    constexpr int kThreads = 256 * KSPLIT, kWaves = 4 * KSPLIT;
+    constexpr int kThreads = KSPLIT == 1 ? 256 : 512, kWaves = kThreads / 64;
     constexpr int kLoads = kStageBytes / 1024 / kWaves;      // wave-level loads per stage and wavefront: 6 or 12
     constexpr int kPerChunk = 16 / sizeof(out_t);            // outputs per 16 bytes
     constexpr int kPitch = BN * sizeof(out_t) + 16;          // bytes per row of the output image
@@ -132,13 +144,15 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     static_assert(BM * kPitch <= kRingBytes && 8 * 16 * kWave * 16 <= kRingBytes, "epilogue areas live in the ring");
     extern __shared__ uint4 ring[];                          // [stage][row][128 B], later exchange area and image
     char* lds_bytes = reinterpret_cast<char*>(ring);
-    float* cs_lds = reinterpret_cast<float*>(lds_bytes + kRingBytes);  // [BN] column scales, [BN] bias
+    float* cs_lds = reinterpret_cast<float*>(lds_bytes + kRingBytes);  // [BN] column scales, [BN] bias, [BM] row scales
+    float* rs_lds = cs_lds + 2 * BN;
 
     const int tid = threadIdx.x;
+    TPQ_DMA_STAMP(0);
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kh = KSPLIT == 2 ? wave >> 2 : 0;  // k-half: substeps 2*kh and 2*kh+1 of every stage
-    const int wm = (wave >> 1) & 1, wn = wave & 1;
+    const int wm = KSPLIT == 0 ? wave >> 1 : (wave >> 1) & 1, wn = wave & 1;
 
     // Workgroups are dealt to the 8 XCDs round-robin (workgroup id mod 8), each with its own L2:
     // give every XCD a compact patch of tiles, as close to square in bytes as the grid allows,
@@ -164,10 +178,18 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     const int kt0 = blockIdx.y * nk_slice;
     const int nk = nk_all - kt0 < nk_slice ? nk_all - kt0 : nk_slice;
 
-    if (Tile::kScaled && tid < BN) {  // column scales and bias of this tile: read once, used in the epilogue
-        const int n = n0 + tid < N ? n0 + tid : N - 1;
-        cs_lds[tid] = tile.cs[n];
-        cs_lds[BN + tid] = tile.bias ? tile.bias[n] : 0.0f;
+    // Scales and bias of this tile: asked for here, ahead of the first stage, and parked in LDS when the main loop is
+    // over.  Written to LDS at this point they would hold the first wavefronts back for two trips to memory before
+    // their share of the first stage is requested; fetched in the epilogue they are a trip that nothing covers.
+    static_assert(kThreads >= BM && BM >= BN, "one thread per row scale");
+    float cs_reg = 0.0f, bias_reg = 0.0f, rs_reg = 0.0f;
+    if (Tile::kScaled) {
+        if (tid < BN) {
+            const int n = n0 + tid < N ? n0 + tid : N - 1;
+            cs_reg = tile.cs[n];
+            bias_reg = tile.bias ? tile.bias[n] : 0.0f;
+        }
+        if (tid < BM) rs_reg = tile.rs[m0 + tid < M ? m0 + tid : M - 1];
     }
 
     // wave-level load i of this wavefront fills rows (wave*6 + i)*8 .. +7 of the stage; lane l
@@ -228,9 +250,17 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     const uint32_t b_row = ring_addr + (BM + wn * WN + frag_row) * kDmaRowBytes;
     // the six reads of a substep, in two groups of three: (A0, A1, W0), then (W1, A2, A3)
     auto read_group = [&](auto group, int slot, uint32_t chunk_off, v4i (&fa)[TM], v4i (&fb)[TN]) {
-        static_assert(TM == 4 && TN == 2, "offsets below");
+        static_assert((TM == 4 || TM == 2) && TN == 2, "offsets below");
         const uint32_t a = a_row + slot * kStageBytes + chunk_off, b = b_row + slot * kStageBytes + chunk_off;
-        if constexpr (decltype(group)::value == 0) {
+        if constexpr (TM == 2) {  // (A0, A1), then (W0, W1)
+            if constexpr (decltype(group)::value == 0) {
+                asm volatile("ds_read_b128 %0, %1" : "=v"(fa[0]) : "v"(a) : "memory");
+                asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[1]) : "v"(a) : "memory");
+            } else {
+                asm volatile("ds_read_b128 %0, %1" : "=v"(fb[0]) : "v"(b) : "memory");
+                asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fb[1]) : "v"(b) : "memory");
+            }
+        } else if constexpr (decltype(group)::value == 0) {
             asm volatile("ds_read_b128 %0, %1" : "=v"(fa[0]) : "v"(a) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[1]) : "v"(a) : "memory");
             asm volatile("ds_read_b128 %0, %1" : "=v"(fb[0]) : "v"(b) : "memory");
@@ -252,9 +282,13 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     // that the MFMAs consuming them cannot be moved above the wait.
     auto frags_ready = [&](auto newer, v4i (&fa)[TM], v4i (&fb)[TN]) {
         constexpr int kNewer = decltype(newer)::value;
-        asm volatile("s_waitcnt lgkmcnt(%6)"
-                     : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1])
-                     : "n"(kNewer));
+        if constexpr (TM == 2) {
+            asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]) : "n"(kNewer));
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(%6)"
+                         : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1])
+                         : "n"(kNewer));
+        }
     };
     constexpr std::integral_constant<int, TM + TN> kOneBatch{};  // the reads of one substep
     constexpr std::integral_constant<int, 0> kNone{};
@@ -288,6 +322,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
 #pragma unroll
     for (int s = 0; s < kDmaStages; ++s)
         if (s < nk) issue(s, s);
+    TPQ_DMA_STAMP(1);
     {  // this wavefront's share of stage 0: everything issued after it may still be outstanding
         const int younger = nk - 1 < kDmaStages - 1 ? nk - 1 : kDmaStages - 1;
         if (younger == 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * kLoads));
@@ -297,11 +332,72 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     // The LDS counter is shared with scalar loads (kernel arguments, which return out of order)
     // and the column-scale writes above: drain it, so that only fragment reads are counted.
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    TPQ_DMA_STAMP(2);
 
     v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
     int kt = 0, slot = 0;  // slot: kt % kDmaStages
     read_frags(0, chunk_first, fa0, fb0);
-    if constexpr (KSPLIT == 1) {
+    if constexpr (KSPLIT == 0) {
+    // Eight positions of 64 x 64, every wavefront multiplies all four substeps of a stage: no k-half exchange in the
+    // epilogue, a third more fragment reads (four per four MFMAs).  The fragments of all four substeps are in
+    // registers; the barrier stands in the middle of the stage, so that the requests for the next stage's first two
+    // substeps have the MFMAs of two substeps to hide behind, as in the k-split form.
+    v4i fa2[TM], fb2[TN], fa3[TM], fb3[TN];
+    constexpr std::integral_constant<int, 3 * (TM + TN)> kThreeBatches{};
+    constexpr std::integral_constant<int, 2 * (TM + TN)> kTwoBatches{};
+    read_frags(0, chunk_second, fa1, fb1);
+    for (; kt + kDmaStages < nk; ++kt) {  // steady state: stages kt+1 .. kt+3 all exist
+        const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
+        read_frags(slot, chunk_third, fa2, fb2);
+        read_frags(slot, chunk_fourth, fa3, fb3);
+        frags_ready(kThreeBatches, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        frags_ready(kTwoBatches, fa1, fb1);
+        multiply(kLow, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        frags_ready(kNone, fa2, fb2);  // this wavefront is done reading stage kt
+        frags_ready(kNone, fa3, fb3);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads));
+        asm volatile("s_barrier" ::: "memory");
+        multiply_one(k0, k0, fa2, fb2);
+        read_group(k0, next, chunk_first, fa0, fb0);
+        multiply_one(k0, k1, fa2, fb2);
+        read_group(k1, next, chunk_first, fa0, fb0);
+        multiply_one(k1, k0, fa2, fb2);
+        read_group(k0, next, chunk_second, fa1, fb1);
+        multiply_one(k1, k1, fa2, fb2);
+        read_group(k1, next, chunk_second, fa1, fb1);
+        multiply_one(k0, k0, fa3, fb3);
+        issue_pair(k0, kt + kDmaStages, slot);
+        multiply_one(k0, k1, fa3, fb3);
+        issue_pair(k2, kt + kDmaStages, slot);
+        multiply_one(k1, k0, fa3, fb3);
+        issue_pair(k4, kt + kDmaStages, slot);
+        multiply_one(k1, k1, fa3, fb3);
+        slot = next;
+    }
+    for (; kt < nk; ++kt) {  // last stages: nothing left to issue
+        const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
+        read_frags(slot, chunk_third, fa2, fb2);
+        read_frags(slot, chunk_fourth, fa3, fb3);
+        frags_ready(kThreeBatches, fa0, fb0);
+        multiply(kLow, fa0, fb0);
+        frags_ready(kTwoBatches, fa1, fb1);
+        multiply(kLow, fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        frags_ready(kNone, fa2, fb2);
+        frags_ready(kNone, fa3, fb3);
+        if (kt + 1 < nk) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            asm volatile("s_barrier" ::: "memory");
+            read_frags(next, chunk_first, fa0, fb0);
+            read_frags(next, chunk_second, fa1, fb1);
+        }
+        multiply(kLow, fa2, fb2);
+        multiply(kLow, fa3, fb3);
+        slot = next;
+    }
+    } else if constexpr (KSPLIT == 1) {
     for (; kt + kDmaStages < nk; ++kt) {  // steady state: stages kt+1 .. kt+3 all exist
         const int next = slot == kDmaStages - 1 ? 0 : slot + 1;
         read_frags(slot, chunk_second, fa1, fb1);
@@ -416,7 +512,16 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
     }
 
     // ---- epilogue ------------------------------------------------------------------------------------
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring no longer needed
+    TPQ_DMA_STAMP(3);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    if (Tile::kScaled) {  // behind the ring: read after the barriers below
+        if (tid < BN) {
+            cs_lds[tid] = cs_reg;
+            cs_lds[BN + tid] = bias_reg;
+        }
+        if (tid < BM) rs_lds[tid] = rs_reg;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring no longer needed
     // Exchange: a wavefront keeps blocks i in [KEEP, KEEP+2) and hands the other two to its
     // partner (same position, other k-half), 16 KB per wavefront.
     int4* mine = reinterpret_cast<int4*>(lds_bytes) + wave * (16 * kWave) + lane;
@@ -452,8 +557,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         float rs_r[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int m = m0 + wm * WM + (KEEP + i) * 32 + frag_row;
-            rs_r[i] = Tile::kScaled ? tile.rs[m < M ? m : M - 1] : 0.0f;
+            rs_r[i] = Tile::kScaled ? rs_lds[wm * WM + (KEEP + i) * 32 + frag_row] : 0.0f;
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
@@ -491,12 +595,14 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
         __syncthreads();
         if (kh == 0) take_over(kLow); else take_over(kHigh);
         __syncthreads();  // exchange area consumed before the image overwrites it
+        TPQ_DMA_STAMP(4);
         if (kh == 0) to_image(kLow); else to_image(kHigh);
     } else {
         to_image(kLow);
-        to_image(kHigh);
+        if constexpr (TM == 4) to_image(kHigh);
     }
     __syncthreads();
+    TPQ_DMA_STAMP(5);
     constexpr int kChunksPerOutRow = BN / kPerChunk;  // 16-byte chunks per image row
     for (int c = tid; c < BM * kChunksPerOutRow; c += kThreads) {
         const int row = c / kChunksPerOutRow, col = (c % kChunksPerOutRow) * kPerChunk;
@@ -510,6 +616,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void int8_gemm_dma_kernel(const int8_
             for (int e = 0; e < kPerChunk && n + e < N; ++e) dstp[e] = reinterpret_cast<const out_t*>(srcp)[e];
         }
     }
+    TPQ_DMA_STAMP(6);
 }
 
 // K must be a multiple of the 128-byte stage.
@@ -518,23 +625,33 @@ inline bool dma_path_ok(int64_t M, int64_t N, int64_t K) { return (M > 128 || (M
 
 template <int KSPLIT, class Tile>
 int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
-    constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + 2 * 128 * sizeof(float);
+    constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + (2 * 128 + 256) * sizeof(float);
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
     auto kernel = int8_gemm_dma_kernel<Tile, KSPLIT>;
     static std::atomic<uint64_t> configured{0};  // per instantiation
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int8 gemm")) return rc;
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
-    kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), 256 * KSPLIT, smem, s>>>(
+    kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), KSPLIT == 1 ? 256 : 512, smem, s>>>(
         a, w, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), tile, vector_stores, slices);
     return check_launch("int8 mfma gemm (dma)");
 }
 
-// TPQ_INT8_KSPLIT=1 selects the four-wavefront variant for comparison runs.
+// Which form of the kernel.  Eight positions without a k split (0) save the exchange of the k-halves in the epilogue
+// (5,100 of a workgroup's 62,700 clocks at 2048 x 4096 x 4096) and pay a third more fragment reads per stage: measured
+// against the k-split form (2) with the same result bits: 2048 x 4096 x 4096 -2 %, K = 2048 -6 %, 2048 x 6912 x 2560
+// -4 %, the sliced launches at 128 .. 1024 rows of 4096 x 4096 -4 .. -7.5 %, 256 x 8192 x 8192 (sliced) -2 %; from 64
+// stages per workgroup on the k-split form is as fast or faster (2048 x 4096 x 11008 +0.6 %, 300 x 28672 x 8192 +1.4 %,
+// 8192^3 +0.6 % for the eight positions), so it keeps those.  TPQ_INT8_KSPLIT = 0 / 1 / 2 in a tuning build forces a
+// form (1: four wavefronts, no k split, 128 x 64 per wavefront).
 template <class Tile>
 int launch_dma(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
     const char* env = tuning_env("TPQ_INT8_KSPLIT");
     if (env && env[0] == '1') return launch_dma_split<1>(a, w, M, N, K, tile, s, slices);
+    if (env && env[0] == '0') return launch_dma_split<0>(a, w, M, N, K, tile, s, slices);
+    if (env && env[0] == '2') return launch_dma_split<2>(a, w, M, N, K, tile, s, slices);
+    const int64_t stages = K / kDmaRowBytes, per_workgroup = (stages + slices - 1) / slices;
+    if (per_workgroup < 64) return launch_dma_split<0>(a, w, M, N, K, tile, s, slices);
     return launch_dma_split<2>(a, w, M, N, K, tile, s, slices);
 }
 
