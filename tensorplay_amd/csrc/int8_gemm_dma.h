@@ -178,9 +178,10 @@ __global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(
     const int kt0 = blockIdx.y * nk_slice;
     const int nk = nk_all - kt0 < nk_slice ? nk_all - kt0 : nk_slice;
 
-    // Scales and bias of this tile: asked for here, ahead of the first stage, and parked in LDS when the main loop is
-    // over.  Written to LDS at this point they would hold the first wavefronts back for two trips to memory before
-    // their share of the first stage is requested; fetched in the epilogue they are a trip that nothing covers.
+    // Scales and bias of this tile: asked for here, ahead of the first stage, and parked in LDS behind the requests of
+    // the first stages, in front of the first barrier (they arrive before the stage that barrier waits for anyway).
+    // Written to LDS at this point they would hold the first wavefronts back for two trips to memory before their
+    // share of the first stage is requested; fetched in the epilogue they are a trip that nothing covers.
     static_assert(kThreads >= BM && BM >= BN, "one thread per row scale");
     float cs_reg = 0.0f, bias_reg = 0.0f, rs_reg = 0.0f;
     if (Tile::kScaled) {
@@ -323,6 +324,13 @@ __global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(
     for (int s = 0; s < kDmaStages; ++s)
         if (s < nk) issue(s, s);
     TPQ_DMA_STAMP(1);
+    if (Tile::kScaled) {  // behind the ring; read in the epilogue, many barriers later
+        if (tid < BN) {
+            cs_lds[tid] = cs_reg;
+            cs_lds[BN + tid] = bias_reg;
+        }
+        if (tid < BM) rs_lds[tid] = rs_reg;
+    }
     {  // this wavefront's share of stage 0: everything issued after it may still be outstanding
         const int younger = nk - 1 < kDmaStages - 1 ? nk - 1 : kDmaStages - 1;
         if (younger == 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * kLoads));
@@ -513,15 +521,57 @@ __global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(
 
     // ---- epilogue ------------------------------------------------------------------------------------
     TPQ_DMA_STAMP(3);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    if (Tile::kScaled) {  // behind the ring: read after the barriers below
-        if (tid < BN) {
-            cs_lds[tid] = cs_reg;
-            cs_lds[BN + tid] = bias_reg;
+    const bool has_bias = tile.bias != nullptr;
+    if constexpr (KSPLIT == 0 && sizeof(out_t) == 2) if ((vector_stores & 2) == 0) {
+        // Every wavefront finishes its own 64 x 64 block, without a barrier: the two stage buffers that do not hold
+        // the last stage are free since the last barrier of the main loop (every wavefront had finished reading them
+        // and every direct load had landed), so each wavefront turns its block into row order in 12 KB of its own
+        // there and stores it itself, 16 bytes per lane, eight whole 128-byte lines per store.
+        const int last = slot == 0 ? kDmaStages - 1 : slot - 1;  // buffer of the last stage (slot was advanced past it)
+        const int mine = wave < 4 ? (last == 0 ? 1 : 0) : (last == 2 ? 1 : 2);
+        constexpr int kWavePitch = WN * 2 + 16;  // bytes per row of the wavefront's image
+        static_assert(4 * 12288 <= kStageBytes && WM * kWavePitch <= 12288, "four wavefronts per free buffer");
+        char* img = lds_bytes + mine * kStageBytes + (wave & 3) * 12288;
+        float rs_r[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) rs_r[i] = rs_lds[wm * WM + i * 32 + frag_row];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n_wave = j * 32 + 8 * q + 4 * frag_half;  // 4 consecutive columns of the wavefront's 64
+                const float4 c = *reinterpret_cast<const float4*>(cs_lds + wn * WN + n_wave);
+                const float4 b = *reinterpret_cast<const float4*>(cs_lds + BN + wn * WN + n_wave);
+                const float c4[4] = {c.x, c.y, c.z, c.w}, b4[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    float f[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) f[t] = Tile::value(acc[i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
+                    *reinterpret_cast<uint2*>(img + (i * 32 + frag_row) * kWavePitch + n_wave * 2) =
+                        make_uint2(Tile::pack2(f[0], f[1]), Tile::pack2(f[2], f[3]));
+                }
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's own LDS writes, in order with its reads
+        TPQ_DMA_STAMP(5);
+#pragma unroll
+        for (int it = 0; it < WM / 8; ++it) {
+            const int row = it * 8 + (lane >> 3), col = (lane & 7) * 8;
+            const int m = m0 + wm * WM + row, n = n0 + wn * WN + col;
+            const uint4 v = *reinterpret_cast<const uint4*>(img + row * kWavePitch + col * 2);
+            if (m >= M || n >= N) continue;
+            out_t* dstp = tile.out + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
+            if ((vector_stores & 1) && n + 8 <= N) {
+                nt_store(reinterpret_cast<uint4*>(dstp), v);  // written once, read by a later kernel
+            } else {
+                const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+                for (int e = 0; e < 8 && n + e < N; ++e) dstp[e] = static_cast<out_t>(words[e >> 1] >> (16 * (e & 1)));
+            }
         }
-        if (tid < BM) rs_lds[tid] = rs_reg;
+        TPQ_DMA_STAMP(6);
+        return;
     }
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring no longer needed
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring no longer needed
     // Exchange: a wavefront keeps blocks i in [KEEP, KEEP+2) and hands the other two to its
     // partner (same position, other k-half), 16 KB per wavefront.
     int4* mine = reinterpret_cast<int4*>(lds_bytes) + wave * (16 * kWave) + lane;
@@ -551,7 +601,6 @@ __global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(
                 }
     };
     // scale, convert and place blocks [KEEP, KEEP+2) in the image
-    const bool has_bias = tile.bias != nullptr;
     auto to_image = [&](auto keep) {
         constexpr int KEEP = decltype(keep)::value;
         float rs_r[2];
@@ -610,7 +659,7 @@ __global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(
         if (m >= M || n >= N) continue;
         const char* srcp = lds_bytes + row * kPitch + col * sizeof(out_t);
         out_t* dstp = tile.out + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
-        if (vector_stores && n + kPerChunk <= N) {
+        if ((vector_stores & 1) && n + kPerChunk <= N) {
             nt_store(reinterpret_cast<uint4*>(dstp), *reinterpret_cast<const uint4*>(srcp));  // written once, read by a later kernel
         } else {
             for (int e = 0; e < kPerChunk && n + e < N; ++e) dstp[e] = reinterpret_cast<const out_t*>(srcp)[e];
@@ -631,7 +680,8 @@ int launch_dma_split(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int
     auto kernel = int8_gemm_dma_kernel<Tile, KSPLIT>;
     static std::atomic<uint64_t> configured{0};  // per instantiation
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int8 gemm")) return rc;
-    const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
+    int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
+    if (tuning_env("TPQ_INT8_NO_WAVE_EPILOGUE")) vector_stores |= 2;  // comparison runs: the workgroup-wide epilogue
     kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), KSPLIT == 1 ? 256 : 512, smem, s>>>(
         a, w, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), tile, vector_stores, slices);
     return check_launch("int8 mfma gemm (dma)");
