@@ -87,6 +87,22 @@ __global__ __launch_bounds__(WAVES * kWave) void int8_decode_kernel(const int8_t
         }
     }
 
+    // The finishing wavefront asks for its scales and bias values here, ahead of the exchange of the partial sums:
+    // fetched element by element in the store loop each is a trip to memory that the next store waits for (a load
+    // behind a store to `out` cannot be moved ahead of it).
+    float row_scale[MB], col_scale[NB][4], bias_n[NB][4];
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < MB; ++r) row_scale[r] = ep.row_scale_of(row_live[r] ? 16 * r + i : 0);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int n = n0 + 16 * b + 4 * q + v;
+                col_scale[b][v] = ep.col_scale_of(n < N ? n : N - 1);
+                bias_n[b][v] = ep.bias_of(n < N ? n : N - 1);
+            }
+    }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -105,7 +121,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int8_decode_kernel(const int8_t
 #pragma unroll
                     for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b * MB + r][v][lane];
                     const int n = n0 + 16 * b + 4 * q + v, m = 16 * r + i;
-                    if (row_live[r] && n < N) ep.store(static_cast<int64_t>(m) * N + n, m, n, sum);
+                    if (row_live[r] && n < N) ep.store_scaled(static_cast<int64_t>(m) * N + n, sum, row_scale[r], col_scale[b][v], bias_n[b][v]);
                 }
     }
 }
@@ -127,6 +143,18 @@ __global__ __launch_bounds__(WAVES * kWave) void int8_row_kernel(const int8_t* _
     const int g = wave / passes, pass = wave - g * passes;
     const int n0 = (blockIdx.x * groups + g) * kI8RowChannels;
     const bool active = g < groups && n0 < N;
+    // thread = (group, channel, row) finishes one output; its scales are asked for ahead of the weights
+    const int tid = threadIdx.x;
+    const bool finishes = tid < groups * kI8RowChannels * ROWS;
+    const int out_group = tid / (kI8RowChannels * ROWS), out_rem = tid - out_group * (kI8RowChannels * ROWS);
+    const int out_c = out_rem / ROWS, out_r = out_rem - out_c * ROWS;
+    const int out_n = (blockIdx.x * groups + out_group) * kI8RowChannels + out_c;
+    float row_scale = 0.0f, col_scale = 0.0f, bias_n = 0.0f;
+    if (finishes && out_n < N) {
+        row_scale = ep.row_scale_of(out_r);
+        col_scale = ep.col_scale_of(out_n);
+        bias_n = ep.bias_of(out_n);
+    }
     int acc[kI8RowChannels][ROWS];
 #pragma unroll
     for (int c = 0; c < kI8RowChannels; ++c)
@@ -175,16 +203,10 @@ __global__ __launch_bounds__(WAVES * kWave) void int8_row_kernel(const int8_t* _
             for (int r = 0; r < ROWS; ++r) red[wave][c * ROWS + r] = acc[c][r];
     }
     __syncthreads();
-    const int tid = threadIdx.x;
-    if (tid < groups * kI8RowChannels * ROWS) {  // thread = (group, channel, row)
-        const int gg = tid / (kI8RowChannels * ROWS), rem = tid - gg * (kI8RowChannels * ROWS);
-        const int c = rem / ROWS, r = rem - c * ROWS;
-        const int n = (blockIdx.x * groups + gg) * kI8RowChannels + c;
-        if (n < N) {
-            int sum = 0;
-            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][rem];
-            ep.store(static_cast<int64_t>(r) * N + n, r, n, sum);
-        }
+    if (finishes && out_n < N) {
+        int sum = 0;
+        for (int ps = 0; ps < passes; ++ps) sum += red[out_group * passes + ps][out_rem];
+        ep.store_scaled(static_cast<int64_t>(out_r) * N + out_n, sum, row_scale, col_scale, bias_n);
     }
 }
 

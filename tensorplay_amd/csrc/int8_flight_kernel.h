@@ -132,6 +132,22 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8_flight_kernel(const 
     }
 
     // ---- the wavefronts' partial sums ------------------------------------------------------------------------
+    // wavefront t finishes output block t (channel block t / MB, row block t % MB): lane (m, q) stores row 16 r + m,
+    // channels n0 + 16 b + 4 q .. + 3.  Its scales are asked for here, ahead of the exchange: behind it they are a
+    // trip to memory that nothing covers.
+    static_assert(NB * MB <= kFlightWaves, "one output block per finishing wavefront");
+    const int fin_m = 16 * (wave % MB) + i, fin_n = n0 + 16 * (wave / MB) + 4 * q;
+    const bool finishes = wave < NB * MB && fin_m < M && fin_n < N;
+    float row_scale = 0.0f, col_scale[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bias_n[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (finishes) {
+        row_scale = ep.row_scale_of(fin_m);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int n = fin_n + v < N ? fin_n + v : fin_n;
+            col_scale[v] = ep.col_scale_of(n);
+            bias_n[v] = ep.bias_of(n);
+        }
+    }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -139,19 +155,15 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8_flight_kernel(const 
 #pragma unroll
             for (int v = 0; v < 4; ++v) red[((wave * NB * MB + b * MB + r) * 4 + v) * kWave + lane] = d[b][r][v];
     __syncthreads();
-    // wavefront t finishes output block t (channel block t / MB, row block t % MB): lane (m, q) stores row 16 r + m,
-    // channels n0 + 16 b + 4 q .. + 3
-    for (int t = wave; t < NB * MB; t += kFlightWaves) {
-        const int b = t / MB, r = t % MB;
-        const int m = 16 * r + i, n = n0 + 16 * b + 4 * q;
-        int sum[4];
+    if (finishes) {
+        const int t = wave;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            sum[v] = 0;
+            int sum = 0;
 #pragma unroll
-            for (int ww = 0; ww < kFlightWaves; ++ww) sum[v] += red[((ww * NB * MB + t) * 4 + v) * kWave + lane];
+            for (int ww = 0; ww < kFlightWaves; ++ww) sum += red[((ww * NB * MB + t) * 4 + v) * kWave + lane];
+            if (fin_n + v < N) ep.store_scaled(static_cast<int64_t>(fin_m) * N + fin_n + v, sum, row_scale, col_scale[v], bias_n[v]);
         }
-        if (m < M && n < N) ep.store_run(static_cast<int64_t>(m) * N + n, m, n, sum, N - n < 4 ? N - n : 4);
     }
 }
 

@@ -36,6 +36,11 @@ __device__ __forceinline__ int swz(int row) { return (((row >> 1) ^ (row >> 3)) 
 struct EpilogueInt32 {
     int32_t* c;
     __device__ __forceinline__ void store(int64_t idx, int m, int n, int v) const { c[idx] = v; }
+    // the two-step form of the scaled epilogues: nothing to fetch here
+    __device__ __forceinline__ float row_scale_of(int) const { return 0.0f; }
+    __device__ __forceinline__ float col_scale_of(int) const { return 0.0f; }
+    __device__ __forceinline__ float bias_of(int) const { return 0.0f; }
+    __device__ __forceinline__ void store_scaled(int64_t idx, int v, float, float, float) const { c[idx] = v; }
     // `count` (1..4) consecutive channels n .. of row m
     __device__ __forceinline__ void store_run(int64_t idx, int m, int n, const int (&v)[4], int count) const {
 #pragma unroll
@@ -53,6 +58,16 @@ struct EpilogueDequant {
     __device__ __forceinline__ void store(int64_t idx, int m, int n, int v) const {
         float f = __fmul_rn(__fmul_rn(static_cast<float>(v), rs[m]), cs[n]);
         if (bias) f = __fadd_rn(f, bias[n]);
+        out[idx] = Elem<DT>::store(f);
+    }
+    // The same in two steps, for kernels that know early what they will store: the scales are fetched ahead of the
+    // arithmetic instead of behind it, where the fetch is a trip to memory that nothing covers.
+    __device__ __forceinline__ float row_scale_of(int m) const { return rs[m]; }
+    __device__ __forceinline__ float col_scale_of(int n) const { return cs[n]; }
+    __device__ __forceinline__ float bias_of(int n) const { return bias ? bias[n] : 0.0f; }
+    __device__ __forceinline__ void store_scaled(int64_t idx, int v, float r, float c, float b) const {
+        float f = __fmul_rn(__fmul_rn(static_cast<float>(v), r), c);
+        if (bias) f = __fadd_rn(f, b);
         out[idx] = Elem<DT>::store(f);
     }
     // `count` (1..4) consecutive channels n .. of row m; every scale is fetched before the first store (a load behind a

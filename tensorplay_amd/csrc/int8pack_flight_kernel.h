@@ -150,6 +150,18 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(co
     }
 
     // ---- the wavefronts' partial sums, added in wavefront order -----------------------------------------------
+    // wavefront w finishes block w: lane (m, q) stores row m, channels n0 + 16 w + 4 q + v; their scales are asked for
+    // ahead of the exchange
+    static_assert(NB <= kFlightWaves, "one block per finishing wavefront");
+    float scale_n[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (wave < NB) {
+        const auto sp = pinned_global(scale);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int n = n0 + 16 * wave + 4 * q + v;
+            scale_n[v] = sp[n < N ? n : N - 1];
+        }
+    }
     const int slot = q * XR + i;  // live lanes (rows < XR) only
     if (i < XR) {
 #pragma unroll
@@ -167,7 +179,7 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(co
             float sum = 0.0f;
 #pragma unroll
             for (int ww = 0; ww < kFlightWaves; ++ww) sum += red[((ww * NB + b) * 4 + v) * (4 * XR) + slot];
-            if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = Elem<DT>::store(__fmul_rn(sum, scale[n + v]));
+            if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = Elem<DT>::store(__fmul_rn(sum, scale_n[v]));
         }
     }
 }

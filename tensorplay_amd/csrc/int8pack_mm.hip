@@ -139,6 +139,17 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
         }
     }
 
+    float scale_n[NB][4];  // the finishing wavefront's channel scales, asked for ahead of the exchange
+    if (wave == 0) {
+        const auto sp = pinned_global(scale);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int n = n0 + 16 * b + 4 * q + v;
+                scale_n[b][v] = sp[n < N ? n : N - 1];
+            }
+    }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -157,7 +168,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
 #pragma unroll
                     for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b * MB + r][v][lane];
                     const int n = n0 + 16 * b + 4 * q + v;
-                    if (row_live[r] && n < N) y[static_cast<size_t>(16 * r + i) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
+                    if (row_live[r] && n < N) y[static_cast<size_t>(16 * r + i) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale_n[b][v]));
                 }
     }
 }
@@ -182,6 +193,14 @@ __global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const u
     const int g = wave / passes, pass = wave - g * passes;
     const int n0 = (blockIdx.x * groups + g) * kRowChannels;
     const bool active = g < groups && n0 < N;
+    // thread = (group, channel, row) finishes one output; its channel scale is asked for ahead of the weights
+    const int tid = threadIdx.x;
+    const int out_group = tid / (kRowChannels * ROWS), out_rem = tid - out_group * (kRowChannels * ROWS);
+    const int out_c = out_rem / ROWS, out_r = out_rem - out_c * ROWS;
+    const int out_n = (blockIdx.x * groups + out_group) * kRowChannels + out_c;
+    const bool finishes = tid < groups * kRowChannels * ROWS && out_n < N;
+    float scale_n = 0.0f;
+    if (finishes) scale_n = pinned_global(scale)[out_n];
     float acc[kRowChannels][ROWS];
 #pragma unroll
     for (int c = 0; c < kRowChannels; ++c)
@@ -259,16 +278,10 @@ __global__ __launch_bounds__(kRowWaves * kWave) void int8pack_row_kernel(const u
             for (int r = 0; r < ROWS; ++r) red[wave][c * ROWS + r] = acc[c][r];
     }
     __syncthreads();
-    const int tid = threadIdx.x;
-    if (tid < groups * kRowChannels * ROWS) {  // thread = (group, channel, row): the passes in order
-        const int gg = tid / (kRowChannels * ROWS), rem = tid - gg * (kRowChannels * ROWS);
-        const int c = rem / ROWS, r = rem - c * ROWS;
-        const int n = (blockIdx.x * groups + gg) * kRowChannels + c;
-        if (n < N) {
-            float sum = 0.0f;
-            for (int ps = 0; ps < passes; ++ps) sum += red[gg * passes + ps][rem];
-            y[static_cast<size_t>(r) * N + n] = Elem<DT>::store(__fmul_rn(sum, scale[n]));
-        }
+    if (finishes) {  // the passes in order
+        float sum = 0.0f;
+        for (int ps = 0; ps < passes; ++ps) sum += red[out_group * passes + ps][out_rem];
+        y[static_cast<size_t>(out_r) * N + out_n] = Elem<DT>::store(__fmul_rn(sum, scale_n));
     }
 }
 

@@ -117,6 +117,21 @@ __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(cons
         }
     }
 
+    // The finishing wavefront asks for its row scales and bias values here, ahead of the exchange of the partial sums:
+    // fetched element by element in the store loop each is a trip to memory that the next store waits for (a load
+    // behind a store to `out` cannot be moved ahead of it).
+    float row_scale[MB], bias_n[NB][4];
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < MB; ++r) row_scale[r] = ep.row_scale_of(m_base + (row_live[r] ? 16 * r + i : 0));
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int n = n0 + 16 * b + 4 * q + v;
+                bias_n[b][v] = ep.bias_of(n < N ? n : N - 1);
+            }
+    }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -135,7 +150,7 @@ __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(cons
 #pragma unroll
                     for (int ww = 0; ww < WAVES; ++ww) sum += red[ww][b * MB + r][v][lane];
                     const int n = n0 + 16 * b + 4 * q + v, m = m_base + 16 * r + i;
-                    if (row_live[r] && n < N) ep.store(static_cast<int64_t>(m) * N + n, m, n, sum);
+                    if (row_live[r] && n < N) ep.store_scaled(static_cast<int64_t>(m) * N + n, sum, row_scale[r], bias_n[b][v]);
                 }
     }
 }

@@ -108,6 +108,15 @@ struct Elem<TPQ_DTYPE_BF16> {
     static __device__ __forceinline__ uint16_t store(float v) { return f32_to_bf16_bits(v); }
 };
 
+// A global address whose origin the compiler has lost sight of: a load through it stays where it is written.  Loads
+// through a __restrict__ const kernel argument may be moved down to their use, across barriers, which turns a fetch
+// that was meant to travel under the main loop into a trip to memory in the epilogue.
+template <class T>
+__device__ __forceinline__ const __attribute__((address_space(1))) T* pinned_global(const T* p) {
+    asm volatile("" : "+v"(p));
+    return (const __attribute__((address_space(1))) T*)p;
+}
+
 // ---- streaming loads -------------------------------------------------------------------------
 
 // Loads marked non-temporal, for data that is read once (weights): measured 7.2 -> 6.8 us on the
