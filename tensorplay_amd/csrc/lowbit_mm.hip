@@ -459,25 +459,50 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
     constexpr int kTurns = 64 / kCpl;            // 1, 1, 2, 4
     constexpr int kWords = kLoadBytes / 4;
     __shared__ float red[WAVES][kLbRowChannels];
+    extern __shared__ __align__(16) unsigned char lb_row_x[];  // the activation row: chunk c of 16 bytes at 16 (c + c / 8)
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = wave / passes, pass = wave - g * passes;
     const int n0 = (blockIdx.x * groups + g) * kLbRowChannels;
     const bool active = g < groups && n0 < N;
+    // The activations reach the lanes through LDS.  A lane owns runs of 64 consecutive k (128 bytes): asked for
+    // directly, a wavefront load takes 16 bytes out of 64 cache lines, and the eight loads of a run are 512 line
+    // look-ups per wavefront against 32 for the packed weights; the texture path's look-ups, not the bytes, were what
+    // the kernel waited for.  The workgroup reads the row once, contiguously (a wavefront load = 1 KB = 8 lines),
+    // and parks it with 16 bytes of padding per 128, so that the lanes' 16-byte reads spread over the banks.
+    // Measured at 4096 -> 11008: 1 bit 7.15 -> 6.43 us, 2 bits 7.85 -> 6.86; 4 bits 7.84 -> 8.3 (a lane's runs are 64
+    // bytes there, half the look-ups to save and twice the 16-byte LDS reads that collide), 8 bits no change: those two
+    // keep the direct loads.
+    constexpr bool kStageX = BITS <= 2;
+    constexpr int kXRounds = 4;  // rounds of 16 bytes per thread in flight together
+    constexpr int kXPerSweep = kXRounds * WAVES * kWave;
+    const int x_chunks = K >> 3;
+    typedef uint32_t words4 __attribute__((ext_vector_type(4)));
+    const auto xg = pinned_global(reinterpret_cast<const words4*>(x));  // the loads stay here, ahead of the weights
+    words4 xr[kXRounds];  // the first sweep is asked for here and parked behind the weights' requests
+    if constexpr (kStageX) {
+#pragma unroll
+        for (int r = 0; r < kXRounds; ++r) {
+            const int c = r * WAVES * kWave + static_cast<int>(threadIdx.x);
+            xr[r] = xg[c < x_chunks ? c : 0];
+        }
+    }
+    uint4 xv[kTurns][kCpl / 8];
     float acc[kLbRowChannels];
 #pragma unroll
     for (int c = 0; c < kLbRowChannels; ++c) acc[c] = 0.0f;
+    uint32_t wv[kLbRowChannels][kTurns][kWords];
+    float2 p[kLbRowChannels][kTurns];
+    bool live[kTurns];
+    int k_first[kTurns];
     if (active) {
         const size_t pitch = static_cast<size_t>(K) / kPerByte;
-        uint32_t wv[kLbRowChannels][kTurns][kWords];
-        float2 p[kLbRowChannels][kTurns];
-        uint4 xv[kTurns][kCpl / 8];
-        bool live[kTurns];
 #pragma unroll
         for (int t = 0; t < kTurns; ++t) {
             const int k0 = ((pass * kTurns + t) * kWave + lane) * kCpl;
             live[t] = k0 < K;
             const int kl = live[t] ? k0 : 0;  // past the end: a valid segment, multiplied by zeros
+            k_first[t] = kl;
 #pragma unroll
             for (int c = 0; c < kLbRowChannels; ++c) {
                 const int n = n0 + c < N ? n0 + c : N - 1;
@@ -490,16 +515,58 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
                     wv[c][t][0] = q.x; wv[c][t][1] = q.y;
                 }
                 p[c][t] = *reinterpret_cast<const float2*>(sz + (static_cast<size_t>(kl / group) * N + n) * 2);
+            }
+            if constexpr (!kStageX) {
+                const uint4* xp = reinterpret_cast<const uint4*>(x + kl);
+#pragma unroll
+                for (int e = 0; e < kCpl / 8; ++e) xv[t][e] = live[t] ? xp[e] : make_uint4(0, 0, 0, 0);
+            }
+        }
+    }
+    if constexpr (kStageX) {
+#pragma unroll
+    for (int r = 0; r < kXRounds; ++r) {
+        const int c = r * WAVES * kWave + static_cast<int>(threadIdx.x);
+        if (c < x_chunks) *reinterpret_cast<words4*>(lb_row_x + 16 * (c + (c >> 3))) = xr[r];
+    }
+    for (int base = kXPerSweep; base < x_chunks; base += kXPerSweep) {  // long rows with few wavefronts
+#pragma unroll
+        for (int r = 0; r < kXRounds; ++r) {
+            const int c = base + r * WAVES * kWave + static_cast<int>(threadIdx.x);
+            xr[r] = xg[c < x_chunks ? c : 0];
+        }
+#pragma unroll
+        for (int r = 0; r < kXRounds; ++r) {
+            const int c = base + r * WAVES * kWave + static_cast<int>(threadIdx.x);
+            if (c < x_chunks) *reinterpret_cast<words4*>(lb_row_x + 16 * (c + (c >> 3))) = xr[r];
+        }
+    }
+    // the weights stay in flight across the barrier: it orders LDS traffic only
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    if (active) {
+        if constexpr (kStageX) {
+#pragma unroll
+            for (int t = 0; t < kTurns; ++t)
+#pragma unroll
+                for (int e = 0; e < kCpl / 8; ++e) {
+                    const int c = (k_first[t] >> 3) + e;
+                    xv[t][e] = live[t] ? *reinterpret_cast<const uint4*>(lb_row_x + 16 * (c + (c >> 3))) : make_uint4(0, 0, 0, 0);
+                }
+        }
+#pragma unroll
+        for (int t = 0; t < kTurns; ++t)
+#pragma unroll
+            for (int c = 0; c < kLbRowChannels; ++c) {
+                // the parameters enter the arithmetic here, not earlier: used ahead of the barrier they would be waited
+                // for in front of it, and with them every load that was asked for before them
+                if constexpr (kStageX) asm volatile("" : "+v"(p[c][t].x), "+v"(p[c][t].y));
                 if constexpr (BITS == 8) {  // signed bytes: value + 128 in the fields, 128 more in the zero point
 #pragma unroll
                     for (int w = 0; w < kWords; ++w) wv[c][t][w] ^= kSignFlip;
                     p[c][t].y += 128.0f;
                 }
             }
-            const uint4* xp = reinterpret_cast<const uint4*>(x + kl);
-#pragma unroll
-            for (int e = 0; e < kCpl / 8; ++e) xv[t][e] = live[t] ? xp[e] : make_uint4(0, 0, 0, 0);
-        }
         // Codes become 16-bit floats in place.  A field of BITS bits moved to the top of the mantissa of each half
         // of the word (one shift), masked and given the exponent whose lowest field bit weighs one (one v_and_or_b32)
         // is the pair (2^BITS + code, 2^BITS + code') of the two halves' codes at that position; one v_dot2 multiplies
@@ -592,7 +659,18 @@ bool launch_lowbit_row(const void* x, const uint8_t* packed, const float* sz, co
     const auto* xp = static_cast<const uint16_t*>(x);
     auto* yp = static_cast<uint16_t*>(out);
     const int n = static_cast<int>(N), k = static_cast<int>(K), gr = static_cast<int>(group);
-#define TPQ_LBROW_C(B, L, W, C) lowbit_row_kernel<DT, B, L, W, C><<<grid, W * kWave, 0, s>>>(xp, packed, sz, bias, yp, n, k, gr, passes, groups)
+    const size_t x_lds = bits <= 2 ? (static_cast<size_t>(K) * 2 / 16) * 18 + 32 : 0;  // 16-byte chunks with 16 bytes of padding per eight
+#define TPQ_LBROW_C(B, L, W, C)                                                                                               \
+    do {                                                                                                                      \
+        auto kernel = lowbit_row_kernel<DT, B, L, W, C>;                                                                      \
+        static std::atomic<uint64_t> configured{0};                                                                           \
+        if (x_lds > 48 * 1024)                                                                                                \
+            if (int e = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), 160 * 1024 - 4096, configured, "lowbit mm")) { \
+                *rc = e;                                                                                                      \
+                return true;                                                                                                  \
+            }                                                                                                                 \
+        kernel<<<grid, W * kWave, x_lds, s>>>(xp, packed, sz, bias, yp, n, k, gr, passes, groups);                            \
+    } while (0)
 #define TPQ_LBROW(B, L, W) do { if (B <= 2 && channels == 8) TPQ_LBROW_C(B, L, W, (B <= 2 ? 8 : 4)); else TPQ_LBROW_C(B, L, W, 4); } while (0)
 #define TPQ_LBROW_W(B, L) do { if (waves == 4) TPQ_LBROW(B, L, 4); else TPQ_LBROW(B, L, 16); } while (0)
 #define TPQ_LBROW_L(B) do { if (lsb_first) TPQ_LBROW_W(B, true); else TPQ_LBROW_W(B, false); } while (0)

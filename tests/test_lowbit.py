@@ -188,7 +188,9 @@ def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("bits,lsb", [(1, False), (1, True), (2, False), (2, True), (4, False), (4, True), (8, False)])
-@pytest.mark.parametrize("N,K,group", [(10, 4096, 128), (7, 8192, 64), (130, 4160, 32), (5, 20480, 1024), (1, 64, 64), (36, 11008, 128)])
+@pytest.mark.parametrize("N,K,group", [(10, 4096, 128), (7, 8192, 64), (130, 4160, 32), (5, 20480, 1024), (1, 64, 64), (36, 11008, 128),
+                                       # rows of 64 KB and 128 KB: the activation row in LDS beyond the default limit (1 and 2 bits)
+                                       (3, 32768, 256), (2, 65536, 4096)])
 @pytest.mark.parametrize("tdt,tag,tol", [(torch.float16, "f16", 1e-3), (torch.bfloat16, "bf16", 8e-3)])
 def test_gpu_mm_one_row_kernel(bits, lsb, N, K, group, tdt, tag, tol, kernel_override):
     """One activation row on the kernel that streams the packed rows: several passes per channel, a last segment
