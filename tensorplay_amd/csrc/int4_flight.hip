@@ -21,12 +21,12 @@ inline int flight_compute_units() {
     return v;
 }
 
-template <int DT, int NB, int SPW, int XR, int MODE, bool NORM>
+template <int DT, int NB, int SPW, int XR, int MODE, bool NORM, int RB = 1>
 int launch_as(const uint16_t* x, int rows, const FlightSet& set, int blocks, int K, int shift, const uint16_t* residual, hipStream_t s) {
     constexpr size_t bytes = flight_lds_bytes<NB, SPW, XR>();
     static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
     static std::atomic<uint64_t> reserved{0};
-    const auto kernel = int4_mfma_flight_kernel<DT, NB, SPW, XR, MODE, NORM>;
+    const auto kernel = int4_mfma_flight_kernel<DT, NB, SPW, XR, MODE, NORM, RB>;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), bytes, reserved, "tpq_int4_mm (mfma, all in flight)")) return rc;
     constexpr int C = MODE == kFlightPair ? NB / 2 : NB;
     kernel<<<dim3((blocks + C - 1) / C), dim3(kFlightWaves * kWave), bytes, s>>>(x, set, rows, K, shift, residual);
@@ -92,10 +92,13 @@ template <int DT>
 bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group, bool pair, const void* residual, hipStream_t s, int* rc) {
     const bool norm = wts.norm_weight != nullptr;
     if (norm && (!aligned(wts.norm_weight, 16) || K > 8192)) return false;  // built for up to four steps per wavefront
-    if (rows < 1 || rows > 16 || K % 128 != 0 || (group != 128 && group != 256) || !aligned(x, 16)) return false;
+    if (rows < 1 || rows > 32 || K % 128 != 0 || (group != 128 && group != 256) || !aligned(x, 16)) return false;
     const int steps = K / 128;
     const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
     if (steps < kFlightWaves || spw > 7 || spw == 5) return false;
+    // 17..32 rows: two blocks of 16 rows against the same weight registers; one weight, up to two steps per wavefront
+    const bool two_blocks = rows > 16;
+    if (two_blocks && (spw > 2 || pair || norm || wts.count != 1 || tuning_env("TPQ_INT4_NO_TWO_BLOCKS"))) return false;
     // five and more steps per wavefront at more than eight rows: the tiles of 16 rows keep one step in LDS at a time and
     // the registers fill up (11008 -> 4096 at 16 rows: 17.7 us against 14.0 for the loop kernel)
     if (spw > 4 && rows > 8) return false;
@@ -120,9 +123,15 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
         slots[w]->first = pair ? 0 : blocks;
         if (!pair || w == 0) blocks += (wts.N[w] + 15) / 16;
     }
-    int nb = flight_width(blocks, rows, spw, pair, wts.count == 1);
+    int nb = flight_width(blocks, rows < 16 ? rows : 16, spw, pair, wts.count == 1);
     if (const char* env = tuning_env("TPQ_INT4_FLIGHT")) nb = std::atoi(env);  // 0 switches the kernel off, 1..4 pin the width
     if (nb <= 0) return false;
+    // Two blocks of rows: measured against the loop kernel with two row blocks per workgroup (us, 17 / 24 / 32 rows):
+    // 4096 -> 11008 11.5 / 11.4 / 11.3 against 11.4 / 11.9 / 13.2; 4096 x 4096 7.5 / 7.6 / 7.7 against 8.1 / 9.1 / 10.4;
+    // 3072 -> 9216 9.3 / 9.2 / 9.5 against 13.1 / 15.1 / 17.5; 4096 -> 6144 8.6 / 8.7 / 8.9 against 8.8 / 9.8 / 11.3.  It loses
+    // where the workgroups need more than one pass or the widest form (4096 -> 16384: 17.8 against 13.5 at 32 rows;
+    // 4096 -> 32000: 32.5 against 25.5) and with a single step per wavefront (2048 -> 8192: 7.2 against 6.1 at 17 rows).
+    if (two_blocks && (nb > 3 || (blocks + nb - 1) / nb > flight_compute_units() || steps < 24)) return false;
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* rp = static_cast<const uint16_t*>(residual);
     const int shift = group == 128 ? 0 : 1;
@@ -137,6 +146,12 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
                           : launch_rows<DT, NBV, SPWV, kFlightMany>(xp, rows, set, blocks, K, shift, rp, s)
         switch (spw) {
             case 1: case 2:
+                if (two_blocks) {
+#define TPQ_FLIGHT2(NBV) code = launch_as<DT, NBV, 2, 16, kFlightOne, false, 2>(xp, rows, set, blocks, K, shift, rp, s)
+                    if (nb == 1) TPQ_FLIGHT2(1); else if (nb == 2) TPQ_FLIGHT2(2); else if (nb == 3) TPQ_FLIGHT2(3); else TPQ_FLIGHT2(4);
+#undef TPQ_FLIGHT2
+                    break;
+                }
                 if (nb == 1) TPQ_FLIGHT(1, 2); else if (nb == 2) TPQ_FLIGHT(2, 2); else if (nb == 3) TPQ_FLIGHT(3, 2); else TPQ_FLIGHT(4, 2);
                 break;
             case 3: if (nb == 1) TPQ_FLIGHT(1, 3); else TPQ_FLIGHT(2, 3); break;

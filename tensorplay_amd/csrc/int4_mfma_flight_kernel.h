@@ -90,6 +90,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 template <int XR>
 constexpr int flight_resident_steps() { return XR == 16 ? 1 : 2; }
 
+// (the same for one and for two row blocks: the second block reuses the tiles and the partial-sum area of the first)
 template <int NB, int SPW, int XR>
 constexpr size_t flight_lds_bytes() {
     return static_cast<size_t>(kFlightWaves) * flight_resident_steps<XR>() * XR * kFlightRowStride  // activation tiles
@@ -101,11 +102,15 @@ constexpr size_t flight_lds_bytes() {
 // x: [M][K] 16-bit, M <= XR; weights as in FlightSet (packed: [N/8][K/32][8] x 16 bytes; sz: [K/group][N] words
 // (scale, zero)); K % 128 == 0, 16 <= K / 128 <= 16 SPW and K / 128 > 16 (SPW - 1); a group is 128 << group_shift k;
 // residual (one weight, may be null): [M][N], added to the rounded output.
-template <int DT, int NB, int SPW, int XR, int MODE, bool NORM = false>
+// RB = 2 (XR = 16, one weight): 17..32 rows as two blocks of 16.  The weights are requested once and stay in registers;
+// the second block's activations are requested step by step into the registers the first block's have left for LDS, and
+// are multiplied with the same weights (unpacked again) when the first block is done.
+template <int DT, int NB, int SPW, int XR, int MODE, bool NORM = false, int RB = 1>
 __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(const uint16_t* __restrict__ x, FlightSet set, int M,
                                                                               int K, int group_shift,
                                                                               const uint16_t* __restrict__ residual) {
     static_assert(XR == 4 || XR == 8 || XR == 16, "rows through LDS: 4, 8 or 16");
+    static_assert(RB == 1 || (RB == 2 && XR == 16 && !NORM && MODE == kFlightOne), "two row blocks: 16 rows each, one weight");
     constexpr bool PAIR = MODE == kFlightPair;
     static_assert(!PAIR || NB % 2 == 0, "a pair is the same blocks of two weights");
     static_assert(NB <= 8, "two parameter words per lane at most");
@@ -307,13 +312,15 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
         }
     }
 
-    float yacc[NB][4];
+    float yacc[RB][NB][4];
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) yacc[b][v] = 0.0f;
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) yacc[rb][b][v] = 0.0f;
 
-    auto compute = [&](int j) {
+    auto compute = [&](int j, int rb) {
         // lane (m, q): the 64 bytes of row m % XR in k-tile 4 s + q; MFMA u takes bytes 16 u .. 16 u + 15 of them
         word4_t xb[4];
         const unsigned char* xrow = my_x + ((j % XS) * XR + (i & (XR - 1))) * kFlightRowStride + q * 64;
@@ -350,7 +357,7 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const uint32_t word = dword_of(p, v);  // (scale, zero) of channel n0 + 4 q + v of block b
-                yacc[b][v] = __builtin_fmaf(L::lo(word), d[b][v] - corr, __builtin_fmaf(L::hi(word), sx, yacc[b][v]));
+                yacc[rb][b][v] = __builtin_fmaf(L::lo(word), d[b][v] - corr, __builtin_fmaf(L::hi(word), sx, yacc[rb][b][v]));
             }
         }
     };
@@ -364,30 +371,62 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
                 *reinterpret_cast<uint4*>(my_x + ((j % XS) * XR + 4 * t + q) * kFlightRowStride + i * 16) = xg[j][t];
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (RB == 2) {  // XS = 1: step j0 of the first block is in LDS, its registers take the second block's
+            order_fence();
+#pragma unroll
+            for (int t = 0; t < XR / 4; ++t) {
+                int row = XR + 4 * t + q;
+                row = row < M ? row : M - 1;
+                const GlobalWords4 src = opaque4(reinterpret_cast<const uint4*>(x + static_cast<size_t>(row) * K) + i);
+                xg[j0][t] = as_uint4(src[step_of[j0] * 16]);
+            }
+            order_fence();
+        }
 #pragma unroll
         for (int j = j0; j < j0 + XS && j < SPW; ++j) {
             if (j < SPW - 1) {
-                compute(j);
+                compute(j, 0);
             } else if (last_live) {  // wave-uniform, after every request: nothing is held back by this branch
-                compute(j);
+                compute(j, 0);
             }
             __builtin_amdgcn_sched_barrier(0);  // a step is finished, epilogue included, while the next one is on its way
         }
         __builtin_amdgcn_wave_barrier();
     }
+    if constexpr (RB == 2) {
+        static_assert(RB == 1 || XS == 1, "the second block's requests go step by step");
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) {
+#pragma unroll
+            for (int t = 0; t < XR / 4; ++t) *reinterpret_cast<uint4*>(my_x + (4 * t + q) * kFlightRowStride + i * 16) = xg[j][t];
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if (j < SPW - 1) {
+                compute(j, 1);
+            } else if (last_live) {
+                compute(j, 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
 
     // ---- the wavefronts' partial sums, added in wavefront order -----------------------------------------------
     const int slot = q * XR + i;  // live lanes (rows < XR) only
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+    if (rb > 0) __syncthreads();  // the sums of the first block have been read
     if (i < XR) {
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) red[((wave * NB + b) * 4 + v) * (4 * XR) + slot] = yacc[b][v];
+            for (int v = 0; v < 4; ++v) red[((wave * NB + b) * 4 + v) * (4 * XR) + slot] = yacc[rb][b][v];
     }
     __syncthreads();
+    const int out_row = XR * rb + i;  // RB = 1: i
     // wavefront w finishes output block w: lane (m, q) stores row m, channels n0 + 4 q + v
     for (int b = wave; b < C; b += kFlightWaves) {
-        if (i >= XR || i >= M) continue;
+        if (i >= XR || out_row >= M) continue;
         const Block out = resolve(b);
         const int n = out.n0 + 4 * q;
         if (n >= out.N) continue;  // N % 8 == 0 and n % 4 == 0: all four channels exist
@@ -418,15 +457,16 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[v] = L::out(sum[0][v]);
             if (residual != nullptr) {  // the rounded output plus the residual, rounded again: what a separate add does
-                const uint2 rw = *reinterpret_cast<const uint2*>(residual + static_cast<size_t>(i) * out.N + n);
+                const uint2 rw = *reinterpret_cast<const uint2*>(residual + static_cast<size_t>(out_row) * out.N + n);
                 const uint16_t rv[4] = {static_cast<uint16_t>(rw.x), static_cast<uint16_t>(rw.x >> 16), static_cast<uint16_t>(rw.y),
                                         static_cast<uint16_t>(rw.y >> 16)};
 #pragma unroll
                 for (int v = 0; v < 4; ++v) o[v] = L::out(Elem<DT>::load(o[v]) + Elem<DT>::load(rv[v]));
             }
         }
-        *reinterpret_cast<uint2*>(out.y + static_cast<size_t>(i) * out.N + n) =
+        *reinterpret_cast<uint2*>(out.y + static_cast<size_t>(out_row) * out.N + n) =
             make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
+    }
     }
 }
 

@@ -259,6 +259,10 @@ FLIGHT_CASES = [  # M, N, K, group: the all-in-flight matrix-core kernel (K >= 2
     (13, 72, 11008, 128),
     (6, 264, 14336, 128),    # seven steps per wavefront
     (12, 264, 14336, 128),   # (that many steps at more than eight rows: the loop kernel)
+    # 17..32 rows: two blocks of 16 rows against the same weight registers (K = 3072..4096), every width of workgroup
+    # that takes it, a partial second block, a partial last channel block, and a slab of 32 plus a rest
+    (17, 72, 3072, 128), (32, 264, 4096, 128), (25, 136, 3584, 128), (31, 8200, 4096, 128), (20, 11008, 4096, 128),
+    (50, 72, 4096, 128),
 ]
 
 
@@ -305,7 +309,8 @@ def _tile_subset(rng, n_tiles, count):
 
 @pytest.mark.parametrize("tdt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 136, 512), (16, 4096, 1024), (19, 48, 384),
-                                   (8, 264, 4096), (3, 72, 11008), (12, 4104, 4096)])  # the all-in-flight kernel
+                                   (8, 264, 4096), (3, 72, 11008), (12, 4104, 4096),  # the all-in-flight kernel
+                                   (24, 136, 4096), (32, 4104, 3072)])               # ... with two blocks of 16 rows
 def test_mm_add_equals_the_two_ops(ops, tdt, M, N, K):
     """out = residual + x.W^T with both roundings of the separate ops: equal bit for bit whenever the matmul
     runs on the same kernel (rows > 1), within one rounding of it otherwise."""
