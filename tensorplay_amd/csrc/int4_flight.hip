@@ -166,12 +166,12 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
     return true;
 }
 
-template <int DT, int NB, int SPW, int XR>
+template <int DT, int NB, int SPW, int XR, int RB = 1>
 int launch_int8_as(const uint16_t* x, int rows, const int8_t* w, const float* scales, uint16_t* y, int N, int K, hipStream_t s) {
     constexpr size_t bytes = int8_flight_lds_bytes<NB, SPW, XR>();
     static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
     static std::atomic<uint64_t> reserved{0};
-    const auto kernel = int8pack_flight_kernel<DT, NB, SPW, XR>;
+    const auto kernel = int8pack_flight_kernel<DT, NB, SPW, XR, RB>;
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), bytes, reserved, "_weight_int8pack_mm (all in flight)")) return rc;
     kernel<<<dim3((N + 16 * NB - 1) / (16 * NB)), dim3(kFlightWaves * kWave), bytes, s>>>(x, w, scales, y, rows, N, K);
     return check_launch("_weight_int8pack_mm (all in flight)");
@@ -182,6 +182,7 @@ int launch_int8_rows(const uint16_t* x, int rows, const int8_t* w, const float* 
     if (rows <= 4) return launch_int8_as<DT, NB, SPW, 4>(x, rows, w, scales, y, N, K, s);
     if (rows <= 8) return launch_int8_as<DT, NB, SPW, 8>(x, rows, w, scales, y, N, K, s);
     if constexpr (SPW <= 2) {
+        if (rows > 16) return launch_int8_as<DT, NB, SPW, 16, 2>(x, rows, w, scales, y, N, K, s);  // two blocks of 16 rows
         return launch_int8_as<DT, NB, SPW, 16>(x, rows, w, scales, y, N, K, s);
     } else {
         return TPQ_ERR_UNSUPPORTED;  // not reached
@@ -192,9 +193,12 @@ int launch_int8_rows(const uint16_t* x, int rows, const int8_t* w, const float* 
 // 4096 x 4096 at 8 rows 7.5 -> 6.4; 4096 -> 32000 at 8 rows 34.7 -> 28.5; 11008 -> 4096 at 8 rows 16.2 -> 14.2.
 template <int DT>
 bool launch_int8(const void* x, int rows, const int8_t* w, const float* scales, void* y, int N, int K, hipStream_t s, int* rc) {
-    if (rows < 1 || rows > 16 || K % 128 != 0 || !aligned(x, 16) || !aligned(w, 16)) return false;
+    if (rows < 1 || rows > 32 || K % 128 != 0 || !aligned(x, 16) || !aligned(w, 16)) return false;
     const int steps = K / 128;
     const int spw = (steps + kFlightWaves - 1) / kFlightWaves;
+    // 17..32 rows: two blocks of 16 rows against the same weight registers, up to two steps per wavefront, one pass of workgroups
+    const bool two_blocks = rows > 16;
+    if (two_blocks && (spw > 2 || steps < 24 || tuning_env("TPQ_INT8PACK_NO_TWO_BLOCKS"))) return false;
     // more than two steps per wavefront at more than eight rows: the loop kernel is as fast or faster (8192 x 8192 at 12 rows:
     // 22.0 us against 19.5; 11008 -> 4096: 17.8 / 17.8)
     if (steps < kFlightWaves || spw > 7 || spw == 5 || (spw > 2 && rows > 8)) return false;
@@ -207,6 +211,10 @@ bool launch_int8(const void* x, int rows, const int8_t* w, const float* scales, 
     if (nb == 0 && spw <= 2) nb = widest;  // several passes pay off with two steps per wavefront only (see flight_width)
     if (const char* env = tuning_env("TPQ_INT8PACK_FLIGHT")) nb = std::atoi(env);  // 0 switches the kernel off, 1..4 pin the width
     if (nb <= 0 || nb > widest) return false;
+    // Two blocks of rows, measured against the loop kernel with two row blocks per workgroup (us, 17 / 24 / 32 rows):
+    // 4096 -> 11008 15.2 / 15.4 / 15.8 against 24.3 / 28.1 / 32.0; 4096 x 4096 8.7 / 9.2 / 9.6 against 10.4 / 11.9 / 13.3;
+    // 3072 -> 9216 14.2 / 14.6 / 15.0 against 20.1 / 21.9 / 23.9; the widest form loses (4096 -> 16384: 34.0 against 31.1)
+    if (two_blocks && (nb > 3 || (blocks + nb - 1) / nb > cus)) return false;
     const auto* xp = static_cast<const uint16_t*>(x);
     auto* yp = static_cast<uint16_t*>(y);
     int code = TPQ_ERR_UNSUPPORTED;

@@ -25,11 +25,13 @@ constexpr size_t int8_flight_lds_bytes() {
 
 // x: [M][K] 16-bit, M <= XR; w: [N][K] int8; scale: [N]; y: [M][N]; K % 128 == 0, 16 <= K / 128 <= 16 SPW and
 // K / 128 > 16 (SPW - 1)
-template <int DT, int NB, int SPW, int XR>
+// RB = 2 (XR = 16): 17..32 rows as two blocks of 16 against the same weight registers, as in the int4 kernel.
+template <int DT, int NB, int SPW, int XR, int RB = 1>
 __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(const uint16_t* __restrict__ x, const int8_t* __restrict__ w,
                                                                              const float* __restrict__ scale, uint16_t* __restrict__ y,
                                                                              int M, int N, int K) {
     static_assert(XR == 4 || XR == 8 || XR == 16, "rows through LDS: 4, 8 or 16");
+    static_assert(RB == 1 || (RB == 2 && XR == 16), "two row blocks: 16 rows each");
     constexpr int XS = flight_resident_steps<XR>();
     extern __shared__ __align__(16) unsigned char flight_lds[];
     unsigned char* const xbuf = flight_lds;
@@ -85,11 +87,13 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(co
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(0x64646464u));
 
     unsigned char* const my_x = xbuf + static_cast<size_t>(wave) * XS * XR * kFlightRowStride;
-    float4_t d[NB];
+    float4_t d[RB][NB];
 #pragma unroll
-    for (int b = 0; b < NB; ++b) d[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) d[rb][b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto compute = [&](int j) {
+    auto compute = [&](int j, int rb) {
         // lane (m, q): the 64 bytes of row m % XR at k = 128 s + 32 q; MFMA u takes bytes 16 u .. 16 u + 15 of them
         word4_t xb[4];
         const unsigned char* xrow = my_x + ((j % XS) * XR + (i & (XR - 1))) * kFlightRowStride + q * 64;
@@ -123,7 +127,7 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(co
                         a[2 * h + 1] = __builtin_amdgcn_perm(f[3], f[2], 0x07060302u);
                     }
                 }
-                d[b] = MfmaLane<DT>::mfma(word4_t{a[0], a[1], a[2], a[3]}, xb[u], d[b]);
+                d[rb][b] = MfmaLane<DT>::mfma(word4_t{a[0], a[1], a[2], a[3]}, xb[u], d[rb][b]);
             }
         }
     };
@@ -137,16 +141,44 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(co
                 *reinterpret_cast<uint4*>(my_x + ((j % XS) * XR + 4 * t + q) * kFlightRowStride + i * 16) = xg[j][t];
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (RB == 2) {  // XS = 1: step j0 of the first block is in LDS, its registers take the second block's
+            order_fence();
+#pragma unroll
+            for (int t = 0; t < XR / 4; ++t) {
+                int row = XR + 4 * t + q;
+                row = row < M ? row : M - 1;
+                const GlobalWords4 src = opaque4(reinterpret_cast<const uint4*>(x + static_cast<size_t>(row) * K) + i);
+                xg[j0][t] = as_uint4(src[step_of[j0] * 16]);
+            }
+            order_fence();
+        }
 #pragma unroll
         for (int j = j0; j < j0 + XS && j < SPW; ++j) {
             if (j < SPW - 1) {
-                compute(j);
+                compute(j, 0);
             } else if (last_live) {  // wave-uniform, after every request
-                compute(j);
+                compute(j, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_wave_barrier();
+    }
+    if constexpr (RB == 2) {
+        static_assert(RB == 1 || XS == 1, "the second block's requests go step by step");
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) {
+#pragma unroll
+            for (int t = 0; t < XR / 4; ++t) *reinterpret_cast<uint4*>(my_x + (4 * t + q) * kFlightRowStride + i * 16) = xg[j][t];
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if (j < SPW - 1) {
+                compute(j, 1);
+            } else if (last_live) {
+                compute(j, 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 
     // ---- the wavefronts' partial sums, added in wavefront order -----------------------------------------------
@@ -163,23 +195,28 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int8pack_flight_kernel(co
         }
     }
     const int slot = q * XR + i;  // live lanes (rows < XR) only
-    if (i < XR) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
+    for (int rb = 0; rb < RB; ++rb) {
+        if (rb > 0) __syncthreads();  // the sums of the first block have been read
+        if (i < XR) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) red[((wave * NB + b) * 4 + v) * (4 * XR) + slot] = d[b][v];
-    }
-    __syncthreads();
-    // wavefront w finishes block w: lane (m, q) stores row m, channels n0 + 16 b + 4 q + v
-    for (int b = wave; b < NB; b += kFlightWaves) {
-        if (i >= XR || i >= M) continue;
-        const int n = n0 + 16 * b + 4 * q;
+            for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            float sum = 0.0f;
+                for (int v = 0; v < 4; ++v) red[((wave * NB + b) * 4 + v) * (4 * XR) + slot] = d[rb][b][v];
+        }
+        __syncthreads();
+        const int out_row = XR * rb + i;
+        // wavefront w finishes block w: lane (m, q) stores row m, channels n0 + 16 b + 4 q + v
+        for (int b = wave; b < NB; b += kFlightWaves) {
+            if (i >= XR || out_row >= M) continue;
+            const int n = n0 + 16 * b + 4 * q;
 #pragma unroll
-            for (int ww = 0; ww < kFlightWaves; ++ww) sum += red[((ww * NB + b) * 4 + v) * (4 * XR) + slot];
-            if (n + v < N) y[static_cast<size_t>(i) * N + n + v] = Elem<DT>::store(__fmul_rn(sum, scale_n[v]));
+            for (int v = 0; v < 4; ++v) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int ww = 0; ww < kFlightWaves; ++ww) sum += red[((ww * NB + b) * 4 + v) * (4 * XR) + slot];
+                if (n + v < N) y[static_cast<size_t>(out_row) * N + n + v] = Elem<DT>::store(__fmul_rn(sum, scale_n[v]));
+            }
         }
     }
 }

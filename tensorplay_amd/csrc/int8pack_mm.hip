@@ -473,7 +473,7 @@ TPQ_EXPORT int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64
         static const int forced_mb = [] { const char* e = tuning_env("TPQ_INT8PACK_MB"); return e ? std::atoi(e) : 0; }();
         for (int64_t m0 = 0; m0 < M;) {
             const int left = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
-            if (left <= 16 && N <= 0x7FFFFFF0 && K <= 0x7FFFFF80) {  // the all-in-flight form, where it is built
+            if (N <= 0x7FFFFFF0 && K <= 0x7FFFFF80) {  // the all-in-flight form, where it is built (17..32 rows: two blocks of 16)
                 int rc = TPQ_OK;
                 if (flight_launch_int8pack(dtype, static_cast<const uint16_t*>(x) + m0 * K, left, w, scales, static_cast<uint16_t*>(out) + m0 * N,
                                            static_cast<int>(N), static_cast<int>(K), s, &rc)) {

@@ -41,7 +41,10 @@ CASES = [(1, 4096, 512), (4, 1024, 136), (16, 256, 40), (17, 384, 72), (2, 100, 
          # the all-in-flight matrix-core kernel (3..16 rows, K = 2048..14336): 4 / 8 / 16 rows through LDS, every width of
          # workgroup, a dead last step (K = 2048, 5120, 11008), ragged N, more workgroups than one pass
          (3, 2048, 72), (5, 4096, 4104), (8, 4096, 11008), (4, 4096, 16392), (9, 4096, 136), (16, 5120, 264),
-         (7, 8192, 136), (8, 11008, 4104), (6, 14336, 264), (13, 11008, 72)]
+         (7, 8192, 136), (8, 11008, 4104), (6, 14336, 264), (13, 11008, 72),
+         # ... 17..32 rows as two blocks of 16 rows against the same weight registers (K = 3072..4096): a partial second
+         # block, ragged N, every width of workgroup, a slab of 32 plus a rest
+         (17, 3072, 72), (32, 4096, 264), (25, 3584, 136), (31, 4096, 8200), (20, 4096, 11008), (50, 4096, 72)]
 
 
 @pytest.mark.gpu
