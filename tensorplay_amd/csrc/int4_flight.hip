@@ -98,7 +98,7 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
     if (steps < kFlightWaves || spw > 7 || spw == 5) return false;
     // 17..32 rows: two blocks of 16 rows against the same weight registers; one weight, up to two steps per wavefront
     const bool two_blocks = rows > 16;
-    if (two_blocks && (spw > 2 || pair || norm || wts.count != 1 || tuning_env("TPQ_INT4_NO_TWO_BLOCKS"))) return false;
+    if (two_blocks && (spw > 3 || pair || norm || wts.count != 1 || tuning_env("TPQ_INT4_NO_TWO_BLOCKS"))) return false;
     // five and more steps per wavefront at more than eight rows: the tiles of 16 rows keep one step in LDS at a time and
     // the registers fill up (11008 -> 4096 at 16 rows: 17.7 us against 14.0 for the loop kernel)
     if (spw > 4 && rows > 8) return false;
@@ -131,7 +131,10 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
     // 3072 -> 9216 9.3 / 9.2 / 9.5 against 13.1 / 15.1 / 17.5; 4096 -> 6144 8.6 / 8.7 / 8.9 against 8.8 / 9.8 / 11.3.  It loses
     // where the workgroups need more than one pass or the widest form (4096 -> 16384: 17.8 against 13.5 at 32 rows;
     // 4096 -> 32000: 32.5 against 25.5) and with a single step per wavefront (2048 -> 8192: 7.2 against 6.1 at 17 rows).
-    if (two_blocks && (nb > 3 || (blocks + nb - 1) / nb > flight_compute_units() || steps < 24)) return false;
+    // Three steps per wavefront (K up to 6144): only the form of one block per workgroup keeps everything in registers
+    // (5120 -> 2560 at 17 / 24 / 32 rows: 8.7 / 8.9 / 9.3 against 9.4 / 10.7 / 12.5); two blocks per workgroup spill 17
+    // registers and four steps 18..52, and lose by up to 2 x (8192 x 8192 at 32 rows: 34.9 against 19.4).
+    if (two_blocks && (nb > 3 || (blocks + nb - 1) / nb > flight_compute_units() || steps < 24 || (spw == 3 && nb != 1))) return false;
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* rp = static_cast<const uint16_t*>(residual);
     const int shift = group == 128 ? 0 : 1;
@@ -154,7 +157,13 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
                 }
                 if (nb == 1) TPQ_FLIGHT(1, 2); else if (nb == 2) TPQ_FLIGHT(2, 2); else if (nb == 3) TPQ_FLIGHT(3, 2); else TPQ_FLIGHT(4, 2);
                 break;
-            case 3: if (nb == 1) TPQ_FLIGHT(1, 3); else TPQ_FLIGHT(2, 3); break;
+            case 3:
+                if (two_blocks) {  // one block per workgroup only (nb == 1: see above)
+                    code = launch_as<DT, 1, 3, 16, kFlightOne, false, 2>(xp, rows, set, blocks, K, shift, rp, s);
+                    break;
+                }
+                if (nb == 1) TPQ_FLIGHT(1, 3); else TPQ_FLIGHT(2, 3);
+                break;
             case 4: if (nb == 1) TPQ_FLIGHT(1, 4); else TPQ_FLIGHT(2, 4); break;
             case 6: TPQ_FLIGHT(1, 6); break;
             case 7: TPQ_FLIGHT(1, 7); break;

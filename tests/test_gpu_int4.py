@@ -262,7 +262,7 @@ FLIGHT_CASES = [  # M, N, K, group: the all-in-flight matrix-core kernel (K >= 2
     # 17..32 rows: two blocks of 16 rows against the same weight registers (K = 3072..4096), every width of workgroup
     # that takes it, a partial second block, a partial last channel block, and a slab of 32 plus a rest
     (17, 72, 3072, 128), (32, 264, 4096, 128), (25, 136, 3584, 128), (31, 8200, 4096, 128), (20, 11008, 4096, 128),
-    (50, 72, 4096, 128),
+    (50, 72, 4096, 128), (29, 136, 5120, 128), (32, 4096, 6144, 128),   # three steps per wavefront, one block per workgroup
 ]
 
 
