@@ -372,12 +372,25 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
     return (out, acc) if return_acc else out
 
 
-# Above this many activation rows _weight_int8pack_mm dequantises and calls the library GEMM.  Measured (fp16, us,
-# 32-row slabs against the dense route): K = 4096, N = 11008: 33 / 44 at 32 rows, 53 / 46 at 48; K = N = 4096: 26 / 33
-# at 64 rows, 39 / 41 at 96; K = N = 8192: 58 / 65 at 64 rows, 86 / 69 at 96.
+# Above this many activation rows _weight_int8pack_mm dequantises and calls the library GEMM.  Measured (fp16 / bf16
+# alike unless said, us, slabs of 32 rows on the decode kernels against the dense route): K = 4096, N = 11008: 30 / 45 at
+# 64 rows, 44 / 47 (bf16: 53 / 47) at 96; K = N = 4096: 26 / 34 at 96, 36 / 37 at 128; 4096 -> 6144: 33 / 39 at 96, 44 / 41
+# at 128; K = N = 8192: 56 / 61 at 64, 84 / 68 at 96; 11008 -> 4096: 47 / 48 at 48, 57 / 53 at 64; 4096 -> 32000: 112 / 113
+# at 64, 168 / 103 at 96.
 INT8PACK_PREFILL_ROWS = 64
-INT8PACK_PREFILL_ROWS_WIDE = 40  # N >= 10240
+INT8PACK_PREFILL_ROWS_TWO_BLOCKS = 96  # K = 3072..4096, N < 10240: slabs of 32 rows on the all-in-flight kernel
+INT8PACK_PREFILL_ROWS_LONG = 48  # K > 8192
 INT8PACK_PREFILL_ROWS_F32 = 24  # float32 activations (per-row kernel): 64 / 89 us at 16 rows, 119 / 94 us at 32
+
+
+def _int8pack_prefill_rows(N: int, K: int, dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return INT8PACK_PREFILL_ROWS_F32
+    if K > 8192:
+        return INT8PACK_PREFILL_ROWS_LONG
+    if 3072 <= K <= 4096 and N < 10240:
+        return INT8PACK_PREFILL_ROWS_TWO_BLOCKS
+    return INT8PACK_PREFILL_ROWS
 
 
 def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
@@ -402,7 +415,7 @@ def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Te
     x, w = self.contiguous(), mat2.contiguous()
     sc = scales.to(torch.float32).contiguous()
     with torch.cuda.device(x.device):
-        if B > (INT8PACK_PREFILL_ROWS_F32 if x.dtype == torch.float32 else INT8PACK_PREFILL_ROWS_WIDE if N >= 10240 else INT8PACK_PREFILL_ROWS):
+        if B > _int8pack_prefill_rows(N, K, x.dtype):
             # Many rows: the decode kernel streams the weight once per 32 rows, which stops paying here.  One pass
             # writes the dense weight T(w * scale) and a library GEMM does the rest.
             dense = torch.empty((N, K), dtype=x.dtype, device=x.device)
