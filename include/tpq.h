@@ -224,7 +224,8 @@ int tpq_int4_mm_swiglu(const void* x, int dtype, int64_t M, int64_t K, const int
                        const void* sz_gate, const void* sz_up, void* out, void* stream);
 
 /*
- * `count` (1..4) int4 weights applied to the same activations in one launch per 16 rows:
+ * `count` (1..4) int4 weights applied to the same activations in one launch per 16 rows (per 32 rows where the
+ * kernel takes two blocks of 16 rows against the same weight registers: K = 3072..4096, one pass of workgroups):
  * out[w] = T(x . W[w]^T), out[w]: [M, N[w]] of dtype, for w < count.  Same kernel, same shapes
  * (float16 / bfloat16, innerKTiles = 2, group 128, K % 128 == 0, else TPQ_ERR_UNSUPPORTED) and same
  * result as `count` calls of tpq_int4_mm at up to 16 rows per call.  packed, N, scales_and_zeros and

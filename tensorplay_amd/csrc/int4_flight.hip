@@ -98,7 +98,7 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
     if (steps < kFlightWaves || spw > 7 || spw == 5) return false;
     // 17..32 rows: two blocks of 16 rows against the same weight registers; one weight, up to two steps per wavefront
     const bool two_blocks = rows > 16;
-    if (two_blocks && (spw > 3 || pair || norm || wts.count != 1 || tuning_env("TPQ_INT4_NO_TWO_BLOCKS"))) return false;
+    if (two_blocks && (spw > 3 || pair || norm || tuning_env("TPQ_INT4_NO_TWO_BLOCKS"))) return false;
     // five and more steps per wavefront at more than eight rows: the tiles of 16 rows keep one step in LDS at a time and
     // the registers fill up (11008 -> 4096 at 16 rows: 17.7 us against 14.0 for the loop kernel)
     if (spw > 4 && rows > 8) return false;
@@ -150,7 +150,9 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
         switch (spw) {
             case 1: case 2:
                 if (two_blocks) {
-#define TPQ_FLIGHT2(NBV) code = launch_as<DT, NBV, 2, 16, kFlightOne, false, 2>(xp, rows, set, blocks, K, shift, rp, s)
+#define TPQ_FLIGHT2(NBV)                                                                                                   \
+    code = wts.count == 1 ? launch_as<DT, NBV, 2, 16, kFlightOne, false, 2>(xp, rows, set, blocks, K, shift, rp, s)          \
+                          : launch_as<DT, NBV, 2, 16, kFlightMany, false, 2>(xp, rows, set, blocks, K, shift, rp, s)
                     if (nb == 1) TPQ_FLIGHT2(1); else if (nb == 2) TPQ_FLIGHT2(2); else if (nb == 3) TPQ_FLIGHT2(3); else TPQ_FLIGHT2(4);
 #undef TPQ_FLIGHT2
                     break;
@@ -159,7 +161,8 @@ bool launch(const void* x, int rows, const FlightWeights& wts, int K, int group,
                 break;
             case 3:
                 if (two_blocks) {  // one block per workgroup only (nb == 1: see above)
-                    code = launch_as<DT, 1, 3, 16, kFlightOne, false, 2>(xp, rows, set, blocks, K, shift, rp, s);
+                    code = wts.count == 1 ? launch_as<DT, 1, 3, 16, kFlightOne, false, 2>(xp, rows, set, blocks, K, shift, rp, s)
+                                          : launch_as<DT, 1, 3, 16, kFlightMany, false, 2>(xp, rows, set, blocks, K, shift, rp, s);
                     break;
                 }
                 if (nb == 1) TPQ_FLIGHT(1, 3); else TPQ_FLIGHT(2, 3);

@@ -102,7 +102,7 @@ constexpr size_t flight_lds_bytes() {
 // x: [M][K] 16-bit, M <= XR; weights as in FlightSet (packed: [N/8][K/32][8] x 16 bytes; sz: [K/group][N] words
 // (scale, zero)); K % 128 == 0, 16 <= K / 128 <= 16 SPW and K / 128 > 16 (SPW - 1); a group is 128 << group_shift k;
 // residual (one weight, may be null): [M][N], added to the rounded output.
-// RB = 2 (XR = 16, one weight): 17..32 rows as two blocks of 16.  The weights are requested once and stay in registers;
+// RB = 2 (XR = 16, one weight or several, not the pair): 17..32 rows as two blocks of 16.  The weights are requested once and stay in registers;
 // the second block's activations are requested step by step into the registers the first block's have left for LDS, and
 // are multiplied with the same weights (unpacked again) when the first block is done.
 template <int DT, int NB, int SPW, int XR, int MODE, bool NORM = false, int RB = 1>
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
                                                                               int K, int group_shift,
                                                                               const uint16_t* __restrict__ residual) {
     static_assert(XR == 4 || XR == 8 || XR == 16, "rows through LDS: 4, 8 or 16");
-    static_assert(RB == 1 || (RB == 2 && XR == 16 && !NORM && MODE == kFlightOne), "two row blocks: 16 rows each, one weight");
+    static_assert(RB == 1 || (RB == 2 && XR == 16 && !NORM && MODE != kFlightPair), "two row blocks: 16 rows each, not for the pair");
     constexpr bool PAIR = MODE == kFlightPair;
     static_assert(!PAIR || NB % 2 == 0, "a pair is the same blocks of two weights");
     static_assert(NB <= 8, "two parameter words per lane at most");

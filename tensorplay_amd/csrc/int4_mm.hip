@@ -587,7 +587,9 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
                  void* const* y, int K, int group, hipStream_t s, const void* norm_weight = nullptr, float norm_eps = 0.0f) {
     int64_t n_total = 0;
     for (int w = 0; w < count; ++w) n_total += N[w];
-    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+    int64_t step = 16;
+    for (int64_t m0 = 0; m0 < M; m0 += step) {
+        step = 16;
         const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
         {
             FlightWeights all{};
@@ -599,6 +601,14 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
             all.norm_weight = norm_weight;
             all.norm_eps = norm_eps;
             int rc = TPQ_OK;
+            // 17..32 rows left: one launch with two blocks of 16 rows, where the all-in-flight kernel is built for it
+            const int rows32 = static_cast<int>(M - m0 < 32 ? M - m0 : 32);
+            if (rows32 > 16 && norm_weight == nullptr &&
+                flight_launch(DT, static_cast<const uint16_t*>(x) + m0 * K, rows32, all, K, group, false, nullptr, s, &rc)) {
+                if (rc != TPQ_OK) return rc;
+                step = 32;
+                continue;
+            }
             if (flight_launch(DT, static_cast<const uint16_t*>(x) + m0 * K, rows, all, K, group, false, nullptr, s, &rc)) {
                 if (rc != TPQ_OK) return rc;
                 continue;

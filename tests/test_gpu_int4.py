@@ -355,7 +355,9 @@ def test_mm_swiglu_against_oracle(ops, tdt, tol, M, N, K):
 @pytest.mark.parametrize("M,K,widths", [(1, 256, (64,)), (8, 512, (136, 136, 136)), (16, 1024, (1024, 256, 256)),
                                         (19, 384, (48, 8, 200, 16)), (8, 4096, (4096, 4096, 4096)), (4, 4096, (11008, 11008)),
                                         # the all-in-flight kernel: blocks of different weights in one workgroup
-                                        (5, 4096, (72, 8, 200, 16)), (9, 11008, (136, 264)), (3, 8192, (4104, 24, 4096))])
+                                        (5, 4096, (72, 8, 200, 16)), (9, 11008, (136, 264)), (3, 8192, (4104, 24, 4096)),
+                                        # ... 17..32 rows as two blocks of 16 in one launch, a slab of 32 plus a rest
+                                        (32, 4096, (4096, 4096, 4096)), (21, 3072, (72, 8, 200, 16)), (45, 4096, (136, 264))])
 def test_mm_multi_equals_separate_products(ops, tdt, tol, M, K, widths):
     """Several weights on one input in one launch: every output against the separate op (the same kernel; the order
     in which the wavefronts' partial sums are added may differ with the workgroup shape) and against the oracle."""
