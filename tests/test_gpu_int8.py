@@ -118,6 +118,9 @@ def test_rescale_bit_exact(ops):
 @pytest.mark.parametrize("out_dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("shape", [(16, 1024, 1024), (300, 208, 200), (5, 7, 3), (256, 512, 384), (40, 256, 36), (1, 4096, 64), (50, 256, 6160), (9, 128, 16390),
                                    (130, 1024, 200), (300, 2048, 136), (65, 1152, 66), (257, 1280, 100),
+                                   # the ring kernel with one, two and three stages in all (which stage buffers are free for the
+                                   # wavefronts' own epilogue depends on the count)
+                                   (200, 128, 136), (300, 256, 264), (129, 384, 72),
                                    # all-in-flight decode kernel: runs of four channels stored with the scales fetched first
                                    (8, 4096, 264), (16, 2048, 4104), (27, 4096, 134), (5, 6144, 70)])
 @pytest.mark.parametrize("with_bias", [False, True])
