@@ -533,7 +533,7 @@ def main() -> int:
         # int8 weight-only decode (next-row op _weight_int8pack_mm): same shape, one byte per weight
         w8s = [torch.randint(-128, 128, (N, K), dtype=torch.int8, device=dev) for _ in range(14)]  # 631 MB
         s8 = torch.rand(N, device=dev) * 0.01
-        for mb in (1, 8):
+        for mb in (1, 8, 32):
             xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
             yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
 
