@@ -522,51 +522,76 @@ __global__ __launch_bounds__(KSPLIT == 1 ? 256 : 512) void int8_gemm_dma_kernel(
     // ---- epilogue ------------------------------------------------------------------------------------
     TPQ_DMA_STAMP(3);
     const bool has_bias = tile.bias != nullptr;
-    if constexpr (KSPLIT == 0 && sizeof(out_t) == 2) if ((vector_stores & 2) == 0) {
+    if constexpr (KSPLIT == 0) if ((vector_stores & 2) == 0) {
         // Every wavefront finishes its own 64 x 64 block, without a barrier: the two stage buffers that do not hold
         // the last stage are free since the last barrier of the main loop (every wavefront had finished reading them
         // and every direct load had landed), so each wavefront turns its block into row order in 12 KB of its own
-        // there and stores it itself, 16 bytes per lane, eight whole 128-byte lines per store.
+        // there and stores it itself, 16 bytes per lane, whole 128-byte lines.  16-bit outputs: all 64 rows at once;
+        // 32-bit outputs (the partial sums of a sliced launch, float32): two passes of 32 rows through the same 12 KB.
         const int last = slot == 0 ? kDmaStages - 1 : slot - 1;  // buffer of the last stage (slot was advanced past it)
         const int mine = wave < 4 ? (last == 0 ? 1 : 0) : (last == 2 ? 1 : 2);
-        constexpr int kWavePitch = WN * 2 + 16;  // bytes per row of the wavefront's image
-        static_assert(4 * 12288 <= kStageBytes && WM * kWavePitch <= 12288, "four wavefronts per free buffer");
+        constexpr int kElem = sizeof(out_t);
+        constexpr int kPassBlocks = kElem == 2 ? TM : 1;             // 32-row blocks per pass
+        constexpr int kWavePitch = WN * kElem + 16;                  // bytes per row of the wavefront's image
+        constexpr int kRowChunks = WN * kElem / 16;                  // 16-byte chunks per row: 8 or 16
+        constexpr int kRowsPerStore = kWave / kRowChunks;            // rows per wavefront store: 8 or 4
+        static_assert(4 * 12288 <= kStageBytes && kPassBlocks * 32 * kWavePitch <= 12288, "four wavefronts per free buffer");
         char* img = lds_bytes + mine * kStageBytes + (wave & 3) * 12288;
-        float rs_r[TM];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) rs_r[i] = rs_lds[wm * WM + i * 32 + frag_row];
+        for (int first = 0; first < TM; first += kPassBlocks) {
+            float rs_r[kPassBlocks];
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int i = 0; i < kPassBlocks; ++i) rs_r[i] = Tile::kScaled ? rs_lds[wm * WM + (first + i) * 32 + frag_row] : 0.0f;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n_wave = j * 32 + 8 * q + 4 * frag_half;  // 4 consecutive columns of the wavefront's 64
-                const float4 c = *reinterpret_cast<const float4*>(cs_lds + wn * WN + n_wave);
-                const float4 b = *reinterpret_cast<const float4*>(cs_lds + BN + wn * WN + n_wave);
-                const float c4[4] = {c.x, c.y, c.z, c.w}, b4[4] = {b.x, b.y, b.z, b.w};
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    float f[4];
+                for (int q = 0; q < 4; ++q) {
+                    const int n_wave = j * 32 + 8 * q + 4 * frag_half;  // 4 consecutive columns of the wavefront's 64
+                    float c4[4] = {0, 0, 0, 0}, b4[4] = {0, 0, 0, 0};
+                    if (Tile::kScaled) {
+                        const float4 c = *reinterpret_cast<const float4*>(cs_lds + wn * WN + n_wave);
+                        const float4 b = *reinterpret_cast<const float4*>(cs_lds + BN + wn * WN + n_wave);
+                        c4[0] = c.x; c4[1] = c.y; c4[2] = c.z; c4[3] = c.w;
+                        b4[0] = b.x; b4[1] = b.y; b4[2] = b.z; b4[3] = b.w;
+                    }
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) f[t] = Tile::value(acc[i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
-                    *reinterpret_cast<uint2*>(img + (i * 32 + frag_row) * kWavePitch + n_wave * 2) =
-                        make_uint2(Tile::pack2(f[0], f[1]), Tile::pack2(f[2], f[3]));
+                    for (int i = 0; i < kPassBlocks; ++i) {
+                        char* dst = img + (i * 32 + frag_row) * kWavePitch + n_wave * kElem;
+                        if constexpr (kElem == 2) {
+                            float f[4];
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) f[t] = Tile::value(acc[first + i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
+                            *reinterpret_cast<uint2*>(dst) = make_uint2(Tile::pack2(f[0], f[1]), Tile::pack2(f[2], f[3]));
+                        } else {
+                            out_t vals[4];
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) vals[t] = Tile::convert(acc[first + i][j][4 * q + t], rs_r[i], c4[t], b4[t], has_bias);
+                            *reinterpret_cast<uint4*>(dst) = make_uint4(__builtin_bit_cast(uint32_t, vals[0]), __builtin_bit_cast(uint32_t, vals[1]),
+                                                                        __builtin_bit_cast(uint32_t, vals[2]), __builtin_bit_cast(uint32_t, vals[3]));
+                        }
+                    }
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's own LDS writes, in order with its reads
+            if (first == 0) TPQ_DMA_STAMP(5);
+#pragma unroll
+            for (int it = 0; it < kPassBlocks * 32 / kRowsPerStore; ++it) {
+                const int row = it * kRowsPerStore + lane / kRowChunks, col = (lane % kRowChunks) * (16 / kElem);
+                const int m = m0 + wm * WM + first * 32 + row, n = n0 + wn * WN + col;
+                const uint4 v = *reinterpret_cast<const uint4*>(img + row * kWavePitch + col * kElem);
+                if (m >= M || n >= N) continue;
+                out_t* dstp = tile.out + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
+                if ((vector_stores & 1) && n + 16 / kElem <= N) {
+                    nt_store(reinterpret_cast<uint4*>(dstp), v);  // written once, read by a later kernel
+                } else {
+                    const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+                    if constexpr (kElem == 2) {
+                        for (int e = 0; e < 8 && n + e < N; ++e) dstp[e] = static_cast<out_t>(words[e >> 1] >> (16 * (e & 1)));
+                    } else {
+                        for (int e = 0; e < 4 && n + e < N; ++e) dstp[e] = __builtin_bit_cast(out_t, words[e]);
+                    }
                 }
             }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wavefront's own LDS writes, in order with its reads
-        TPQ_DMA_STAMP(5);
-#pragma unroll
-        for (int it = 0; it < WM / 8; ++it) {
-            const int row = it * 8 + (lane >> 3), col = (lane & 7) * 8;
-            const int m = m0 + wm * WM + row, n = n0 + wn * WN + col;
-            const uint4 v = *reinterpret_cast<const uint4*>(img + row * kWavePitch + col * 2);
-            if (m >= M || n >= N) continue;
-            out_t* dstp = tile.out + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
-            if ((vector_stores & 1) && n + 8 <= N) {
-                nt_store(reinterpret_cast<uint4*>(dstp), v);  // written once, read by a later kernel
-            } else {
-                const uint32_t words[4] = {v.x, v.y, v.z, v.w};
-                for (int e = 0; e < 8 && n + e < N; ++e) dstp[e] = static_cast<out_t>(words[e >> 1] >> (16 * (e & 1)));
-            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the image has been read before the next pass overwrites it
         }
         TPQ_DMA_STAMP(6);
         return;
