@@ -255,16 +255,31 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     TPQ_STAMP(7);
 }
 
-// out = epilogue(sum over the splits), element by element
+// out = epilogue(sum over the splits): a thread takes four consecutive columns of one row (grid.y = row, so no
+// division per element; 16-byte loads of the partial sums, one vector store where the row pitch allows)
 template <class Epilogue>
 __global__ __launch_bounds__(256) void ternary_slab_finish_kernel(const int32_t* __restrict__ partial, int splits, int M, int N, Epilogue ep) {
-    const int64_t total = static_cast<int64_t>(M) * N;
-    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += gridDim.x * 256ll) {
-        int v = 0;
-        for (int s = 0; s < splits; ++s) v += partial[s * total + idx];
-        const int m = static_cast<int>(idx / N), n = static_cast<int>(idx - static_cast<int64_t>(m) * N);
-        ep.store_scaled(idx, v, ep.row_scale_of(m), ep.bias_of(n));
+    const int m = blockIdx.y;
+    const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (n >= N) return;
+    const int count = N - n < 4 ? N - n : 4;
+    const int64_t total = static_cast<int64_t>(M) * N, idx = static_cast<int64_t>(m) * N + n;
+    const bool whole = count == 4 && (N & 3) == 0;  // the partial matrices are 16-byte aligned (launcher) and M N is a multiple of 4
+    const float row_scale = ep.row_scale_of(m);
+    float bias_n[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bias_n[e] = ep.bias_of(e < count ? n + e : n);
+    int v[4] = {0, 0, 0, 0};
+    if (whole) {
+        for (int s = 0; s < splits; ++s) {
+            const int4 q = *reinterpret_cast<const int4*>(partial + s * total + idx);
+            v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
+        }
+    } else {
+        for (int s = 0; s < splits; ++s)
+            for (int e = 0; e < count; ++e) v[e] += partial[s * total + idx + e];
     }
+    ep.store_scaled_run(idx, v, row_scale, bias_n, count, whole && ep.runs_aligned());
 }
 
 // Splits of K for the slab kernel (1: no workspace needed); 0 when the kernel does not take the shape.
@@ -309,8 +324,8 @@ int launch_ternary_slab(const int8_t* x, const uint8_t* packed, int64_t M, int64
         static_cast<int>(m_tiles), static_cast<int>(n_tiles), splits, splits > 1 ? partial : nullptr, ep);
     if (int rc = check_launch("tpq_ternary_mm (slab)")) return rc;
     if (splits > 1) {
-        const int64_t blocks = (M * N + 255) / 256;
-        ternary_slab_finish_kernel<Epilogue><<<static_cast<unsigned>(blocks > 2048 ? 2048 : blocks), 256, 0, s>>>(
+        TPQ_REQUIRE(M <= 65535, TPQ_ERR_INVALID_VALUE, "ternary slab: too many rows for the finishing launch");
+        ternary_slab_finish_kernel<Epilogue><<<dim3(static_cast<unsigned>((N + 1023) / 1024), static_cast<unsigned>(M)), 256, 0, s>>>(
             partial, splits, static_cast<int>(M), static_cast<int>(N), ep);
         return check_launch("tpq_ternary_mm (slab, finish)");
     }
