@@ -49,21 +49,33 @@ __global__ __launch_bounds__(256) void int8_finish_kernel(const int32_t* __restr
                                                           typename Elem<DT>::storage* __restrict__ out, int64_t M, int64_t N) {
     const int64_t total = M * N, stride = static_cast<int64_t>(gridDim.x) * 256;
     const bool has_bias = bias != nullptr;
-    if (N % 4 == 0) {  // four consecutive columns of one row per thread
-        for (int64_t q = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; q < total / 4; q += stride) {
-            const int64_t idx = q * 4, m = idx / N, n = idx - m * N;
-            int4 v = make_int4(0, 0, 0, 0);
-            for (int z = 0; z < slices; ++z) {
-                const uint4 p = nt_load(reinterpret_cast<const uint4*>(partial + z * total + idx));
-                v.x += static_cast<int>(p.x); v.y += static_cast<int>(p.y); v.z += static_cast<int>(p.z); v.w += static_cast<int>(p.w);
+    if (N % 4 == 0) {  // four consecutive columns of one row per thread; grid.y walks the rows, so nothing is divided
+        const bool vector_out = (reinterpret_cast<uintptr_t>(out) & (4 * sizeof(typename Elem<DT>::storage) - 1)) == 0;
+        for (int64_t m = blockIdx.y; m < M; m += gridDim.y) {
+            for (int64_t n = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4; n < N; n += stride * 4) {
+                const int64_t idx = m * N + n;
+                // the scales first: they are not behind the partial sums when those arrive
+                const float4 c = *reinterpret_cast<const float4*>(cs + n);
+                const float4 b = has_bias ? *reinterpret_cast<const float4*>(bias + n) : make_float4(0, 0, 0, 0);
+                const float r = rs[m];
+                int4 v = make_int4(0, 0, 0, 0);
+                for (int z = 0; z < slices; ++z) {
+                    const uint4 p = nt_load(reinterpret_cast<const uint4*>(partial + z * total + idx));
+                    v.x += static_cast<int>(p.x); v.y += static_cast<int>(p.y); v.z += static_cast<int>(p.z); v.w += static_cast<int>(p.w);
+                }
+                const typename Elem<DT>::storage o[4] = {TileDequant<DT>::convert(v.x, r, c.x, b.x, has_bias), TileDequant<DT>::convert(v.y, r, c.y, b.y, has_bias),
+                                                        TileDequant<DT>::convert(v.z, r, c.z, b.z, has_bias), TileDequant<DT>::convert(v.w, r, c.w, b.w, has_bias)};
+                if (vector_out) {
+                    if constexpr (sizeof(typename Elem<DT>::storage) == 2) {
+                        *reinterpret_cast<uint2*>(out + idx) = make_uint2(static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16),
+                                                                          static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16));
+                    } else {
+                        *reinterpret_cast<float4*>(out + idx) = make_float4(o[0], o[1], o[2], o[3]);
+                    }
+                } else {
+                    out[idx] = o[0]; out[idx + 1] = o[1]; out[idx + 2] = o[2]; out[idx + 3] = o[3];
+                }
             }
-            const float4 c = *reinterpret_cast<const float4*>(cs + n);
-            const float4 b = has_bias ? *reinterpret_cast<const float4*>(bias + n) : make_float4(0, 0, 0, 0);
-            const float r = rs[m];
-            out[idx] = TileDequant<DT>::convert(v.x, r, c.x, b.x, has_bias);
-            out[idx + 1] = TileDequant<DT>::convert(v.y, r, c.y, b.y, has_bias);
-            out[idx + 2] = TileDequant<DT>::convert(v.z, r, c.z, b.z, has_bias);
-            out[idx + 3] = TileDequant<DT>::convert(v.w, r, c.w, b.w, has_bias);
         }
         return;
     }
@@ -238,9 +250,10 @@ TPQ_EXPORT int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const fl
     hipStream_t s = static_cast<hipStream_t>(stream);
     int32_t* acc = static_cast<int32_t*>(workspace);  // [slices][M][N]; M N % 4 == 0 keeps every matrix 16-byte aligned
     if (int rc = launch_dma_sliced(a, w, M, N, K, acc, slices, s)) return rc;
-    const int64_t items = N % 4 == 0 ? M * N / 4 : M * N;
+    // N % 4 == 0: grid.x over the row's groups of four columns, grid.y over the rows; else a flat grid
+    const int64_t items = N % 4 == 0 ? N / 4 : M * N;
     const int64_t blocks = (items + 255) / 256;
-    const unsigned grid = static_cast<unsigned>(blocks > 4096 ? 4096 : blocks);
+    const dim3 grid(static_cast<unsigned>(blocks > 4096 ? 4096 : blocks), N % 4 == 0 ? static_cast<unsigned>(M > 65535 ? 65535 : M) : 1u);
     switch (out_dtype) {
         case TPQ_DTYPE_F32: int8_finish_kernel<TPQ_DTYPE_F32><<<grid, 256, 0, s>>>(acc, slices, row_scale, col_scale, bias, static_cast<float*>(out), M, N); break;
         case TPQ_DTYPE_F16: int8_finish_kernel<TPQ_DTYPE_F16><<<grid, 256, 0, s>>>(acc, slices, row_scale, col_scale, bias, static_cast<uint16_t*>(out), M, N); break;
