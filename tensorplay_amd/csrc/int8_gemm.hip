@@ -5,7 +5,7 @@
 #include <type_traits>
 
 #include "int8_decode_kernel.h"
-#include "int8_gemm_dma.h"
+#include "int8_gemm_stagger.h"
 
 namespace tpq {
 namespace {
@@ -112,7 +112,7 @@ int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t 
         return launch_int8_decode(a, w, M, N, K, ep, [N](const Epilogue& e, int64_t m0) { return rebase_rows(e, m0, N); }, s);
     // The ring-buffered kernel also wins when its 256 x 128 tiles fill only part of the chip: at K = N = 4096,
     // M = 512 / 1024 it takes 27.9 / 29.5 us against 33.9 / 39.4 us for the register-staged kernel on 128 x 64 tiles.
-    if (dma_path_ok(M, N, K) && !(force && force[0] == 'r')) return launch_dma(a, w, M, N, K, to_tile(ep), s);
+    if (dma_path_ok(M, N, K) && !(force && force[0] == 'r')) return launch_tiled(a, w, M, N, K, to_tile(ep), s);
     return launch_mfma(a, w, M, N, K, ep, s);
 }
 
@@ -249,7 +249,7 @@ TPQ_EXPORT int tpq_int8_mm_dequant_ws(const int8_t* a, const int8_t* w, const fl
     TPQ_REQUIRE(out && row_scale && col_scale, TPQ_ERR_INVALID_VALUE, "int8_mm_dequant: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     int32_t* acc = static_cast<int32_t*>(workspace);  // [slices][M][N]; M N % 4 == 0 keeps every matrix 16-byte aligned
-    if (int rc = launch_dma_sliced(a, w, M, N, K, acc, slices, s)) return rc;
+    if (int rc = launch_tiled_sliced(a, w, M, N, K, acc, slices, s)) return rc;
     // N % 4 == 0: grid.x over the row's groups of four columns, grid.y over the rows; else a flat grid
     const int64_t items = N % 4 == 0 ? N / 4 : M * N;
     const int64_t blocks = (items + 255) / 256;
@@ -271,7 +271,7 @@ TPQ_EXPORT int tpq_int_mm_ws(const void* a, int a_unsigned, const int8_t* b, int
         return tpq_int_mm(a, a_unsigned, b, b_stride_k, b_stride_n, c, M, K, N, stream);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int32_t* partial = static_cast<int32_t*>(workspace);
-    if (int rc = launch_dma_sliced(static_cast<const int8_t*>(a), b, M, N, K, partial, slices, s)) return rc;
+    if (int rc = launch_tiled_sliced(static_cast<const int8_t*>(a), b, M, N, K, partial, slices, s)) return rc;
     const int64_t blocks = (M * N / 4 + 255) / 256;
     int32_sum_slices_kernel<<<static_cast<unsigned>(blocks > 4096 ? 4096 : blocks), 256, 0, s>>>(partial, slices, c, M * N);
     return check_launch("_int_mm (sum of slices)");
