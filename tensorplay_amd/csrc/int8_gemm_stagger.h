@@ -1,30 +1,40 @@
 // int8 GEMM, staggered form: 256 x 128 tile per workgroup, three-stage LDS ring of whole 128-byte rows filled by
-// direct global -> LDS loads, eight multiplying wavefronts in eight positions of 64 x 64 (v_mfma_i32_16x16x64_i8),
-// the two wavefronts of a SIMD half a stage apart.
+// direct global -> LDS loads, eight wavefronts in eight positions of 64 x 64 (v_mfma_i32_16x16x64_i8), the two
+// wavefronts of a SIMD half a stage apart.
 //
-// Why this form.  Measured on MI355X at 2048 x 4096 x 4096: the matrix cores need 1024 clocks per stage, the vector
-// memory path 1040 (48 wave-level loads of 1 KB at one per ~21.6 clocks and compute unit), so both have to run all the
-// time.  Two things kept the lock-step kernel at 1450 - 1490 clocks per stage.  (i) A SIMD issues matrix and vector
-// ALU instructions through one port and serves the older wavefront first: while MFMAs are issued back to back, every
-// vector instruction of another wavefront (the address arithmetic of a fragment read or of a direct load) waits for a
-// gap, and a wavefront that mixes them with its own MFMAs delays those.  (ii) A direct load blocks the wavefront
-// that issues it until the memory path accepts it, and with it every MFMA behind it in program order.  So here
+// What the form answers (measured on MI355X at 2048 x 4096 x 4096, per stage of 128 bytes of k and compute unit): the
+// matrix cores need 1024 - 1090 clocks, the vector memory path 1040 (48 wave-level loads of 1 KB, one per ~21.6
+// clocks), so both have to run all the time; the lock-step kernel (int8_gemm_dma.h) took 1450 - 1490.  Found:
+//  (i)   A SIMD issues matrix and vector ALU instructions through one port, older wavefront first.  While one
+//        wavefront issues MFMAs back to back, every vector instruction of another one (the address arithmetic of a
+//        fragment read or of a direct load) waits for a gap; a wavefront that mixes them with its own MFMAs delays
+//        those.  (Two loading wavefronts beside two multiplying ones on a SIMD: the MFMAs kept their rate, the loads
+//        dropped to a third of theirs.)
+//  (ii)  A direct load blocks the wavefront that issues it until the memory path accepts it, and with it every MFMA
+//        behind it in program order.
+//  (iii) The chip runs this kernel at its power limit (random operands: 1.4 - 1.7 GHz of 2.4), so time follows energy
+//        more than clocks.  v_mfma_i32_16x16x64_i8 reads and writes a quarter of the accumulator registers of
+//        v_mfma_i32_32x32x32_i8 per multiply-add and sustains 4.1 POPS alone where that one sustains 3.5.
+// So:
 //   - a wavefront alternates between a multiply phase (the 32 MFMAs of a stage, all fragments already in registers,
-//     nothing else) and a memory phase (the 16 fragment reads of its next stage, and its share of the requests), with a
+//     nothing else) and a memory phase (the 16 fragment reads of its next stage and its six direct loads), with a
 //     workgroup barrier at the end of every phase; wavefronts 0..3 multiply in the even phases, 4..7 in the odd ones,
-//     so every SIMD always has one wavefront whose MFMAs wait for nothing;
+//     so every SIMD always has one wavefront whose MFMAs wait for nothing.  (One barrier per stage and no forced
+//     alternation was measured too: the multiply phases of a SIMD's two wavefronts drift together, + 4 %.)
 //   - the memory phase contains no vector ALU instruction: fragment addresses are 12 registers computed once (per
 //     ring slot, operand and k-half; the loop is unrolled three times so that the slot is a constant), and the
 //     direct loads take a scalar base (advanced per stage by scalar instructions) plus a per-lane 32-bit offset that
-//     never changes.
+//     never changes.  The loads are spread between the reads, so the memory path has work from the start of a phase.
 //
 // Ring protocol (stage t lives in slot t % 3).  Group 0 reads stage t in phase 2t - 1, group 1 in phase 2t; the
-// barrier that ends phase 2t frees the slot.  With LOADERS = 0 every wavefront requests its sixth of a stage in its
-// own memory phase: group 0 requests stage t + 3 in phase 2t + 1, group 1 requests stage t + 2 in phase 2t (the slot
-// of stage t - 1).  With LOADERS = 4 four extra wavefronts (one per SIMD) do nothing but request: loads 0..5 of
-// stage u + 2 in phase 2u - 1, loads 6..11 in phase 2u.  A stage must have landed when the barrier that ends phase
-// 2t - 2 is crossed; each requesting wavefront waits for its own share in front of that barrier (vector loads of
-// a wavefront complete in order).  All wavefronts cross the same number of barriers: 2 nk - 1 after the first.
+// barrier that ends phase 2t frees the slot.  Every wavefront requests its sixth of a stage in its own memory phase:
+// group 0 requests stage t + 3 in phase 2t + 1, group 1 requests stage t + 2 in phase 2t (into the slot of stage
+// t - 1).  A stage must have landed when the barrier that ends phase 2t - 2 is crossed; each wavefront waits for its own
+// share in front of that barrier (vector loads of a wavefront complete in order, so "my share of t + 1 has landed" is
+// "at most the six loads of t + 2 are outstanding").  Both groups cross 2 nk - 1 barriers after the first.
+//
+// Four extra wavefronts that do nothing but request (one per SIMD, 168 registers per wavefront) were built and measured:
+// the loop drops from 1085 to 1064 clocks per stage, the first stage arrives 1000 clocks later, same time; not kept.
 //
 // Requires K % 128 == 0, K < 2^23 and 16-byte aligned operands.  Edges in M and N: source rows are clamped, stores masked.
 #pragma once
@@ -39,15 +49,10 @@ namespace {
 #endif
 constexpr int kPhasePrio = TPQ_PHASE_PRIO;  // wavefront priority during a multiply phase
 
-#ifndef TPQ_STAGGER_MID_BARRIER
-#define TPQ_STAGGER_MID_BARRIER 1
-#endif
-constexpr bool kMidBarrier = TPQ_STAGGER_MID_BARRIER != 0;  // a second barrier per stage, between the two phases
-
 #if defined(TPQ_DMA_STAMPS) && TPQ_DMA_STAMPS >= 2
 #define TPQ_STAGGER_PHASE_STAMPS 1
-__device__ unsigned long long g_stagger_stamps[12 * 128];  // [wavefront][phase][arrival at the barrier, departure]
-constexpr int kStaggerStampBytes = 12 * 128 * 8;
+__device__ unsigned long long g_stagger_stamps[8 * 128];  // [wavefront][phase][arrival at the barrier, departure]
+constexpr int kStaggerStampBytes = 8 * 128 * 8;
 #else
 constexpr int kStaggerStampBytes = 0;
 #endif
@@ -58,16 +63,15 @@ __device__ unsigned long long g_stagger_coarse[4 * 8];  // [start, first barrier
 #define TPQ_STAGGER_STAMP(I) do { } while (0)
 #endif
 
-template <class Tile, int LOADERS>
-__global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, int M,
+template <class Tile>
+__global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, int M,
                                                                               int N, int K, Tile tile, int vector_stores, int slices) {
     using out_t = typename Tile::out_t;
-    static_assert(LOADERS == 0 || LOADERS == 4, "requests come from the multiplying wavefronts or from four extra ones");
     constexpr int BM = 256, BN = 128, WM = 64, WN = 64;
     constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;  // 48 KB
     constexpr int kRingBytes = kDmaStages * kStageBytes;   // 144 KB
-    constexpr int kRequesters = LOADERS ? LOADERS : 8;
-    constexpr int kLoadsA = BM / 8 / kRequesters, kLoadsW = BN / 8 / kRequesters, kLoads = kLoadsA + kLoadsW;  // 4 + 2, or 8 + 4
+    constexpr int kRequesters = 8;
+    constexpr int kLoadsA = BM / 8 / kRequesters, kLoadsW = BN / 8 / kRequesters, kLoads = kLoadsA + kLoadsW;  // 4 + 2
     extern __shared__ uint4 ring[];
     char* lds_bytes = reinterpret_cast<char*>(ring);
     float* cs_lds = reinterpret_cast<float*>(lds_bytes + kRingBytes);  // [BN] column scales, [BN] bias, [BM] row scales
@@ -100,11 +104,10 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
     const int nk = nk_all - kt0 < nk_slice ? nk_all - kt0 : nk_slice;
 
     // ---- requests -----------------------------------------------------------------------------------------------
-    // Requester r (wavefront r, or wavefront 8 + r) owns row blocks of eight rows: kLoadsA of the activations, kLoadsW of
+    // Wavefront r owns row blocks of eight rows: kLoadsA of the activations, kLoadsW of
     // the weights.  Load i of a requester fills 1 KB of the stage: lane l fetches the 16-byte chunk that belongs in
     // slot l % 8 of row l / 8 (the swizzle of the fragment reads is applied on the global side).
-    const bool requests = LOADERS ? wave >= 8 : true;
-    const int rq = LOADERS ? (wave & 3) : wave;
+    const int rq = wave;
     uint32_t voff[kLoads];            // byte offset of this lane's chunk from the tile's first row, k = 0
     uint32_t lds_of_load[kLoads];     // byte offset of the load's 1 KB inside a stage (wave-uniform)
 #pragma unroll
@@ -143,8 +146,7 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
     constexpr std::integral_constant<int, 1> c1{};
     constexpr std::integral_constant<int, 2> c2{};
     constexpr std::integral_constant<int, kLoads> cAll{};
-    constexpr std::integral_constant<int, kLoads / 2> cHalf{};
-    auto request_stage = [&](auto slot_c, int kt) { request(c0, cAll, slot_c, kt); };
+        auto request_stage = [&](auto slot_c, int kt) { request(c0, cAll, slot_c, kt); };
 
     // ---- fragment reads -----------------------------------------------------------------------------------------
     // v_mfma_i32_16x16x64_i8: lane (r = lane % 16, c = lane / 16) holds row r, 16-byte chunk c of a k-half of 64 bytes.
@@ -164,10 +166,10 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
             addr_b[s][kh] = ring_addr + s * kStageBytes + (BM + wn * WN + frag_row) * kDmaRowBytes + chunk;
         }
     v4i fa[2][4], fb[2][4];  // [k-half][block of 16 rows]
-    auto read_stage = [&](auto slot_c) {
+    auto read_half = [&](auto slot_c, auto half_c) {
         constexpr int SLOT = decltype(slot_c)::value;
 #pragma unroll
-        for (int kh = 0; kh < 2; ++kh) {
+        for (int kh = decltype(half_c)::value; kh < decltype(half_c)::value + 1; ++kh) {
             const uint32_t aa = addr_a[SLOT][kh], ab = addr_b[SLOT][kh];
             // (an array element as an asm operand inside a generic lambda does not compile: references)
             v4i &a0 = fa[kh][0], &a1 = fa[kh][1], &a2 = fa[kh][2], &a3 = fa[kh][3], &b0 = fb[kh][0], &b1 = fb[kh][1], &b2 = fb[kh][2], &b3 = fb[kh][3];
@@ -179,6 +181,28 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
             asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(b2) : "v"(ab) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(a3) : "v"(aa) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(b3) : "v"(ab) : "memory");
+        }
+    };
+    auto read_stage = [&](auto slot_c) {
+        read_half(slot_c, std::integral_constant<int, 0>{});
+        read_half(slot_c, std::integral_constant<int, 1>{});
+    };
+#ifndef TPQ_STAGGER_INTERLEAVE
+#define TPQ_STAGGER_INTERLEAVE 1
+#endif
+    // memory phase of a wavefront that also requests: TPQ_STAGGER_INTERLEAVE 0: the reads, then the requests; 1: a third
+    // of the requests ahead of each half of the reads and behind them, so that the memory path has work from the start
+    auto read_and_request = [&](auto read_slot, auto fill_slot, int kt_new) {
+        if constexpr (TPQ_STAGGER_INTERLEAVE == 0) {
+            read_stage(read_slot);
+            request_stage(fill_slot, kt_new);
+        } else {
+            constexpr std::integral_constant<int, kLoads / 3> third{};
+            request(std::integral_constant<int, 0>{}, third, fill_slot, kt_new);
+            read_half(read_slot, std::integral_constant<int, 0>{});
+            request(third, third, fill_slot, kt_new);
+            read_half(read_slot, std::integral_constant<int, 1>{});
+            request(std::integral_constant<int, 2 * (kLoads / 3)>{}, third, fill_slot, kt_new);
         }
     };
     auto stage_ready = [&]() {  // every fragment read has delivered; the MFMAs that use them stay behind this point
@@ -247,8 +271,8 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
     // The scales of the tile go to LDS by direct loads as well (64 floats per wave-level load, source index clamped at the
     // edges), ahead of the stages in every requesting wavefront's order, so the wait for stage 0 covers them; nothing
     // here is a load the compiler counts, so it inserts no wait of its own in front of the first barrier.
-    if (Tile::kScaled && requests) {
-        // eight pieces of 64 floats: column scales 0..1, bias 2..3, row scales 4..7; one per wavefront, or two per loader
+    if (Tile::kScaled) {
+        // eight pieces of 64 floats: column scales 0..1, bias 2..3, row scales 4..7; one per wavefront
         constexpr int kPieces = 8 / kRequesters;
 #pragma unroll
         for (int e = 0; e < kPieces; ++e) {
@@ -262,11 +286,9 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
             if (src != nullptr) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(src) : "memory", "m0");
         }
     }
-    if (requests) {
-        request_stage(c0, 0);
-        if (nk > 1) request_stage(c1, 1);
-        if (nk > 2) request_stage(c2, 2);
-    }
+    request_stage(c0, 0);
+    if (nk > 1) request_stage(c1, 1);
+    if (nk > 2) request_stage(c2, 2);
     if (nk > 2) wait_loads(kTwoStages);
     else if (nk > 1) wait_loads(kOneStage);
     else wait_loads(c0);
@@ -279,81 +301,34 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
         constexpr int SLOT = decltype(slot_c)::value, NEXT = (SLOT + 1) % kDmaStages;
         constexpr bool STEADY = decltype(steady)::value;
         multiply_stage();
-        if constexpr (LOADERS == 0) {  // own share of kt + 1 landed (kt + 2 may be in flight)
-            if (STEADY || kt + 2 < nk) wait_loads(kOneStage);
-            else wait_loads(c0);
-        }
+        if (STEADY || kt + 2 < nk) wait_loads(kOneStage);  // own share of kt + 1 landed (kt + 2 may be in flight)
+        else wait_loads(c0);
         phase_end();
         if (STEADY || kt + 1 < nk) {
-            read_stage(std::integral_constant<int, NEXT>{});
-            if constexpr (LOADERS == 0) {
-                if (STEADY || kt + kDmaStages < nk) request_stage(slot_c, kt + kDmaStages);
-            }
+            if (STEADY || kt + kDmaStages < nk) read_and_request(std::integral_constant<int, NEXT>{}, slot_c, kt + kDmaStages);
+            else read_stage(std::integral_constant<int, NEXT>{});
             stage_ready();
-            if constexpr (kMidBarrier) phase_end();
+            phase_end();
         }
     };
     // group 1: read kt, request kt + 2 into the slot of kt - 1 | multiply kt
     auto group1_step = [&](auto slot_c, auto steady, int kt) {
         constexpr int SLOT = decltype(slot_c)::value, PREV = (SLOT + kDmaStages - 1) % kDmaStages;
         constexpr bool STEADY = decltype(steady)::value;
-        read_stage(slot_c);
-        if constexpr (LOADERS == 0) {
-            if (STEADY || (kt >= 1 && kt + 2 < nk)) request_stage(std::integral_constant<int, PREV>{}, kt + 2);
-        }
+        if (STEADY || (kt >= 1 && kt + 2 < nk)) read_and_request(slot_c, std::integral_constant<int, PREV>{}, kt + 2);
+        else read_stage(slot_c);
         stage_ready();
-        if constexpr (LOADERS == 0) {  // own share of kt + 1 landed (kt + 2 may be in flight)
-            if (STEADY || kt + 2 < nk) wait_loads(kOneStage);
-            else wait_loads(c0);
-        }
+        if (STEADY || kt + 2 < nk) wait_loads(kOneStage);  // own share of kt + 1 landed (kt + 2 may be in flight)
+        else wait_loads(c0);
         phase_end();
         multiply_stage();
-        if constexpr (kMidBarrier) {
-            if (STEADY || kt + 1 < nk) phase_end();
-        }
+        if (STEADY || kt + 1 < nk) phase_end();
     };
     constexpr std::true_type kSteady{};
     constexpr std::false_type kChecked{};
 
     int kt = 0;
-    if (LOADERS != 0 && wave >= 8) {
-        // requesting wavefronts: phase 0, then per stage u >= 1 the phases 2u - 1 (loads 0 .. of stage u + 2 into the
-        // slot of stage u - 1) and 2u (the other half; own share of stage u + 1 landed)
-        if (nk > 2) wait_loads(kOneStage);
-        else wait_loads(c0);
-        phase_end();
-        auto loader_step = [&](auto free_slot, auto steady, int u) {
-            constexpr bool STEADY = decltype(steady)::value;
-            if (STEADY || u + 2 < nk) request(c0, cHalf, free_slot, u + 2);
-            if constexpr (kMidBarrier) phase_end();
-            if (STEADY || u + 2 < nk) {
-                request(cHalf, cHalf, free_slot, u + 2);
-                wait_loads(kOneStage);
-            } else {
-                wait_loads(c0);
-            }
-            phase_end();
-        };
-        int u = 1;
-        for (; u + 4 < nk; u += 3) {
-            loader_step(c0, kSteady, u);
-            loader_step(c1, kSteady, u + 1);
-            loader_step(c2, kSteady, u + 2);
-        }
-        // at most four stages left, the first with slot 0 free: straight-line code, nested, so that no step sits in a
-        // branch of a loop (the register allocator then copies the accumulators around at every join)
-        if (u < nk) {
-            loader_step(c0, kChecked, u);
-            if (u + 1 < nk) {
-                loader_step(c1, kChecked, u + 1);
-                if (u + 2 < nk) {
-                    loader_step(c2, kChecked, u + 2);
-                    if (u + 3 < nk) loader_step(c0, kChecked, u + 3);
-                }
-            }
-        }
-        return;
-    } else if (wave < 4) {
+    if (wave < 4) {
         read_stage(c0);
         stage_ready();
         for (; kt + 2 + kDmaStages < nk; kt += 3) {
@@ -470,28 +445,32 @@ __global__ __launch_bounds__(512 + 64 * LOADERS) void int8_gemm_stagger_kernel(c
     TPQ_STAGGER_STAMP(3);
 }
 
-template <int LOADERS, class Tile>
+template <class Tile>
 int launch_stagger(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
     constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + (2 * 128 + 256) * sizeof(float) + kStaggerStampBytes;
     const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
     TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
     TPQ_REQUIRE(K % kDmaRowBytes == 0 && K < (1 << 23), TPQ_ERR_INVALID_VALUE, "int8 gemm (staggered): K must be a multiple of 128 below 2^23");
-    auto kernel = int8_gemm_stagger_kernel<Tile, LOADERS>;
+    auto kernel = int8_gemm_stagger_kernel<Tile>;
     static std::atomic<uint64_t> configured{0};  // per instantiation
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int8 gemm")) return rc;
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
-    kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), 512 + 64 * LOADERS, smem, s>>>(
+    kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), 512, smem, s>>>(
         a, w, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), tile, vector_stores, slices);
     return check_launch("int8 mfma gemm (staggered)");
 }
 
-// Which tiled kernel runs a shape.  TPQ_INT8_FORM = dma in a tuning build keeps the lock-step kernel (comparison runs).
+// Which tiled kernel runs a shape.  Measured against the lock-step kernel with the same result bits (us, lock-step /
+// staggered): 2048 x 4096 x 4096 35.9 / 29.0, 2048 x 11008 x 4096 105 / 93, 2048 x 4096 x 11008 91 / 72, 8192^3 550 / 437,
+// 2048 x 2560 x 6912 44.5 / 35.0, 4096 x 4096 x 512 18.0 / 16.2.  Launches whose k range is cut into slices (few stages
+// per workgroup, 32-bit partial sums out) gain nothing from it (128 .. 1024 rows of 4096 x 4096: equal; 256 x 8192 x
+// 8192: 34.2 / 37.5) and stay on the lock-step kernel.  TPQ_INT8_FORM = dma / stagger in a tuning build forces one.
 template <class Tile>
 int launch_tiled(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
     const char* env = tuning_env("TPQ_INT8_FORM");
     if (K >= (1 << 23) || (env && env[0] == 'd')) return launch_dma(a, w, M, N, K, tile, s, slices);
-    if (env && env[0] == 'l') return launch_stagger<4>(a, w, M, N, K, tile, s, slices);
-    return launch_stagger<0>(a, w, M, N, K, tile, s, slices);
+    if (slices > 1 && !(env && env[0] == 's')) return launch_dma(a, w, M, N, K, tile, s, slices);
+    return launch_stagger(a, w, M, N, K, tile, s, slices);
 }
 
 // partial [slices][M][N] int32 (16-byte aligned) := the slices of A W^T
