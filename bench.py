@@ -99,6 +99,21 @@ def graph_of(fn):
     return g
 
 
+def load_probe():
+    """The pure-read measurement probe: a library of its own (tensorplay_amd/csrc/probe.hip), not part of the kernel
+    library's interface."""
+    import ctypes
+
+    from tensorplay_amd import build
+
+    if not os.path.exists(build.PROBE_LIB_PATH):
+        raise RuntimeError(f"{build.PROBE_LIB_PATH} is missing: build it with `python -m tensorplay_amd.build`")
+    lib = ctypes.CDLL(build.PROBE_LIB_PATH)
+    lib.tpq_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.tpq_probe_read.restype = ctypes.c_int
+    return lib
+
+
 def host_description():
     """What the CPU baseline ran on: logical CPUs the OS reports, CPUs this process may use, physical cores, model name
     and the ISA tier that decides the reference's CPU int4 layout (64-column blocks on AVX-512, 32 on AVX2 / plain)."""
@@ -445,6 +460,16 @@ def main() -> int:
     if not args.no_extras:  # the same graph seven more times: median step time
         reps = sorted(time_region(g.replay, sync, 1) / steps for _ in range(7))
         extras["int4_gemv_us_median_of_7_replays"] = reps[3] * 1e3
+        # The K-step graph above carries its own start-up (about half a microsecond per step at 20 steps).  The same
+        # kernel timed the way every other figure here is: a graph of 640 launches, warmed for >= 30 ms, median of 7.
+        gs = graph_of(lambda: [gemv(i) for i in range(10 * copies)])
+        gs.replay(); sync()
+        steady_us = steady(gs.replay, sync) / (10 * copies) * 1e3
+        extras["int4_gemv_steady_us"] = steady_us
+        extras["int4_gemv_steady_GBs"] = GEMV_BYTES / (steady_us * 1e-6) / 1e9
+        extras["int4_gemv_steady_frac_of_hbm_peak"] = GEMV_BYTES / (steady_us * 1e-6) / 1e9 / HBM_PEAK_GBS
+        extras["int4_gemv_steady_launches_per_graph"] = 10 * copies
+        del gs
     if not args.no_extras:
         # The ceiling this kernel is held against: a pure read of the same number of bytes (packed weight + scales and
         # zeros, 23,953,408 B, rotating through the same number of copies so that it comes from HBM), with every compute
@@ -453,11 +478,12 @@ def main() -> int:
         probe_bytes = (N * K // 2 + (K // GROUP) * N * 4) // 1024 * 1024
         probe_bufs = [torch.empty(probe_bytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
         sink = torch.zeros(256, dtype=torch.uint8, device=dev)
+        probe = load_probe()
         best = None
         # (the last shape is the column-per-lane pattern of the decode kernel itself: `contiguous` = K / 128, one workgroup per 64 columns)
         for wg, waves, loads, contiguous in ((256, 8, 4, 0), (256, 8, 12, 0), (256, 16, 8, 1), (512, 4, 12, 0), (1, 16, 8, K // 128)):
             def read(i, wg=wg, waves=waves, loads=loads, contiguous=contiguous):
-                lib.tpq_probe_read(probe_bufs[i % copies].data_ptr(), probe_bytes, wg, waves, loads, contiguous, sink.data_ptr(), cur())
+                probe.tpq_probe_read(probe_bufs[i % copies].data_ptr(), probe_bytes, wg, waves, loads, contiguous, sink.data_ptr(), cur())
 
             gp = graph_of(lambda: [read(i) for i in range(10 * copies)])
             gp.replay(); sync()
@@ -466,13 +492,14 @@ def main() -> int:
                 best = (us, f"column-per-lane pattern, one workgroup of {waves} wavefronts per 64 columns, all loads in flight" if contiguous >= 2 else
                         f"{wg} workgroups x {waves} wavefronts, {loads} KB in flight each, {'contiguous runs' if contiguous else 'interleaved'}")
             del gp
-        ge = graph_of(lambda: [lib.tpq_probe_read(None, 0, 256, 8, 4, 0, sink.data_ptr(), cur()) for _ in range(640)])
+        ge = graph_of(lambda: [probe.tpq_probe_read(None, 0, 256, 8, 4, 0, sink.data_ptr(), cur()) for _ in range(640)])
         ge.replay(); sync()
         extras["empty_kernel_in_graph_us"] = steady(ge.replay, sync) / 640 * 1e3
         extras["int4_gemv_read_ceiling_us"] = best[0]
         extras["int4_gemv_read_ceiling_GBs"] = probe_bytes / (best[0] * 1e-6) / 1e9
         extras["int4_gemv_read_ceiling_pattern"] = best[1]
         extras["int4_gemv_frac_of_read_ceiling"] = best[0] / extras["int4_gemv_us_median_of_7_replays"]
+        extras["int4_gemv_steady_frac_of_read_ceiling"] = best[0] / extras["int4_gemv_steady_us"]
         del probe_bufs, ge
         torch.cuda.empty_cache()
     if args.profile_rows > 0:

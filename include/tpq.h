@@ -41,14 +41,9 @@ int tpq_abi_version(void);
 const char* tpq_last_error(void);
 
 /*
- * Which kernel serves a call is a function of the call's arguments alone; the library never reads the environment.
- * Three routes can be pinned for comparison runs and tests (no counterpart in the reference): "int8_row" (0: the
- * int8 row-streaming kernel never runs, 1: it takes up to four activation rows instead of two; integer sums, so the
- * results are bit-identical either way), "lowbit_row" (0: the packed n-bit row kernel never runs, 1: it runs wherever
- * the shape allows) and "int4_row" (the same for the int4 one-row kernel that deals whole tiles of eight channels to the
- * compute units).  value -1 restores the default rule.  Process-wide, atomic.
+ * Which kernel serves a call is a function of the call's arguments alone; the library never reads the environment and
+ * has no switch that changes a route.
  */
-int tpq_set_kernel_override(const char* route, int value);
 
 /*
  * Fused row-wise signed quantizer.
@@ -248,6 +243,12 @@ int tpq_int4_mm_multi(const void* x, int dtype, int64_t M, int64_t K, int count,
  * the weights and scales the finished fp32 sums of a row, so no launch and no round trip of the activations through
  * memory is spent on the norm; the result differs from the two-step formulation only in where the rounding to T
  * falls and agrees with it to the tolerance of the product (1e-2 relative; 1e-3 against exact sums for float16).
+ * Input range: any finite x and norm_weight of the dtype.  For float16 the product x * norm_weight can leave the
+ * type's range (beyond 65504, or below 6e-5 where it loses its mantissa) although the normalized value does not, so
+ * there every wavefront first scales both factors by exact powers of two taken from its own part of the row (the
+ * scaled products stay within [-4, 4]) and multiplies its fp32 partial sums by the inverse power before they are
+ * added; rows of magnitude 1e-4 .. 1e4 with weights 0.02 .. 30 hold the tolerance row by row.  bfloat16 has
+ * float32's exponent range and needs none of it.
  * Built for K = 2048..8192 (the pair: 2049..4096) at up to 16 rows (the pair: 8); other shapes return
  * TPQ_ERR_UNSUPPORTED and the caller runs the norm and the plain entry point.
  */
@@ -384,18 +385,6 @@ int tpq_lowbit_pack(const uint8_t* codes, int bits, int lsb_first, int64_t rows,
                     uint8_t* packed, void* stream);
 int tpq_lowbit_unpack(const uint8_t* packed, int bits, int lsb_first, int64_t rows, int64_t cols,
                       uint8_t* codes, void* stream);
-
-/*
- * Measurement probe, no counterpart in the reference: reads `bytes` (a multiple of 1024) of device memory and does
- * nothing else, with `workgroups` x `waves` wavefronts that each keep `loads_in_flight` (2, 4, 8, 12, 16 or 24) 1 KB
- * loads outstanding; `contiguous` = 1 gives every wavefront one contiguous run, 0 interleaves the wavefronts
- * kilobyte by kilobyte; `contiguous` >= 2 selects the access pattern of the column-per-lane decode kernel for a packed
- * int4 weight with K = 128 x contiguous (one workgroup per 64 columns, `workgroups` ignored, 16-byte loads that touch
- * eight 128-byte lines per wavefront).  bytes = 0 launches an empty kernel of the same grid.  `sink`: 256 bytes that are practically
- * never written.  The benchmark uses it as the ceiling a bandwidth-bound kernel of the same footprint is held against.
- */
-int tpq_probe_read(const void* src, int64_t bytes, int workgroups, int waves, int loads_in_flight, int contiguous,
-                   void* sink, void* stream);
 
 #ifdef __cplusplus
 }

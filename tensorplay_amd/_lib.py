@@ -20,7 +20,6 @@ _i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_
 # name -> argument types, in the order of include/tpq.h
 SIGNATURES = {
     "tpq_abi_version": [],
-    "tpq_set_kernel_override": [ctypes.c_char_p, _int],
     "tpq_quantize_rowwise": [_ptr, _int, _i64, _i64, _f32, _f32, _int, _int, _int, _ptr, _ptr, _ptr],
     "tpq_int_mm": [_ptr, _int, _ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr],
     "tpq_int8_mm_rescale": [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr],
@@ -55,7 +54,6 @@ SIGNATURES = {
     "tpq_lowbit_dequantize": [_ptr, _int, _int, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],
     "tpq_lowbit_pack": [_ptr, _int, _int, _i64, _i64, _ptr, _ptr],
     "tpq_lowbit_unpack": [_ptr, _int, _int, _i64, _i64, _ptr, _ptr],
-    "tpq_probe_read": [_ptr, _i64, _int, _int, _int, _int, _ptr, _ptr],
     "tpq_dequantize_affine": [_ptr, _int, _int, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr],
 }
 
@@ -76,14 +74,19 @@ def load() -> ctypes.CDLL:
     # process, so that device pointers and streams are shared with the tensors we are handed.
     import torch  # noqa: F401
 
-    lib = ctypes.CDLL(LIB_PATH)
+    _lib = bind(LIB_PATH)
+    return _lib
+
+
+def bind(path: str) -> ctypes.CDLL:
+    """Opens a build of the kernel library and declares the operators' signatures on it."""
+    lib = ctypes.CDLL(path)
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = ctypes.c_size_t if name.endswith("_bytes") else _int
     lib.tpq_last_error.argtypes = []
     lib.tpq_last_error.restype = ctypes.c_char_p
-    _lib = lib
     return lib
 
 

@@ -1,7 +1,11 @@
-"""Builds ``libtpq_gfx950.so`` (the C-ABI kernel library) in-tree with hipcc.
+"""Builds the gfx950 libraries in-tree with hipcc (which cross-compiles without a GPU present).
 
-Usage: ``python -m tensorplay_amd.build`` or ``tensorplay_amd.build.build_library()``.
-hipcc cross-compiles for gfx950 without a GPU present.
+``libtpq_gfx950.so``        the C-ABI kernel library: the operators of include/tpq.h and nothing else.
+``libtpq_gfx950_hooks.so``  the same sources with -DTPQ_TEST_HOOKS: exports tpq_set_kernel_override as well, with which the
+                            tests pin a route so that a kernel is checked on every shape it can take.  Only tests load it.
+``libtpq_probe.so``         the pure-read measurement probe (csrc/probe.hip).  Only bench.py loads it.
+
+Usage: ``python -m tensorplay_amd.build`` (all three) or ``tensorplay_amd.build.build_library()``.
 """
 from __future__ import annotations
 
@@ -15,8 +19,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libtpq_gfx950.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
+HOOKS_LIB_PATH = os.path.join(HERE, "libtpq_gfx950_hooks.so")
+PROBE_LIB_PATH = os.path.join(HERE, "libtpq_probe.so")
 
-SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "rms_norm.hip", "probe.hip"]
+SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "rms_norm.hip"]
+# the sources that read a pinned route: the only ones compiled a second time for the test-hook library
+HOOK_SOURCES = ["tpq_core.hip", "int4_mm.hip", "int8_gemm.hip", "lowbit_mm.hip"]
 
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32.
 # -ffp-contract=off: fused multiply-adds only where the source asks for one,
@@ -44,35 +52,51 @@ def hipcc() -> str:
     return exe
 
 
-def build_library(verbose: bool = False, jobs: int = 5, tuning: bool = False) -> str:
-    """tuning=True compiles the sweep knobs in (-DTPQ_TUNING: TPQ_* environment variables pick kernels and workgroup
-    shapes); the library that ships is built without it and never reads the environment."""
+def _compile(cc: str, src: str, obj: str, extra: list, verbose: bool) -> str:
+    cmd = [cc, *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "packed-fp32-ops' is not a recognized feature"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return obj
+
+
+def _link(cc: str, objs: list, path: str) -> str:
+    tmp = path + ".tmp"
+    proc = subprocess.run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    os.replace(tmp, path)
+    return path
+
+
+def build_library(verbose: bool = False, jobs: int = 6, tuning: bool = False, hooks: bool = True, probe: bool = True) -> str:
+    """Compiles every source and links the kernel library; with hooks / probe also the test-hook library and the
+    measurement probe.  tuning=True compiles the sweep knobs in (-DTPQ_TUNING: TPQ_* environment variables pick kernels
+    and workgroup shapes); the library that ships is built without it and never reads the environment."""
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     cc = hipcc()
-
-    def compile_one(src: str) -> str:
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        cmd = [cc, *HIPCC_FLAGS, *(["-DTPQ_TUNING"] if tuning else []), "-c", os.path.join(CSRC, src), "-o", obj]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        proc = subprocess.run(cmd, capture_output=True, text=True)
-        noise = "packed-fp32-ops' is not a recognized feature"
-        err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
-        if proc.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src}:\n{err}")
-        if verbose and err.strip():
-            print(err, file=sys.stderr)
-        return obj
-
+    tune = ["-DTPQ_TUNING"] if tuning else []
+    work = [(src, os.path.join(obj_dir, src.replace(".hip", ".o")), tune) for src in SOURCES]
+    if hooks:
+        work += [(src, os.path.join(obj_dir, src.replace(".hip", ".hooks.o")), tune + ["-DTPQ_TEST_HOOKS"]) for src in HOOK_SOURCES]
+    if probe:
+        work.append(("probe.hip", os.path.join(obj_dir, "probe.o"), []))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
-    tmp = LIB_PATH + ".tmp"
-    link = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
-    proc = subprocess.run(link, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"link failed:\n{proc.stderr}")
-    os.replace(tmp, LIB_PATH)
+        list(pool.map(lambda w: _compile(cc, w[0], w[1], w[2], verbose), work))
+    plain = [os.path.join(obj_dir, src.replace(".hip", ".o")) for src in SOURCES]
+    _link(cc, plain, LIB_PATH)
+    if hooks:
+        hooked = [os.path.join(obj_dir, src.replace(".hip", ".hooks.o" if src in HOOK_SOURCES else ".o")) for src in SOURCES]
+        _link(cc, hooked, HOOKS_LIB_PATH)
+    if probe:
+        _link(cc, [os.path.join(obj_dir, "probe.o")], PROBE_LIB_PATH)
     return LIB_PATH
 
 

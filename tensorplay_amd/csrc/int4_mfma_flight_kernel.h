@@ -96,7 +96,7 @@ constexpr size_t flight_lds_bytes() {
     return static_cast<size_t>(kFlightWaves) * flight_resident_steps<XR>() * XR * kFlightRowStride  // activation tiles
          + static_cast<size_t>(kFlightWaves) * SPW * (NB > 4 ? 2 : 1) * kWave * 4                    // parameter words
          + static_cast<size_t>(kFlightWaves) * NB * 4 * (4 * XR) * 4                                 // partial sums, live rows
-         + static_cast<size_t>(kFlightWaves) * XR * 4;                                               // NORM: sums of squares
+         + static_cast<size_t>(kFlightWaves) * XR * 4 * 2;                                           // NORM: sums of squares, and the power of two each row was scaled by
 }
 
 // x: [M][K] 16-bit, M <= XR; weights as in FlightSet (packed: [N/8][K/32][8] x 16 bytes; sz: [K/group][N] words
@@ -283,21 +283,78 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
         for (int h = 0; h < PW; ++h) my_par[(j * PW + h) * kWave + lane] = pw[j][h];
 
     float* const ssq = red + kFlightWaves * NB * 4 * (4 * XR);  // [wave][XR], NORM only
+    float* const undo = ssq + kFlightWaves * XR;                // [wave][XR], NORM with fp16: 2^(ex + eg) of the row's products
     if constexpr (NORM) {
-        // lane (i, q) holds eight k of row 4 t + q per step: squares added per row, the values multiplied by g in place
+        // lane (i, q) holds eight k of row 4 t + q per step: squares added per row, the values multiplied by g in place.
+        // The products x g are rounded to the activation type before the row's factor is known.  bfloat16 has float's
+        // exponent range.  fp16 does not (x g beyond 65504 would become inf, x g below 6e-5 subnormal), so there both
+        // factors are first scaled by exact powers of two taken from bounds this wavefront already has: |x| <= sqrt of
+        // its sum of squares of the row, |g| < 2^eg over its k.  The scaled products stay within [-4, 4]; the wavefront's
+        // partial sums of the row are multiplied by 2^(ex + eg) again before they leave it.
         const bool last_counts = wave + (SPW - 1) * kFlightWaves < steps;
+        [[maybe_unused]] int eg = 0;
+        auto pow2_half2 = [](int e) -> uint32_t {  // (2^e, 2^e) as two fp16, e in [-16, 15]
+            const uint32_t h = e >= -14 ? static_cast<uint32_t>(e + 15) << 10 : 0x0400u >> (-14 - e);
+            return h | (h << 16);
+        };
+        if constexpr (DT == TPQ_DTYPE_F16) {
+            uint32_t mag = 0;
+#pragma unroll
+            for (int j = 0; j < SPW; ++j) {
+                const uint32_t gw[4] = {gk[j].x, gk[j].y, gk[j].z, gk[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t a = gw[e] & 0x7FFF7FFFu;
+                    const uint32_t lo = a & 0xFFFFu, hi = a >> 16;
+                    mag = mag > lo ? mag : lo;
+                    mag = mag > hi ? mag : hi;
+                }
+            }
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) {
+                const uint32_t other = __shfl_xor(mag, off, kWave);
+                mag = mag > other ? mag : other;
+            }
+            eg = static_cast<int>(mag >> 10) - 14;  // |g| < 2^eg (biased exponent - 15 + 1)
+            eg = eg < -15 ? -15 : eg > 16 ? 16 : eg;
+            const half2_t gs = __builtin_bit_cast(half2_t, pow2_half2(-eg));
+#pragma unroll
+            for (int j = 0; j < SPW; ++j) {
+                gk[j].x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, gk[j].x) * gs);
+                gk[j].y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, gk[j].y) * gs);
+                gk[j].z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, gk[j].z) * gs);
+                gk[j].w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, gk[j].w) * gs);
+            }
+        }
 #pragma unroll
         for (int t = 0; t < XR / 4; ++t) {
             float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < SPW; ++j) {
+                const uint32_t xw[4] = {xg[j][t].x, xg[j][t].y, xg[j][t].z, xg[j][t].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (j < SPW - 1 || last_counts) acc = L::dot(xw[e], xw[e], acc);  // a step past the end was read twice
+            }
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+            if (i == 0) ssq[wave * XR + 4 * t + q] = acc;  // read behind the barrier at the end
+            [[maybe_unused]] half2_t xs;
+            if constexpr (DT == TPQ_DTYPE_F16) {
+                const int fl = static_cast<int>(__builtin_bit_cast(uint32_t, acc) >> 23) - 127;  // acc >= 0: floor(log2), -127 for 0
+                int ex = (fl + 2) >> 1;                                                               // sqrt(acc) < 2^ex
+                ex = ex < -15 ? -15 : ex > 16 ? 16 : ex;
+                xs = __builtin_bit_cast(half2_t, pow2_half2(-ex));
+                if (i == 0) undo[wave * XR + 4 * t + q] = __builtin_bit_cast(float, static_cast<uint32_t>(127 + ex + eg) << 23);
+            }
 #pragma unroll
             for (int j = 0; j < SPW; ++j) {
                 const uint32_t gw[4] = {gk[j].x, gk[j].y, gk[j].z, gk[j].w};
                 uint32_t xw[4] = {xg[j][t].x, xg[j][t].y, xg[j][t].z, xg[j][t].w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (j < SPW - 1 || last_counts) acc = L::dot(xw[e], xw[e], acc);  // a step past the end was read twice
                     if constexpr (DT == TPQ_DTYPE_F16) {
-                        xw[e] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, xw[e]) * __builtin_bit_cast(half2_t, gw[e]));
+                        xw[e] = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(half2_t, xw[e]) * xs) * __builtin_bit_cast(half2_t, gw[e]));
                     } else {
                         const float lo = __fmul_rn(bf16_bits_to_f32(static_cast<uint16_t>(xw[e] & 0xFFFFu)), bf16_bits_to_f32(static_cast<uint16_t>(gw[e] & 0xFFFFu)));
                         const float hi = __fmul_rn(bf16_bits_to_f32(static_cast<uint16_t>(xw[e] >> 16)), bf16_bits_to_f32(static_cast<uint16_t>(gw[e] >> 16)));
@@ -306,9 +363,6 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
                 }
                 xg[j][t] = make_uint4(xw[0], xw[1], xw[2], xw[3]);
             }
-#pragma unroll
-            for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
-            if (i == 0) ssq[wave * XR + 4 * t + q] = acc;  // read behind the barrier at the end
         }
     }
 
@@ -420,7 +474,11 @@ __global__ __launch_bounds__(kFlightWaves* kWave) void int4_mfma_flight_kernel(c
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) red[((wave * NB + b) * 4 + v) * (4 * XR) + slot] = yacc[rb][b][v];
+            for (int v = 0; v < 4; ++v) {
+                float part = yacc[rb][b][v];
+                if constexpr (NORM && DT == TPQ_DTYPE_F16) part *= undo[wave * XR + i];  // this wavefront's own write, same row: exact
+                red[((wave * NB + b) * 4 + v) * (4 * XR) + slot] = part;
+            }
     }
     __syncthreads();
     const int out_row = XR * rb + i;  // RB = 1: i

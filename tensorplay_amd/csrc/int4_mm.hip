@@ -646,7 +646,7 @@ int launch_multi(const void* x, int64_t M, int count, const int32_t* const* pack
 template <int DT>
 bool launch_row(const void* x, const int32_t* packed, const void* sz, void* y, int N, int K, int group, hipStream_t s, int* rc) {
     const char* force = tuning_env("TPQ_INT4_KERNEL");  // "row" pins it, any other value excludes it (sweeps)
-    const int pinned = g_override_int4_row.load(std::memory_order_relaxed);
+    const int pinned = route_override_int4_row();
     if ((force && force[0] != 'r') || pinned == 0) return false;
     if (K % 256 != 0 || K > 12288 || N % 8 != 0) return false;  // three 1 KB blocks per wavefront and tile at most (registers)
     int cus = compute_units() / 32 * 32;

@@ -299,8 +299,8 @@ int launch_int8_decode(const int8_t* a, const int8_t* w, int64_t M, int64_t N, i
     // 11008 -> 4096 9.8 / 13.6, 4096 -> 11008 10.0 / 12.6, 8192 x 8192 13.5 / 16.2, 8192 -> 28672 38.1 / 46.2, 28672 -> 8192
     // 36.9 / 51.2 (6.4 TB/s); two rows: 10.5 / 13.4, 10.4 / 11.4, 14.5 / 16.3, 38.8 / 47.1, 38.3 / 52.6.  At four rows
     // the two are even (4096 x 4096: 6.8 / 5.9; 8192 x 8192: 15.8 / 17.4; 8192 -> 28672: 53.6 / 50.5) and the matrix-core
-    // kernel stays.  tpq_set_kernel_override("int8_row", 0 / 1): never / up to four rows, for comparison runs and tests.
-    const int row_override = g_override_int8_row.load(std::memory_order_relaxed);
+    // kernel stays.  A test-hook build pins it: never / up to four rows (route_override_int8_row).
+    const int row_override = route_override_int8_row();
     const int row_limit = row_override < 0 ? 2 : row_override == 0 ? 0 : 4;
     if (M <= row_limit && launch_int8_rows(a, w, static_cast<int>(M), N, K, ep, s)) return check_launch("int8 row gemm");
     const int steps = static_cast<int>(K / 128);

@@ -722,8 +722,8 @@ TPQ_EXPORT int tpq_lowbit_mm(const void* x, int dtype, int64_t M, int64_t K, con
     }
     const bool fast = dtype != TPQ_DTYPE_F32 && K > 0 && group_shift >= 0 && K % step_k == 0 && N % 4 == 0 && K <= 0x7FFFFF80 &&
                       N <= 0x7FFFFFF0 && aligned(x, 16) && aligned(packed, 16) && aligned(scales_and_zeros, 16) && aligned(out, 8);
-    const int forced_row = g_override_lowbit_row.load(std::memory_order_relaxed);
-    if (M == 1 && dtype != TPQ_DTYPE_F32 && forced_row != 0) {  // tpq_set_kernel_override("lowbit_row", 0 / 1): never / wherever the shape allows
+    const int forced_row = route_override_lowbit_row();
+    if (M == 1 && dtype != TPQ_DTYPE_F32 && forced_row != 0) {  // a test-hook build pins the route: never / wherever the shape allows
         int rc = TPQ_OK;
         if (dtype == TPQ_DTYPE_F16 ? launch_lowbit_row<TPQ_DTYPE_F16>(x, packed, scales_and_zeros, bias, out, N, K, group, bits, lsb_first, forced_row == 1, s, &rc)
                                    : launch_lowbit_row<TPQ_DTYPE_BF16>(x, packed, scales_and_zeros, bias, out, N, K, group, bits, lsb_first, forced_row == 1, s, &rc))

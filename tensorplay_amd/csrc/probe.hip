@@ -6,9 +6,35 @@
 // workgroups x wavefronts x loads x 1 KB covers it.  Blocks of 1 KB are dealt to the wavefronts either interleaved
 // (wavefront w takes blocks w, w + W, w + 2 W, ...: neighbouring wavefronts read neighbouring kilobytes) or as one
 // contiguous run per wavefront.
+//
+// Built into a library of its own (libtpq_probe.so, loaded by the benchmark only): it is a measuring instrument, not an
+// operator, and the kernel library's interface lists operators only.  Signature:
+//   int tpq_probe_read(const void* src, int64_t bytes, int workgroups, int waves, int loads_in_flight, int contiguous,
+//                      void* sink, void* stream)
+// reads `bytes` (a multiple of 1024) of device memory with `workgroups` x `waves` wavefronts that each keep
+// `loads_in_flight` (2, 4, 8, 12, 16 or 24) 1 KB loads outstanding; `contiguous` = 1 gives every wavefront one contiguous
+// run, 0 interleaves the wavefronts kilobyte by kilobyte; `contiguous` in 2..1024 selects the access pattern of the
+// column-per-lane decode kernel for a packed int4 weight with K = 128 x contiguous (one workgroup per 64 columns,
+// `workgroups` ignored, 16-byte loads that touch eight 128-byte lines per wavefront; bytes must then be a multiple of
+// 512 x contiguous).  bytes = 0 launches an empty kernel of the same grid.  `sink`: 256 bytes that are practically never written.
+#include <cstdarg>
+#include <cstdio>
+
 #include "tpq_common.h"
 
 namespace tpq {
+// the error plumbing of tpq_common.h, for this library alone
+char* error_buffer() {
+    static thread_local char buffer[512] = "";
+    return buffer;
+}
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
 namespace {
 
 template <int LOADS>
@@ -84,7 +110,12 @@ TPQ_EXPORT int tpq_probe_read(const void* src, int64_t bytes, int workgroups, in
     }
     TPQ_REQUIRE(src && aligned(src, 16), TPQ_ERR_INVALID_VALUE, "probe_read: source must be 16-byte aligned");
     if (contiguous >= 2) {  // the column-per-lane pattern: `workgroups` is ignored, one per 64 columns; K = 128 x contiguous
+        TPQ_REQUIRE(contiguous <= 1024, TPQ_ERR_INVALID_VALUE, "probe_read: column pattern: contiguous = K / 128 must be at most 1024");
+        TPQ_REQUIRE(loads_in_flight == 2 || loads_in_flight == 4 || loads_in_flight == 8 || loads_in_flight == 12 || loads_in_flight == 16 || loads_in_flight == 24,
+                    TPQ_ERR_INVALID_VALUE, "probe_read: loads in flight must be 2, 4, 8, 12, 16 or 24");
         const int k_super = contiguous * 4;  // contiguous = K / 128
+        TPQ_REQUIRE(bytes % (static_cast<int64_t>(k_super) * 128) == 0 && bytes / (static_cast<int64_t>(k_super) * 128) <= 0x7FFFFFF,
+                    TPQ_ERR_INVALID_VALUE, "probe_read: column pattern: bytes must be whole tile rows of 512 x contiguous bytes");
         const int n_tiles = static_cast<int>(bytes / (static_cast<int64_t>(k_super) * 128));
         const dim3 g((n_tiles + 7) / 8), b(static_cast<unsigned>(waves * kWave));
         if (loads_in_flight >= 8) read_probe_columns_kernel<2><<<g, b, 0, s>>>(static_cast<const uint4*>(src), n_tiles, k_super, static_cast<uint32_t*>(sink));

@@ -58,10 +58,22 @@ inline const char* tuning_env(const char* name) {
 #endif
 }
 
-// The routes that tests pin explicitly (tpq_set_kernel_override): -1 = the default rule.
+// Routes that tests pin explicitly, so that a kernel is checked on every shape it can take and not only where the
+// default rule sends it: -1 = the default rule.  They exist only in a build with -DTPQ_TEST_HOOKS (the library the
+// tests' route-pinning fixture loads, with tpq_set_kernel_override exported); in the library that ships the kernel
+// that runs depends on the arguments alone.
+#ifdef TPQ_TEST_HOOKS
 extern std::atomic<int> g_override_int8_row;    // 0 never / 1 up to four rows on the int8 row kernel
 extern std::atomic<int> g_override_lowbit_row;  // 0 never / 1 wherever the shape allows, the packed n-bit row kernel
 extern std::atomic<int> g_override_int4_row;    // 0 never / 1 wherever the shape allows, the int4 tile-streaming one-row kernel
+inline int route_override_int8_row() { return g_override_int8_row.load(std::memory_order_relaxed); }
+inline int route_override_lowbit_row() { return g_override_lowbit_row.load(std::memory_order_relaxed); }
+inline int route_override_int4_row() { return g_override_int4_row.load(std::memory_order_relaxed); }
+#else
+inline int route_override_int8_row() { return -1; }
+inline int route_override_lowbit_row() { return -1; }
+inline int route_override_int4_row() { return -1; }
+#endif
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 

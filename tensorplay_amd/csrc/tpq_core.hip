@@ -217,6 +217,7 @@ using namespace tpq;
 
 TPQ_EXPORT int tpq_abi_version(void) { return 1; }
 
+#ifdef TPQ_TEST_HOOKS
 namespace tpq {
 std::atomic<int> g_override_int8_row{-1};
 std::atomic<int> g_override_lowbit_row{-1};
@@ -232,6 +233,7 @@ TPQ_EXPORT int tpq_set_kernel_override(const char* route, int value) {
     else return tpq::fail(TPQ_ERR_INVALID_VALUE, "tpq_set_kernel_override: unknown route '%s'", route);
     return TPQ_OK;
 }
+#endif
 
 TPQ_EXPORT const char* tpq_last_error(void) { return error_buffer(); }
 

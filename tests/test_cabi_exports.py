@@ -82,18 +82,31 @@ def test_bench_refuses_more_than_one_gpu():
 
 
 def test_dispatch_does_not_depend_on_the_environment():
-    """The shipped library imports no getenv: which kernel runs is a function of the arguments.  The two selectable
-    routes go through tpq_set_kernel_override, which validates its arguments on the host."""
+    """The shipped library imports no getenv and exports neither the route switch of the test-hook build nor the
+    measurement probe: which kernel runs is a function of the arguments, and the interface lists operators only."""
+    import ctypes
     import subprocess
-    from tensorplay_amd import _lib
+    from tensorplay_amd import _lib, build
 
-    lib = _lib.load()
+    _lib.load()
     syms = subprocess.run(["nm", "-D", "--undefined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
     assert "getenv" not in syms, "the library was built with -DTPQ_TUNING (sweep knobs compiled in)"
-    assert lib.tpq_set_kernel_override(b"int8_row", 1) == 0 and lib.tpq_set_kernel_override(b"int8_row", -1) == 0
-    assert lib.tpq_set_kernel_override(b"lowbit_row", 0) == 0 and lib.tpq_set_kernel_override(b"lowbit_row", -1) == 0
-    assert lib.tpq_set_kernel_override(b"int4_row", 1) == 0 and lib.tpq_set_kernel_override(b"int4_row", -1) == 0
-    assert lib.tpq_set_kernel_override(b"no_such_route", 1) == _lib.TPQ_ERR_INVALID_VALUE
-    assert "unknown route" in _lib.last_error()
-    assert lib.tpq_set_kernel_override(b"int8_row", 5) == _lib.TPQ_ERR_INVALID_VALUE
-    assert lib.tpq_set_kernel_override(None, 0) == _lib.TPQ_ERR_INVALID_VALUE
+    exported = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    assert "tpq_set_kernel_override" not in exported and "tpq_probe_read" not in exported
+    # the test-hook build validates its arguments on the host
+    hooked = ctypes.CDLL(build.HOOKS_LIB_PATH)
+    hooked.tpq_set_kernel_override.argtypes = [ctypes.c_char_p, ctypes.c_int]
+    hooked.tpq_last_error.restype = ctypes.c_char_p
+    assert hooked.tpq_set_kernel_override(b"int8_row", 1) == 0 and hooked.tpq_set_kernel_override(b"int8_row", -1) == 0
+    assert hooked.tpq_set_kernel_override(b"lowbit_row", 0) == 0 and hooked.tpq_set_kernel_override(b"lowbit_row", -1) == 0
+    assert hooked.tpq_set_kernel_override(b"int4_row", 1) == 0 and hooked.tpq_set_kernel_override(b"int4_row", -1) == 0
+    assert hooked.tpq_set_kernel_override(b"no_such_route", 1) == _lib.TPQ_ERR_INVALID_VALUE
+    assert b"unknown route" in hooked.tpq_last_error()
+    assert hooked.tpq_set_kernel_override(b"int8_row", 5) == _lib.TPQ_ERR_INVALID_VALUE
+    assert hooked.tpq_set_kernel_override(None, 0) == _lib.TPQ_ERR_INVALID_VALUE
+    # the probe library: argument checks of the column pattern, no launch
+    probe = ctypes.CDLL(build.PROBE_LIB_PATH)
+    probe.tpq_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    assert probe.tpq_probe_read(16, 1024, 1, 8, 8, 32, 16, None) == _lib.TPQ_ERR_INVALID_VALUE   # fewer bytes than one tile row
+    assert probe.tpq_probe_read(16, 1 << 30, 1, 8, 8, 5000, 16, None) == _lib.TPQ_ERR_INVALID_VALUE
+    assert probe.tpq_probe_read(16, 16384 * 8, 1, 8, 7, 32, 16, None) == _lib.TPQ_ERR_INVALID_VALUE

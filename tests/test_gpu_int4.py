@@ -415,6 +415,34 @@ def test_mm_multi_with_rms_norm_against_oracle(ops, tdt, tol, M, K, widths):
         assert_close_norm(y.float().cpu().numpy()[:, cols], want, 2 * tol)
 
 
+@pytest.mark.parametrize("tdt,tol", [(torch.float16, 1e-3), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("K,widths", [(4096, (264, 136)), (2048, (520,)), (8192, (136,))])
+def test_mm_multi_with_rms_norm_row_magnitudes(ops, tdt, tol, K, widths):
+    """Rows from 1e-4 to 1e4 in one batch and norm weights from 0.02 to 30: the fused kernel rounds x g before the row's
+    factor is known, so in fp16 it has to scale both (x g reaches 3e5 here, and 2e-6 at the other end).  Every row is
+    held to the tolerance on its own, against the oracle's product of the normalized activations
+    (tensorplay/nn/functional.py:2350-2372: (x inv) g in float32, one rounding)."""
+    rng = np.random.default_rng(K + len(widths))
+    tag = "f16" if tdt == torch.float16 else "bf16"
+    scales = np.array([1e-4, 1e-3, 1.0, 30.0, 1e3, 3e3, 1e4, 0.05], dtype=np.float32)
+    M = len(scales)
+    cases = [_fused_case(rng, M, n, K, tdt) for n in widths]
+    x = (cases[0][2].float() * torch.from_numpy(scales)[:, None]).to(tdt).to(DEV)
+    g_np = rng.uniform(0.5, 1.5, K).astype(np.float32) * rng.choice(np.array([0.04, 1.0, 20.0], dtype=np.float32), K)
+    g = torch.from_numpy(g_np).to(tdt).to(DEV)
+    assert torch.isfinite(x).all()
+    packed = [ops._convert_weight_to_int4pack(torch.from_numpy(c).to(DEV), 2) for c, _, _ in cases]
+    szs = [sz.to(DEV) for _, sz, _ in cases]
+    got = ops.int4pack_mm_multi(x, packed, 128, szs, norm_weight=g, eps=1e-5)
+    xn = _rms_norm_bits(host(x), host(g), tag, 1e-5)
+    for (codes, sz, _), y, n in zip(cases, got, widths):
+        y = y.float().cpu().numpy()
+        assert np.isfinite(y).all()
+        want = oracle.to_f32(oracle.int4_mm_tc(xn, tag, oracle.int4_pack_tc(codes, 2), host(sz), 128), tag)
+        for r in range(M):
+            assert_close_norm(y[r:r + 1], want[r:r + 1], 2 * tol, "row of magnitude %g" % scales[r])
+
+
 @pytest.mark.parametrize("tdt,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)])
 @pytest.mark.parametrize("M,N,K", [(8, 11008, 4096), (2, 72, 4096), (5, 136, 2048), (12, 200, 4096), (3, 64, 512)])
 def test_mm_swiglu_with_rms_norm_against_oracle(ops, tdt, tol, M, N, K):
