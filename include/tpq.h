@@ -273,6 +273,17 @@ int tpq_rms_norm(const void* x, int dtype, int64_t M, int64_t K, const void* wei
                  void* stream);
 
 /*
+ * The plain GEMM of the reference's many-row route for packed weights, which dequantises the weight to a dense
+ * matrix of the activation type and multiplies once (p10/src/backend/cuda/QuantGemmKernels.cu:1296-1341, the call
+ * gemm_impl(xf, wf.t(), out, 1.0, 0.0, nullptr) at :1339; likewise behind _weight_int8pack_mm and the low-bit linear):
+ *   out[m][n] = T(sum_k float(x[m][k]) * float(w[n][k])),  float32 accumulation, one rounding to `dtype`.
+ * x: [M, K], w: [N, K] (the dense weight that tpq_int4_dequantize / tpq_int8pack_dequantize / tpq_lowbit_dequantize
+ * wrote), out: [M, N], all contiguous and of `dtype` = float16 or bfloat16; x and w 16-byte aligned.
+ * TPQ_ERR_UNSUPPORTED for float32 or K not a multiple of 64 (nothing written).
+ */
+int tpq_dense_mm(const void* x, int dtype, int64_t M, int64_t K, const void* w, int64_t N, void* out, void* stream);
+
+/*
  * Dense weight [N, K] of `dtype` from the packed device layout: W = T(code - 8) * scale + zero, the
  * product and the sum each rounded to T.  The reference runs this before its library GEMM
  * (int4_tc_dequantize_kernel, p10/src/backend/cuda/QuantGemmKernels.cu:1170-1202, 1296-1341); the

@@ -1,4 +1,4 @@
-// int8 GEMM, staggered form: 256 x 128 tile per workgroup, three-stage LDS ring of whole 128-byte rows filled by
+// Tiled GEMM C = A W^T (int8 -> int32, or float16 / bfloat16 -> float32), staggered form: 256 x 128 tile per workgroup, three-stage LDS ring of whole 128-byte rows filled by
 // direct global -> LDS loads, eight wavefronts in eight positions of 64 x 64 (v_mfma_i32_16x16x64_i8), the two
 // wavefronts of a SIMD half a stage apart.
 //
@@ -63,13 +63,43 @@ __device__ unsigned long long g_stagger_coarse[4 * 8];  // [start, first barrier
 #define TPQ_STAGGER_STAMP(I) do { } while (0)
 #endif
 
-template <class Tile>
-__global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, int M,
-                                                                              int N, int K, Tile tile, int vector_stores, int slices) {
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// The operand types the form multiplies.  A stage is 128 bytes of k per row whatever the type, and the lane layout of
+// the 16-byte fragments is the same for all three instructions (lane (r, c): row r, bytes 16 c .. 16 c + 15 of a k-half
+// of 64 bytes), so the kernel body does not depend on the type beyond the accumulator and the instruction.
+struct ArithI8 {  // 128 k per stage, v_mfma_i32_16x16x64_i8
+    using acc_t = v4i;
+    static __device__ __forceinline__ acc_t mfma(const v4i& b, const v4i& a, const acc_t& c) { return __builtin_amdgcn_mfma_i32_16x16x64_i8(b, a, c, 0, 0, 0); }
+};
+struct ArithF16 {  // 64 k per stage, v_mfma_f32_16x16x32_f16
+    using acc_t = v4f;
+    static __device__ __forceinline__ acc_t mfma(const v4i& b, const v4i& a, const acc_t& c) {
+        typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, b), __builtin_bit_cast(h8_t, a), c, 0, 0, 0);
+    }
+};
+struct ArithBF16 {  // 64 k per stage, v_mfma_f32_16x16x32_bf16
+    using acc_t = v4f;
+    static __device__ __forceinline__ acc_t mfma(const v4i& b, const v4i& a, const acc_t& c) {
+        typedef __bf16 b8_t __attribute__((ext_vector_type(8)));
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8_t, b), __builtin_bit_cast(b8_t, a), c, 0, 0, 0);
+    }
+};
+
+// A, W: row-major [M][K], [N][K] with K contiguous; row_bytes = K * sizeof(element).
+// MB: blocks of 16 rows per wavefront: 4 (tile of 256 rows, what the description above and the numbers are about) or 2
+// (tile of 128 rows for problems with few rows or few tiles: per stage 32 wave-level loads against 16 MFMAs per
+// wavefront, so the vector memory path bounds it at about 700 clocks per stage).
+template <class Tile, class Arith, int MB>
+__global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restrict__ A, const char* __restrict__ W, int M, int N,
+                                                                         int row_bytes, Tile tile, int vector_stores, int slices) {
     using out_t = typename Tile::out_t;
-    constexpr int BM = 256, BN = 128, WM = 64, WN = 64;
-    constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;  // 48 KB
-    constexpr int kRingBytes = kDmaStages * kStageBytes;   // 144 KB
+    using acc_t = typename Arith::acc_t;
+    constexpr int BM = 64 * MB, BN = 128, WM = 16 * MB, WN = 64;
+    static_assert(MB == 4 || MB == 2, "two tile heights are built");
+    constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;  // 48 KB (32 KB)
+    constexpr int kRingBytes = kDmaStages * kStageBytes;   // 144 KB (96 KB)
     constexpr int kRequesters = 8;
     constexpr int kLoadsA = BM / 8 / kRequesters, kLoadsW = BN / 8 / kRequesters, kLoads = kLoadsA + kLoadsW;  // 4 + 2
     extern __shared__ uint4 ring[];
@@ -99,7 +129,7 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
         }
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int nk_all = K / kDmaRowBytes, nk_slice = (nk_all + slices - 1) / slices;
+    const int nk_all = row_bytes / kDmaRowBytes, nk_slice = (nk_all + slices - 1) / slices;
     const int kt0 = blockIdx.y * nk_slice;
     const int nk = nk_all - kt0 < nk_slice ? nk_all - kt0 : nk_slice;
 
@@ -120,17 +150,17 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
         int gr = (act ? m0 : n0) + row;
         const int limit = act ? M : N;
         gr = gr < limit ? gr : limit - 1;
-        voff[i] = static_cast<uint32_t>(gr - (act ? m0 : n0)) * static_cast<uint32_t>(K) + chunk * 16;
+        voff[i] = static_cast<uint32_t>(gr - (act ? m0 : n0)) * static_cast<uint32_t>(row_bytes) + chunk * 16;
         lds_of_load[i] = static_cast<uint32_t>(act ? block : BM / 8 + block) * 1024;
     }
     const uint32_t ring_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)ring));
-    const int8_t* const base_a = A + static_cast<size_t>(m0) * K + static_cast<size_t>(kt0) * kDmaRowBytes;
-    const int8_t* const base_w = W + static_cast<size_t>(n0) * K + static_cast<size_t>(kt0) * kDmaRowBytes;
+    const char* const base_a = A + static_cast<size_t>(m0) * row_bytes + static_cast<size_t>(kt0) * kDmaRowBytes;
+    const char* const base_w = W + static_cast<size_t>(n0) * row_bytes + static_cast<size_t>(kt0) * kDmaRowBytes;
     // loads [FIRST, FIRST + COUNT) of stage kt into ring slot SLOT: scalar base, constant per-lane offset, no vector ALU
     auto request = [&](auto first, auto count, auto slot_c, int kt) {
         constexpr int FIRST = decltype(first)::value, COUNT = decltype(count)::value, SLOT = decltype(slot_c)::value;
-        const int8_t* const sa = base_a + static_cast<size_t>(kt) * kDmaRowBytes;
-        const int8_t* const sw = base_w + static_cast<size_t>(kt) * kDmaRowBytes;
+        const char* const sa = base_a + static_cast<size_t>(kt) * kDmaRowBytes;
+        const char* const sw = base_w + static_cast<size_t>(kt) * kDmaRowBytes;
 #pragma unroll
         for (int i = FIRST; i < FIRST + COUNT; ++i) {
             const uint32_t dst = ring_addr + SLOT * kStageBytes + lds_of_load[i];
@@ -165,21 +195,21 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
             addr_a[s][kh] = ring_addr + s * kStageBytes + (wm * WM + frag_row) * kDmaRowBytes + chunk;
             addr_b[s][kh] = ring_addr + s * kStageBytes + (BM + wn * WN + frag_row) * kDmaRowBytes + chunk;
         }
-    v4i fa[2][4], fb[2][4];  // [k-half][block of 16 rows]
+    v4i fa[2][MB], fb[2][4];  // [k-half][block of 16 rows]
     auto read_half = [&](auto slot_c, auto half_c) {
         constexpr int SLOT = decltype(slot_c)::value;
 #pragma unroll
         for (int kh = decltype(half_c)::value; kh < decltype(half_c)::value + 1; ++kh) {
             const uint32_t aa = addr_a[SLOT][kh], ab = addr_b[SLOT][kh];
             // (an array element as an asm operand inside a generic lambda does not compile: references)
-            v4i &a0 = fa[kh][0], &a1 = fa[kh][1], &a2 = fa[kh][2], &a3 = fa[kh][3], &b0 = fb[kh][0], &b1 = fb[kh][1], &b2 = fb[kh][2], &b3 = fb[kh][3];
+            v4i &a0 = fa[kh][0], &a1 = fa[kh][1], &a2 = fa[kh][MB - 2], &a3 = fa[kh][MB - 1], &b0 = fb[kh][0], &b1 = fb[kh][1], &b2 = fb[kh][2], &b3 = fb[kh][3];
             asm volatile("ds_read_b128 %0, %1" : "=v"(a0) : "v"(aa) : "memory");
             asm volatile("ds_read_b128 %0, %1" : "=v"(b0) : "v"(ab) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(a1) : "v"(aa) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(b1) : "v"(ab) : "memory");
-            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(a2) : "v"(aa) : "memory");
+            if constexpr (MB == 4) asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(a2) : "v"(aa) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(b2) : "v"(ab) : "memory");
-            asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(a3) : "v"(aa) : "memory");
+            if constexpr (MB == 4) asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(a3) : "v"(aa) : "memory");
             asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(b3) : "v"(ab) : "memory");
         }
     };
@@ -197,25 +227,26 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
             read_stage(read_slot);
             request_stage(fill_slot, kt_new);
         } else {
-            constexpr std::integral_constant<int, kLoads / 3> third{};
-            request(std::integral_constant<int, 0>{}, third, fill_slot, kt_new);
+            constexpr int kFirst = (kLoads + 2) / 3, kSecond = (kLoads - kFirst + 1) / 2, kThird = kLoads - kFirst - kSecond;  // 2 2 2 (2 1 1)
+            request(std::integral_constant<int, 0>{}, std::integral_constant<int, kFirst>{}, fill_slot, kt_new);
             read_half(read_slot, std::integral_constant<int, 0>{});
-            request(third, third, fill_slot, kt_new);
+            request(std::integral_constant<int, kFirst>{}, std::integral_constant<int, kSecond>{}, fill_slot, kt_new);
             read_half(read_slot, std::integral_constant<int, 1>{});
-            request(std::integral_constant<int, 2 * (kLoads / 3)>{}, third, fill_slot, kt_new);
+            request(std::integral_constant<int, kFirst + kSecond>{}, std::integral_constant<int, kThird>{}, fill_slot, kt_new);
         }
     };
     auto stage_ready = [&]() {  // every fragment read has delivered; the MFMAs that use them stay behind this point
-        asm volatile("s_waitcnt lgkmcnt(0)"
-                     : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[0][2]), "+v"(fb[0][3]));
-        asm volatile("" : "+v"(fa[1][0]), "+v"(fa[1][1]), "+v"(fa[1][2]), "+v"(fa[1][3]), "+v"(fb[1][0]), "+v"(fb[1][1]), "+v"(fb[1][2]), "+v"(fb[1][3]));
+        // (every register must appear once: a register named twice would be copied in front of the wait)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[0][2]), "+v"(fb[0][3]));
+        asm volatile("" : "+v"(fa[1][0]), "+v"(fa[1][1]), "+v"(fb[1][0]), "+v"(fb[1][1]), "+v"(fb[1][2]), "+v"(fb[1][3]));
+        if constexpr (MB == 4) asm volatile("" : "+v"(fa[0][MB - 2]), "+v"(fa[0][MB - 1]), "+v"(fa[1][MB - 2]), "+v"(fa[1][MB - 1]));
     };
 
-    v4i acc[4][4];  // [block of 16 rows][block of 16 columns]
+    acc_t acc[MB][4];  // [block of 16 rows][block of 16 columns]
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MB; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+        for (int j = 0; j < 4; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
     // W fragment first: a lane ends up with 4 consecutive n for one m.  Column blocks in snake order, so that one operand
     // changes from one instruction to the next.
     auto multiply_stage = [&]() {
@@ -224,11 +255,11 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < MB; ++i)
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) {
                     const int j = (i & 1) ? 3 - jj : jj;
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[kh][j], fa[kh][i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = Arith::mfma(fb[kh][j], fa[kh][i], acc[i][j]);
                 }
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
@@ -272,7 +303,7 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
     // edges), ahead of the stages in every requesting wavefront's order, so the wait for stage 0 covers them; nothing
     // here is a load the compiler counts, so it inserts no wait of its own in front of the first barrier.
     if (Tile::kScaled) {
-        // eight pieces of 64 floats: column scales 0..1, bias 2..3, row scales 4..7; one per wavefront
+        // pieces of 64 floats: column scales 0..1, bias 2..3, row scales 4..7 (4..5); one per wavefront
         constexpr int kPieces = 8 / kRequesters;
 #pragma unroll
         for (int e = 0; e < kPieces; ++e) {
@@ -283,7 +314,7 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
             const int idx = first + lane < limit ? first + lane : limit - 1;
             const uint32_t off = static_cast<uint32_t>(idx) * 4;
             const uint32_t dst = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_ptr)cs_lds)) + piece * 256;
-            if (src != nullptr) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(src) : "memory", "m0");
+            if (src != nullptr && piece < 4 + BM / 64) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(src) : "memory", "m0");
         }
     }
     request_stage(c0, 0);
@@ -383,14 +414,14 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
 #endif
     const bool has_bias = tile.bias != nullptr;
     constexpr int kElem = sizeof(out_t);
-    constexpr int kPassBlocks = kElem == 2 ? 4 : 2;              // 16-row blocks per pass
+    constexpr int kPassBlocks = kElem == 2 ? MB : 2;             // 16-row blocks per pass
     constexpr int kWavePitch = WN * kElem + 16;                  // bytes per row of the wavefront's image
     constexpr int kRowChunks = WN * kElem / 16;                  // 16-byte chunks per row: 8 or 16
     constexpr int kRowsPerStore = kWave / kRowChunks;            // rows per wavefront store: 8 or 4
     static_assert(8 * 12288 <= kRingBytes && kPassBlocks * 16 * kWavePitch <= 12288, "eight wavefront images in the ring");
     char* img = lds_bytes + wave * 12288;
 #pragma unroll
-    for (int first = 0; first < 4; first += kPassBlocks) {
+    for (int first = 0; first < MB; first += kPassBlocks) {
         float rs_r[kPassBlocks];
 #pragma unroll
         for (int i = 0; i < kPassBlocks; ++i) rs_r[i] = Tile::kScaled ? rs_lds[wm * WM + (first + i) * 16 + frag_row] : 0.0f;
@@ -445,38 +476,26 @@ __global__ __launch_bounds__(512) void int8_gemm_stagger_kernel(const int8_t* __
     TPQ_STAGGER_STAMP(3);
 }
 
-template <class Tile>
-int launch_stagger(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
-    constexpr size_t smem = static_cast<size_t>(kDmaStages) * (256 + 128) * kDmaRowBytes + (2 * 128 + 256) * sizeof(float) + kStaggerStampBytes;
-    const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
-    TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "int8 gemm: too many tiles");
-    TPQ_REQUIRE(K % kDmaRowBytes == 0 && K < (1 << 23), TPQ_ERR_INVALID_VALUE, "int8 gemm (staggered): K must be a multiple of 128 below 2^23");
-    auto kernel = int8_gemm_stagger_kernel<Tile>;
+// row_bytes = K * sizeof(element): a multiple of 128 below 2^23
+template <class Arith, int MB, class Tile>
+int launch_stagger_bytes(const void* a, const void* w, int64_t M, int64_t N, int64_t row_bytes, Tile tile, hipStream_t s, int slices, const char* what) {
+    constexpr int BM = 64 * MB;
+    constexpr size_t smem = static_cast<size_t>(kDmaStages) * (BM + 128) * kDmaRowBytes + (2 * 128 + BM) * sizeof(float) + kStaggerStampBytes;
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + 127) / 128);
+    TPQ_REQUIRE(tiles <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "staggered gemm: too many tiles");
+    TPQ_REQUIRE(row_bytes % kDmaRowBytes == 0 && row_bytes < (1 << 23), TPQ_ERR_INVALID_VALUE, "staggered gemm: a row of k must be a multiple of 128 bytes below 2^23");
+    auto kernel = gemm_stagger_kernel<Tile, Arith, MB>;
     static std::atomic<uint64_t> configured{0};  // per instantiation
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int8 gemm")) return rc;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, what)) return rc;
     const int vector_stores = (N * sizeof(typename Tile::out_t)) % 16 == 0 && aligned(tile.out, 16);
     kernel<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(slices)), 512, smem, s>>>(
-        a, w, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), tile, vector_stores, slices);
-    return check_launch("int8 mfma gemm (staggered)");
+        static_cast<const char*>(a), static_cast<const char*>(w), static_cast<int>(M), static_cast<int>(N), static_cast<int>(row_bytes), tile, vector_stores, slices);
+    return check_launch(what);
 }
 
-// Which tiled kernel runs a shape.  Measured against the lock-step kernel with the same result bits (us, lock-step /
-// staggered): 2048 x 4096 x 4096 35.9 / 29.0, 2048 x 11008 x 4096 105 / 93, 2048 x 4096 x 11008 91 / 72, 8192^3 550 / 437,
-// 2048 x 2560 x 6912 44.5 / 35.0, 4096 x 4096 x 512 18.0 / 16.2.  Launches whose k range is cut into slices (few stages
-// per workgroup, 32-bit partial sums out) gain nothing from it (128 .. 1024 rows of 4096 x 4096: equal; 256 x 8192 x
-// 8192: 34.2 / 37.5) and stay on the lock-step kernel.  TPQ_INT8_FORM = dma / stagger in a tuning build forces one.
 template <class Tile>
-int launch_tiled(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
-    const char* env = tuning_env("TPQ_INT8_FORM");
-    if (K >= (1 << 23) || (env && env[0] == 'd')) return launch_dma(a, w, M, N, K, tile, s, slices);
-    if (slices > 1 && !(env && env[0] == 's')) return launch_dma(a, w, M, N, K, tile, s, slices);
-    return launch_stagger(a, w, M, N, K, tile, s, slices);
-}
-
-// partial [slices][M][N] int32 (16-byte aligned) := the slices of A W^T
-inline int launch_tiled_sliced(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, int32_t* partial, int slices, hipStream_t s) {
-    const TileInt32 tile{partial, nullptr, nullptr, nullptr};
-    return launch_tiled(a, w, M, N, K, tile, s, slices);
+int launch_stagger(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
+    return launch_stagger_bytes<ArithI8, 4>(a, w, M, N, K, tile, s, slices, "int8 mfma gemm (staggered)");
 }
 
 }  // namespace

@@ -5,10 +5,29 @@
 #include <type_traits>
 
 #include "int8_decode_kernel.h"
-#include "int8_gemm_stagger.h"
+#include "gemm_stagger.h"
 
 namespace tpq {
 namespace {
+
+// Which tiled kernel runs a shape.  Measured against the lock-step kernel with the same result bits (us, lock-step /
+// staggered): 2048 x 4096 x 4096 35.9 / 29.0, 2048 x 11008 x 4096 105 / 93, 2048 x 4096 x 11008 91 / 72, 8192^3 550 / 437,
+// 2048 x 2560 x 6912 44.5 / 35.0, 4096 x 4096 x 512 18.0 / 16.2.  Launches whose k range is cut into slices (few stages
+// per workgroup, 32-bit partial sums out) gain nothing from it (128 .. 1024 rows of 4096 x 4096: equal; 256 x 8192 x
+// 8192: 34.2 / 37.5) and stay on the lock-step kernel.  TPQ_INT8_FORM = dma / stagger in a tuning build forces one.
+template <class Tile>
+int launch_tiled(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
+    const char* env = tuning_env("TPQ_INT8_FORM");
+    if (K >= (1 << 23) || (env && env[0] == 'd')) return launch_dma(a, w, M, N, K, tile, s, slices);
+    if (slices > 1 && !(env && env[0] == 's')) return launch_dma(a, w, M, N, K, tile, s, slices);
+    return launch_stagger(a, w, M, N, K, tile, s, slices);
+}
+
+// partial [slices][M][N] int32 (16-byte aligned) := the slices of A W^T
+inline int launch_tiled_sliced(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, int32_t* partial, int slices, hipStream_t s) {
+    const TileInt32 tile{partial, nullptr, nullptr, nullptr};
+    return launch_tiled(a, w, M, N, K, tile, s, slices);
+}
 
 // Large problems with K a multiple of the 128-byte stage take the ring-buffered kernel.
 inline TileInt32 to_tile(const EpilogueInt32& ep) { return TileInt32{ep.c, nullptr, nullptr, nullptr}; }

@@ -116,6 +116,20 @@ struct TileDequant {
     }
 };
 
+// float32 accumulators of a float16 / bfloat16 product, rounded once to the output type (no scales)
+template <int DT>
+struct TileFloat {
+    using out_t = typename Elem<DT>::storage;
+    static constexpr bool kScaled = false;
+    out_t* out;
+    const float* rs;
+    const float* cs;
+    const float* bias;
+    static __device__ __forceinline__ float value(float acc, float, float, float, bool) { return acc; }
+    static __device__ __forceinline__ out_t convert(float acc, float, float, float, bool) { return Elem<DT>::store(acc); }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return TileDequant<DT>::pack2(lo, hi); }
+};
+
 constexpr int kDmaRowBytes = 128;  // bytes of k per stage: one cache line per row
 constexpr int kDmaStages = 3;
 

@@ -229,25 +229,37 @@ def _convert_weight_to_int4pack(self: torch.Tensor, innerKTiles: int) -> torch.T
     return out
 
 
-# Above this many activation rows _weight_int4pack_mm dequantises and calls the library GEMM; below, the library's own
-# kernels read the packed weight (decode kernels up to 112 rows, a tiled kernel above).  Measured (us, packed-weight
-# kernels against the dense route, whose dequantize pass takes 21 us in float16 and 25 us in bfloat16 at K = 4096,
-# N = 11008).  float16: K = 4096, N = 11008: 53 / 64 at 256 rows, 69 / 66 at 384, 73 / 75 at 512, 139 / 87 at 768;
-# K = N = 8192: 71 / 99 at 256, 115 / 92 at 384; K = N = 4096: 36 / 36 at 256, 60 / 38 at 384; K = 11008, N = 4096:
-# 50 / 49 at 64, 74 / 60 at 96, 85 / 64 at 256; K = 8192, N = 28672: 282 / 341 at 512, 414 / 457 at 768, 533 / 510 at 1024.
-# bfloat16 pays ten vector operations per pair of weights for the dense weight's two roundings in the tiled kernel
-# (float16: three packed ones), so it hands over earlier: K = 4096, N = 11008: 41 / 52 at 96, 54 / 55 at 128, 73 / 60
-# at 192; K = N = 8192: 62 / 67 at 96, 99 / 72 at 128; K = 11008, N = 4096: 48 / 51 at 64, 72 / 63 at 96; K = 8192,
-# N = 28672: 275 / 291 at 256, 336 / 349 at 512, 484 / 441 at 768.
+# Above this many activation rows _weight_int4pack_mm dequantises the weight and multiplies with the library's dense
+# 16-bit tile kernel (tpq_dense_mm); below, the kernels that read the packed weight run (decode kernels up to 112 rows, a
+# tiled kernel above).  Measured (us, packed-weight kernels / dense route including its dequantize pass of 21 us in
+# float16 and 25 us in bfloat16 at K = 4096, N = 11008).  float16: K = 4096, N = 11008: 53 / 54 at 256 rows, 66 / 65 at
+# 384, 71 / 68 at 512, 141 / 120 at 1024, 233 / 180 at 2048; K = N = 4096: 35 / 41 at 256, 61 / 38 at 384; K = N = 8192:
+# 68 / 76 at 256, 114 / 97 at 384; K = 11008, N = 4096: 84 / 86 at 256, 150 / 92 at 384; K = 8192, N = 28672: 393 / 469
+# at 768, 522 / 562 at 1024, 1012 / 875 at 2048.  bfloat16 pays ten vector operations per pair of weights for the dense
+# weight's two roundings in the tiled kernel (float16: three packed ones), so it hands over earlier: K = 4096,
+# N = 11008: 34 / 48 at 96, 51 / 48 at 128; K = N = 8192: 59 / 77 at 96, 96 / 79 at 128; K = 11008, N = 4096: 71 / 82 at
+# 96, 127 / 87 at 128; K = 8192, N = 28672: 466 / 479 at 768, 623 / 565 at 1024.
 INT4_PREFILL_ROWS = 256
-INT4_PREFILL_ROWS_WIDE = 512       # N >= 10240
-INT4_PREFILL_ROWS_VERY_WIDE = 768  # N >= 16384
-INT4_PREFILL_ROWS_DEEP = 64        # K >= 2 N: few output tiles, a long k range
+INT4_PREFILL_ROWS_VERY_WIDE = 1024  # N >= 16384
 INT4_PREFILL_ROWS_BF16 = 112
-INT4_PREFILL_ROWS_BF16_VERY_WIDE = 512
+INT4_PREFILL_ROWS_BF16_VERY_WIDE = 768
 # float32 activations have no matrix-core decode kernel: the per-row kernel costs about 16 us a row at K = 4096,
-# N = 11008 (71 us at 4 rows, 253 us at 16), the dense float32 route 95 us at 16 rows and 134 us at 64.
+# N = 11008 (71 us at 4 rows, 253 us at 16), the dense float32 route (the framework's GEMM) 95 us at 16 rows and 134 us at 64.
 INT4_PREFILL_ROWS_F32 = 4
+
+
+def _dense_mm(x: torch.Tensor, dense: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out = x @ dense.T`` behind the dequantise-then-multiply routes (QuantGemmKernels.cu:1339).
+
+    float16 / bfloat16 with K a multiple of 64 run the library's tile kernel; float32 activations and other K go to
+    the framework's GEMM."""
+    m, k = x.shape
+    n = dense.size(0)
+    if x.dtype != torch.float32 and k % 64 == 0 and k < (1 << 22) and x.data_ptr() % 16 == 0:
+        with torch.cuda.device(x.device):
+            _check(_lib.load().tpq_dense_mm(_ptr(x), _DT[x.dtype], m, k, _ptr(dense), n, _ptr(out), _stream(x)))
+        return out
+    return torch.matmul(x, dense.t(), out=out)
 
 
 def _int4_dequantize(packed: torch.Tensor, inner: int, n: int, k: int, group: int, sz: torch.Tensor) -> torch.Tensor:
@@ -291,19 +303,16 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
     sz = qScaleAndZeros.to(self.dtype).contiguous()
     if self.dtype == torch.float32:
         prefill_rows = INT4_PREFILL_ROWS_F32
-    elif k >= 2 * n:
-        prefill_rows = INT4_PREFILL_ROWS_DEEP
     elif self.dtype == torch.bfloat16:
         prefill_rows = INT4_PREFILL_ROWS_BF16_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS_BF16
     else:
-        prefill_rows = INT4_PREFILL_ROWS_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS_WIDE if n >= 10240 else INT4_PREFILL_ROWS
+        prefill_rows = INT4_PREFILL_ROWS_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS
     if m > prefill_rows and inner == 2:
         # Many rows: what the reference does for every shape (QuantGemmKernels.cu:1296-1341) - dequantise
-        # the weight to a dense matrix of the activation dtype, then one plain library GEMM.  The decode
+        # the weight to a dense matrix of the activation dtype, then one plain GEMM.  The decode
         # kernels read the packed weight once per 32 rows, which stops paying at this point.
         dense = _int4_dequantize(w, inner, n, k, qGroupSize, sz)
-        torch.matmul(x, dense.t(), out=out)
-        return out
+        return _dense_mm(x, dense, out)
     with torch.cuda.device(self.device):
         ws = _int4_workspace(self.device, n)
         _check(_lib.load().tpq_int4_mm_ws(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz),
@@ -372,25 +381,20 @@ def ternary_mm(x_i8: torch.Tensor, row_scale: torch.Tensor, packed: torch.Tensor
     return (out, acc) if return_acc else out
 
 
-# Above this many activation rows _weight_int8pack_mm dequantises and calls the library GEMM.  Measured (fp16 / bf16
-# alike unless said, us, slabs of 32 rows on the decode kernels against the dense route): K = 4096, N = 11008: 30 / 45 at
-# 64 rows, 44 / 47 (bf16: 53 / 47) at 96; K = N = 4096: 26 / 34 at 96, 36 / 37 at 128; 4096 -> 6144: 33 / 39 at 96, 44 / 41
-# at 128; K = N = 8192: 56 / 61 at 64, 84 / 68 at 96; 11008 -> 4096: 47 / 48 at 48, 57 / 53 at 64; 4096 -> 32000: 112 / 113
-# at 64, 168 / 103 at 96.
-INT8PACK_PREFILL_ROWS = 64
-INT8PACK_PREFILL_ROWS_TWO_BLOCKS = 96  # K = 3072..4096, N < 10240: slabs of 32 rows on the all-in-flight kernel
-INT8PACK_PREFILL_ROWS_LONG = 48  # K > 8192
-INT8PACK_PREFILL_ROWS_F32 = 24  # float32 activations (per-row kernel): 64 / 89 us at 16 rows, 119 / 94 us at 32
+# Above this many activation rows _weight_int8pack_mm dequantises and multiplies with the dense 16-bit tile kernel.
+# Measured (fp16 / bf16 alike unless said, us, slabs of 32 rows on the decode kernels / dense route): K = 4096,
+# N = 11008: 32 / 50 at 64 rows, 48 / 50 (bf16: 55 / 50) at 96, 62 / 51 at 128; K = N = 4096: 27 / 38 at 96, 37 / 39 at 128,
+# 56 / 41 at 192; K = N = 8192: 58 / 78 at 64, 86 / 79 at 96; 11008 -> 4096: 58 / 83 at 64, 87 / 84 at 96; 8192 -> 28672:
+# 202 / 249 at 64, 303 / 248 at 96.
+INT8PACK_PREFILL_ROWS = 80
+INT8PACK_PREFILL_ROWS_SHORT = 96  # K <= 4096
+INT8PACK_PREFILL_ROWS_F32 = 24  # float32 activations (per-row kernel, the framework's GEMM): 64 / 89 us at 16 rows, 119 / 94 us at 32
 
 
 def _int8pack_prefill_rows(N: int, K: int, dtype: torch.dtype) -> int:
     if dtype == torch.float32:
         return INT8PACK_PREFILL_ROWS_F32
-    if K > 8192:
-        return INT8PACK_PREFILL_ROWS_LONG
-    if 3072 <= K <= 4096 and N < 10240:
-        return INT8PACK_PREFILL_ROWS_TWO_BLOCKS
-    return INT8PACK_PREFILL_ROWS
+    return INT8PACK_PREFILL_ROWS_SHORT if K <= 4096 else INT8PACK_PREFILL_ROWS
 
 
 def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
@@ -417,11 +421,10 @@ def _weight_int8pack_mm(self: torch.Tensor, mat2: torch.Tensor, scales: torch.Te
     with torch.cuda.device(x.device):
         if B > _int8pack_prefill_rows(N, K, x.dtype):
             # Many rows: the decode kernel streams the weight once per 32 rows, which stops paying here.  One pass
-            # writes the dense weight T(w * scale) and a library GEMM does the rest.
+            # writes the dense weight T(w * scale) and the dense tile kernel does the rest.
             dense = torch.empty((N, K), dtype=x.dtype, device=x.device)
             _check(_lib.load().tpq_int8pack_dequantize(_ptr(w), _ptr(sc), N, K, _DT[x.dtype], _ptr(dense), _stream(x)))
-            torch.matmul(x, dense.t(), out=out)
-            return out
+            return _dense_mm(x, dense, out)
         _check(_lib.load().tpq_weight_int8pack_mm(_ptr(x), _DT[x.dtype], B, K, _ptr(w), _ptr(sc), N, _ptr(out), _stream(x)))
     return out
 
@@ -566,11 +569,11 @@ def dequantize_affine(input, block_size, scales: torch.Tensor, zero_points: Opti
 
 # ---- packed n-bit weight-only linear (int2 / intx / binary modules) ------------------------------
 
-# above this many activation rows the weight is dequantised once for the library GEMM (measured, 2 bits, float16, us,
-# decode kernel / dense route: K = 4096, N = 11008: 35 / 51 at 32 rows, 52 / 52 at 48, 68 / 53 at 64; K = N = 8192:
-# 66 / 71 at 48, 87 / 72 at 64; K = N = 4096: 23 / 36 at 48, 29 / 37 at 64)
-LOWBIT_PREFILL_ROWS = 48
-LOWBIT_PREFILL_ROWS_SMALL = 64  # N K <= 2^24
+# above this many activation rows the weight is dequantised once for the dense 16-bit tile kernel (measured, 2 and 4
+# bits, float16 and bfloat16 alike, us, decode kernel / dense route: K = 4096, N = 11008: 34 / 58 at 32 rows, 51 / 58 at
+# 48, 68 / 58 at 64; K = N = 4096: 29 / 42 at 64, 42 / 42 at 96, 56 / 42 at 128)
+LOWBIT_PREFILL_ROWS = 56
+LOWBIT_PREFILL_ROWS_SMALL = 80  # N K <= 2^24
 LOWBIT_PREFILL_ROWS_F32 = 40  # float32 activations (per-row kernel): 144 / 165 us at 32 rows, 278 / 192 us at 64 (K = 4096, N = 11008)
 
 
@@ -651,7 +654,7 @@ def _lowbit_mm(input: torch.Tensor, packed: torch.Tensor, bits: int, columns: in
     b = None if bias is None else bias.to(torch.float32).contiguous()
     if m > (LOWBIT_PREFILL_ROWS_F32 if x.dtype == torch.float32 else LOWBIT_PREFILL_ROWS_SMALL if n * columns <= (1 << 24) else LOWBIT_PREFILL_ROWS):
         dense = _lowbit_dequantize(w, bits, columns, sz, x.dtype, lsb_first)
-        out = torch.matmul(x, dense.t())
+        out = _dense_mm(x, dense, torch.empty((m, n), dtype=x.dtype, device=x.device))
         return out if b is None else out + b.to(out.dtype)
     out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):

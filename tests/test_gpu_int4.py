@@ -245,6 +245,27 @@ def test_mm_many_rows_takes_the_dense_route(ops, dtype):
     assert rel_err(got, y64) < {"f16": 2e-3, "bf16": 1e-2, "f32": 1e-4}[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_mm_prefill_block_matches_cpu_formulation(ops, dtype):
+    """2048 rows of 4096 -> 11008, the prefill block of the model the decode numbers are quoted on: dequantise, then
+    the library's dense tile kernel (no framework GEMM on this route)."""
+    M, N, K, group = 2048, 11008, 4096, 128
+    rng = np.random.default_rng(2048)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = ops._convert_weight_to_int4pack(torch.from_numpy(codes).to(DEV), 2)
+    calls = []
+    real = torch.matmul
+    torch.matmul = lambda *a, **k: calls.append(1) or real(*a, **k)
+    try:
+        got = ops._weight_int4pack_mm(dev(xb, dtype), packed, group, dev(szb, dtype)).float().cpu().numpy()
+    finally:
+        torch.matmul = real
+    assert not calls, "the many-row route went through torch.matmul"
+    assert_close_to_cpu_formulation(got, xb, dtype, codes, szb, group)
+
+
 # ---- fusions around the decode matmul --------------------------------------------------------------
 
 FLIGHT_CASES = [  # M, N, K, group: the all-in-flight matrix-core kernel (K >= 2048, 2..16 rows, groups of 128)
