@@ -94,7 +94,7 @@ class BitNetPacked2bitLinear(nn.Module):
 
     def _apply(self, fn, recurse=True):
         super()._apply(fn, recurse)
-        self._scale_value = float(self.scale)   # a dtype change rounds the scale
+        self._scale_value = None   # a dtype change rounds the scale: read again at the next forward (no copy here: meta tensors, no sync per .to())
         return self
 
     @classmethod
@@ -104,4 +104,6 @@ class BitNetPacked2bitLinear(nn.Module):
         return cls(pack_ternary(codes), scale, linear.in_features, bias, eps)
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if self._scale_value is None:
+            self._scale_value = float(self.scale)
         return bitnet_linear_packed(input, self.int_data, self._scale_value, self.in_features, self.bias, self.eps)

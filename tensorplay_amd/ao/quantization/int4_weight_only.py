@@ -6,6 +6,7 @@ layout int32 [N/8, K/32, 32, 1] written by ``_convert_weight_to_int4pack(codes, 
 """
 from __future__ import annotations
 
+import warnings
 from dataclasses import dataclass
 from typing import Tuple
 
@@ -91,8 +92,10 @@ class WeightOnlyInt4Linear(nn.Module):
     # Layout of a CPU-packed ``weight`` met in a state_dict: (columns per block, half-split nibbles).  The reference's
     # CPU pack depends on the ISA tier it was compiled for (p10/src/backend/cpu/QuantizedElementwiseKernels.cpp:19,
     # 370-390): (64, True) AVX-512 (also what torch's CPU pack writes on such a host), (32, True) AVX2, (32, False)
-    # the plain tier.  A state_dict does not say which; set this before load_state_dict for another tier.
-    cpu_pack_layout = (64, True)
+    # the plain tier.  A state_dict does not say which: set this before load_state_dict.  Left at None, a CPU-layout
+    # weight is taken to be the AVX-512 one, with a warning (a pack from another tier would load without error and
+    # decode to wrong weights).
+    cpu_pack_layout = None
 
     def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
         """Accepts the module's own buffers (device layout int32 [N/8, K/32, 32, 1]) and the buffers a CPU model of the
@@ -110,7 +113,10 @@ class WeightOnlyInt4Linear(nn.Module):
             elif not self.weight.is_cuda:
                 error_msgs.append(f"{key}: move the module to the GPU before loading a CPU-layout weight (the converter is a GPU kernel)")
             else:
-                block_cols, half_split = self.cpu_pack_layout
+                if self.cpu_pack_layout is None:
+                    warnings.warn(f"{key}: CPU-layout int4 weight with cpu_pack_layout unset: assuming the AVX-512 pack (64, True); "
+                                  "set cpu_pack_layout = (32, True) for an AVX2 pack, (32, False) for the plain tier", stacklevel=2)
+                block_cols, half_split = self.cpu_pack_layout or (64, True)
                 state_dict = dict(state_dict)
                 state_dict[key] = ops.int4pack_cpu_to_device(w.to(self.weight.device), block_cols=block_cols, half_split=half_split)
         super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)

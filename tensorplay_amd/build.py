@@ -21,6 +21,7 @@ LIB_NAME = "libtpq_gfx950.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 HOOKS_LIB_PATH = os.path.join(HERE, "libtpq_gfx950_hooks.so")
 PROBE_LIB_PATH = os.path.join(HERE, "libtpq_probe.so")
+QUANT_STAMPS_LIB_PATH = os.path.join(HERE, "libtpq_quant_stamps.so")  # the row quantizer with clock readings per phase (quant_stamps.py)
 
 SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "rms_norm.hip", "dense_mm.hip"]
 # the sources that read a pinned route: the only ones compiled a second time for the test-hook library
@@ -88,6 +89,7 @@ def build_library(verbose: bool = False, jobs: int = 6, tuning: bool = False, ho
         work += [(src, os.path.join(obj_dir, src.replace(".hip", ".hooks.o")), tune + ["-DTPQ_TEST_HOOKS"]) for src in HOOK_SOURCES]
     if probe:
         work.append(("probe.hip", os.path.join(obj_dir, "probe.o"), []))
+        work.append(("quantize_rowwise.hip", os.path.join(obj_dir, "quantize_rowwise.stamps.o"), ["-DTPQ_QUANT_STAMPS"]))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda w: _compile(cc, w[0], w[1], w[2], verbose), work))
     plain = [os.path.join(obj_dir, src.replace(".hip", ".o")) for src in SOURCES]
@@ -97,6 +99,7 @@ def build_library(verbose: bool = False, jobs: int = 6, tuning: bool = False, ho
         _link(cc, hooked, HOOKS_LIB_PATH)
     if probe:
         _link(cc, [os.path.join(obj_dir, "probe.o")], PROBE_LIB_PATH)
+        _link(cc, [os.path.join(obj_dir, "quantize_rowwise.stamps.o"), os.path.join(obj_dir, "tpq_core.o")], QUANT_STAMPS_LIB_PATH)
     return LIB_PATH
 
 

@@ -22,10 +22,32 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kVec = 8;  // elements per lane per chunk
+// Rows up to this length: one wavefront (or a part of one) per row.  Longer rows on one wavefront were measured
+// (2048 x 4096 bfloat16: 7.0 us against 6.6 with four wavefronts per row, 8.9 against 7.1 from HBM; two wavefronts per
+// row: 8.3 against 7.9): a quarter of the wavefronts to launch, but too few loads in flight per compute unit.
+constexpr int kSubwaveMaxK = 1024;
+
+// -DTPQ_QUANT_STAMPS (a measuring build of its own, never the shipped library): every workgroup of the register-cached
+// kernel leaves six readings of the shader clock (entry, loads issued, own data arrived and reduced, row maximum known,
+// stores issued, stores acknowledged: the counters of different compute units do not share a zero, so only differences
+// inside a workgroup mean something) and two of the chip-wide 100 MHz clock (entry, end).
+#ifdef TPQ_QUANT_STAMPS
+constexpr int kStampSlots = 8, kStampRows = 8192;
+__device__ unsigned long long g_quant_stamps[kStampRows * kStampSlots];
+#define TPQ_QUANT_STAMP(I)                                                                                              \
+    do {                                                                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        if (threadIdx.x == 0 && blockIdx.x < kStampRows) g_quant_stamps[blockIdx.x * kStampSlots + (I)] = __builtin_amdgcn_s_memtime(); \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+    } while (0)
+#else
+#define TPQ_QUANT_STAMP(I) do { } while (0)
+#endif
 
 struct QParams {
     float eps, divisor;
     int qmin, qmax, sign_mode;
+    int no_clamp;  // no quotient |v| / scale, |v| <= absmax, can round outside [qmin, qmax]
 };
 
 __device__ __forceinline__ int quantize_one(float v, float scale, const QParams& p) {
@@ -60,12 +82,63 @@ __device__ __forceinline__ void quantize_eight_packed(const float (&v)[kVec], fl
     }
     lo = word[0] ^ 0x80808080u;
     hi = word[1] ^ 0x80808080u;
-    if (redo) {
-        lo = hi = 0;
+    // Rare (one element in a few thousand).  Behind a branch the whole wavefront takes or skips, with a statement the
+    // compiler may not move: left as a plain "if", the eight divisions were computed for every chunk and selected away.
+    // Rare (one element in a few thousand).  Behind a branch the whole wavefront takes or skips, and with the divisor
+    // passed through a statement the compiler may not move: as a plain "if", the eight divisions were hoisted above the
+    // branch, computed for every chunk and selected away.
+    if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+        float divisor = scale;
+        asm volatile("; elements redone with the division" : "+v"(divisor));
+        if (redo) {
+            lo = hi = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            lo |= (static_cast<uint32_t>(quantize_one(v[i], scale, p)) & 0xFFu) << (8 * i);
-            hi |= (static_cast<uint32_t>(quantize_one(v[i + 4], scale, p)) & 0xFFu) << (8 * i);
+            for (int i = 0; i < 4; ++i) {
+                lo |= (static_cast<uint32_t>(quantize_one(v[i], divisor, p)) & 0xFFu) << (8 * i);
+                hi |= (static_cast<uint32_t>(quantize_one(v[i + 4], divisor, p)) & 0xFFu) << (8 * i);
+            }
+        }
+    }
+}
+
+// The same codes with fewer instructions, for parameters under which no quotient can leave the code range
+// (rint(divisor (1 + 2^-20)) <= qmax and >= -qmin, true for the usual divisor = qmax = -qmin = 127): no clamp is
+// needed, and the code is read off the mantissa.  t = fma(v, 1/scale, 1.5 * 2^23) rounds the exact product to the
+// nearest integer (ties to even) and leaves it in two's complement in the low mantissa bits; c = t - 1.5 * 2^23 is that
+// integer, r = fma(v, 1/scale, -c) its distance from the product.  The product is within 2^-16 of the correctly rounded
+// quotient the reference rounds, so |r| <= 1/2 - 2^-13 proves both round to c; anything else (also NaN) is redone with
+// the division.  Five instructions per code and three byte permutes per four codes.
+__device__ __forceinline__ void quantize_eight_lean(const float (&v)[kVec], float scale, float inv_scale, const QParams& p,
+                                                    uint32_t& lo, uint32_t& hi) {
+    constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23
+    bool redo = false;
+    uint32_t t[kVec];
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+        const float tf = __builtin_fmaf(v[i], inv_scale, kMagic);
+        const float c = tf - kMagic;
+        const float r = __builtin_fmaf(v[i], inv_scale, -c);
+        redo |= !(fabsf(r) <= 0.5f - 0x1p-13f);
+        t[i] = __builtin_bit_cast(uint32_t, tf);
+    }
+    // v_perm_b32(a, b, sel): selector bytes 0..3 take bytes of b, 4..7 of a, 0x0c a zero byte
+    lo = __builtin_amdgcn_perm(t[1], t[0], 0x0c0c0400u) | __builtin_amdgcn_perm(t[3], t[2], 0x04000c0cu);
+    hi = __builtin_amdgcn_perm(t[5], t[4], 0x0c0c0400u) | __builtin_amdgcn_perm(t[7], t[6], 0x04000c0cu);
+    // Rare (one element in a few thousand).  Behind a branch the whole wavefront takes or skips, with a statement the
+    // compiler may not move: left as a plain "if", the eight divisions were computed for every chunk and selected away.
+    // Rare (one element in a few thousand).  Behind a branch the whole wavefront takes or skips, and with the divisor
+    // passed through a statement the compiler may not move: as a plain "if", the eight divisions were hoisted above the
+    // branch, computed for every chunk and selected away.
+    if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+        float divisor = scale;
+        asm volatile("; elements redone with the division" : "+v"(divisor));
+        if (redo) {
+            lo = hi = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                lo |= (static_cast<uint32_t>(quantize_one(v[i], divisor, p)) & 0xFFu) << (8 * i);
+                hi |= (static_cast<uint32_t>(quantize_one(v[i + 4], divisor, p)) & 0xFFu) << (8 * i);
+            }
         }
     }
 }
@@ -112,6 +185,10 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_cached(
     const auto* xr = x + row * K;
     int8_t* cr = codes + row * K;
 
+#ifdef TPQ_QUANT_STAMPS
+    if (threadIdx.x == 0 && blockIdx.x < kStampRows) g_quant_stamps[blockIdx.x * kStampSlots + 6] = __builtin_amdgcn_s_memrealtime();
+#endif
+    TPQ_QUANT_STAMP(0);
     float v[CHUNKS][kVec];
     float absmax = 0.0f;
     // No branch around the loads: at the join of a branch the compiler waits for every outstanding load, which made
@@ -122,24 +199,31 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_cached(
         const int k0 = (c * THREADS + threadIdx.x) * kVec;
         load_chunk<DT>(xr + (k0 < K ? k0 : K - kVec), v[c]);
     }
+    TPQ_QUANT_STAMP(1);
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
         for (int i = 0; i < kVec; ++i) absmax = fmaxf(absmax, fabsf(v[c][i]));
+    absmax = wave_max(absmax);
+    TPQ_QUANT_STAMP(2);
     absmax = block_max<THREADS>(absmax, smem);
+    TPQ_QUANT_STAMP(3);
     const float scale = __fdiv_rn(fmaxf(absmax, p.eps), p.divisor);
     if (threadIdx.x == 0) scales[row] = scale;
     // the shortcut needs |quotient| <= 128 and a finite reciprocal: true for every scale the formula
     // above produces from finite inputs with divisor <= 128; anything else takes the divisions
     const float inv_scale = __fdiv_rn(1.0f, scale);
     const bool shortcut = !p.sign_mode && p.divisor <= 128.0f && inv_scale < 3.0e38f && absmax <= 3.0e38f;
+    const bool lean = shortcut && p.no_clamp;
 
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * THREADS + threadIdx.x) * kVec;
         if (k0 < K) {
             uint32_t lo = 0, hi = 0;
-            if (shortcut) {
+            if (lean) {
+                quantize_eight_lean(v[c], scale, inv_scale, p, lo, hi);
+            } else if (shortcut) {
                 quantize_eight_packed(v[c], scale, inv_scale, p, lo, hi);
             } else {
 #pragma unroll
@@ -151,6 +235,12 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_cached(
             *reinterpret_cast<uint2*>(cr + k0) = make_uint2(lo, hi);
         }
     }
+#ifdef TPQ_QUANT_STAMPS
+    TPQ_QUANT_STAMP(4);
+    __builtin_amdgcn_s_waitcnt(0);  // every store of this wavefront acknowledged
+    TPQ_QUANT_STAMP(5);
+    if (threadIdx.x == 0 && blockIdx.x < kStampRows) g_quant_stamps[blockIdx.x * kStampSlots + 7] = __builtin_amdgcn_s_memrealtime();
+#endif
 }
 
 // Short rows (K <= LANES * CHUNKS * 8, K % 8 == 0): LANES lanes of a wavefront per row, so a workgroup
@@ -185,13 +275,16 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_subwave(
     if (live && sub == 0) scales[row] = scale;
     const float inv_scale = __fdiv_rn(1.0f, scale);
     const bool shortcut = !p.sign_mode && p.divisor <= 128.0f && inv_scale < 3.0e38f && absmax <= 3.0e38f;  // as above
+    const bool lean = shortcut && p.no_clamp;
 
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int k0 = (c * LANES + sub) * kVec;
         if (live && k0 < K) {
             uint32_t lo = 0, hi = 0;
-            if (shortcut) {
+            if (lean) {
+                quantize_eight_lean(v[c], scale, inv_scale, p, lo, hi);
+            } else if (shortcut) {
                 quantize_eight_packed(v[c], scale, inv_scale, p, lo, hi);
             } else {
 #pragma unroll
@@ -230,7 +323,7 @@ int launch(const void* x, int64_t M, int64_t K, const QParams& p, int8_t* codes,
     const S* xp = static_cast<const S*>(x);
     const dim3 grid(static_cast<unsigned>(M)), block(kThreads);
     const bool vec_ok = (K % kVec == 0) && aligned(x, 16) && aligned(codes, 8) && K <= 8 * 1024 * kVec;
-    if (vec_ok && K <= 1024) {
+    if (vec_ok && K <= kSubwaveMaxK) {
         const int k = static_cast<int>(K);
         auto run = [&](auto lanes, auto chunks) {
             constexpr int L = decltype(lanes)::value, C = decltype(chunks)::value;
@@ -261,6 +354,17 @@ int launch(const void* x, int64_t M, int64_t K, const QParams& p, int8_t* codes,
 }  // namespace
 }  // namespace tpq
 
+#ifdef TPQ_QUANT_STAMPS
+// [rows][8] clock readings of the last launch of the register-cached kernel (rows beyond 8192 are not recorded)
+TPQ_EXPORT int tpq_quantize_stamps_read(unsigned long long* host, int64_t rows) {
+    using namespace tpq;
+    TPQ_REQUIRE(host && rows >= 0 && rows <= kStampRows, TPQ_ERR_INVALID_VALUE, "quantize stamps: at most %d rows", kStampRows);
+    const hipError_t e = hipMemcpyFromSymbol(host, HIP_SYMBOL(g_quant_stamps), static_cast<size_t>(rows) * kStampSlots * sizeof(unsigned long long));
+    TPQ_REQUIRE(e == hipSuccess, TPQ_ERR_RUNTIME, "quantize stamps: %s", hipGetErrorString(e));
+    return TPQ_OK;
+}
+#endif
+
 TPQ_EXPORT int tpq_quantize_rowwise(const void* x, int x_dtype, int64_t M, int64_t K, float eps,
                                     float divisor, int qmin, int qmax, int sign_mode,
                                     int8_t* codes, float* scales, void* stream) {
@@ -273,7 +377,10 @@ TPQ_EXPORT int tpq_quantize_rowwise(const void* x, int x_dtype, int64_t M, int64
     if (M == 0 || K == 0) return TPQ_OK;
     TPQ_REQUIRE(x && codes && scales, TPQ_ERR_INVALID_VALUE, "quantize_rowwise: null pointer");
     TPQ_REQUIRE(M <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "quantize_rowwise: more than 2^31-1 rows");
-    const QParams p{eps, divisor, qmin, qmax, sign_mode ? 1 : 0};
+    // |v| / scale <= divisor (1 + 2^-22) for every element of the row, whatever the rounding of scale and of the quotient
+    const float reach = rintf(divisor * (1.0f + 0x1p-20f));
+    const int no_clamp = divisor <= 127.0f && reach <= static_cast<float>(qmax) && -reach >= static_cast<float>(qmin);
+    const QParams p{eps, divisor, qmin, qmax, sign_mode ? 1 : 0, no_clamp};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (x_dtype) {
         case TPQ_DTYPE_F32: return launch<TPQ_DTYPE_F32>(x, M, K, p, codes, scales, s);

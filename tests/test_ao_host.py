@@ -107,3 +107,16 @@ def test_fused_int4_ops_check_the_packed_extent_on_the_host():
     # with consistent operands the only thing left to fail on the host is the missing GPU
     with pytest.raises(RuntimeError):
         ops.int4pack_mm_add(x, good, 128, sz, res)
+
+
+def test_bitnet_packed_linear_moves_without_reading_its_scale():
+    """.to() / .half() of a model must not copy the scale to the host (a device sync per call, an error on meta
+    tensors): the cached value is dropped and read again at the next forward."""
+    from tensorplay_amd.ao.quantization import BitNetPacked2bitLinear
+
+    mod = BitNetPacked2bitLinear(torch.zeros(8, 4, dtype=torch.uint8), 0.5, 16, bias=torch.zeros(8))
+    assert mod._scale_value == 0.5
+    mod.half()
+    assert mod._scale_value is None
+    mod.to("meta")   # raised before: float() of a meta tensor
+    assert mod.scale.is_meta and mod._scale_value is None

@@ -224,7 +224,8 @@ def test_int4_linear_loads_a_cpu_saved_state_dict(dtype, tag, tmp_path):
     torch.save({"weight": cpu_packed, "scales_and_zeros": torch.from_numpy(sz32), "bias": torch.from_numpy(bias)}, path)
 
     mod = q.WeightOnlyInt4Linear(K, N, groupsize=g, bias=True, device=DEV, dtype=dtype)
-    result = mod.load_state_dict(torch.load(path, weights_only=True))
+    with pytest.warns(UserWarning, match="assuming the AVX-512 pack"):   # the tier was not stated
+        result = mod.load_state_dict(torch.load(path, weights_only=True))
     assert not result.missing_keys and not result.unexpected_keys
     assert mod.weight.dtype == torch.int32 and tuple(mod.weight.shape) == (N // 8, K // 32, 32, 1)
     np.testing.assert_array_equal(host(mod.weight), oracle.int4_pack_tc(codes, 2))      # the converter, bit for bit

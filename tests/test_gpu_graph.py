@@ -82,3 +82,79 @@ def test_replays_equal_eager(ops):
         torch.cuda.synchronize()
         for idx, (got, ref) in enumerate(zip(recorded, want)):
             assert torch.equal(got, ref), f"replay with seed {seed}: output {idx} differs from the eager call"
+
+
+def test_noalloc_entry_point_under_capture():
+    """tpq_int8_mm_dequant_noalloc recorded into graphs.  The first graph holds what is (when this file runs in a fresh
+    process) the first call on this device, so the lookup of the built-in buffer's address happens during the capture;
+    the second is recorded after eager calls.  Between the replays the inputs change and a smaller eager call leaves its
+    partial sums in the shared buffer.  Every replay must equal tpq_int8_mm_dequant_ws with a caller's workspace, bit
+    for bit (both add the same exact int32 partial sums)."""
+    import ctypes
+
+    from tensorplay_amd import _lib
+
+    lib = _lib.load()
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+    M, N, K = 300, 264, 2048
+    need = lib.tpq_int8_mm_workspace_bytes(M, N, K)
+    assert 0 < need <= lib.tpq_int8_mm_noalloc_max_bytes()
+    a = torch.empty((M, K), dtype=torch.int8, device=DEV)
+    w = torch.empty((N, K), dtype=torch.int8, device=DEV)
+    rs = torch.empty(M, device=DEV)
+    cs = torch.empty(N, device=DEV)
+    bias = torch.empty(N, device=DEV)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    # the smaller problem that dirties the shared buffer between replays
+    m2, n2, k2 = 130, 200, 1024
+    assert lib.tpq_int8_mm_workspace_bytes(m2, n2, k2) > 0
+    a2 = torch.randint(-128, 128, (m2, k2), dtype=torch.int8, device=DEV)
+    w2 = torch.randint(-128, 128, (n2, k2), dtype=torch.int8, device=DEV)
+    rs2, cs2 = torch.rand(m2, device=DEV), torch.rand(n2, device=DEV)
+    out2 = torch.empty((m2, n2), dtype=torch.float32, device=DEV)
+
+    def fill(seed):
+        gen = torch.Generator(device=DEV).manual_seed(seed)
+        a.copy_(torch.randint(-128, 128, a.shape, device=DEV, generator=gen).to(torch.int8))
+        w.copy_(torch.randint(-128, 128, w.shape, device=DEV, generator=gen).to(torch.int8))
+        rs.copy_(torch.rand(M, device=DEV, generator=gen) * 0.02 + 0.001)
+        cs.copy_(torch.rand(N, device=DEV, generator=gen) * 0.002 + 0.0001)
+        bias.copy_(torch.randn(N, device=DEV, generator=gen) * 0.01)
+
+    def record(out, dt):
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(graph, stream=stream):
+                s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                rc = lib.tpq_int8_mm_dequant_noalloc(ptr(a), ptr(w), ptr(rs), ptr(cs), ptr(bias), ptr(out), dt, M, N, K, s)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        return graph
+
+    def check(graph, out, dt, seeds):
+        for seed in seeds:
+            fill(seed)
+            s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            want = torch.full_like(out, 5)
+            rc = lib.tpq_int8_mm_dequant_ws(ptr(a), ptr(w), ptr(rs), ptr(cs), ptr(bias), ptr(want), dt, M, N, K, ptr(ws), need, s)
+            assert rc == 0, _lib.last_error()
+            # an eager call on a smaller problem: its partial sums stay in the shared buffer
+            assert lib.tpq_int8_mm_dequant_noalloc(ptr(a2), ptr(w2), ptr(rs2), ptr(cs2), None, ptr(out2), 0, m2, n2, k2, s) == 0
+            out.fill_(3)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.uint8), want.view(torch.uint8)), f"replay with seed {seed} differs from the _ws call"
+
+    fill(10)
+    out32 = torch.empty((M, N), dtype=torch.float32, device=DEV)
+    first = record(out32, 0)            # no noalloc call has been made before this capture in this file
+    check(first, out32, 0, (11, 12, 13))
+    out16 = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    second = record(out16, 2)           # recorded after eager calls
+    check(second, out16, 2, (14, 15))
+    check(first, out32, 0, (16,))       # and the first graph still replays correctly
