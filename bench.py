@@ -34,16 +34,17 @@ INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 M, K, N, GROUP = 1, 4096, 11008, 128
 GEMV_BYTES = N * K // 2 + (K // GROUP) * N * 4 + 2 * M * K + 2 * M * N   # 23,983,616
 GEMV_PROFILE = os.path.join(ROOT, "profiles", "int4_decode_gemv_M1_K4096_N11008.md")
+INT8_PROFILE = os.path.join(ROOT, "profiles", "int8_gemm_stagger_M2048_K4096_N4096.md")
 
 
-def measured_traffic_bytes():
-    """HBM bytes per launch of the GEMV kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
+def measured_traffic_bytes(profile=None):
+    """HBM bytes per launch of the GEMV kernel (or of the kernel of another profile summary) as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
     what the same counter reads for a 256 MiB device copy, --calibrate-copy).  The figure lives in the committed profile
     summary, on a line `traffic_bytes_per_launch: <bytes> (commit <hash>)`; None when that file or line is missing."""
     import re
 
     try:
-        m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", open(GEMV_PROFILE).read(), flags=re.M)
+        m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", open(profile or GEMV_PROFILE).read(), flags=re.M)
     except OSError:
         return None
     return int(m.group(1)) if m else None
@@ -555,6 +556,25 @@ def main() -> int:
             bytes_b = N * K // 2 + (K // GROUP) * N * 4 + 2 * mb * K + 2 * mb * N
             extras[f"int4_gemv_M{mb}_us"] = ms * 1e3
             extras[f"int4_gemv_M{mb}_GBs"] = bytes_b / (ms * 1e-3) / 1e9
+        # prefill block of 2048 rows on the same weight: the many-row route (dequantise to a dense fp16 weight, then the
+        # library's dense tile kernel), both steps through the C ABI, and the dense kernel alone
+        mb = 2048
+        xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
+        yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
+        dense = torch.empty((N, K), dtype=torch.float16, device=dev)
+
+        def prefill(i, both=True):
+            if both:
+                lib.tpq_int4_dequantize(packs[i % 4].data_ptr(), 2, N, K, GROUP, szs[i % 4].data_ptr(), _lib.F16, dense.data_ptr(), cur())
+            lib.tpq_dense_mm(xb.data_ptr(), _lib.F16, mb, K, dense.data_ptr(), N, yb.data_ptr(), cur())
+
+        for key, both in (("int4_prefill_M2048", True), ("dense_mm_f16_2048x4096x11008", False)):
+            gp = graph_of(lambda: [prefill(i, both) for i in range(16)])
+            gp.replay(); sync()
+            ms = steady(gp.replay, sync) / 16
+            extras[key + "_us"] = ms * 1e3
+            extras[key + "_TFLOPs"] = 2.0 * mb * N * K / (ms * 1e-3) / 1e12
+        del dense, gp
         del packs[1:], szs[1:]
         torch.cuda.empty_cache()
         # int8 weight-only decode (next-row op _weight_int8pack_mm): same shape, one byte per weight
@@ -621,8 +641,8 @@ def main() -> int:
         extras["int8_gemm_TOPS"] = tops
         extras["int8_gemm_frac_of_mfma_peak"] = tops / INT8_PEAK_TOPS
         roofline_int8 = {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
-                         "kernel": "int8_gemm_dma_kernel<bf16 dequant epilogue> (tpq_int8_mm_dequant)",
+                         "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": measured_traffic_bytes(INT8_PROFILE),
+                         "kernel": "gemm_stagger_kernel<bf16 dequant epilogue, int8> (tpq_int8_mm_dequant)",
                          "algorithmic_ops_per_launch": 2 * M8 * N8 * K8, "avg_launch_us": ms * 1e3,
                          "workload": "int8 x int8 prefill GEMM M=2048 K=4096 N=4096, fused per-row x per-channel dequant, bf16 out (BASELINE configs[2])"}
         # the vendor library's int8 GEMM on the same operands (torch._int_mm -> hipBLASLt), for scale: it
