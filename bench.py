@@ -461,6 +461,20 @@ def main() -> int:
     if not args.no_extras:  # the same graph seven more times: median step time
         reps = sorted(time_region(g.replay, sync, 1) / steps for _ in range(7))
         extras["int4_gemv_us_median_of_7_replays"] = reps[3] * 1e3
+        # Is the start-up of the K-step figure the host submitting the graph while the GPU idles behind the start event?
+        # The same K-step graph with the GPU still busy when the host gets there (a replay of it directly in front, no
+        # synchronization between).  It reads the same (6.58 against 6.59 us at 20 steps): the start-up of about 9 us
+        # belongs to every graph launch on the GPU side, whatever the host does.
+        def busy_start():
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            sync()
+            g.replay()
+            a.record()
+            g.replay()
+            b.record()
+            sync()
+            return a.elapsed_time(b) / steps
+        extras["int4_gemv_us_K_steps_gpu_busy_at_start"] = sorted(busy_start() for _ in range(7))[3] * 1e3
         # The K-step graph above carries its own start-up (about half a microsecond per step at 20 steps).  The same
         # kernel timed the way every other figure here is: a graph of 640 launches, warmed for >= 30 ms, median of 7.
         gs = graph_of(lambda: [gemv(i) for i in range(10 * copies)])
