@@ -26,7 +26,7 @@
 //     direct loads take a scalar base (advanced per stage by scalar instructions) plus a per-lane 32-bit offset that
 //     never changes.  The loads are spread between the reads, so the memory path has work from the start of a phase.
 //
-// Ring protocol (stage t lives in slot t % 3).  Group 0 reads stage t in phase 2t - 1, group 1 in phase 2t; the
+// Ring protocol (stage t lives in slot t % 3; the prologue requests stages 0 and 1 and group 0's share of stage 2).  Group 0 reads stage t in phase 2t - 1, group 1 in phase 2t; the
 // barrier that ends phase 2t frees the slot.  Every wavefront requests its sixth of a stage in its own memory phase:
 // group 0 requests stage t + 3 in phase 2t + 1, group 1 requests stage t + 2 in phase 2t (into the slot of stage
 // t - 1).  A stage must have landed when the barrier that ends phase 2t - 2 is crossed; each wavefront waits for its own
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
     constexpr std::integral_constant<int, kLoads> kOneStage{};
     constexpr std::integral_constant<int, 2 * kLoads> kTwoStages{};
 
-    // ---- prologue: scales, three stages requested, stage 0 landed ------------------------------------------------
+    // ---- prologue: scales, the first stages requested, stage 0 landed ------------------------------------------------
     // The scales of the tile go to LDS by direct loads as well (64 floats per wave-level load, source index clamped at the
     // edges), ahead of the stages in every requesting wavefront's order, so the wait for stage 0 covers them; nothing
     // here is a load the compiler counts, so it inserts no wait of its own in front of the first barrier.
@@ -317,12 +317,20 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
             if (src != nullptr && piece < 4 + BM / 64) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(src) : "memory", "m0");
         }
     }
+    // Group 1 leaves its share of stage 2 to its first memory phase (phase 0, as the ring protocol has it for every later
+    // stage): 24 loads fewer in front of the first barrier, which every wavefront reaches only after the memory path has
+    // accepted all its requests.
     request_stage(c0, 0);
     if (nk > 1) request_stage(c1, 1);
-    if (nk > 2) request_stage(c2, 2);
-    if (nk > 2) wait_loads(kTwoStages);
-    else if (nk > 1) wait_loads(kOneStage);
-    else wait_loads(c0);
+    if (wave < 4) {
+        if (nk > 2) request_stage(c2, 2);
+        if (nk > 2) wait_loads(kTwoStages);
+        else if (nk > 1) wait_loads(kOneStage);
+        else wait_loads(c0);
+    } else {
+        if (nk > 1) wait_loads(kOneStage);
+        else wait_loads(c0);
+    }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     TPQ_STAGGER_STAMP(1);
 
@@ -346,7 +354,7 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
     auto group1_step = [&](auto slot_c, auto steady, int kt) {
         constexpr int SLOT = decltype(slot_c)::value, PREV = (SLOT + kDmaStages - 1) % kDmaStages;
         constexpr bool STEADY = decltype(steady)::value;
-        if (STEADY || (kt >= 1 && kt + 2 < nk)) read_and_request(slot_c, std::integral_constant<int, PREV>{}, kt + 2);
+        if (STEADY || kt + 2 < nk) read_and_request(slot_c, std::integral_constant<int, PREV>{}, kt + 2);
         else read_stage(slot_c);
         stage_ready();
         if (STEADY || kt + 2 < nk) wait_loads(kOneStage);  // own share of kt + 1 landed (kt + 2 may be in flight)

@@ -93,6 +93,7 @@ def test_dispatch_does_not_depend_on_the_environment():
     assert "getenv" not in syms, "the library was built with -DTPQ_TUNING (sweep knobs compiled in)"
     exported = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
     assert "tpq_set_kernel_override" not in exported and "tpq_probe_read" not in exported
+    assert "tpq_quantize_stamps_read" not in exported and "g_quant_stamps" not in exported   # clock readings: the measuring build only
     # the test-hook build validates its arguments on the host
     hooked = ctypes.CDLL(build.HOOKS_LIB_PATH)
     hooked.tpq_set_kernel_override.argtypes = [ctypes.c_char_p, ctypes.c_int]
@@ -104,6 +105,12 @@ def test_dispatch_does_not_depend_on_the_environment():
     assert b"unknown route" in hooked.tpq_last_error()
     assert hooked.tpq_set_kernel_override(b"int8_row", 5) == _lib.TPQ_ERR_INVALID_VALUE
     assert hooked.tpq_set_kernel_override(None, 0) == _lib.TPQ_ERR_INVALID_VALUE
+    # the measuring build of the row quantizer: the operator plus the reader of its clock readings, argument checks on the host
+    stamps = ctypes.CDLL(build.QUANT_STAMPS_LIB_PATH)
+    stamps.tpq_quantize_stamps_read.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+    assert stamps.tpq_quantize_stamps_read(None, 8) == _lib.TPQ_ERR_INVALID_VALUE
+    assert stamps.tpq_quantize_stamps_read(16, 1 << 20) == _lib.TPQ_ERR_INVALID_VALUE
+    assert hasattr(stamps, "tpq_quantize_rowwise")
     # the probe library: argument checks of the column pattern, no launch
     probe = ctypes.CDLL(build.PROBE_LIB_PATH)
     probe.tpq_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
