@@ -273,6 +273,26 @@ int tpq_rms_norm(const void* x, int dtype, int64_t M, int64_t K, const void* wei
                  void* stream);
 
 /*
+ * The linear, float-output form of _quantized_packed_run with the weight prepacked by _quantized_weight_prepack
+ * (config/native_functions.yaml:11883-11886; CPU kernels
+ * p10/src/backend/cpu/QuantPacked.cpp:420-516 and :519-572, packed_real_value p10/include/QuantPacked.h:133-139):
+ *   acc[m][n] = sum_k x[m][k] w[n][k] - x_zero_point offsets[n] - w_zero_points[n] sum_k x[m][k]
+ *               + K x_zero_point w_zero_points[n]                                   (integers, exact)
+ *   out[m][n] = fmaf(float(acc), float(x_scale) * w_scales[n], bias ? bias[n] : 0);  relu: max(out, 0)
+ * x: [M, K] int8 or uint8 codes of a per-tensor quantized activation; packed: [N, packed_row_stride] int8 with
+ * packed_row_stride >= K (the reference pads rows to a multiple of 32 with zeros); offsets[n] = sum_k w[n][k] (int64),
+ * w_scales [N] float32, w_zero_points [N] int64, bias [N] float32 or null; out: [M, N] float32.  K <= 65536.
+ * workspace: device memory, 16-byte aligned, tpq_packed_linear_workspace_bytes(M, N, K, x_unsigned) bytes (the int32
+ * products, and a signed copy of unsigned activations); contents need not be preserved between calls.
+ * Bit-exact with the reference's arithmetic.  The convolution, requantised-output and activation forms are not built.
+ */
+size_t tpq_packed_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_unsigned);
+int tpq_packed_linear_float(const void* x, int x_unsigned, double x_scale, int64_t x_zero_point, const int8_t* packed,
+                            int64_t packed_row_stride, const int64_t* offsets, const float* w_scales,
+                            const int64_t* w_zero_points, const float* bias, int relu, float* out, int64_t M, int64_t N,
+                            int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The plain GEMM of the reference's many-row route for packed weights, which dequantises the weight to a dense
  * matrix of the activation type and multiplies once (p10/src/backend/cuda/QuantGemmKernels.cu:1296-1341, the call
  * gemm_impl(xf, wf.t(), out, 1.0, 0.0, nullptr) at :1339; likewise behind _weight_int8pack_mm and the low-bit linear):

@@ -44,6 +44,9 @@ SIGNATURES = {
     "tpq_int4_mm_swiglu_norm": [_ptr, _int, _i64, _i64, _ptr, _f32, _ptr, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, _ptr],
     "tpq_rms_norm": [_ptr, _int, _i64, _i64, _ptr, _f32, _ptr, _ptr],
     "tpq_dense_mm": [_ptr, _int, _i64, _i64, _ptr, _i64, _ptr, _ptr],
+    "tpq_packed_linear_workspace_bytes": [_i64, _i64, _i64, _int],
+    "tpq_packed_linear_float": [_ptr, _int, ctypes.c_double, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _i64, _ptr,
+                                ctypes.c_size_t, _ptr],
     "tpq_int4_mm_multi_norm": [_ptr, _int, _i64, _i64, _ptr, _f32, _int, _ptr, _int, _ptr, _i64, _ptr, _ptr, _ptr],
     "tpq_int4_dequantize": [_ptr, _int, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],
     "tpq_int4_pack_cpu_layout": [_ptr, _i64, _i64, _int, _int, _ptr, _ptr],

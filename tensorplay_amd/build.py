@@ -23,7 +23,7 @@ HOOKS_LIB_PATH = os.path.join(HERE, "libtpq_gfx950_hooks.so")
 PROBE_LIB_PATH = os.path.join(HERE, "libtpq_probe.so")
 QUANT_STAMPS_LIB_PATH = os.path.join(HERE, "libtpq_quant_stamps.so")  # the row quantizer with clock readings per phase (quant_stamps.py)
 
-SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "rms_norm.hip", "dense_mm.hip"]
+SOURCES = ["tpq_core.hip", "quantize_rowwise.hip", "int4_mm.hip", "int4_flight.hip", "int8_gemm.hip", "ternary_mm.hip", "int8pack_mm.hip", "affine_quant.hip", "lowbit_mm.hip", "rms_norm.hip", "dense_mm.hip", "packed_linear.hip"]
 # the sources that read a pinned route: the only ones compiled a second time for the test-hook library
 HOOK_SOURCES = ["tpq_core.hip", "int4_mm.hip", "int8_gemm.hip", "lowbit_mm.hip"]
 

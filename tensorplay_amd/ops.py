@@ -150,6 +150,53 @@ def _int8_mm_rescale(out: torch.Tensor, row_scale: torch.Tensor, col_scale: torc
     return result
 
 
+def _quantized_weight_prepack(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """int8 weight ``[N, K]`` -> (``packed`` int8 ``[N, ceil(K / 32) * 32]``, zero padded, ``offsets`` int64 ``[N]`` = row sums),
+    the reference's ``_quantized_weight_prepack`` (p10/src/backend/cpu/QuantPacked.cpp:519-533).  One-time, tensor ops."""
+    if weight.dim() != 2 or weight.dtype != torch.int8:
+        raise TypeError("_quantized_weight_prepack: expected a 2-D int8 weight")
+    _require_device(weight, "_quantized_weight_prepack")
+    n, k = weight.shape
+    packed = torch.zeros((n, (k + 31) // 32 * 32), dtype=torch.int8, device=weight.device)
+    packed[:, :k] = weight
+    return packed, weight.to(torch.int64).sum(1)
+
+
+def _quantized_packed_run_linear(x_codes: torch.Tensor, x_scale: float, x_zero_point: int, packed: torch.Tensor,
+                                 offsets: torch.Tensor, scales: torch.Tensor, zero_points: torch.Tensor,
+                                 bias: Optional[torch.Tensor], in_features: int, relu: bool = False) -> torch.Tensor:
+    """The linear, ``output_float=True`` form of the reference's ``_quantized_packed_run``
+    (p10/src/backend/cpu/QuantPacked.cpp:420-516, 537-572) on the codes of a per-tensor quantized activation:
+    ``fmaf(float(acc), float(x_scale) * scales[n], bias[n])`` with ``acc = x.w - xz off[n] - wz[n] sum(x) + K xz wz[n]``.
+    x_codes ``[M, K]`` int8 or uint8; packed / offsets from ``_quantized_weight_prepack``; result float32 ``[M, N]``."""
+    if x_codes.dim() != 2 or x_codes.dtype not in (torch.int8, torch.uint8):
+        raise TypeError("_quantized_packed_run_linear: expected 2-D int8 or uint8 activation codes")
+    if packed.dim() != 2 or packed.dtype != torch.int8:
+        raise TypeError("_quantized_packed_run_linear: expected a 2-D int8 packed weight")
+    m, k = x_codes.shape
+    n = packed.size(0)
+    if k != in_features or packed.size(1) < k:
+        raise ValueError("_quantized_packed_run_linear: K dimension mismatch")
+    if offsets.numel() != n or scales.numel() != n or zero_points.numel() != n or (bias is not None and bias.numel() != n):
+        raise ValueError("_quantized_packed_run_linear: per-channel parameters must have one entry per output channel")
+    _require_device(x_codes, "_quantized_packed_run_linear")
+    out = torch.empty((m, n), dtype=torch.float32, device=x_codes.device)
+    if m == 0 or n == 0:
+        return out
+    x, w = x_codes.contiguous(), packed.contiguous()
+    off, zp = offsets.to(torch.int64).contiguous(), zero_points.to(torch.int64).contiguous()
+    sc = scales.to(torch.float32).contiguous()
+    b = None if bias is None else bias.to(torch.float32).contiguous()
+    lib = _lib.load()
+    unsigned = int(x.dtype == torch.uint8)
+    with torch.cuda.device(x.device):
+        need = int(lib.tpq_packed_linear_workspace_bytes(m, n, k, unsigned))
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        _check(lib.tpq_packed_linear_float(_ptr(x), unsigned, float(x_scale), int(x_zero_point), _ptr(w), w.size(1), _ptr(off), _ptr(sc),
+                                           _ptr(zp), _ptr(b), int(bool(relu)), _ptr(out), m, n, k, _ptr(ws), need, _stream(x)))
+    return out
+
+
 def int8_mm_dequant(A_i8: torch.Tensor, B_t_i8: torch.Tensor, row_scale: torch.Tensor, col_scale: torch.Tensor,
                     bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """``_int_mm`` + ``_int8_mm_rescale`` (+ bias) in one launch.

@@ -199,3 +199,38 @@ def test_prefill_config3_full_size(ops):
     np.testing.assert_array_equal(host(fused)[rows], want)
     two_step = ops._int8_mm_rescale(acc, a_s, w_s).to(torch.bfloat16)
     assert torch.equal(fused, two_step)
+
+
+
+# ---- the prepacked quantized linear in its general form (A12) ------------------------------------------------------
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("shape", [(5, 7, 23), (5, 7, 64), (1, 8, 32), (33, 136, 4096), (300, 264, 2048), (2, 4104, 515), (64, 40, 65536)])
+def test_packed_linear_general_form_bit_exact(ops, shape, unsigned, relu):
+    """acc = x.w - xz off[n] - wz[n] sum(x) + K xz wz[n] in integers, fmaf(float(acc), float(xs) * ws[n], bias[n]):
+    bit-exact with the oracle's restatement of QuantPacked.cpp:420-516 (linear, float output), signed and unsigned
+    activation codes, rows that are and are not multiples of 32 long, the matrix-core and the generic product."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 31 + N + K + unsigned)
+    x = rng.integers(0 if unsigned else -128, 256 if unsigned else 128, size=(M, K)).astype(np.uint8 if unsigned else np.int8)
+    w = rng.integers(-128, 128, size=(N, K)).astype(np.int8)
+    xs, xz = 0.021, (137 if unsigned else -13)
+    scales = rng.uniform(0.004, 0.04, N).astype(np.float32)
+    zps = rng.integers(-5, 6, N).astype(np.int64)
+    bias = rng.normal(0, 0.7, N).astype(np.float32)
+    packed_ref, offsets_ref = oracle.weight_prepack(w)
+    packed, offsets = ops._quantized_weight_prepack(torch.from_numpy(w).to(DEV))
+    np.testing.assert_array_equal(packed.cpu().numpy(), packed_ref)
+    np.testing.assert_array_equal(offsets.cpu().numpy(), offsets_ref)
+    for b in (bias, None):
+        want = oracle.packed_run_linear_float(x, xs, xz, packed_ref, offsets_ref, scales, zps, b, K)
+        if relu:
+            want = np.maximum(want, 0.0)
+        got = ops._quantized_packed_run_linear(torch.from_numpy(x).to(DEV), xs, xz, packed, offsets, torch.from_numpy(scales).to(DEV),
+                                               torch.from_numpy(zps).to(DEV), None if b is None else torch.from_numpy(b).to(DEV), K, relu=relu)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+    # the hot path's special case: unit scales, zero zero-points, no bias = float(_int_mm)
+    plain = ops._quantized_packed_run_linear(torch.from_numpy(x).to(DEV), 1.0, 0, packed, offsets, torch.ones(N, device=DEV),
+                                             torch.zeros(N, dtype=torch.int64, device=DEV), None, K)
+    np.testing.assert_array_equal(plain.cpu().numpy(), (x.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32))
