@@ -90,7 +90,8 @@ struct ArithBF16 {  // 64 k per stage, v_mfma_f32_16x16x32_bf16
 // A, W: row-major [M][K], [N][K] with K contiguous; row_bytes = K * sizeof(element).
 // MB: blocks of 16 rows per wavefront: 4 (tile of 256 rows, what the description above and the numbers are about) or 2
 // (tile of 128 rows for problems with few rows or few tiles: per stage 32 wave-level loads against 16 MFMAs per
-// wavefront, so the vector memory path bounds it at about 700 clocks per stage).
+// wavefront, so the vector memory path bounds it at about 700 clocks per stage; int8, 4096 x 4096: 15.4 .. 18.8 us at
+// 256 .. 1024 rows, where the 256-row tiles take 21 .. 22 and the sliced launches 21 .. 32).
 template <class Tile, class Arith, int MB>
 __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restrict__ A, const char* __restrict__ W, int M, int N,
                                                                          int row_bytes, Tile tile, int vector_stores, int slices) {

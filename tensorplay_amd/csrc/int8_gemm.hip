@@ -10,17 +10,52 @@
 namespace tpq {
 namespace {
 
-// Which tiled kernel runs a shape.  Measured against the lock-step kernel with the same result bits (us, lock-step /
-// staggered): 2048 x 4096 x 4096 35.9 / 29.0, 2048 x 11008 x 4096 105 / 93, 2048 x 4096 x 11008 91 / 72, 8192^3 550 / 437,
-// 2048 x 2560 x 6912 44.5 / 35.0, 4096 x 4096 x 512 18.0 / 16.2.  Launches whose k range is cut into slices (few stages
-// per workgroup, 32-bit partial sums out) gain nothing from it (128 .. 1024 rows of 4096 x 4096: equal; 256 x 8192 x
-// 8192: 34.2 / 37.5) and stay on the lock-step kernel.  TPQ_INT8_FORM = dma / stagger in a tuning build forces one.
+// Which tiled kernel runs a shape.  Three forms, compared by an estimate of their clocks that reproduces the measured
+// times to about 10 % (2048 x 4096 x 4096 down to 65 rows, K = 2048 .. 11008, N = 2048 .. 11008):
+//   tall    256 x 128 tiles, staggered kernel: rounds of 256 tiles x (1,080 clocks per stage of 128 k + 9,000)
+//   short   128 x 128 tiles, staggered kernel: its stages are bound by the loads, 690 clocks each, + 8,000; wins where
+//           it needs one round and the tall form would leave most of the chip idle (256 .. 1024 rows of 4096 x 4096:
+//           15.3 .. 18.4 us against 21.2 .. 32.4 for the sliced form; 2048 x 2048: 9 against 13 .. 22)
+//   sliced  the k range of the tall tiles cut into slices (lock-step kernel, 1,450 clocks per stage, exact int32
+//           partial sums in a workspace) + the pass that adds them, whose traffic (2 x slices x M N x 4 bytes at about
+//           2,500 bytes per clock) is what it costs: left for few tiles with a long k range (256 rows of 11008 -> 4096:
+//           28 us against 35 short) and only where the caller brings a workspace.
+// Measured against the lock-step kernel with the same result bits (us, lock-step / staggered tall): 2048 x 4096 x 4096
+// 35.9 / 29.0, 2048 x 11008 x 4096 105 / 93, 2048 x 4096 x 11008 91 / 72, 8192^3 550 / 437, 2048 x 2560 x 6912 44.5 /
+// 35.0, 4096 x 4096 x 512 18.0 / 16.2.  Slices on the staggered kernel gain nothing (few stages per workgroup).
+// TPQ_INT8_FORM = dma / stagger / half in a tuning build forces a form.
+enum TiledForm { kTall = 0, kShort = 1, kSliced = 2 };
+struct TiledPlan {
+    TiledForm form;
+    int slices;
+};
+inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, bool may_slice) {
+    const double nk = static_cast<double>(K / kDmaRowBytes);
+    const int64_t cols = (N + 127) / 128, t256 = ((M + 255) / 256) * cols, t128 = ((M + 127) / 128) * cols;
+    const double tall = static_cast<double>((t256 + 255) / 256) * (nk * 1080.0 + 9000.0);
+    const double shrt = static_cast<double>((t128 + 255) / 256) * (nk * 690.0 + 8000.0);
+    double sliced = 1e30;
+    const int slices = may_slice ? dma_slices(M, N, K) : 1;
+    if (slices >= 2) {
+        const double per = static_cast<double>((K / kDmaRowBytes + slices - 1) / slices);
+        sliced = per * 1450.0 + 9000.0 + 3200.0 + 2.0 * static_cast<double>(M) * static_cast<double>(N) * 4.0 * slices / 2500.0;
+    }
+    if (K >= (1 << 23)) return TiledPlan{slices >= 2 ? kSliced : kTall, slices >= 2 ? slices : 1};  // beyond the staggered kernel's offsets
+    if (sliced < tall && sliced < shrt) return TiledPlan{kSliced, slices};
+    return TiledPlan{shrt < tall ? kShort : kTall, 1};
+}
+
 template <class Tile>
 int launch_tiled(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t K, Tile tile, hipStream_t s, int slices = 1) {
     const char* env = tuning_env("TPQ_INT8_FORM");
-    if (K >= (1 << 23) || (env && env[0] == 'd')) return launch_dma(a, w, M, N, K, tile, s, slices);
-    if (slices > 1 && !(env && env[0] == 's')) return launch_dma(a, w, M, N, K, tile, s, slices);
-    return launch_stagger(a, w, M, N, K, tile, s, slices);
+    if (slices > 1) {
+        if (env && env[0] == 's') return launch_stagger(a, w, M, N, K, tile, s, slices);
+        return launch_dma(a, w, M, N, K, tile, s, slices);
+    }
+    if (K >= (1 << 23) || (env && env[0] == 'd')) return launch_dma(a, w, M, N, K, tile, s, 1);
+    const bool use_short = env ? env[0] == 'h' : plan_tiled(M, N, K, false).form == kShort;
+    if (use_short) return launch_stagger_bytes<ArithI8, 2>(a, w, M, N, K, tile, s, 1, "int8 mfma gemm (staggered, 128 rows)");
+    return launch_stagger(a, w, M, N, K, tile, s, 1);
 }
 
 // partial [slices][M][N] int32 (16-byte aligned) := the slices of A W^T
@@ -57,7 +92,8 @@ inline int int8_slices(const void* a, const void* w, int64_t M, int64_t N, int64
     if (K <= 0 || !mfma_path_ok(a, w, M, N, K) || (force && force[0] == 'r')) return 1;
     const int decode_rows = int8_decode_rows(N) < 32 ? int8_decode_rows(N) : 32;
     if (M <= decode_rows && int8_decode_ok(a, w, M, N, K)) return 1;
-    return dma_slices(M, N, K);
+    const TiledPlan plan = plan_tiled(M, N, K, true);
+    return plan.form == kSliced ? plan.slices : 1;
 }
 
 // partial [slices][M][N] int32 -> out: acc = sum of the slices (exact), then (float(acc) * rs[m]) * cs[n] (+ bias[n]),
@@ -131,7 +167,8 @@ int launch_best(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t 
         return launch_int8_decode(a, w, M, N, K, ep, [N](const Epilogue& e, int64_t m0) { return rebase_rows(e, m0, N); }, s);
     // The ring-buffered kernel also wins when its 256 x 128 tiles fill only part of the chip: at K = N = 4096,
     // M = 512 / 1024 it takes 27.9 / 29.5 us against 33.9 / 39.4 us for the register-staged kernel on 128 x 64 tiles.
-    if (dma_path_ok(M, N, K) && !(force && force[0] == 'r')) return launch_tiled(a, w, M, N, K, to_tile(ep), s);
+    // (65 .. 128 rows included: on 128 x 128 tiles 128 rows of 4096 x 4096 take 15 us, 24.6 on the register-staged kernel)
+    if (K % kDmaRowBytes == 0 && !(force && force[0] == 'r')) return launch_tiled(a, w, M, N, K, to_tile(ep), s);
     return launch_mfma(a, w, M, N, K, ep, s);
 }
 

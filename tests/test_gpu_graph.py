@@ -99,7 +99,7 @@ def test_noalloc_entry_point_under_capture():
     def ptr(t):
         return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
-    M, N, K = 300, 264, 2048
+    M, N, K = 300, 264, 8192   # few tiles, long K: the shape is one that cuts the k range into slices
     need = lib.tpq_int8_mm_workspace_bytes(M, N, K)
     assert 0 < need <= lib.tpq_int8_mm_noalloc_max_bytes()
     a = torch.empty((M, K), dtype=torch.int8, device=DEV)
@@ -109,7 +109,7 @@ def test_noalloc_entry_point_under_capture():
     bias = torch.empty(N, device=DEV)
     ws = torch.empty(need, dtype=torch.uint8, device=DEV)
     # the smaller problem that dirties the shared buffer between replays
-    m2, n2, k2 = 130, 200, 1024
+    m2, n2, k2 = 130, 200, 4096
     assert lib.tpq_int8_mm_workspace_bytes(m2, n2, k2) > 0
     a2 = torch.randint(-128, 128, (m2, k2), dtype=torch.int8, device=DEV)
     w2 = torch.randint(-128, 128, (n2, k2), dtype=torch.int8, device=DEV)

@@ -26,8 +26,10 @@ SHAPES = [(5, 7, 3), (1, 1, 1), (64, 12, 32), (16, 1024, 1024), (64, 128, 32), (
           # decode kernel: 1..64 rows in slabs of 32 / 16, K a multiple of 128, ragged N, both widths of workgroup
           (1, 128, 40), (17, 256, 24), (48, 384, 72), (33, 4096, 100), (7, 11008, 64),
           (64, 256, 6150), (49, 128, 8200), (8, 384, 16400), (31, 256, 6144), (16, 128, 9000), (64, 512, 17),
-          # tiled kernel with the k range in slices (few tiles, long K), ragged last slice
+          # 128-row tiles of the staggered kernel (65 rows and more where one round of them covers the problem)
           (130, 1024, 200), (300, 2048, 136), (65, 1152, 64), (257, 1280, 100), (33, 1024, 10248),
+          # tiled kernel with the k range in slices (few tiles, long K), ragged last slice
+          (130, 4096, 200), (300, 8192, 136), (65, 4608, 64), (257, 5120, 100), (300, 4224, 136),
           # one or two rows on the row kernel: a last chunk past K, several passes per channel, ragged N, the long rows
           # that fall back to the matrix-core kernel (more than 32768 k), and 3 / 4 rows (that kernel by default)
           (2, 4224, 10), (1, 20480, 13), (2, 32768, 9), (1, 36864, 8), (2, 4096, 8200), (1, 8192, 16390), (3, 4096, 50), (4, 256, 7),
@@ -71,10 +73,11 @@ def test_int_mm_unsigned_lhs_out_and_empty(ops):
         ops._int_mm(torch.zeros(2, 3, dtype=torch.int8, device=DEV), torch.zeros(2, 2, dtype=torch.int8, device=DEV))
 
 
-@pytest.mark.parametrize("shape", [(32, 4096, 11008), (128, 4096, 4096), (48, 11008, 4096), (512, 4096, 4096)])
+@pytest.mark.parametrize("shape", [(32, 4096, 11008), (128, 4096, 4096), (48, 11008, 4096), (512, 4096, 4096), (128, 8192, 8192)])
 def test_int_mm_decode_and_sliced_kernels_at_model_sizes(ops, shape):
-    """The decode kernel (32 rows per pass, both widths of workgroup) and the sliced tiled kernel at real layer sizes,
-    with the extremes in: exact against numpy, and against the un-sliced single launch through the C ABI."""
+    """The decode kernel (32 rows per pass, both widths of workgroup), the 128-row tiles and the sliced tiled kernel
+    (128 rows of 8192 x 8192) at real layer sizes, with the extremes in: exact against numpy, and against the single
+    launch through the C ABI."""
     M, K, N = shape
     rng = np.random.default_rng(M + K + N)
     a = _rand_i8(rng, (M, K))

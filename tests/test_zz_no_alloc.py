@@ -67,11 +67,11 @@ def test_noalloc_equals_workspace_entry_point_two_calls_in_a_row():
     from tensorplay_amd import _lib
 
     lib = _lib.load()
-    print("noalloc: 300x264x2048 f32 then 130x200x1024 bf16", flush=True)
-    _run_pair(lib, 300, 264, 2048, torch.float32, True, 1)   # first call: fills the built-in buffer
-    _run_pair(lib, 130, 200, 1024, torch.float32, False, 2)  # second, smaller: the buffer still holds the first call's sums
-    _run_pair(lib, 300, 264, 2048, torch.bfloat16, True, 3)
-    _run_pair(lib, 132, 128, 1152, torch.float16, False, 4)
+    print("noalloc: 300x264x8192 f32 then 130x200x4096 f32", flush=True)
+    _run_pair(lib, 300, 264, 8192, torch.float32, True, 1)   # first call: fills the built-in buffer
+    _run_pair(lib, 130, 200, 4096, torch.float32, False, 2)  # second, smaller: the buffer still holds the first call's sums
+    _run_pair(lib, 300, 264, 8192, torch.bfloat16, True, 3)
+    _run_pair(lib, 132, 128, 4608, torch.float16, False, 4)
 
 
 def test_noalloc_rejects_what_does_not_fit_and_passes_on_what_needs_no_scratch():
@@ -80,7 +80,7 @@ def test_noalloc_rejects_what_does_not_fit_and_passes_on_what_needs_no_scratch()
     lib = _lib.load()
     limit = lib.tpq_int8_mm_noalloc_max_bytes()
     assert limit == 16 << 20
-    M, N, K = 512, 4096, 4096   # 64 tiles -> 4 slices of 512 x 4096 int32 = 32 MiB
+    M, N, K = 256, 4096, 11008   # 32 tiles, 86 stages -> 8 slices of 256 x 4096 int32 = 32 MiB
     need = lib.tpq_int8_mm_workspace_bytes(M, N, K)
     assert need > limit
     rc = lib.tpq_int8_mm_dequant_noalloc(None, None, None, None, None, None, 0, M, N, K, None)
