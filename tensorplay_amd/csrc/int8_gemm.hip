@@ -10,20 +10,26 @@
 namespace tpq {
 namespace {
 
-// Which tiled kernel runs a shape.  Three forms, compared by an estimate of their clocks that reproduces the measured
-// times to about 10 % (2048 x 4096 x 4096 down to 65 rows, K = 2048 .. 11008, N = 2048 .. 11008):
+// Which tiled kernel runs a shape.  Three forms, compared by an estimate of their clocks fitted to measurements with the
+// weight streaming from HBM (65 .. 2048 rows, K = 2048 .. 11008, N = 2048 .. 11008; the estimate picks the measured
+// best or a tie everywhere):
 //   tall    256 x 128 tiles, staggered kernel: rounds of 256 tiles x (1,080 clocks per stage of 128 k + 9,000)
-//   short   128 x 128 tiles, staggered kernel: its stages are bound by the loads, 690 clocks each, + 8,000; wins where
-//           it needs one round and the tall form would leave most of the chip idle (256 .. 1024 rows of 4096 x 4096:
-//           15.3 .. 18.4 us against 21.2 .. 32.4 for the sliced form; 2048 x 2048: 9 against 13 .. 22)
-//   sliced  the k range of the tall tiles cut into slices (lock-step kernel, 1,450 clocks per stage, exact int32
-//           partial sums in a workspace) + the pass that adds them, whose traffic (2 x slices x M N x 4 bytes at about
-//           2,500 bytes per clock) is what it costs: left for few tiles with a long k range (256 rows of 11008 -> 4096:
-//           28 us against 35 short) and only where the caller brings a workspace.
+//   short   128 x 128 tiles, staggered kernel: its stages are bound by the loads, 690 clocks each, + 8,000
+//   both    not below 128 K / 12.5 clocks: a workgroup streams its 128 K bytes of weight with three stages (48 KB) in
+//           flight, about 25 GB/s per compute unit from HBM (4096 x 4096 on short tiles: 21.5 us at any row count,
+//           13 .. 19 us with the weight in the caches)
+//   sliced  the k range of the tall tiles cut into slices (lock-step kernel, exact int32 partial sums in a workspace:
+//           1,450 clocks per stage, up to 2,000 with 32 and more stages per workgroup) + the pass that adds them, whose
+//           traffic (2 x slices x M N x 4 bytes at about 2,500 bytes per clock) is what it costs; only where the caller
+//           brings a workspace.
+// us, weights rotating through HBM, slices wherever they apply / this plan: 4096 x 4096 at 128 / 512 / 1024 rows 17.2 /
+// 25.1 / 32.8 -> 17.2 / 21.3 / 22.4; 4096 -> 11008 at 65 / 256 rows 23.9 / 29.3 -> 21.6 / 24.2; 8192 x 8192 at 384 / 512
+// rows 49.0 / 52.1 -> 43.4 / 43.3; 11008 -> 4096 at 1024 rows 63.3 -> 57.1; 2048 x 2048 at 512 / 1024 rows 15.1 / 19.9 ->
+// 12.6 / 12.5.
 // Measured against the lock-step kernel with the same result bits (us, lock-step / staggered tall): 2048 x 4096 x 4096
 // 35.9 / 29.0, 2048 x 11008 x 4096 105 / 93, 2048 x 4096 x 11008 91 / 72, 8192^3 550 / 437, 2048 x 2560 x 6912 44.5 /
 // 35.0, 4096 x 4096 x 512 18.0 / 16.2.  Slices on the staggered kernel gain nothing (few stages per workgroup).
-// TPQ_INT8_FORM = dma / stagger / half in a tuning build forces a form.
+// TPQ_INT8_FORM = dma / stagger / half and TPQ_INT8_PLAN = o (slices wherever they apply) / h in a tuning build force a form.
 enum TiledForm { kTall = 0, kShort = 1, kSliced = 2 };
 struct TiledPlan {
     TiledForm form;
@@ -32,17 +38,26 @@ struct TiledPlan {
 inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, bool may_slice) {
     const double nk = static_cast<double>(K / kDmaRowBytes);
     const int64_t cols = (N + 127) / 128, t256 = ((M + 255) / 256) * cols, t128 = ((M + 127) / 128) * cols;
-    const double tall = static_cast<double>((t256 + 255) / 256) * (nk * 1080.0 + 9000.0);
-    const double shrt = static_cast<double>((t128 + 255) / 256) * (nk * 690.0 + 8000.0);
+    const double stream = 128.0 * static_cast<double>(K) / 12.5;  // a tile's weight bytes at what one compute unit pulls from HBM
+    const double tall_tile = nk * 1080.0 + 9000.0, short_tile = nk * 690.0 + 8000.0;
+    const double tall = static_cast<double>((t256 + 255) / 256) * (tall_tile > stream ? tall_tile : stream);
+    const double shrt = static_cast<double>((t128 + 255) / 256) * (short_tile > stream ? short_tile : stream);
     double sliced = 1e30;
     const int slices = may_slice ? dma_slices(M, N, K) : 1;
     if (slices >= 2) {
         const double per = static_cast<double>((K / kDmaRowBytes + slices - 1) / slices);
-        sliced = per * 1450.0 + 9000.0 + 3200.0 + 2.0 * static_cast<double>(M) * static_cast<double>(N) * 4.0 * slices / 2500.0;
+        const double stage = 1450.0 + 550.0 * (per < 32.0 ? per / 32.0 : 1.0);
+        sliced = per * stage + 9000.0 + 3200.0 + 2.0 * static_cast<double>(M) * static_cast<double>(N) * 4.0 * slices / 2500.0;
     }
-    if (K >= (1 << 23)) return TiledPlan{slices >= 2 ? kSliced : kTall, slices >= 2 ? slices : 1};  // beyond the staggered kernel's offsets
-    if (sliced < tall && sliced < shrt) return TiledPlan{kSliced, slices};
-    return TiledPlan{shrt < tall ? kShort : kTall, 1};
+    const char* env = tuning_env("TPQ_INT8_PLAN");  // o: slices wherever they apply, else tall; h: short
+    if (K >= (1 << 23) || (env && env[0] == 'o')) return TiledPlan{slices >= 2 ? kSliced : kTall, slices >= 2 ? slices : 1};  // K: beyond the staggered kernel's offsets
+    if (env && env[0] == 'h') return TiledPlan{kShort, 1};
+    // One round of short tiles is never slower than the tall ones on the same problem (fewer compute units busy on tall
+    // tiles, and those run at the power limit: 768 rows of 11008 -> 4096 from HBM 55 us short, 81 tall).
+    const bool one_round_short = t128 <= 256;
+    const double unsliced = one_round_short ? shrt : (shrt < tall ? shrt : tall);
+    if (sliced < unsliced) return TiledPlan{kSliced, slices};
+    return TiledPlan{one_round_short || shrt < tall ? kShort : kTall, 1};
 }
 
 template <class Tile>

@@ -60,8 +60,8 @@ def test_int8_workspace_sizing_is_host_logic():
     assert ws(16, 4096, 4096) == 0            # decode kernel
     assert ws(32, 4096, 4096) == 0
     assert ws(2048, 4096, 4096) == 0          # 256 tiles fill the chip
-    assert ws(128, 4096, 4096) == 0           # one round of 128 x 128 tiles is estimated faster than slices + the adding pass
-    assert ws(512, 4096, 4096) == 0
+    assert ws(128, 4096, 4096) == 8 * 128 * 4096 * 4     # 32 tiles of 256 x 128 -> 8 slices of 4 stages
+    assert ws(512, 4096, 4096) == 0           # one round of 128 x 128 tiles is estimated faster than 4 slices + the adding pass
     assert ws(256, 4096, 11008) == 8 * 256 * 4096 * 4    # few tiles, long K: 32 tiles of 256 x 128 -> 8 slices
     assert ws(128, 8192, 8192) == 4 * 128 * 8192 * 4     # 64 tiles -> 4 slices of 16 stages
     assert ws(128, 4096, 512) == 0            # K of four stages: nothing to cut
