@@ -1,5 +1,5 @@
-// Tiled GEMM C = A W^T (int8 -> int32, or float16 / bfloat16 -> float32), staggered form: 256 x 128 tile per workgroup, three-stage LDS ring of whole 128-byte rows filled by
-// direct global -> LDS loads, eight wavefronts in eight positions of 64 x 64 (v_mfma_i32_16x16x64_i8), the two
+// Tiled GEMM C = A W^T (int8 -> int32, or float16 / bfloat16 -> float32), staggered form: 256 x 128 tile per workgroup,
+// three-stage LDS ring of whole 128-byte rows filled by direct global -> LDS loads, eight wavefronts in eight positions of 64 x 64 (v_mfma_i32_16x16x64_i8), the two
 // wavefronts of a SIMD half a stage apart.
 //
 // What the form answers (measured on MI355X at 2048 x 4096 x 4096, per stage of 128 bytes of k and compute unit): the
@@ -26,12 +26,16 @@
 //     direct loads take a scalar base (advanced per stage by scalar instructions) plus a per-lane 32-bit offset that
 //     never changes.  The loads are spread between the reads, so the memory path has work from the start of a phase.
 //
-// Ring protocol (stage t lives in slot t % 3; the prologue requests stages 0 and 1 and group 0's share of stage 2).  Group 0 reads stage t in phase 2t - 1, group 1 in phase 2t; the
-// barrier that ends phase 2t frees the slot.  Every wavefront requests its sixth of a stage in its own memory phase:
-// group 0 requests stage t + 3 in phase 2t + 1, group 1 requests stage t + 2 in phase 2t (into the slot of stage
-// t - 1).  A stage must have landed when the barrier that ends phase 2t - 2 is crossed; each wavefront waits for its own
-// share in front of that barrier (vector loads of a wavefront complete in order, so "my share of t + 1 has landed" is
-// "at most the six loads of t + 2 are outstanding").  Both groups cross 2 nk - 1 barriers after the first.
+// Ring protocol for a ring of S stages (S = 3; stage t lives in slot t % S; the prologue requests stages 0 .. S - 2 and
+// group 0's share of stage S - 1).  Group 0 reads stage t in phase 2t - 1,
+// group 1 in phase 2t; the barrier that ends phase 2t frees the slot.  Every wavefront requests its eighth of a stage in
+// its own memory phase: group 0 requests stage t + S in phase 2t + 1, group 1 requests stage t + S - 1 in phase 2t (into
+// the slot of stage t - 1).  A stage must have landed when the barrier that ends phase 2t - 2 is crossed; each wavefront
+// waits for its own share in front of that barrier (vector loads of a wavefront complete in order, so "my share of
+// t + 1 has landed" is "at most the loads of the S - 2 stages behind it are outstanding").  Both groups cross 2 nk - 1
+// barriers after the first.  A fourth stage for the 128-row tile (128 KB of LDS) was measured where the weight streams
+// from HBM and a compute unit pulls about 25 GB/s of it: no change (4096 x 4096 at 256 .. 1024 rows 21.1 .. 22.5 us
+// against 21.4 .. 22.6), so that rate is not set by the depth of the ring.
 //
 // Four extra wavefronts that do nothing but request (one per SIMD, 168 registers per wavefront) were built and measured:
 // the loop drops from 1085 to 1064 clocks per stage, the first stage arrives 1000 clocks later, same time; not kept.
@@ -64,6 +68,25 @@ __device__ unsigned long long g_stagger_coarse[4 * 8];  // [start, first barrier
 #endif
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+
+// f(integral_constant<int, I>) for I = FIRST .. LAST - 1, unrolled at compile time
+template <int FIRST, int LAST, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>{});
+        static_for<FIRST + 1, LAST>(f);
+    }
+}
+// if (base + 0 < limit) { f(0); if (base + 1 < limit) { f(1); ... } }: up to DEPTH steps as nested straight-line code
+template <int D, int DEPTH, class F>
+__device__ __forceinline__ void nested_while_below(int base, int limit, F&& f) {
+    if constexpr (D < DEPTH) {
+        if (base + D < limit) {
+            f(std::integral_constant<int, D>{});
+            nested_while_below<D + 1, DEPTH>(base, limit, f);
+        }
+    }
+}
 
 // The operand types the form multiplies.  A stage is 128 bytes of k per row whatever the type, and the lane layout of
 // the 16-byte fragments is the same for all three instructions (lane (r, c): row r, bytes 16 c .. 16 c + 15 of a k-half
@@ -100,7 +123,8 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
     constexpr int BM = 64 * MB, BN = 128, WM = 16 * MB, WN = 64;
     static_assert(MB == 4 || MB == 2, "two tile heights are built");
     constexpr int kStageBytes = (BM + BN) * kDmaRowBytes;  // 48 KB (32 KB)
-    constexpr int kRingBytes = kDmaStages * kStageBytes;   // 144 KB (96 KB)
+    constexpr int S = kDmaStages;                          // ring depth (the loop control below is written for any depth >= 3)
+    constexpr int kRingBytes = S * kStageBytes;            // 144 KB (96 KB)
     constexpr int kRequesters = 8;
     constexpr int kLoadsA = BM / 8 / kRequesters, kLoadsW = BN / 8 / kRequesters, kLoads = kLoadsA + kLoadsW;  // 4 + 2
     extern __shared__ uint4 ring[];
@@ -174,8 +198,6 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
         }
     };
     constexpr std::integral_constant<int, 0> c0{};
-    constexpr std::integral_constant<int, 1> c1{};
-    constexpr std::integral_constant<int, 2> c2{};
     constexpr std::integral_constant<int, kLoads> cAll{};
         auto request_stage = [&](auto slot_c, int kt) { request(c0, cAll, slot_c, kt); };
 
@@ -187,9 +209,9 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
     // they share one swizzle value.
     const int frag_row = lane & 15, frag_chunk = lane >> 4;
     const uint32_t sw = (frag_row >> 1) & 7;
-    uint32_t addr_a[kDmaStages][2], addr_b[kDmaStages][2];
+    uint32_t addr_a[S][2], addr_b[S][2];
 #pragma unroll
-    for (int s = 0; s < kDmaStages; ++s)
+    for (int s = 0; s < S; ++s)
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) {
             const uint32_t chunk = ((kh * 4 + frag_chunk) ^ sw) * 16;
@@ -296,8 +318,18 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
     };
 #endif
     auto wait_loads = [&](auto allowed) { __builtin_amdgcn_s_waitcnt(vmcnt_imm(decltype(allowed)::value)); };
-    constexpr std::integral_constant<int, kLoads> kOneStage{};
-    constexpr std::integral_constant<int, 2 * kLoads> kTwoStages{};
+    // at most `stages` (0 .. S - 1, wave-uniform) whole stages of this wavefront's requests may still be outstanding
+    auto wait_stages = [&](int stages) {
+        bool done = false;
+        static_for<0, S>([&](auto i) {
+            constexpr int N = S - 1 - decltype(i)::value;  // S - 1 down to 0
+            if (!done && stages >= N) {
+                wait_loads(std::integral_constant<int, N * kLoads>{});
+                done = true;
+            }
+        });
+    };
+    constexpr std::integral_constant<int, (S - 2) * kLoads> kSteadyWait{};  // own share of the next stage landed, the S - 2 after it may be in flight
 
     // ---- prologue: scales, the first stages requested, stage 0 landed ------------------------------------------------
     // The scales of the tile go to LDS by direct loads as well (64 floats per wave-level load, source index clamped at the
@@ -318,48 +350,44 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
             if (src != nullptr && piece < 4 + BM / 64) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(src) : "memory", "m0");
         }
     }
-    // Group 1 leaves its share of stage 2 to its first memory phase (phase 0, as the ring protocol has it for every later
-    // stage): 24 loads fewer in front of the first barrier, which every wavefront reaches only after the memory path has
-    // accepted all its requests.
-    request_stage(c0, 0);
-    if (nk > 1) request_stage(c1, 1);
-    if (wave < 4) {
-        if (nk > 2) request_stage(c2, 2);
-        if (nk > 2) wait_loads(kTwoStages);
-        else if (nk > 1) wait_loads(kOneStage);
-        else wait_loads(c0);
-    } else {
-        if (nk > 1) wait_loads(kOneStage);
-        else wait_loads(c0);
+    // Stages 0 .. S - 2 by everybody, stage S - 1 by group 0 only: group 1 leaves its share of it to its first memory
+    // phase (phase 0, as the ring protocol has it for every later stage), which is that many loads fewer in front of the
+    // first barrier; every wavefront reaches it only after the memory path has accepted all its requests.
+    {
+        const int mine = wave < 4 ? (nk < S ? nk : S) : (nk < S - 1 ? nk : S - 1);  // stages this wavefront requests here
+        static_for<0, S>([&](auto st) {
+            if (decltype(st)::value < mine) request_stage(st, decltype(st)::value);
+        });
+        wait_stages(mine - 1);  // stage 0 (and the scales in front of it) landed
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     TPQ_STAGGER_STAMP(1);
 
     // one phase pair of a wavefront; SLOT = slot of stage kt.  STEADY: every stage named exists, no conditions.
-    // group 0: multiply kt | read kt + 1, request kt + 3 into SLOT
+    // group 0: multiply kt | read kt + 1, request kt + S into SLOT
     auto group0_step = [&](auto slot_c, auto steady, int kt) {
-        constexpr int SLOT = decltype(slot_c)::value, NEXT = (SLOT + 1) % kDmaStages;
+        constexpr int SLOT = decltype(slot_c)::value, NEXT = (SLOT + 1) % S;
         constexpr bool STEADY = decltype(steady)::value;
         multiply_stage();
-        if (STEADY || kt + 2 < nk) wait_loads(kOneStage);  // own share of kt + 1 landed (kt + 2 may be in flight)
-        else wait_loads(c0);
+        if (STEADY) wait_loads(kSteadyWait);  // own share of kt + 1 landed (kt + 2 .. may be in flight)
+        else wait_stages(nk - kt - 2 < 0 ? 0 : nk - kt - 2 < S - 2 ? nk - kt - 2 : S - 2);
         phase_end();
         if (STEADY || kt + 1 < nk) {
-            if (STEADY || kt + kDmaStages < nk) read_and_request(std::integral_constant<int, NEXT>{}, slot_c, kt + kDmaStages);
+            if (STEADY || kt + S < nk) read_and_request(std::integral_constant<int, NEXT>{}, slot_c, kt + S);
             else read_stage(std::integral_constant<int, NEXT>{});
             stage_ready();
             phase_end();
         }
     };
-    // group 1: read kt, request kt + 2 into the slot of kt - 1 | multiply kt
+    // group 1: read kt, request kt + S - 1 into the slot of kt - 1 | multiply kt
     auto group1_step = [&](auto slot_c, auto steady, int kt) {
-        constexpr int SLOT = decltype(slot_c)::value, PREV = (SLOT + kDmaStages - 1) % kDmaStages;
+        constexpr int SLOT = decltype(slot_c)::value, PREV = (SLOT + S - 1) % S;
         constexpr bool STEADY = decltype(steady)::value;
-        if (STEADY || kt + 2 < nk) read_and_request(slot_c, std::integral_constant<int, PREV>{}, kt + 2);
+        if (STEADY || kt + S - 1 < nk) read_and_request(slot_c, std::integral_constant<int, PREV>{}, kt + S - 1);
         else read_stage(slot_c);
         stage_ready();
-        if (STEADY || kt + 2 < nk) wait_loads(kOneStage);  // own share of kt + 1 landed (kt + 2 may be in flight)
-        else wait_loads(c0);
+        if (STEADY) wait_loads(kSteadyWait);  // own share of kt + 1 landed (kt + 2 .. may be in flight)
+        else wait_stages(nk - kt - 2 < 0 ? 0 : nk - kt - 2 < S - 2 ? nk - kt - 2 : S - 2);
         phase_end();
         multiply_stage();
         if (STEADY || kt + 1 < nk) phase_end();
@@ -367,45 +395,25 @@ __global__ __launch_bounds__(512) void gemm_stagger_kernel(const char* __restric
     constexpr std::true_type kSteady{};
     constexpr std::false_type kChecked{};
 
+    // The steady loops are unrolled S times so that the ring slot is a constant; what is left behind them (at most
+    // 2 S - 1 stages) is nested straight-line code with the conditions of the ends (a loop with a runtime slot made
+    // the compiler copy the accumulators between its arms).
     int kt = 0;
     if (wave < 4) {
         read_stage(c0);
         stage_ready();
-        for (; kt + 2 + kDmaStages < nk; kt += 3) {
-            group0_step(c0, kSteady, kt);
-            group0_step(c1, kSteady, kt + 1);
-            group0_step(c2, kSteady, kt + 2);
-        }
-        if (kt < nk) {  // at most five stages left, the first in slot 0
-            group0_step(c0, kChecked, kt);
-            if (kt + 1 < nk) {
-                group0_step(c1, kChecked, kt + 1);
-                if (kt + 2 < nk) {
-                    group0_step(c2, kChecked, kt + 2);
-                    if (kt + 3 < nk) {
-                        group0_step(c0, kChecked, kt + 3);
-                        if (kt + 4 < nk) group0_step(c1, kChecked, kt + 4);
-                    }
-                }
-            }
-        }
+        for (; kt + 2 * S - 1 < nk; kt += S)
+            static_for<0, S>([&](auto i) { group0_step(i, kSteady, kt + decltype(i)::value); });
+        nested_while_below<0, 2 * S - 1>(kt, nk, [&](auto d) {  // the first of them in slot 0
+            group0_step(std::integral_constant<int, decltype(d)::value % S>{}, kChecked, kt + decltype(d)::value);
+        });
     } else {
         group1_step(c0, kChecked, 0);
-        for (kt = 1; kt + 4 < nk; kt += 3) {
-            group1_step(c1, kSteady, kt);
-            group1_step(c2, kSteady, kt + 1);
-            group1_step(c0, kSteady, kt + 2);
-        }
-        if (kt < nk) {  // at most four stages left, the first in slot 1
-            group1_step(c1, kChecked, kt);
-            if (kt + 1 < nk) {
-                group1_step(c2, kChecked, kt + 1);
-                if (kt + 2 < nk) {
-                    group1_step(c0, kChecked, kt + 2);
-                    if (kt + 3 < nk) group1_step(c1, kChecked, kt + 3);
-                }
-            }
-        }
+        for (kt = 1; kt + 2 * S - 2 < nk; kt += S)
+            static_for<0, S>([&](auto i) { group1_step(std::integral_constant<int, (1 + decltype(i)::value) % S>{}, kSteady, kt + decltype(i)::value); });
+        nested_while_below<0, 2 * S - 2>(kt, nk, [&](auto d) {  // the first of them in slot 1
+            group1_step(std::integral_constant<int, (1 + decltype(d)::value) % S>{}, kChecked, kt + decltype(d)::value);
+        });
     }
 
     // ---- epilogue: every wavefront finishes its own 64 x 64 block ------------------------------------------------

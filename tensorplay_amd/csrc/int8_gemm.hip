@@ -15,8 +15,8 @@ namespace {
 // best or a tie everywhere):
 //   tall    256 x 128 tiles, staggered kernel: rounds of 256 tiles x (1,080 clocks per stage of 128 k + 9,000)
 //   short   128 x 128 tiles, staggered kernel: its stages are bound by the loads, 690 clocks each, + 8,000
-//   both    not below 128 K / 12.5 clocks: a workgroup streams its 128 K bytes of weight with three stages (48 KB) in
-//           flight, about 25 GB/s per compute unit from HBM (4096 x 4096 on short tiles: 21.5 us at any row count,
+//   both    not below 128 K / 12.5 clocks: a workgroup streams its 128 K bytes of weight at about 25 GB/s per compute
+//           unit from HBM, whatever the depth of its ring (4096 x 4096 on short tiles: 21.5 us at any row count,
 //           13 .. 19 us with the weight in the caches)
 //   sliced  the k range of the tall tiles cut into slices (lock-step kernel, exact int32 partial sums in a workspace:
 //           1,450 clocks per stage, up to 2,000 with 32 and more stages per workgroup) + the pass that adds them, whose
