@@ -342,7 +342,7 @@ int tpq_weight_int8pack_mm(const void* x, int dtype, int64_t M, int64_t K, const
 
 /*
  * Dense [N, K] weight of `dtype` from the int8 weight and its per-row scales: T(float(w) * scale[n]).
- * For many activation rows the host op multiplies this with a library GEMM instead of streaming the
+ * For many activation rows the host op multiplies this with tpq_dense_mm instead of streaming the
  * int8 weight once per 16 or 32 rows (the reference's device op runs its batched GEMV at every size,
  * p10/src/backend/cuda/QuantGemmKernels.cu:345-405).
  */

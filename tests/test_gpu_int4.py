@@ -231,7 +231,7 @@ def test_dequantize_bf16_non_finite_scale(ops):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 def test_mm_many_rows_takes_the_dense_route(ops, dtype):
-    """More than INT4_PREFILL_ROWS rows: dequantise + library GEMM, the reference's device formulation."""
+    """More than INT4_PREFILL_ROWS rows: dequantise + one dense GEMM (tpq_dense_mm where K allows), the reference's device formulation."""
     M, N, K, group = ops.INT4_PREFILL_ROWS + 37, 136, 512, 128
     rng = np.random.default_rng(77)
     codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)

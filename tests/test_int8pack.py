@@ -103,7 +103,7 @@ def test_gpu_all_positive_activations_full_width():
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 def test_gpu_many_rows_take_the_dense_route(dtype):
-    """More rows than INT8PACK_PREFILL_ROWS: dense weight T(w * scale) + library GEMM, within the same bounds."""
+    """More rows than INT8PACK_PREFILL_ROWS: dense weight T(w * scale) + one dense GEMM, within the same bounds."""
     import torch
     from tensorplay_amd import ops
     rng = np.random.default_rng(77)

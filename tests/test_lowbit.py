@@ -256,7 +256,7 @@ def test_gpu_dequantize_bit_exact_and_many_rows(bits):
     np.testing.assert_array_equal(dense.cpu().numpy(), dense_weight(codes, sz, group, bits))
     dense16 = ops._lowbit_dequantize(packed, bits, K, torch.from_numpy(sz).to(DEV), torch.float16)
     np.testing.assert_array_equal(dense16.cpu().numpy(), dense_weight(codes, sz, group, bits).astype(np.float16))
-    M = ops.LOWBIT_PREFILL_ROWS_SMALL + 5   # dequantise + library GEMM
+    M = ops.LOWBIT_PREFILL_ROWS_SMALL + 5   # dequantise + one dense GEMM
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32))
     got = ops._lowbit_mm(x.to(DEV), packed, bits, K, torch.from_numpy(sz).to(DEV))
     want = x.double().numpy() @ dense_weight(codes, sz, group, bits).astype(np.float64).T
