@@ -15,14 +15,18 @@
 //     16-byte MFMA operands (operand f = field f of its four chunks), kept in slot (8 unit + 4 half + f) ^ (row % 16)
 //     of the row (rows are a multiple of 256 bytes apart): the 16 lanes that a 16-byte LDS read serves together
 //     hit 16 different bank groups;
+//   * the packed weights are fetched in whole 128-byte lines (a load costs the vector memory path the lines it
+//     touches) and reach MFMA order through small LDS areas of their own;
 //   * one barrier, then wavefront (nb, kp) multiplies channel block nb with its units (slab_unit_of):
 //     v_mfma_i32_32x32x32_i8, A = activations from LDS, B = weight fields moved to the top of their bytes in
 //     registers, four MFMAs per unit;
 //   * the four k-parts meet in LDS (the slab's space, after a second barrier); every thread finishes and stores
 //     four consecutive columns of one row.
 //
-// Where the time goes (clock stamps at 128 x 6912 x 2560, 216 workgroups): the requests of a workgroup are taken
-// at the rate data returns, and the last wavefront's activations are there after about half of the kernel; from then
+// Where the time goes (clock stamps at 128 x 6912 x 2560, 216 workgroups, 13,200 clocks): the requests of a workgroup
+// are accepted at about 2.7 clocks per cache line they touch (the last wavefront has its requests out after 3,700
+// clocks; 6,300 with the weights as 64-byte runs of 16 rows, which made the kernel 14,900 clocks), and the last
+// wavefront's activations are in LDS after 6,100; from then
 // on 16 wavefronts on four SIMDs pay four clocks of a SIMD per vector instruction and wavefront, so a hundred
 // instructions per wavefront are 1600 clocks: the expansion of the weights, the sums and the epilogue are
 // instruction issue, not memory (without the weight loads the phases behind the barrier take as long as with them).
@@ -39,6 +43,8 @@ namespace {
 constexpr int kSlabRows = 32, kSlabChannels = 128, kSlabThreads = 1024;
 constexpr int kSlabUnitsPerWave = 5, kSlabKParts = 4, kSlabUnits = kSlabUnitsPerWave * kSlabKParts;  // 20 units = 2560 k
 constexpr int kSlabChunkRounds = kSlabRows * kSlabUnits * 8 / kSlabThreads;                          // 5 chunks of 16 bytes per thread
+constexpr int kSlabXchPitch = 144;                                                                   // bytes between the rows of the weight exchange areas in LDS
+constexpr int kSlabXchBytes = (4 * 32 + 16 * 16) * kSlabXchPitch;                                    // units 16 .. 19 of four channel blocks + 16 rows per wavefront
 
 // x: [M][K] int8; packed: [N][K/4]; units_per_split units of 128 k per workgroup (<= kSlabUnits), split z takes the
 // units z units_per_split ...; lds_main_bytes: size of the slab / k-part area; 32 row scales and 128 bias values sit behind it;
@@ -50,10 +56,9 @@ __device__ unsigned long long g_slab_stamps[16 * 16];
 #define TPQ_STAMP(I) do { } while (0)
 #endif
 
-// Unit j of k-part kp.  A row of packed weights holds four units per 128-byte cache line; a wavefront load takes 32
-// bytes of 32 rows, so the four units of a line go to one wavefront, which asks for them back to back: the line is
-// brought into the first-level cache once.  Dealt round-robin (unit kp + 4 j) every line was fetched by four
-// wavefronts at four different times, four times the traffic between the caches.  Units 16..19 go one to each k-part.
+// Unit j of k-part kp.  A row of packed weights holds four units per 128-byte cache line: the four units of a line go to
+// one wavefront, which fetches the line whole (dealt round-robin, unit kp + 4 j, every line was fetched by four
+// wavefronts at four different times, four times the traffic between the caches).  Units 16..19 go one to each k-part.
 __device__ __forceinline__ constexpr int slab_unit_of(int kp, int j) { return j < 4 ? 4 * kp + j : 16 + kp; }
 static_assert(kSlabUnitsPerWave == 5 && kSlabKParts == 4, "slab_unit_of deals 20 units");
 
@@ -103,32 +108,31 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
         }
     }
     // weights of wavefront (nb, kp).  The MFMA wants lane (n, half) to hold the 16 bytes (64 codes) of half `half` of
-    // a unit for row n0 + 32 nb + n: asked for like that, a wavefront load takes 32 bytes out of 32 cache lines.  The
-    // four units of the wavefront's own line are therefore fetched as two pairs of loads that take 64 bytes (two
-    // units) out of 16 lines each: load A rows 0..15, load B rows 16..31, the 16-lane groups of either holding the
-    // chunks (unit, half) of the run in the order (e, 0), (o, 0), (e, 1), (o, 1).  One v_permlane16_swap per register
-    // (group 1 of A against group 0 of B, group 3 against group 2) then leaves unit e in MFMA order in the one and
-    // unit o in the other.  The fifth unit (16 + kp) is asked for in MFMA order directly.
+    // a unit for row n0 + 32 nb + n: asked for like that, a wavefront load takes 32 bytes out of 32 cache lines, and what
+    // a load costs the vector memory path is the lines it touches (about 2.7 clocks each: the requests of the last
+    // wavefront were accepted 6,300 clocks into the kernel when the weights came as 64-byte runs of 16 rows and the fifth
+    // unit in MFMA order, 16 and 32 lines per load).  So the weights are fetched in whole lines: the four units of the
+    // wavefront's own line (4 kp .. 4 kp + 3 are the 128 bytes of one line of a row) as four loads of eight rows x 128
+    // bytes, lane l = row l / 8 of the eight, 16-byte chunk l % 8 (unit 4 kp + chunk / 2, half chunk % 2); and of the
+    // line that holds the units 16 .. 19 the wavefront fetches rows 8 kp .. 8 kp + 7 of its channel block for all four
+    // k-parts.  Both go through LDS on their way into MFMA order (below).
     const int wn = lane & 31, half = lane >> 5;
-    uint4 wq[kSlabUnitsPerWave];  // pair 0: A, B; pair 1: A, B; the single unit
+    const int w_row8 = lane >> 3, w_chunk = lane & 7;
+    uint4 wl[4], wl5;
     {
-        const int n16 = lane & 15, group = lane >> 4;
-        const int odd = group & 1, run_half = group >> 1;  // the group's chunk: unit 2 pair + odd, half run_half
-        const int row_a = n0 + 32 * nb + n16 < N ? n0 + 32 * nb + n16 : N - 1;
-        const int row_b = n0 + 32 * nb + 16 + n16 < N ? n0 + 32 * nb + 16 + n16 : N - 1;
         const size_t pitch = static_cast<size_t>(K >> 2);
-        const unsigned char* const wbase = packed;
-        const unsigned char* base = wbase + (static_cast<size_t>(unit0) << 5) + run_half * 16;
+        const unsigned char* const base = packed + (static_cast<size_t>(unit0) << 5);
+        const int u_own = 4 * kp + (w_chunk >> 1), u_fifth = 16 + (w_chunk >> 1);
+        // a unit past the end of the split re-reads the first bytes of the row's range and is not multiplied
+        const int off_own = u_own < U ? u_own * 32 + (w_chunk & 1) * 16 : 0;
+        const int off_fifth = u_fifth < U ? u_fifth * 32 + (w_chunk & 1) * 16 : 0;
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr) {
-            const int u = 4 * kp + 2 * pr + odd;
-            const int off = (u < U ? u : 0) * 32;  // a unit past the end re-reads unit 0 and is not multiplied
-            wq[2 * pr] = nt_load(reinterpret_cast<const uint4*>(base + row_a * pitch + off));
-            wq[2 * pr + 1] = nt_load(reinterpret_cast<const uint4*>(base + row_b * pitch + off));
+        for (int i = 0; i < 4; ++i) {
+            const int row = n0 + 32 * nb + 8 * i + w_row8;
+            wl[i] = nt_load(reinterpret_cast<const uint4*>(base + (row < N ? row : N - 1) * pitch + off_own));
         }
-        const int n = n0 + 32 * nb + wn < N ? n0 + 32 * nb + wn : N - 1;
-        const int u = 16 + kp;
-        wq[4] = nt_load(reinterpret_cast<const uint4*>(wbase + n * pitch + (static_cast<size_t>(unit0) << 5) + 16 * half + (u < U ? u : 0) * 32));
+        const int row = n0 + 32 * nb + 8 * kp + w_row8;
+        wl5 = nt_load(reinterpret_cast<const uint4*>(base + (row < N ? row : N - 1) * pitch + off_fifth));
     }
 
     TPQ_STAMP(1);
@@ -148,9 +152,34 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
                 *reinterpret_cast<int*>(slab_lds + (dst ^ (f * 16))) = t[f];
         }
     }
+    // ---- weights into MFMA order through LDS ------------------------------------------------------------------
+    // Rows 144 bytes apart: the 16 lanes a 16-byte read serves together (rows n .. n + 15, one chunk) hit 16 different
+    // bank groups.  The own line: a wavefront-private area of 16 rows, used twice (rows 0 .. 15, then 16 .. 31 of the
+    // channel block; LDS accesses of one wavefront execute in order, no barrier).  The line of the units 16 .. 19: an area
+    // per channel block that the four k-parts fill together, read behind the barrier that the activations need anyway.
+    uint4 wq[kSlabUnitsPerWave];  // [j]: unit slab_unit_of(kp, j) in MFMA order
+    {
+        unsigned char* const xch = slab_lds + lds_main_bytes + (kSlabRows + kSlabChannels) * sizeof(float);
+        unsigned char* const fifth = xch + (nb * 32) * kSlabXchPitch;
+        *reinterpret_cast<uint4*>(fifth + (8 * kp + w_row8) * kSlabXchPitch + w_chunk * 16) = wl5;
+        unsigned char* const mine = xch + 4 * 32 * kSlabXchPitch + wave * 16 * kSlabXchPitch;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<uint4*>(mine + w_row8 * kSlabXchPitch + w_chunk * 16) = wl[2 * h];
+            *reinterpret_cast<uint4*>(mine + (8 + w_row8) * kSlabXchPitch + w_chunk * 16) = wl[2 * h + 1];
+            __builtin_amdgcn_wave_barrier();
+            if ((wn >> 4) == h) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) wq[j] = *reinterpret_cast<const uint4*>(mine + (wn & 15) * kSlabXchPitch + (2 * j + half) * 16);
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
     TPQ_STAMP(2);
     __syncthreads();
     TPQ_STAMP(3);
+    wq[4] = *reinterpret_cast<const uint4*>(slab_lds + lds_main_bytes + (kSlabRows + kSlabChannels) * sizeof(float) +
+                                            (nb * 32 + wn) * kSlabXchPitch + (2 * kp + half) * 16);
 
     // ---- wavefront (nb, kp): 32 rows x 32 channels over its units ------------------------------------------
     // A 2-bit field at the top of a byte is the code times 64 as a signed byte (0b11 -> -64, 0b10 -> -128: the
@@ -166,19 +195,6 @@ __global__ __launch_bounds__(kSlabThreads) void ternary_slab_kernel(const int8_t
     int a_off[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) a_off[f] = ((4 * half + f) ^ (wn & 7)) * 16;
-#pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {  // loads A and B of a pair -> its even and its odd unit in MFMA order
-        uint32_t a[4] = {wq[2 * pr].x, wq[2 * pr].y, wq[2 * pr].z, wq[2 * pr].w};
-        uint32_t b[4] = {wq[2 * pr + 1].x, wq[2 * pr + 1].y, wq[2 * pr + 1].z, wq[2 * pr + 1].w};
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const auto r = __builtin_amdgcn_permlane16_swap(a[d], b[d], false, false);
-            a[d] = r[0];
-            b[d] = r[1];
-        }
-        wq[2 * pr] = make_uint4(a[0], a[1], a[2], a[3]);
-        wq[2 * pr + 1] = make_uint4(b[0], b[1], b[2], b[3]);
-    }
 #pragma unroll
     for (int j = 0; j < kSlabUnitsPerWave; ++j) {
         const int u = slab_unit_of(kp, j);
@@ -312,10 +328,10 @@ int launch_ternary_slab(const int8_t* x, const uint8_t* packed, int64_t M, int64
     const size_t slab_bytes = static_cast<size_t>(kSlabRows) * (per_split + (per_split & 1)) * 128;
     const size_t part_bytes = static_cast<size_t>(16) * 16 * kWave * sizeof(int);  // 64 KB
     const size_t main_bytes = slab_bytes > part_bytes ? slab_bytes : part_bytes;
-    const size_t smem = main_bytes + (kSlabRows + kSlabChannels) * sizeof(float);
+    const size_t smem = main_bytes + (kSlabRows + kSlabChannels) * sizeof(float) + kSlabXchBytes;
     auto kernel = ternary_slab_kernel<Epilogue>;
     static std::atomic<uint64_t> configured{0};  // per instantiation
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<size_t>(kSlabRows) * kSlabUnits * 128 + (kSlabRows + kSlabChannels) * sizeof(float), configured, "ternary slab")) return rc;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<size_t>(kSlabRows) * kSlabUnits * 128 + (kSlabRows + kSlabChannels) * sizeof(float) + kSlabXchBytes, configured, "ternary slab")) return rc;
     const int64_t n_tiles = (N + kSlabChannels - 1) / kSlabChannels, m_tiles = (M + kSlabRows - 1) / kSlabRows;
     const int64_t gx = 8 * m_tiles * ((n_tiles * splits + 7) / 8);
     TPQ_REQUIRE(gx <= 0x7FFFFFFF, TPQ_ERR_INVALID_VALUE, "ternary slab: shape too large");
