@@ -91,7 +91,8 @@ TPQ_EXPORT int tpq_packed_linear_float(const void* x, int x_unsigned, double x_s
     TPQ_REQUIRE(out && offsets && w_scales && w_zero_points && (K == 0 || (x && packed)), TPQ_ERR_INVALID_VALUE, "packed linear: null pointer");
     TPQ_REQUIRE(packed_row_stride >= K, TPQ_ERR_INVALID_VALUE, "packed linear: the rows of the packed weight are shorter than K");
     // |x| <= 255, |w| <= 128: the int32 products of tpq_int_mm hold up to this K
-    TPQ_REQUIRE(K <= 65536 && M <= 0x7FFFFFFF && N <= 0x7FFFFFFF, TPQ_ERR_UNSUPPORTED, "packed linear: K above 65536 is not built");
+    TPQ_REQUIRE(K <= 65536, TPQ_ERR_UNSUPPORTED, "packed linear: K above 65536 is not built");
+    TPQ_REQUIRE(M <= 0x7FFFFFFF && N <= 65535ll * kFinishColumns, TPQ_ERR_UNSUPPORTED, "packed linear: more rows or channels than the finishing launch's grid holds");
     TPQ_REQUIRE(workspace && aligned(workspace, 16) && workspace_bytes >= tpq_packed_linear_workspace_bytes(M, N, K, x_unsigned),
                 TPQ_ERR_INVALID_VALUE, "packed linear: workspace of tpq_packed_linear_workspace_bytes(M, N, K, x_unsigned) bytes needed");
     hipStream_t s = static_cast<hipStream_t>(stream);
