@@ -7,6 +7,7 @@
 // weight is ever materialised (the reference unpacks to int8 on every call,
 // tensorplay/ao/quantization/bitnet.py:233).
 //
+// One row, K % 64 == 0, up to 8 MB of packed weights: the flat dot-product kernel of ternary_row_kernel.h.
 // Up to 32 rows with K % 256 == 0: the matrix-core decode kernel of ternary_decode_mfma.h.
 //
 // Dot-product decode kernel (M <= 8, other K % 64 == 0): one wavefront per 4 weight rows, lane l owns the
@@ -27,6 +28,7 @@
 #include "int8_gemm_kernel.h"
 #include "ternary_gemm_kernel.h"
 #include "ternary_decode_mfma.h"
+#include "ternary_row_kernel.h"
 #include "ternary_slab_kernel.h"
 
 namespace tpq {
@@ -134,6 +136,10 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
     // 5.2..29.6 us (the tile kernel 9.3..75 us for any row count up to 128; two slabs stay below it, three do not).
     static const int mfma_min = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_MIN"); return e ? std::atoi(e) : 1; }();
     static const int mfma_rows = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_ROWS"); return e ? std::atoi(e) : 32; }();
+    // One row over up to 8 MB of packed weights: the flat dot-product kernel (every wave-level load 1 KB of whole lines)
+    if (forced_decode_rows < 0 && M == 1 && aligned(x, 16) && aligned(packed, 16) && !tuning_env("TPQ_TERNARY_NO_ROW")) {
+        if (const int rows_wg = ternary_row_rows_per_workgroup(M, N, K)) return launch_ternary_row(x, packed, N, K, rows_wg, ep, s);
+    }
     if (forced_decode_rows < 0 && M >= mfma_min && M <= mfma_rows && ternary_decode_mfma_ok(x, packed, M, N, K))
         return launch_ternary_decode_mfma(x, packed, M, N, K, ep, s);
     // 33 rows and more: the slab kernel (every load of a workgroup in flight at once); K beyond 2560 is split and

@@ -1,0 +1,112 @@
+// Ternary-weight product for ONE activation row (the decode step of the BitNet linear), K % 64 == 0, K <= 8192.
+//
+// The matrix-core kernel of ternary_decode_mfma.h asks for the packed weights in the MFMA's operand order: a wave-level
+// load takes 64 bytes out of each of 16 rows, and the activations are fetched per lane.  The vector memory path takes a
+// wave-level load at a price per cache line it touches, not per byte, so at one row (where the matrix cores have
+// nothing to amortise) that order costs more than the arithmetic.  Here the packed matrix is read as what it is in
+// memory, a flat run of bytes:
+//   * a workgroup owns `rows_wg` consecutive channels = rows_wg * K / 4 contiguous bytes, one 16-byte chunk (64 codes)
+//     per thread, so every wave-level load is 1 KB of whole lines and every wavefront of the chip has exactly one;
+//   * the activation row is read once per workgroup, contiguously, ahead of the weights (loads return in order), brought
+//     into the field order of the packed bytes by a 4 x 4 byte transpose and parked in LDS (K bytes); an LDS-only
+//     barrier, so that nobody waits for its weights in front of it;
+//   * (w << 2 f) & 0xC0C0C0C0 puts field f of four packed bytes at the top of its byte: 64 x code as a signed byte; one
+//     v_dot4_i32_i8 with the four activations of that field position, 3 instructions per 4 codes, and the 64 leaves the
+//     finished sum with an exact shift;
+//   * chunk t of the workgroup belongs to channel t / (K / 64): the lanes add their sums to the channel's word in LDS
+//     (ds_add_u32), the first rows_wg threads scale, round and store.
+// Exact int32 sums, the same as every other ternary kernel here.
+#pragma once
+
+#include "int8_gemm_kernel.h"
+#include "ternary_decode_mfma.h"
+
+namespace tpq {
+namespace {
+
+constexpr int kTernaryRowMaxK = 8192;
+constexpr int kTernaryRowMaxThreads = 1024;
+
+// grid: ceil(N / rows_wg); block: 64 * ceil(rows_wg * K / 64 / 64) threads >= K / 16; LDS: K + 4 * rows_wg bytes
+template <class Epilogue>
+__global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(const int8_t* __restrict__ x, const uint8_t* __restrict__ packed, int N,
+                                                                           int K, int rows_wg, float inv_chunks_per_row, Epilogue ep) {
+    extern __shared__ uint4 x_fields[];  // [K / 16], slot 4 c + ((d + c) & 3) holds the transposed piece d of chunk c
+    int* const sums = reinterpret_cast<int*>(x_fields + (K >> 4));
+    const int t = threadIdx.x;
+    const int cpr = K >> 6;  // 16-byte chunks in a packed row
+    const int row0 = blockIdx.x * rows_wg;
+    const int rows_here = N - row0 < rows_wg ? N - row0 : rows_wg;
+    const bool live = t < rows_here * cpr;
+    const int pieces = K >> 4;
+
+    // requests in the order they are needed (loads come back in the order they were made): activations, weights, bias
+    const uint4 xr = reinterpret_cast<const uint4*>(x)[t < pieces ? t : 0];
+    const uint4 w = nt_load(reinterpret_cast<const uint4*>(packed + static_cast<size_t>(row0) * (static_cast<size_t>(K) >> 2)) + (live ? t : 0));
+    const float row_scale = ep.row_scale_of(0);
+    const int n = row0 + (t < rows_here ? t : 0);
+    const bool with_bias = ep.out && ep.bias;
+    const float bias_raw = *(with_bias ? ep.bias + n : reinterpret_cast<const float*>(x));  // no branch around a load: some readable word instead
+
+    if (t < rows_wg) sums[t] = 0;
+    if (t < pieces) {
+        const v4i f = transpose_4x4_bytes(xr);
+        const int c = t >> 2, d = t & 3;
+        x_fields[4 * c + ((d + c) & 3)] = make_uint4(static_cast<uint32_t>(f[0]), static_cast<uint32_t>(f[1]), static_cast<uint32_t>(f[2]), static_cast<uint32_t>(f[3]));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weights stay in flight
+
+    const int row = static_cast<int>((static_cast<float>(t) + 0.5f) * inv_chunks_per_row);  // t / cpr exactly: t < 1024, cpr <= 128
+    const int c = t - row * cpr;
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+    int acc = 0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const uint4 xf = x_fields[4 * c + ((d + c) & 3)];
+        const uint32_t fields[4] = {xf.x, xf.y, xf.z, xf.w};
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+            acc = __builtin_amdgcn_sdot4(static_cast<int>(fields[f]), static_cast<int>((words[d] << (2 * f)) & 0xC0C0C0C0u), acc, false);
+    }
+    if (live) __hip_atomic_fetch_add(&sums[row], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (t < rows_here) ep.store_scaled(n, sums[t] >> 6, row_scale, with_bias ? bias_raw : 0.0f);
+}
+
+// rows per workgroup (0: the kernel does not take the shape).  Whole rounds of workgroups over the compute units
+// where the channel count allows, at most 16 wavefronts and at least the K / 16 threads that park the activations.
+// One chunk per thread means one round of wavefronts up to 8 MB of packed weights (8192 wavefronts fit the chip at
+// once); beyond that the rounds queue and the matrix-core kernel, whose wavefronts loop, is ahead again.  Measured,
+// weights streamed from HBM (us, this kernel / ternary_decode_mfma.h):
+//   2560 -> 6912  3.50 / 4.33 (cache-resident 3.17 / 3.79)      6912 -> 2560  3.87 / 4.92 (3.42 / 4.22)
+//   1024 x 1024   2.03 / 2.61      2048 x 2048   2.41 / 3.15      2048 -> 4096  2.70 / 3.33      4096 x 4096  3.61 / 3.98
+//   5120 x 5120   4.43 / 5.46      4096 -> 11008 6.19 / 6.27      5120 -> 13824 9.47 / 8.10      8192 x 8192  8.57 / 7.70
+// (two chunks per thread were tried for the larger ones: 4096 -> 11008 5.94, 5120 -> 13824 7.83, 8192 x 8192 8.02)
+inline int ternary_row_rows_per_workgroup(int64_t M, int64_t N, int64_t K, int compute_units = 256) {
+    if (M != 1 || K < 64 || K % 64 != 0 || K > kTernaryRowMaxK || N < 1 || N > 0x7FFFFFF0 || N * K > (int64_t{1} << 25)) return 0;
+    const int64_t cpr = K / 64, most = kTernaryRowMaxThreads / cpr;
+    if (most < 4) return 0;
+    if (const char* e = tuning_env("TPQ_TERNARY_ROW_WG")) {
+        const int64_t rows = std::atoll(e);
+        return rows >= 4 && rows <= most ? static_cast<int>(rows) : 0;
+    }
+    for (int64_t rounds = 1; rounds <= 64; ++rounds) {
+        const int64_t rows = (N + compute_units * rounds - 1) / (compute_units * rounds);
+        if (rows <= most) return static_cast<int>(rows < 4 ? 4 : rows);
+    }
+    return static_cast<int>(most);
+}
+
+template <class Epilogue>
+int launch_ternary_row(const int8_t* x, const uint8_t* packed, int64_t N, int64_t K, int rows_wg, Epilogue ep, hipStream_t s) {
+    const int64_t cpr = K / 64, threads = (rows_wg * cpr + 63) / 64 * 64;
+    TPQ_REQUIRE(K % 64 == 0 && K <= kTernaryRowMaxK && rows_wg >= 4 && threads <= kTernaryRowMaxThreads && threads >= K / 16 && threads >= rows_wg,
+                TPQ_ERR_INVALID_VALUE, "ternary row kernel: workgroup shape");
+    const size_t smem = static_cast<size_t>(K) + 4 * static_cast<size_t>(rows_wg);
+    ternary_row_kernel<Epilogue><<<static_cast<unsigned>((N + rows_wg - 1) / rows_wg), static_cast<unsigned>(threads), smem, s>>>(
+        x, packed, static_cast<int>(N), static_cast<int>(K), rows_wg, 1.0f / static_cast<float>(cpr), ep);
+    return check_launch("tpq_ternary_mm (one row)");
+}
+
+}  // namespace
+}  // namespace tpq

@@ -126,3 +126,31 @@ def test_ternary_slab_arbitrary_bytes(ops, M, K, N):
     np.testing.assert_array_equal(host(got), want)
     got_only = ops.ternary_mm(dev(x), dev(rs), dev(packed), 0.03, K)
     np.testing.assert_array_equal(host(got_only), want)
+
+
+@pytest.mark.parametrize("K,N", [(64, 3), (64, 5), (192, 1000), (320, 77), (1024, 1), (2560, 6912), (6912, 2560), (4096, 4100),
+                                 (8192, 4096), (5120, 5120), (2048, 259)])
+def test_ternary_one_row_kernel_arbitrary_bytes(ops, K, N):
+    """One activation row on up to 8 MB of packed weights takes the flat dot-product kernel (one 16-byte chunk per
+    thread, the channel sums added up in LDS): any byte value in the packed weight (0b10 decodes to -2), activations
+    over the whole int8 range with -128 and the extremes in it, K % 64 == 0 only, channel counts that leave the last
+    workgroup short: exact accumulators, the scaled output with and without bias equal to the oracle's in every
+    output type, and linear in the activations."""
+    rng = np.random.default_rng(K + N)
+    packed = rng.integers(0, 256, size=(N, K // 4)).astype(np.uint8)
+    x = rng.integers(-128, 128, size=(1, K)).astype(np.int8)
+    x[0, ::7] = np.where(rng.random(x[0, ::7].shape) < 0.5, -127, 127)
+    rs = np.float32([0.0071])
+    bias = rng.normal(0, 0.05, N).astype(np.float32)
+    want, want_acc = oracle.ternary_mm(x, rs, packed, 0.03, K, bias=bias)
+    got, acc = ops.ternary_mm(dev(x), dev(rs), dev(packed), 0.03, K, bias=dev(bias), return_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    np.testing.assert_array_equal(host(got), want)
+    for dt in ("f16", "bf16"):
+        w16, _ = oracle.ternary_mm(x, rs, packed, 0.03, K, out_dtype=dt)
+        g16 = ops.ternary_mm(dev(x), dev(rs), dev(packed), 0.03, K, out_dtype=TORCH_DT[dt])
+        np.testing.assert_array_equal(host(g16), w16)
+    flipped = np.clip(-x.astype(np.int32), -127, 127).astype(np.int8)
+    _, want_neg = oracle.ternary_mm(flipped, rs, packed, 0.03, K)
+    _, neg = ops.ternary_mm(dev(flipped), dev(rs), dev(packed), 0.03, K, return_acc=True)
+    np.testing.assert_array_equal(host(neg), want_neg)
