@@ -448,6 +448,13 @@ int launch_generic(const void* x, const uint8_t* packed, const float* sz, const 
 // activations re-read per wavefront would otherwise outweigh the packed bytes (8192 -> 28672 at 1 bit: 26.4 -> 21.9 us);
 // 4 for small weights, which need the wavefronts (4096 x 4096 at 1 bit: 4.8 us against 6.0 with 8).
 
+// The (scale, zero) pairs lie across the packed rows ([K / group][N] pairs): a lane asking for the pair of its segment
+// and channel takes 8 bytes out of a cache line of its own, 128 lines per wavefront against 16 to 32 of packed weights.
+// Parking them in LDS as well (the workgroup's channels are neighbours, so per group their pairs are one run; 16-byte
+// pieces ahead of the weights, one more LDS-only barrier) was built and lost at every width (4096 -> 11008 at 1 / 2 / 4 /
+// 8 bits: 6.4 / 6.7 / 7.8 / 11.5 -> 6.9 / 7.6 / 8.5 / 12.6 us): at these sizes every wavefront's loads arrive together and
+// the 450 vector instructions of the three wavefronts a SIMD holds run one after the other behind the arrival, so the
+// kernel is bound by that arithmetic and anything that sits between arrival and arithmetic adds to it.
 template <int DT, int BITS, bool LSB, int WAVES, int CH>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed,
                                                                   const float* __restrict__ sz, const float* __restrict__ bias,

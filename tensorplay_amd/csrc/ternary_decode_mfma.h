@@ -12,8 +12,15 @@
 // the same order instead: lane (m, q) loads x[m][256 s + 64 q .. + 64) as four 16-byte chunks and
 // transposes each as a 4 x 4 byte matrix (8 v_perm_b32), once for all NB channel blocks.
 // D comes out as lane (m, q) x channels 4 q + v of a block in int32, exact; the wavefronts of a
-// workgroup take the steps round-robin and add their partial sums through LDS.  Columns m >= M stay
-// zero and load nothing.
+// workgroup take the steps round-robin and add their partial sums through LDS.
+//
+// The activations of a step are 256 bytes = two cache lines per row.  Asked for in the MFMA's order (lane (m, q): 16
+// bytes at 64 q + 16 d of row m, four loads) every load touches two lines of every row, 8 M line look-ups per step, and
+// the vector memory path charges a load by the lines it touches: at 8 rows the activations cost it four times what the
+// packed weights do.  So a wavefront reads them as they lie (lane l: 16 bytes at 16 (l % 16) of row l / 16, four rows =
+// 8 whole lines per load, ceil(M / 4) loads), transposes what it got and passes it to the MFMA's lanes through a
+// wave-private LDS area (row pitch 272 bytes, so the sixteen rows of a 16-byte read spread over the banks).  Columns
+// m >= M hold whatever is there; their sums are dropped.
 #pragma once
 
 #include <cstdlib>
@@ -45,10 +52,17 @@ __device__ __forceinline__ v4i ternary_fields_to_i8(uint32_t w) {
     return out;
 }
 
-template <int NB, int MB, int WAVES, class Epilogue>
+constexpr int kTdecXPitch = 272;                    // bytes per activation row in the exchange area
+constexpr int kTdecXBytes = 16 * kTdecXPitch;      // per wavefront: 16 rows of one step
+
+// XL: wave-level loads of activations per step (four rows each), rows <= 4 XL; MB = 2 takes XL = 8 (rows 16.. in the
+// second block)
+template <int NB, int MB, int XL, int WAVES, class Epilogue>
 __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(const int8_t* __restrict__ x, const uint8_t* __restrict__ packed,
                                                                            int m_base, int M, int N, int K, Epilogue ep) {
+    static_assert(XL <= 4 * MB && (MB == 1 || XL == 8), "activation loads per step");
     __shared__ int red[WAVES][NB * MB][4][kWave];
+    extern __shared__ __align__(16) unsigned char tdec_xch[];  // [WAVES][kTdecXBytes]
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
@@ -62,45 +76,57 @@ __global__ __launch_bounds__(WAVES * kWave) void ternary_decode_mfma_kernel(cons
         w_base[b] = reinterpret_cast<const uint4*>(packed + static_cast<size_t>(n < N ? n : N - 1) * bpr) + q;  // rows past N: a valid row, result dropped
     }
     bool row_live[MB];
-    const uint4* x_base[MB];
 #pragma unroll
-    for (int r = 0; r < MB; ++r) {
-        row_live[r] = 16 * r + i < M;
-        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m_base + (row_live[r] ? 16 * r + i : 0)) * K) + q * 4;
+    for (int r = 0; r < MB; ++r) row_live[r] = 16 * r + i < M;
+    // load j of a step: row 4 j + lane / 16, bytes 16 (lane % 16) of the step's 256 (rows past M: row 0, dropped)
+    const uint4* x_base[XL];
+#pragma unroll
+    for (int j = 0; j < XL; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        x_base[j] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(m_base + (row < M ? row : 0)) * K) + (lane & 15);
     }
+    unsigned char* const xch = tdec_xch + wave * kTdecXBytes;
+    unsigned char* const xch_put = xch + (lane >> 4) * kTdecXPitch + (lane & 15) * 16;  // + 4 j rows
+    const unsigned char* const xch_get = xch + i * kTdecXPitch + q * 64;                // + 16 d
 
     struct Step {
         uint4 w[NB];
-        uint4 xv[MB][4];
+        uint4 xv[XL];
     };
     auto load = [&](int s, Step& st) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) st.w[b] = nt_load(w_base[b] + s * 4);
 #pragma unroll
-        for (int r = 0; r < MB; ++r)
-            if (row_live[r]) {
-#pragma unroll
-                for (int d = 0; d < 4; ++d) st.xv[r][d] = x_base[r][s * 16 + d];
-            }
+        for (int j = 0; j < XL; ++j) st.xv[j] = x_base[j][s * 16];
     };
     v4i acc[NB][MB][2] = {};  // two accumulators per output block taking turns
     auto compute = [&](const Step& st) {
+        v4i xb[MB][4];
+#pragma unroll
+        for (int r = 0; r < MB; ++r) {
+            // this block's rows into the exchange area (LDS keeps a wavefront's accesses in order: the reads of the
+            // block before are served before these writes), then each lane's four pieces out of it
+#pragma unroll
+            for (int j = 4 * r; j < 4 * r + 4 && j < XL; ++j) {
+                const v4i f = transpose_4x4_bytes(st.xv[j]);
+                *reinterpret_cast<v4i*>(xch_put + (j - 4 * r) * 4 * kTdecXPitch) = f;
+            }
+#pragma unroll
+            for (int d = 0; d < 4; ++d) xb[r][d] = *reinterpret_cast<const v4i*>(xch_get + d * 16);
+        }
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            v4i xb[MB];
-#pragma unroll
-            for (int r = 0; r < MB; ++r) xb[r] = transpose_4x4_bytes(st.xv[r][d]);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const uint32_t word = d == 0 ? st.w[b].x : d == 1 ? st.w[b].y : d == 2 ? st.w[b].z : st.w[b].w;
                 const v4i codes = ternary_fields_to_i8(word);
 #pragma unroll
-                for (int r = 0; r < MB; ++r) acc[b][r][d & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(codes, xb[r], acc[b][r][d & 1], 0, 0, 0);
+                for (int r = 0; r < MB; ++r) acc[b][r][d & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(codes, xb[r][d], acc[b][r][d & 1], 0, 0, 0);
             }
         }
     };
 
-    // this wavefront's steps: wave, wave + WAVES, ...; RING in flight (a step is 16 NB + 64 MB bytes per lane)
+    // this wavefront's steps: wave, wave + WAVES, ...; RING in flight (a step is 16 (NB + XL) bytes per lane)
     constexpr int kRing = MB >= 2 ? 2 : 4;
     Step ring[kRing] = {};
 #pragma unroll
@@ -180,11 +206,28 @@ int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M
         const int mb = forced_mb ? forced_mb : (left > 16 ? 2 : 1);
         const int rows = left < 16 * mb ? left : 16 * mb;
         const int base = static_cast<int>(m0);
-#define TPQ_TDEC(NBV, MBV, WV) ternary_decode_mfma_kernel<NBV, MBV, WV, Epilogue><<<grid, WV * kWave, 0, s>>>(x, packed, base, rows, n, k, ep)
-        if (nb == 2 && mb == 2) { if (waves == 8) TPQ_TDEC(2, 2, 8); else TPQ_TDEC(2, 2, 4); }
-        else if (nb == 2) { if (waves == 8) TPQ_TDEC(2, 1, 8); else TPQ_TDEC(2, 1, 4); }
-        else if (mb == 2) { if (waves == 8) TPQ_TDEC(1, 2, 8); else TPQ_TDEC(1, 2, 4); }
-        else { if (waves == 8) TPQ_TDEC(1, 1, 8); else TPQ_TDEC(1, 1, 4); }
+        const int xl = rows > 16 ? 8 : rows > 8 ? 4 : rows > 4 ? 2 : 1;
+        const size_t xch_bytes = static_cast<size_t>(waves) * kTdecXBytes;
+#define TPQ_TDEC(NBV, MBV, XLV, WV)                                                                                      \
+    do {                                                                                                                 \
+        auto kernel = ternary_decode_mfma_kernel<NBV, MBV, XLV, WV, Epilogue>;                                           \
+        constexpr size_t kStatic = sizeof(int) * WV * NBV * MBV * 4 * kWave;                                             \
+        if (kStatic + xch_bytes > 64 * 1024) {                                                                           \
+            static std::atomic<uint64_t> configured{0};                                                                  \
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), xch_bytes, configured, "tpq_ternary_mm (mfma decode)")) return rc; \
+        }                                                                                                                \
+        kernel<<<grid, WV * kWave, xch_bytes, s>>>(x, packed, base, rows, n, k, ep);                                     \
+    } while (0)
+#define TPQ_TDEC_X(NBV, WV)                                      \
+    do {                                                         \
+        if (mb == 2) TPQ_TDEC(NBV, 2, 8, WV);                    \
+        else if (xl == 4) TPQ_TDEC(NBV, 1, 4, WV);               \
+        else if (xl == 2) TPQ_TDEC(NBV, 1, 2, WV);               \
+        else TPQ_TDEC(NBV, 1, 1, WV);                            \
+    } while (0)
+        if (nb == 2) { if (waves == 8) TPQ_TDEC_X(2, 8); else TPQ_TDEC_X(2, 4); }
+        else { if (waves == 8) TPQ_TDEC_X(1, 8); else TPQ_TDEC_X(1, 4); }
+#undef TPQ_TDEC_X
 #undef TPQ_TDEC
         m0 += rows;
     }
