@@ -613,22 +613,23 @@ def main() -> int:
         # {1, 2, 4, 8}, float32 (scale, zero) per group of 128; enough rotating copies to stream from HBM
         G = K // 128
         szf = torch.stack([torch.rand(G, N, device=dev) * 0.01, torch.full((G, N), 2.0, device=dev)], dim=-1).contiguous()
-        xb = torch.from_numpy(rng.normal(0, 1, (1, K)).astype(np.float32)).to(dev).half()
-        yb = torch.empty((1, N), dtype=torch.float16, device=dev)
         for bits in (1, 2, 4, 8):
             row_bytes = K * bits // 8
             n_copies = max(2, min(60, (600 << 20) // (N * row_bytes)))
             wl = [torch.randint(0, 256, (N, row_bytes), dtype=torch.uint8, device=dev) for _ in range(n_copies)]
+            for mb in (1, 8):  # one row: the row kernel; eight: the matrix-core kernel
+                xb = torch.from_numpy(rng.normal(0, 1, (mb, K)).astype(np.float32)).to(dev).half()
+                yb = torch.empty((mb, N), dtype=torch.float16, device=dev)
 
-            def lbmm(i, wl=wl, bits=bits, n_copies=n_copies):
-                lib.tpq_lowbit_mm(xb.data_ptr(), _lib.F16, 1, K, wl[i % n_copies].data_ptr(), bits, 0, N, 128,
-                                  szf.data_ptr(), None, yb.data_ptr(), cur())
+                def lbmm(i, wl=wl, bits=bits, n_copies=n_copies, xb=xb, yb=yb, mb=mb):
+                    lib.tpq_lowbit_mm(xb.data_ptr(), _lib.F16, mb, K, wl[i % n_copies].data_ptr(), bits, 0, N, 128,
+                                      szf.data_ptr(), None, yb.data_ptr(), cur())
 
-            gl = graph_of(lambda: [lbmm(i) for i in range(2 * n_copies)])
-            gl.replay(); sync()
-            ms = steady(gl.replay, sync) / (2 * n_copies)
-            extras[f"lowbit{bits}_M1_us"] = ms * 1e3
-            extras[f"lowbit{bits}_M1_GBs"] = (N * row_bytes + 8 * G * N + 2 * K + 2 * N) / (ms * 1e-3) / 1e9
+                gl = graph_of(lambda: [lbmm(i) for i in range(2 * n_copies)])
+                gl.replay(); sync()
+                ms = steady(gl.replay, sync) / (2 * n_copies)
+                extras[f"lowbit{bits}_M{mb}_us"] = ms * 1e3
+                extras[f"lowbit{bits}_M{mb}_GBs"] = (N * row_bytes + 8 * G * N + 2 * mb * K + 2 * mb * N) / (ms * 1e-3) / 1e9
             del wl
         torch.cuda.empty_cache()
 

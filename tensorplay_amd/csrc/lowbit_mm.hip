@@ -71,12 +71,29 @@ constexpr uint32_t kSignFlip = 0x80808080u;
 // bf16 has seven mantissa bits, too few for the exponent trick: there a code is cut out of its dword,
 // converted to float (exact) and the upper halves of two floats are packed; no offsets to take out, the
 // constant-A MFMA only sums x.
-template <int DT, int BITS, bool LSB, int WAVES>
+//
+// The activations of a step are kStepK * 2 bytes of every row.  Asked for in the MFMA's order (lane (m, q): its 16-byte
+// pieces of row m) every load touches two or three lines of every row, and the vector memory path charges a load by the
+// lines it touches: at 8 rows the activations cost it four times what the packed weights do, and the time grew by half a
+// microsecond per row.  So a wavefront reads them as they lie (a load = 64 consecutive 16-byte pieces = 4 or 8 whole
+// rows of the step, XL loads for up to 16 rows) and passes them to the MFMA's lanes through a wave-private LDS area
+// whose rows are 16 bytes longer than a step, so that the sixteen rows of a 16-byte read spread over the banks.
+// Columns m >= M hold whatever is there; their sums are dropped.  Measured, 4096 -> 11008, 1 / 2 / 4 bits (us):
+// 2 rows 10.0 / 10.4 / 10.7, 4 rows 11.1 / 11.4 / 11.6, 8 rows 13.2 / 13.4 / 13.6, 16 rows 17.1 / 17.7 / 17.7 before.
+template <int BITS, bool LSB>
+constexpr int lowbit_x_pitch() { return Fields<BITS, LSB>::kStepK * 2 + 16; }
+
+template <int DT, int BITS, bool LSB, int WAVES, int XL>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
     const float* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int group_shift) {
     using F = Fields<BITS, LSB>;
+    constexpr int kPiecesPerRow = F::kStepK / 8;           // 16-byte pieces of a row and step: 16, or 8 at one code per byte
+    constexpr int kRowsPerLoad = kWave / kPiecesPerRow;    // 4 or 8
+    constexpr int kPitch = lowbit_x_pitch<BITS, LSB>();
+    static_assert(XL * kRowsPerLoad <= 16, "at most 16 rows per launch");
     __shared__ float red[WAVES][4][kWave];
+    extern __shared__ __align__(16) unsigned char lowbit_xch[];  // [WAVES][16 rows][kPitch]
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
@@ -88,8 +105,16 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     n4 = n4 + 4 <= N ? n4 : N - 4;
     const float* sz_base = sz + static_cast<size_t>(n4) * 2;
     const bool row_live = i < M;
-    // columns m >= M stay zero and load nothing
-    const uint4* x_base = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live ? i : 0) * K + q * F::kCodes);
+    // load j of a step: row kRowsPerLoad j + lane / kPiecesPerRow, piece lane % kPiecesPerRow (rows past M: row 0, dropped)
+    const uint4* x_base[XL];
+#pragma unroll
+    for (int j = 0; j < XL; ++j) {
+        const int row = kRowsPerLoad * j + lane / kPiecesPerRow;
+        x_base[j] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row < M ? row : 0) * K) + lane % kPiecesPerRow;
+    }
+    unsigned char* const xch = lowbit_xch + wave * (16 * kPitch);
+    unsigned char* const xch_put = xch + (lane / kPiecesPerRow) * kPitch + (lane % kPiecesPerRow) * 16;  // + kRowsPerLoad j rows
+    const unsigned char* const xch_get = xch + i * kPitch + q * (F::kCodes * 2);                        // + 16 c
 
     // constant A of the offset MFMA: row 0 = the offsets of the eight k of an MFMA (pairs 0..3 of the
     // lane's codes: the pattern repeats every byte, so every MFMA has the same), row 1 = ones
@@ -106,7 +131,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     struct Step {
         uint4 w;       // kBytes of it are used
         uint4 p[2];    // (scale, zero) of four channels
-        uint4 xv[F::kCodes / 8];
+        uint4 xv[XL];  // as loaded: piece lane % kPiecesPerRow of row kRowsPerLoad j + lane / kPiecesPerRow
     };
     auto load = [&](int s, Step& st) {
         const uint8_t* src = w_base + static_cast<size_t>(s) * (4 * F::kBytes);
@@ -117,15 +142,20 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
         const uint4* prm = reinterpret_cast<const uint4*>(sz_base + static_cast<size_t>(s >> group_shift) * N * 2);
         st.p[0] = prm[0];
         st.p[1] = prm[1];
-        if (row_live) {
 #pragma unroll
-            for (int c = 0; c < F::kCodes / 8; ++c) st.xv[c] = x_base[static_cast<size_t>(s) * (F::kStepK / 8) + c];
-        }
+        for (int j = 0; j < XL; ++j) st.xv[j] = x_base[j][static_cast<size_t>(s) * kPiecesPerRow];
     };
 
     float yacc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     auto compute = [&](const Step& st) {
         float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f}, d = {0.0f, 0.0f, 0.0f, 0.0f};
+        // the step's activations into the exchange area and this lane's pieces out of it (LDS keeps a wavefront's
+        // accesses in order: the reads of the step before are served before these writes)
+#pragma unroll
+        for (int j = 0; j < XL; ++j) *reinterpret_cast<uint4*>(xch_put + j * kRowsPerLoad * kPitch) = st.xv[j];
+        uint4 xb[F::kCodes / 8];
+#pragma unroll
+        for (int c = 0; c < F::kCodes / 8; ++c) xb[c] = *reinterpret_cast<const uint4*>(xch_get + c * 16);
 #pragma unroll
         for (int u = 0; u < F::kCodes / 8; ++u) {  // MFMA u (16x16x32): codes 8u .. 8u+7 of the lane
             uint32_t a[4];
@@ -143,7 +173,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
                 }
             }
             const word4_t av = {a[0], a[1], a[2], a[3]}, cv = {a_corr[0], a_corr[1], a_corr[2], a_corr[3]};
-            const word4_t bv = {st.xv[u].x, st.xv[u].y, st.xv[u].z, st.xv[u].w};  // the same eight k of the activations
+            const word4_t bv = {xb[u].x, xb[u].y, xb[u].z, xb[u].w};  // the same eight k of the activations
             if constexpr (DT == TPQ_DTYPE_F16) {
                 aux = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, cv), __builtin_bit_cast(half8_t, bv), aux, 0, 0, 0);
                 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
@@ -407,15 +437,29 @@ int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const flo
     const int64_t steps = K / Fields<BITS, LSB>::kStepK;
     // measured at 4096 -> 11008, one row, 2 bits: 4 waves 11.1 us, 8 waves 10.4 - 11.0 us, 16 waves 14.3 us
     const int waves = forced ? forced : steps >= 16 ? 8 : 4;
+    constexpr int kRowsPerLoad = kWave / (Fields<BITS, LSB>::kStepK / 8);  // 4, or 8 at one code per byte
+    constexpr int kFull = 16 / kRowsPerLoad;                               // loads of activations per step for 16 rows
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
         const dim3 grid(static_cast<unsigned>((N + 15) / 16));
         const uint16_t* xs = static_cast<const uint16_t*>(x) + m0 * K;
         uint16_t* ys = static_cast<uint16_t*>(out) + m0 * N;
         const int n = static_cast<int>(N), k = static_cast<int>(K);
-        if (waves >= 16) lowbit_mfma_kernel<DT, BITS, LSB, 16><<<grid, 16 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
-        else if (waves >= 8) lowbit_mfma_kernel<DT, BITS, LSB, 8><<<grid, 8 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
-        else lowbit_mfma_kernel<DT, BITS, LSB, 4><<<grid, 4 * kWave, 0, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);
+        const bool few = rows <= kRowsPerLoad;  // one load of activations per step
+        const size_t xch = static_cast<size_t>(waves >= 16 ? 16 : waves >= 8 ? 8 : 4) * 16 * lowbit_x_pitch<BITS, LSB>();
+#define TPQ_LB_MFMA(W, XLV)                                                                                                   \
+    do {                                                                                                                      \
+        auto kernel = lowbit_mfma_kernel<DT, BITS, LSB, W, XLV>;                                                              \
+        if (xch + sizeof(float) * W * 4 * kWave > 64 * 1024) {                                                                \
+            static std::atomic<uint64_t> configured{0};                                                                       \
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), xch, configured, "tpq_lowbit_mm (mfma)")) return rc; \
+        }                                                                                                                     \
+        kernel<<<grid, W * kWave, xch, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);                               \
+    } while (0)
+        if (waves >= 16) { if (few) TPQ_LB_MFMA(16, 1); else TPQ_LB_MFMA(16, kFull); }
+        else if (waves >= 8) { if (few) TPQ_LB_MFMA(8, 1); else TPQ_LB_MFMA(8, kFull); }
+        else { if (few) TPQ_LB_MFMA(4, 1); else TPQ_LB_MFMA(4, kFull); }
+#undef TPQ_LB_MFMA
     }
     return check_launch("tpq_lowbit_mm (mfma)");
 }
