@@ -78,8 +78,9 @@ constexpr uint32_t kSignFlip = 0x80808080u;
 // microsecond per row.  So a wavefront reads them as they lie (a load = 64 consecutive 16-byte pieces = 4 or 8 whole
 // rows of the step, XL loads for up to 16 rows) and passes them to the MFMA's lanes through a wave-private LDS area
 // whose rows are 16 bytes longer than a step, so that the sixteen rows of a 16-byte read spread over the banks.
-// Columns m >= M hold whatever is there; their sums are dropped.  Measured, 4096 -> 11008, 1 / 2 / 4 bits (us):
-// 2 rows 10.0 / 10.4 / 10.7, 4 rows 11.1 / 11.4 / 11.6, 8 rows 13.2 / 13.4 / 13.6, 16 rows 17.1 / 17.7 / 17.7 before.
+// Columns m >= M hold whatever is there; their sums are dropped.  Measured, 4096 -> 11008, 1 / 2 / 4 bits (us, with the
+// loads in MFMA order -> as they lie): 2 rows 10.0 / 10.4 / 10.7 -> 9.2 / 9.0 / 10.4, 4 rows 11.1 / 11.4 / 11.6 ->
+// 9.4 / 9.1 / 11.6, 8 rows 13.2 / 13.4 / 13.6 -> 12.3 / 11.0 / 11.5, 16 rows 17.1 / 17.7 / 17.7 -> 12.8 / 12.4 / 13.4.
 template <int BITS, bool LSB>
 constexpr int lowbit_x_pitch() { return Fields<BITS, LSB>::kStepK * 2 + 16; }
 
