@@ -162,6 +162,11 @@ int tpq_int4_mm(const void* x, int dtype, int64_t M, int64_t K, const int32_t* p
  * order), so repeated calls are bit-identical.
  */
 size_t tpq_int4_mm_workspace_bytes(int64_t N);
+/* The same for a call with M rows: 113 .. 256 rows run on the tiled kernel, which with few tiles deals the steps of K to
+ * up to 16 slices and keeps their fp32 sums [slice][M][N] behind the counters; never less than
+ * tpq_int4_mm_workspace_bytes(N).  With a smaller workspace the call takes fewer slices or none: same roundings of the
+ * weights, the sums added in another order. */
+size_t tpq_int4_mm_rows_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int tpq_int4_mm_ws(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,
                    int inner_k_tiles, int64_t N, int64_t group, const void* scales_and_zeros,
                    void* out, void* workspace, size_t workspace_bytes, void* stream);

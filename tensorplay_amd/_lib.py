@@ -33,6 +33,7 @@ SIGNATURES = {
     "tpq_int4_mm": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr],
     "tpq_int4_mm_ws": [_ptr, _int, _i64, _i64, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, ctypes.c_size_t, _ptr],
     "tpq_int4_mm_workspace_bytes": [_i64],
+    "tpq_int4_mm_rows_workspace_bytes": [_i64, _i64, _i64],
     "tpq_ternary_pack": [_ptr, _i64, _i64, _ptr, _ptr],
     "tpq_ternary_unpack": [_ptr, _i64, _i64, _ptr, _ptr],
     "tpq_ternary_mm": [_ptr, _ptr, _ptr, _f32, _ptr, _i64, _i64, _i64, _ptr, _int, _ptr, _ptr],

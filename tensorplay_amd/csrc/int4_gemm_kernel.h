@@ -12,6 +12,11 @@
 // bytes + 16 of padding, so the sixteen lanes of a fragment read (row m, 16 bytes at 64 q + 16 u) hit
 // sixteen different groups of four banks.  Lane (m, q) of the result holds row 16 rb + m, channels 4 q + v of a
 // block; sums stay in the MFMA accumulators over the whole K range (fp32) and are rounded once at the end.
+//
+// Few rows (one or two tiles of 128) leave most compute units without a workgroup: N / 64 workgroups, 64 of them at
+// N = 4096.  With a workspace the steps of K are dealt to gridDim.z slices; every slice leaves its fp32 sums in the
+// workspace and int4_gemm_finish_kernel adds the slices in order and rounds once, so the result does not depend on how
+// the launch was scheduled.
 #pragma once
 
 #include <atomic>
@@ -68,7 +73,7 @@ struct DensePair<TPQ_DTYPE_BF16> {
 template <int DT, int NB, int WAVES, int GKT, int RSPLIT>
 __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t* __restrict__ x, const uint4* __restrict__ packed,
                                                                  const uint32_t* __restrict__ sz, uint16_t* __restrict__ y, int M, int N,
-                                                                 int K) {
+                                                                 int K, int steps_per_slice, float* __restrict__ partial) {
     using L = Lane16<DT>;
     using ML = MfmaLane<DT>;
     constexpr int kThreads = WAVES * kWave;
@@ -80,7 +85,9 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int i = lane & 15, q = lane >> 4;
-    const int k_super = K / 32, steps = K / 128, n_tiles = N / 8;
+    const int k_super = K / 32, n_tiles = N / 8;
+    const int s_begin = blockIdx.z * steps_per_slice;                                            // this slice: steps s_begin .. steps - 1
+    const int steps = K / 128 < s_begin + steps_per_slice ? K / 128 : s_begin + steps_per_slice;  // (every slice has at least one)
     constexpr int kChannelWaves = WAVES / RSPLIT, kRowBlocks = kGemmRowBlocks / RSPLIT;
     const int cw = wave % kChannelWaves, rp = wave / kChannelWaves;    // channel position, row part
     const int n0 = blockIdx.x * (16 * NB * kChannelWaves) + cw * (16 * NB);  // first channel of this wavefront
@@ -178,11 +185,11 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
     auto clamp = [&](int s) __attribute__((always_inline)) { return s < last ? s : last; };
     Weights wr[4] = {};
 #pragma unroll
-    for (int r = 0; r < 4; ++r) load_w(clamp(r), wr[r]);
-    load_x(0, 0);
+    for (int r = 0; r < 4; ++r) load_w(clamp(s_begin + r), wr[r]);
+    load_x(s_begin, 0);
     store_x(0, 0);
-    load_x(clamp(1), 1);
-    load_x(clamp(2), 0);
+    load_x(clamp(s_begin + 1), 1);
+    load_x(clamp(s_begin + 2), 0);
     // LDS traffic only: __syncthreads() would also wait for the global loads in flight, which are the prefetch
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
     lds_barrier();
@@ -195,7 +202,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
         load_x(clamp(s + 3), set);
         lds_barrier();
     };
-    for (int s = 0; s < steps; s += 4) {
+    for (int s = s_begin; s < steps; s += 4) {
         phase(s, std::integral_constant<int, 0>{});
         phase(s + 1, std::integral_constant<int, 1>{});
         phase(s + 2, std::integral_constant<int, 2>{});
@@ -212,12 +219,85 @@ __global__ __launch_bounds__(WAVES * kWave) void int4_gemm_kernel(const uint16_t
             const int row = 16 * (rp * kRowBlocks + rb) + i;
             if (row < rows_here) {
                 const float4_t d = acc[b][rb];
+                if (partial != nullptr) {  // this slice's sums: [slice][M][N] fp32
+                    *reinterpret_cast<float4_t*>(partial + (static_cast<size_t>(blockIdx.z) * M + m0 + row) * N + n) = d;
+                    continue;
+                }
                 const uint32_t lo = L::out(d[0]) | (static_cast<uint32_t>(L::out(d[1])) << 16);
                 const uint32_t hi = L::out(d[2]) | (static_cast<uint32_t>(L::out(d[3])) << 16);
                 *reinterpret_cast<uint2*>(y + static_cast<size_t>(m0 + row) * N + n) = make_uint2(lo, hi);
             }
         }
     }
+}
+
+// y = round(sum over the slices, in slice order); a thread takes four consecutive elements
+template <int DT>
+__global__ __launch_bounds__(256) void int4_gemm_finish_kernel(const float* __restrict__ partial, int slices, int64_t quads, uint16_t* __restrict__ y) {
+    using L = Lane16<DT>;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= quads) return;
+    float4_t sum = reinterpret_cast<const float4_t*>(partial)[e];
+    for (int z = 1; z < slices; ++z) {
+        const float4_t more = reinterpret_cast<const float4_t*>(partial)[static_cast<int64_t>(z) * quads + e];
+        sum = float4_t{sum[0] + more[0], sum[1] + more[1], sum[2] + more[2], sum[3] + more[3]};
+    }
+    const uint32_t lo = L::out(sum[0]) | (static_cast<uint32_t>(L::out(sum[1])) << 16);
+    const uint32_t hi = L::out(sum[2]) | (static_cast<uint32_t>(L::out(sum[3])) << 16);
+    reinterpret_cast<uint2*>(y)[e] = make_uint2(lo, hi);
+}
+
+// Slices of K for the tiled kernel (1: no workspace used).  `room`: bytes for the fp32 sums.  Chosen by an estimate
+// of the time (us) fitted to measurements at 113 .. 255 rows (workgroups of 64 channels): a workgroup takes 5 + 7.2 per
+// 1024 k of its slice; up to one workgroup per compute unit they all run at once, up to two per compute unit the pairs
+// cost 1.7 times one, and so on; the second launch costs 1.6 + its bytes (slices x M x N x 4, written and read) at
+// 4 TB/s.  Measured (one slice -> the choice): 4096 x 4096 at 128 rows 33.1 -> 19.7 (four slices), 11008 -> 4096
+// 82.7 -> 34.3 (four), 8192 x 8192 62.7 -> 44.2 (two), 13824 -> 5120 at 192 rows 102 -> 74 (three); 4096 -> 11008 stays
+// at one slice (35.3; two: 40.4).
+struct Int4GemmPlan {
+    int slices;
+    double us;  // the estimate
+};
+inline Int4GemmPlan int4_gemm_plan(int64_t M, int64_t N, int64_t K, size_t room, int compute_units = 256) {
+    const double tiles = static_cast<double>(((N + 63) / 64) * ((M + kGemmRows - 1) / kGemmRows));
+    auto estimate = [&](int64_t slices) {
+        const double per_unit = tiles * static_cast<double>(slices) / compute_units;
+        const double rounds = per_unit <= 1.0 ? 1.0 : 1.7 * static_cast<double>(static_cast<int64_t>((per_unit + 1.999) / 2.0));
+        const double main_us = rounds * (5.0 + 7.2 * static_cast<double>(K) / 1024.0 / static_cast<double>(slices));
+        return main_us + (slices == 1 ? 0.0 : 1.6 + static_cast<double>(slices) * M * N * 8.0 / 4e6);
+    };
+    if (M > 256 || K < 1024) return {1, estimate(1)};
+    const int64_t steps = K / 128, most = steps / 4 < 16 ? steps / 4 : 16;
+    auto fits = [&](int64_t slices) { return slices == 1 || static_cast<size_t>(slices) * M * N * sizeof(float) <= room; };
+    if (const char* e = tuning_env("TPQ_INT4_GEMM_SLICES")) {
+        const int forced = std::atoi(e);
+        return forced >= 1 && forced <= steps && fits(forced) ? Int4GemmPlan{forced, estimate(forced)} : Int4GemmPlan{1, estimate(1)};
+    }
+    Int4GemmPlan best{1, estimate(1)};
+    for (int64_t slices = 2; slices <= most && fits(slices); ++slices)
+        if (estimate(slices) < best.us) best = {static_cast<int>(slices), estimate(slices)};
+    return best;
+}
+inline int int4_gemm_slices(int64_t M, int64_t N, int64_t K, size_t room) { return int4_gemm_plan(M, N, K, room).slices; }
+
+// From how many rows the tiled kernel takes a shape: always from kInt4GemmRows; from kInt4GemmRowsSliced where its
+// estimate is below that of the slabs of 32 rows it replaces, each of which streams the weight again: a slab of 32 rows
+// takes about 1.6 + 0.31 per MB of packed weight + 1.33 per 1024 k (us, fitted to eight shapes, +- 20 %), a shorter last
+// slab 55 % of that plus its share of the rest.  Measured (us, slabs / tiled, 33 - 48 - 64 - 80 - 96 - 112 rows):
+//   4096 x 4096     12.6 14.0 16.1 21.4 23.2 28.2 / 15.5 15.7 16.1 16.9 17.6 18.4
+//   4096 -> 11008   18.8 19.6 23.0 29.8 32.7 40.2 / 34.3 32.9 33.1 33.3 33.4 33.7
+//   11008 -> 4096   31.6 37.9 47.6 61.3 71.0 84.8 / 30.0 29.6 29.7 29.9 30.7 31.4
+//   8192 x 8192     30.6 32.8 40.5 51.0 59.4 69.9 / 40.1 39.8 39.8 40.4 40.0 40.0
+//   2048 x 2048     10.2 11.2 13.5 17.7 20.0 24.4 /  9.8 10.1 10.5 10.8 11.2 11.7
+//   13824 -> 5120   45.1 50.4 61.9 81.5 93.3 112  / 41.5 42.3 42.2 42.4 42.3 42.9
+constexpr int64_t kInt4GemmRows = 113, kInt4GemmRowsSliced = 33;
+inline bool int4_gemm_takes(int64_t M, int64_t N, int64_t K, size_t room) {
+    if (M >= kInt4GemmRows) return true;
+    if (M < kInt4GemmRowsSliced) return false;
+    const double slab = 1.6 + 0.31 * static_cast<double>(N) * static_cast<double>(K) / 2e6 + 1.33 * static_cast<double>(K) / 1024.0;
+    const int64_t whole = M / 32, rest = M % 32;
+    const double slabs = static_cast<double>(whole) * slab + (rest ? slab * (0.55 + 0.45 * static_cast<double>(rest) / 32.0) : 0.0);
+    return int4_gemm_plan(M, N, K, room).us < slabs;
 }
 
 inline bool int4_gemm_ok(const void* x, const void* packed, const void* sz, const void* y, int64_t M, int64_t N, int64_t K, int64_t group) {
@@ -228,10 +308,14 @@ inline bool int4_gemm_ok(const void* x, const void* packed, const void* sz, cons
 
 template <int DT, int NB, int WAVES, int RSPLIT>
 int launch_int4_gemm_shape(const void* x, const int32_t* packed, const void* sz, void* y, int64_t M, int64_t N, int64_t K, int group,
-                           hipStream_t s) {
+                           int slices, float* partial, hipStream_t s) {
     constexpr size_t smem = 2 * static_cast<size_t>(kGemmStageBytes);
     constexpr int kChannels = 16 * NB * (WAVES / RSPLIT);
-    const dim3 grid(static_cast<unsigned>((N + kChannels - 1) / kChannels), static_cast<unsigned>((M + kGemmRows - 1) / kGemmRows));
+    const int steps_per_slice = static_cast<int>((K / 128 + slices - 1) / slices);
+    slices = static_cast<int>((K / 128 + steps_per_slice - 1) / steps_per_slice);  // no empty slice
+    if (slices == 1) partial = nullptr;
+    const dim3 grid(static_cast<unsigned>((N + kChannels - 1) / kChannels), static_cast<unsigned>((M + kGemmRows - 1) / kGemmRows),
+                    static_cast<unsigned>(slices));
     const auto* xp = static_cast<const uint16_t*>(x);
     const auto* pp = reinterpret_cast<const uint4*>(packed);
     const auto* sp = static_cast<const uint32_t*>(sz);
@@ -241,15 +325,21 @@ int launch_int4_gemm_shape(const void* x, const int32_t* packed, const void* sz,
         auto kernel = int4_gemm_kernel<DT, NB, WAVES, GKTV, RSPLIT>;                                                                 \
         static std::atomic<uint64_t> configured{0};                                                                          \
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), smem, configured, "int4 gemm")) return rc;    \
-        kernel<<<grid, WAVES * kWave, smem, s>>>(xp, pp, sp, yp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K)); \
+        kernel<<<grid, WAVES * kWave, smem, s>>>(xp, pp, sp, yp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), \
+                                                 steps_per_slice, partial);                                                   \
     }
     if (group == 32) TPQ_GEMM4(1) else if (group == 64) TPQ_GEMM4(2) else TPQ_GEMM4(4)
 #undef TPQ_GEMM4
-    return check_launch("tpq_int4_mm (gemm)");
+    if (int rc = check_launch("tpq_int4_mm (gemm)")) return rc;
+    if (partial == nullptr) return TPQ_OK;
+    const int64_t quads = M * N / 4;  // N % 8 == 0
+    int4_gemm_finish_kernel<DT><<<static_cast<unsigned>((quads + 255) / 256), 256, 0, s>>>(partial, slices, quads, yp);
+    return check_launch("tpq_int4_mm (gemm, sum of the slices)");
 }
 
 template <int DT>
-int launch_int4_gemm(const void* x, const int32_t* packed, const void* sz, void* y, int64_t M, int64_t N, int64_t K, int group, hipStream_t s) {
+int launch_int4_gemm(const void* x, const int32_t* packed, const void* sz, void* y, int64_t M, int64_t N, int64_t K, int group, hipStream_t s,
+                     int slices = 1, float* partial = nullptr) {
     static const int forced_nb = [] { const char* e = tuning_env("TPQ_INT4_GEMM_NB"); return e ? std::atoi(e) : 0; }();
     static const int forced_waves = [] { const char* e = tuning_env("TPQ_INT4_GEMM_WAVES"); return e ? std::atoi(e) : 0; }();
     static const int forced_rsplit = [] { const char* e = tuning_env("TPQ_INT4_GEMM_RSPLIT"); return e ? std::atoi(e) : 0; }();
@@ -260,24 +350,24 @@ int launch_int4_gemm(const void* x, const int32_t* packed, const void* sz, void*
     // 8192 x 8192, 256 rows: 73 with 64 channels (256 workgroups), 93 with 128.
     const bool few = M <= 256;
     const int64_t narrow_groups = ((N + 63) / 64) * ((M + kGemmRows - 1) / kGemmRows);
-    const int nb = forced_nb ? forced_nb : (few && narrow_groups <= 256 ? 1 : 2);
+    const int nb = forced_nb ? forced_nb : (few && (narrow_groups <= 256 || slices > 1) ? 1 : 2);
     const int waves = forced_waves ? forced_waves : 8;
     const int rsplit = forced_rsplit ? forced_rsplit : (few ? 2 : 1);
     if (rsplit == 4 && waves == 16) {
-        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 16, 4>(x, packed, sz, y, M, N, K, group, s);
-        return launch_int4_gemm_shape<DT, 1, 16, 4>(x, packed, sz, y, M, N, K, group, s);
+        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 16, 4>(x, packed, sz, y, M, N, K, group, slices, partial, s);
+        return launch_int4_gemm_shape<DT, 1, 16, 4>(x, packed, sz, y, M, N, K, group, slices, partial, s);
     }
     if (rsplit == 2 && waves == 16) {
-        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 16, 2>(x, packed, sz, y, M, N, K, group, s);
-        return launch_int4_gemm_shape<DT, 1, 16, 2>(x, packed, sz, y, M, N, K, group, s);
+        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 16, 2>(x, packed, sz, y, M, N, K, group, slices, partial, s);
+        return launch_int4_gemm_shape<DT, 1, 16, 2>(x, packed, sz, y, M, N, K, group, slices, partial, s);
     }
     if (rsplit == 2) {
-        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 8, 2>(x, packed, sz, y, M, N, K, group, s);
-        return launch_int4_gemm_shape<DT, 1, 8, 2>(x, packed, sz, y, M, N, K, group, s);
+        if (nb == 2) return launch_int4_gemm_shape<DT, 2, 8, 2>(x, packed, sz, y, M, N, K, group, slices, partial, s);
+        return launch_int4_gemm_shape<DT, 1, 8, 2>(x, packed, sz, y, M, N, K, group, slices, partial, s);
     }
-    if (nb == 2 && waves == 8) return launch_int4_gemm_shape<DT, 2, 8, 1>(x, packed, sz, y, M, N, K, group, s);
-    if (nb == 2) return launch_int4_gemm_shape<DT, 2, 4, 1>(x, packed, sz, y, M, N, K, group, s);
-    return launch_int4_gemm_shape<DT, 1, 4, 1>(x, packed, sz, y, M, N, K, group, s);
+    if (nb == 2 && waves == 8) return launch_int4_gemm_shape<DT, 2, 8, 1>(x, packed, sz, y, M, N, K, group, slices, partial, s);
+    if (nb == 2) return launch_int4_gemm_shape<DT, 2, 4, 1>(x, packed, sz, y, M, N, K, group, slices, partial, s);
+    return launch_int4_gemm_shape<DT, 1, 4, 1>(x, packed, sz, y, M, N, K, group, slices, partial, s);
 }
 
 }  // namespace

@@ -700,11 +700,16 @@ int launch_decode(const void* x, int64_t M, const int32_t* packed, const void* s
             if (flight_launch(DT, x, 1, one, K, group, false, nullptr, s, &rc)) return rc;
         }
     }
-    // Many rows: the tiled kernel, the packed weight read once per 128 rows.  Measured against the 32-row slabs below
-    // (us, fp16): K = 4096, N = 11008: 43 / 55 at 128 rows, 62 / 107 at 256, 258 / 821 at 2048; K = N = 8192:
-    // 77 / 81 at 128, 82 / 157 at 256; at 96 rows the slabs still win (42 against 43, 63 against 77).
-    static const int64_t gemm_rows = [] { const char* e = tuning_env("TPQ_INT4_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{113}; }();
-    if (M >= gemm_rows && int4_gemm_ok(x, packed, sz, y, M, N, K, group)) return launch_int4_gemm<DT>(x, packed, sz, y, M, N, K, group, s);
+    // Many rows: the tiled kernel, the packed weight read once per 128 rows, from 113 rows on and from 33 where its
+    // estimate beats the 32-row slabs below (int4_gemm_takes; TPQ_INT4_GEMM_ROWS pins the row count in sweeps).
+    static const int64_t gemm_rows = [] { const char* e = tuning_env("TPQ_INT4_GEMM_ROWS"); return e ? std::atoll(e) : int64_t{0}; }();
+    // few tiles: slices of K over the chip, their fp32 sums in the workspace behind the counters
+    const size_t room = workspace != nullptr && workspace_bytes > kCounterBytes ? workspace_bytes - kCounterBytes : 0;
+    if ((gemm_rows ? M >= gemm_rows : int4_gemm_takes(M, N, K, room)) && int4_gemm_ok(x, packed, sz, y, M, N, K, group)) {
+        const int slices = int4_gemm_slices(M, N, K, room);
+        float* partial = slices > 1 ? reinterpret_cast<float*>(static_cast<char*>(workspace) + kCounterBytes) : nullptr;
+        return launch_int4_gemm<DT>(x, packed, sz, y, M, N, K, group, s, slices, partial);
+    }
     {   // slabs of 32 rows (16 with groups of 32 / 64) on the matrix cores where the shape allows
         static const int slab_rows = [] { const char* e = tuning_env("TPQ_INT4_SLAB_ROWS"); return e ? std::atoi(e) : 32; }();
         const size_t row_x = static_cast<size_t>(K) * 2, row_y = static_cast<size_t>(N) * 2;
@@ -885,6 +890,17 @@ using namespace tpq;
 TPQ_EXPORT size_t tpq_int4_mm_workspace_bytes(int64_t N) {
     // counters + up to 16 slices of 4 rows of fp32 partial columns
     return N <= 0 ? 0 : kCounterBytes + static_cast<size_t>(16) * 4 * static_cast<size_t>(N) * sizeof(float);
+}
+
+TPQ_EXPORT size_t tpq_int4_mm_rows_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    // the decode kernels' share, and for 33 .. 256 rows up to 16 slices of fp32 sums for the tiled kernel
+    size_t bytes = tpq_int4_mm_workspace_bytes(N);
+    if (M >= kInt4GemmRowsSliced && M <= 256 && N > 0 && K >= 128) {
+        const int slices = int4_gemm_slices(M, N, K, ~static_cast<size_t>(0));
+        const size_t tiled = kCounterBytes + static_cast<size_t>(slices) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+        if (slices > 1 && tiled > bytes) bytes = tiled;
+    }
+    return bytes;
 }
 
 TPQ_EXPORT int tpq_int4_mm_ws(const void* x, int dtype, int64_t M, int64_t K, const int32_t* packed,

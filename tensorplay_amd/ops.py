@@ -243,11 +243,11 @@ def int8_mm_dequant(A_i8: torch.Tensor, B_t_i8: torch.Tensor, row_scale: torch.T
 _int4_workspaces = {}
 
 
-def _int4_workspace(device: torch.device, n: int) -> torch.Tensor:
-    """Zero-filled scratch buffer of the int4 decode kernel, one per (device, stream), grown on demand.
-    The kernel leaves the counters at the front of it zero again after every call."""
+def _int4_workspace(device: torch.device, m: int, n: int, k: int) -> torch.Tensor:
+    """Zero-filled scratch buffer of the int4 kernels, one per (device, stream), grown on demand.
+    The kernels leave the counters at the front of it zero again after every call."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
-    need = _lib.load().tpq_int4_mm_workspace_bytes(n)
+    need = _lib.load().tpq_int4_mm_rows_workspace_bytes(m, n, k)
     ws = _int4_workspaces.get(key)
     if ws is None or ws.numel() < need:
         ws = torch.zeros(need, dtype=torch.uint8, device=device)
@@ -361,7 +361,7 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
         dense = _int4_dequantize(w, inner, n, k, qGroupSize, sz)
         return _dense_mm(x, dense, out)
     with torch.cuda.device(self.device):
-        ws = _int4_workspace(self.device, n)
+        ws = _int4_workspace(self.device, m, n, k)
         _check(_lib.load().tpq_int4_mm_ws(_ptr(x), _DT[x.dtype], m, k, _ptr(w), inner, n, qGroupSize, _ptr(sz),
                                           _ptr(out), _ptr(ws), ws.numel(), _stream(self)))
     return out

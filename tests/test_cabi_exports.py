@@ -73,6 +73,24 @@ def test_int8_workspace_sizing_is_host_logic():
     assert lib.tpq_int_mm_ws(None, 0, None, 1, 1, None, 0, 4, 4, None, 0, None) == _lib.TPQ_OK
 
 
+def test_int4_rows_workspace_sizing_is_host_logic():
+    """tpq_int4_mm_rows_workspace_bytes: the decode kernels' share, and for 33 .. 256 rows the fp32 sums of the slices
+    the tiled kernel would take (counters + slices x M x N x 4)."""
+    from tensorplay_amd import _lib
+
+    lib = _lib.load()
+    base, rows = lib.tpq_int4_mm_workspace_bytes, lib.tpq_int4_mm_rows_workspace_bytes
+    counters = 4096 * 4
+    assert rows(1, 11008, 4096) == base(11008) and rows(32, 4096, 4096) == base(4096)
+    assert rows(128, 4096, 4096) == counters + 4 * 128 * 4096 * 4      # 64 workgroups of 64 channels -> four slices
+    assert rows(255, 4096, 4096) == counters + 2 * 255 * 4096 * 4      # 128 workgroups -> two
+    assert rows(128, 4096, 11008) == counters + 4 * 128 * 4096 * 4     # long K, few channels
+    assert rows(128, 11008, 4096) == base(11008)                       # 172 workgroups: one slice, nothing to add up
+    assert rows(300, 4096, 4096) == base(4096)                         # beyond 256 rows: no slices
+    assert rows(128, 4096, 512) == base(4096)                          # K of four steps: nothing to cut
+    assert rows(0, 4096, 4096) == base(4096) and rows(128, 0, 4096) == 0
+
+
 def test_bench_refuses_more_than_one_gpu():
     """The benchmark is a one-GPU program: any other --gpus value exits with a message and status 2."""
     import os

@@ -137,6 +137,46 @@ def test_mm_tiled_kernel_matches_oracle(ops, dtype, M, N, K, group):
     assert_close_norm(got32[:16], few, 2e-2 if dtype == "bf16" else 1e-2, "vs the decode kernel (cross-check of two kernels, each within 1e-2 of the CPU formulation)")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,group", [(40, 264, 2048, 128), (128, 520, 4096, 128), (200, 72, 11008, 128), (113, 264, 1024, 64),
+                                         (64, 2048, 2048, 128), (255, 136, 3072, 32), (96, 4096, 11008, 128)])
+def test_mm_tiled_kernel_with_slices_of_k(ops, dtype, M, N, K, group):
+    """33 .. 256 rows with a workspace: where the tiled kernel would leave most compute units idle the steps of K go to
+    several slices, whose fp32 sums meet in the workspace in slice order.  Against the CPU formulation and the exact
+    sums to the bounds of test_mm_matches_oracle, twice in a row into the same workspace bit for bit, and against the
+    same call without workspace (one slice or the 32-row slabs: other order of the sums only)."""
+    from tensorplay_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(M * 5 + N * 3 + K + group)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xb, szb = cast_bits(x, dtype), cast_bits(sz, dtype)
+    packed = oracle.int4_pack_tc(codes, 2)
+    xd, pd, sd = dev(xb, dtype), dev(packed), dev(szb, dtype)
+    tag = {"f16": _lib.F16, "bf16": _lib.BF16}[dtype]
+    need = lib.tpq_int4_mm_rows_workspace_bytes(M, N, K)
+    assert need >= lib.tpq_int4_mm_workspace_bytes(N)
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for _ in range(2):
+        out = torch.full((M, N), float("nan"), dtype=TORCH_DT[dtype], device=DEV)
+        rc = lib.tpq_int4_mm_ws(xd.data_ptr(), tag, M, K, pd.data_ptr(), 2, N, group, sd.data_ptr(), out.data_ptr(), ws.data_ptr(), need, stream)
+        assert rc == 0, _lib.last_error()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    got32 = outs[0].float().cpu().numpy()
+    _, y64 = oracle.int4_mm_tc(xb, dtype, packed, szb, group, round_w=False, want_f64=True)
+    assert_close_to_cpu_formulation(got32, xb, dtype, codes, szb, group)
+    assert rel_err(got32, y64) < {"f16": 1e-3, "bf16": 1e-2}[dtype]
+    plain = torch.empty((M, N), dtype=TORCH_DT[dtype], device=DEV)
+    rc = lib.tpq_int4_mm(xd.data_ptr(), tag, M, K, pd.data_ptr(), 2, N, group, sd.data_ptr(), plain.data_ptr(), stream)
+    assert rc == 0, _lib.last_error()
+    assert_close_norm(got32, plain.float().cpu().numpy(), 2e-2 if dtype == "bf16" else 1e-2, "vs the call without workspace")
+    # the counters at the front of the workspace are zero again: a decode call may share it
+    assert int(ws[:16384].view(torch.int32).abs().sum()) == 0
+
+
 @pytest.mark.parametrize("M", [1, 4, 16])
 def test_mm_config2_full_size(ops, M):
     """M x 4096 x 11008, group 128, fp16: the decode configuration at its real size."""
