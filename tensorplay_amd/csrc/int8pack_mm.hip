@@ -35,11 +35,26 @@ typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 
 // x: [M][K] fp16 or bf16; w: [N][K] int8; scale: [N] fp32; steps = K / 128; NB blocks of 16 channels and MB blocks
 // of 16 activation rows per workgroup (the converted weights of a step feed every row block)
+//
+// The activations of a step are 256 bytes = two cache lines per row.  Asked for in the MFMA's order (lane (m, q): 16
+// bytes at 64 q + 16 c of row m, four loads) every load touches two lines of every row, and the vector memory path
+// charges a load by the lines it touches: at 32 rows that is 256 line look-ups per step against 16 for the weights.  So
+// a wavefront reads them as they lie (lane l: piece l % 16 of row l / 16, four rows = eight whole lines per load) and
+// passes them to the MFMA's lanes through a wave-private LDS area, one block of 16 rows at a time (rows 272 bytes apart,
+// so that the sixteen rows of a 16-byte read spread over the banks).  Columns m >= M hold whatever is there; their sums
+// are dropped.
+constexpr int kI8pXPitch = 272;
+constexpr int kI8pXBytes = 16 * kI8pXPitch;  // per wavefront
+
 template <int DT, int NB, int MB, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
     const uint16_t* __restrict__ x, const int8_t* __restrict__ w, const float* __restrict__ scale,
     uint16_t* __restrict__ y, int M, int N, int K) {
-    __shared__ float red[WAVES][NB * MB][4][kWave];
+    // one LDS area for both uses: the exchange areas during the steps, the partial sums behind a barrier after them
+    constexpr size_t kRedBytes = sizeof(float) * WAVES * NB * MB * 4 * kWave, kXchBytes = static_cast<size_t>(WAVES) * kI8pXBytes;
+    __shared__ __align__(16) unsigned char lds_raw[kRedBytes > kXchBytes ? kRedBytes : kXchBytes];
+    float (*const red)[NB * MB][4][kWave] = reinterpret_cast<float (*)[NB * MB][4][kWave]>(lds_raw);
+    unsigned char (*const xch_all)[kI8pXBytes] = reinterpret_cast<unsigned char (*)[kI8pXBytes]>(lds_raw);
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
@@ -51,13 +66,18 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
         const int n = n0 + 16 * b + i;
         w_base[b] = reinterpret_cast<const uint4*>(w + static_cast<size_t>(n < N ? n : N - 1) * K) + q * 2;  // rows past N: a valid row, result dropped
     }
-    bool row_live[MB];  // columns m >= M stay zero and load nothing
-    const uint4* x_base[MB];
+    bool row_live[MB];
 #pragma unroll
-    for (int r = 0; r < MB; ++r) {
-        row_live[r] = 16 * r + i < M;
-        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live[r] ? 16 * r + i : 0) * K) + q * 4;
+    for (int r = 0; r < MB; ++r) row_live[r] = 16 * r + i < M;
+    // load j of a step: row 4 j + lane / 16, piece lane % 16 of the step's 256 bytes (rows past M: row 0, dropped)
+    const uint4* x_base[4 * MB];
+#pragma unroll
+    for (int j = 0; j < 4 * MB; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        x_base[j] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row < M ? row : 0) * K) + (lane & 15);
     }
+    unsigned char* const xch_put = xch_all[wave] + (lane >> 4) * kI8pXPitch + (lane & 15) * 16;  // + 4 j' rows
+    const unsigned char* const xch_get = xch_all[wave] + i * kI8pXPitch + q * 64;                 // + 16 c
 
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     const h2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
@@ -76,18 +96,26 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
         }
 #pragma unroll
         for (int r = 0; r < MB; ++r)
-            if (row_live[r]) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) st.xv[r][c] = x_base[r][s * 16 + c];
-            }
+            for (int c = 0; c < 4; ++c) st.xv[r][c] = x_base[4 * r + c][s * 16];  // as loaded: rows 16 r + 4 c .. + 3
     };
     float4_t d[NB][MB][2] = {};  // two accumulators per output block taking turns
     auto compute = [&](const Step& st) {
+        // each block of 16 rows into the exchange area and this lane's four pieces out of it (LDS keeps a wavefront's
+        // accesses in order: the reads of the block before are served before these writes)
+        uint4 xb[MB][4];
+#pragma unroll
+        for (int r = 0; r < MB; ++r) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) *reinterpret_cast<uint4*>(xch_put + c * 4 * kI8pXPitch) = st.xv[r][c];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) xb[r][c] = *reinterpret_cast<const uint4*>(xch_get + c * 16);
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {  // MFMA u (16x16x32): k = 8u .. 8u+7 of the lane's 32
             word4_t bv[MB];
 #pragma unroll
-            for (int r = 0; r < MB; ++r) bv[r] = word4_t{st.xv[r][u].x, st.xv[r][u].y, st.xv[r][u].z, st.xv[r][u].w};
+            for (int r = 0; r < MB; ++r) bv[r] = word4_t{xb[r][u].x, xb[r][u].y, xb[r][u].z, xb[r][u].w};
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 uint32_t a[4];
@@ -150,6 +178,7 @@ __global__ __launch_bounds__(WAVES * kWave) void int8pack_mfma_kernel(
                 scale_n[b][v] = sp[n < N ? n : N - 1];
             }
     }
+    __syncthreads();  // every wavefront is done with its exchange area
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
