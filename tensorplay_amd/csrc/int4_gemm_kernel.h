@@ -282,21 +282,23 @@ inline int int4_gemm_slices(int64_t M, int64_t N, int64_t K, size_t room) { retu
 
 // From how many rows the tiled kernel takes a shape: always from kInt4GemmRows; from kInt4GemmRowsSliced where its
 // estimate is below that of the slabs of 32 rows it replaces, each of which streams the weight again: a slab of 32 rows
-// takes about 1.6 + 0.31 per MB of packed weight + 1.33 per 1024 k (us, fitted to eight shapes, +- 20 %), a shorter last
-// slab 55 % of that plus its share of the rest.  Measured (us, slabs / tiled, 33 - 48 - 64 - 80 - 96 - 112 rows):
-//   4096 x 4096     12.6 14.0 16.1 21.4 23.2 28.2 / 15.5 15.7 16.1 16.9 17.6 18.4
-//   4096 -> 11008   18.8 19.6 23.0 29.8 32.7 40.2 / 34.3 32.9 33.1 33.3 33.4 33.7
-//   11008 -> 4096   31.6 37.9 47.6 61.3 71.0 84.8 / 30.0 29.6 29.7 29.9 30.7 31.4
-//   8192 x 8192     30.6 32.8 40.5 51.0 59.4 69.9 / 40.1 39.8 39.8 40.4 40.0 40.0
-//   2048 x 2048     10.2 11.2 13.5 17.7 20.0 24.4 /  9.8 10.1 10.5 10.8 11.2 11.7
-//   13824 -> 5120   45.1 50.4 61.9 81.5 93.3 112  / 41.5 42.3 42.2 42.4 42.3 42.9
+// takes about 2.7 + 0.37 per MB of packed weight + 0.67 per 1024 k (us, fitted to eight shapes, +- 10 %), a shorter last
+// slab 45 % of that plus its share of the rest.  Measured (us, slabs / tiled, 33 - 48 - 64 - 80 - 96 - 112 rows):
+//   4096 x 4096     12.1 13.9 15.8 21.2 23.0 28.3 / 15.0 15.5 16.0 16.8 17.6 18.3
+//   4096 -> 11008   18.7 19.7 23.8 29.9 33.2 40.5 / 34.0 33.2 33.1 33.3 33.5 33.9
+//   11008 -> 4096   24.4 28.8 33.1 43.5 47.5 58.8 / 29.5 29.2 29.6 30.0 31.0 31.5
+//   8192 x 8192     27.9 29.7 34.3 45.0 49.6 60.9 / 38.8 38.5 38.1 38.7 39.6 40.1
+//   2048 x 2048      8.8  9.8 10.8 14.8 15.6 19.9 /  9.8 10.0 10.4 10.8 11.2 11.7
+//   13824 -> 5120   39.2 41.1 49.0 65.7 73.4 89.8 / 38.8 39.7 40.5 41.6 42.0 42.4
+//   4096 -> 32000   43.0 49.8 57.4 73.2 81.5 98.4 / 54.9 52.4 51.9 51.9 50.2 52.5
+//   5120 x 5120     17.2 19.0 22.8 30.2 34.1 41.3 / 20.6 20.7 21.3 22.1 22.6 23.6
 constexpr int64_t kInt4GemmRows = 113, kInt4GemmRowsSliced = 33;
 inline bool int4_gemm_takes(int64_t M, int64_t N, int64_t K, size_t room) {
     if (M >= kInt4GemmRows) return true;
     if (M < kInt4GemmRowsSliced) return false;
-    const double slab = 1.6 + 0.31 * static_cast<double>(N) * static_cast<double>(K) / 2e6 + 1.33 * static_cast<double>(K) / 1024.0;
+    const double slab = 2.7 + 0.37 * static_cast<double>(N) * static_cast<double>(K) / 2e6 + 0.67 * static_cast<double>(K) / 1024.0;
     const int64_t whole = M / 32, rest = M % 32;
-    const double slabs = static_cast<double>(whole) * slab + (rest ? slab * (0.55 + 0.45 * static_cast<double>(rest) / 32.0) : 0.0);
+    const double slabs = static_cast<double>(whole) * slab + (rest ? slab * (0.45 + 0.55 * static_cast<double>(rest) / 32.0) : 0.0);
     return int4_gemm_plan(M, N, K, room).us < slabs;
 }
 

@@ -92,7 +92,16 @@ __device__ __forceinline__ void int4_mfma_body(
     constexpr bool DEQ = GKT < 4;
     using L = Lane16<DT>;
     using ML = MfmaLane<DT>;
-    __shared__ float red[WAVES][NB * MB][4][kWave];
+    // The activations of a step (256 bytes = two cache lines per row) are read as they lie, four rows = eight whole
+    // lines per wave-level load, and reach the MFMA's lanes (lane (m, q): 64 bytes of row m) through a wave-private
+    // LDS area, one block of 16 rows at a time, rows 272 bytes apart: asked for in MFMA order every load touches two
+    // lines of every row, and the vector memory path charges a load by the lines it touches.  Columns m >= M hold
+    // whatever is there; their sums are dropped.  One LDS area serves both uses: the exchange during the steps, the
+    // partial sums behind a barrier after them.
+    constexpr int kXPitch = 272, kXBytes = 16 * kXPitch;
+    constexpr size_t kRedBytes = sizeof(float) * WAVES * NB * MB * 4 * kWave, kXchBytes = static_cast<size_t>(WAVES) * kXBytes;
+    __shared__ __align__(16) unsigned char lds_raw[kRedBytes > kXchBytes ? kRedBytes : kXchBytes];
+    float (*const red)[NB * MB][4][kWave] = reinterpret_cast<float (*)[NB * MB][4][kWave]>(lds_raw);
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -115,12 +124,17 @@ __device__ __forceinline__ void int4_mfma_body(
         if constexpr (DEQ) sz_base[b] = sz + ((nb0 + i) < N ? nb0 + i : N - 1);  // (scale, zero) of this lane's weight row
     }
     bool row_live[MB];
-    const uint4* x_base[MB];
 #pragma unroll
-    for (int r = 0; r < MB; ++r) {
-        row_live[r] = 16 * r + i < M;
-        x_base[r] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row_live[r] ? 16 * r + i : 0) * K) + q * 4;
+    for (int r = 0; r < MB; ++r) row_live[r] = 16 * r + i < M;
+    // load j of a step: row 4 j + lane / 16, piece lane % 16 of the step's 256 bytes (rows past M: row 0, dropped)
+    const uint4* x_base[4 * MB];
+#pragma unroll
+    for (int j = 0; j < 4 * MB; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        x_base[j] = reinterpret_cast<const uint4*>(x + static_cast<size_t>(row < M ? row : 0) * K) + (lane & 15);
     }
+    unsigned char* const xch_put = lds_raw + wave * kXBytes + (lane >> 4) * kXPitch + (lane & 15) * 16;  // + 4 c rows
+    const unsigned char* const xch_get = lds_raw + wave * kXBytes + i * kXPitch + q * 64;                 // + 16 c
 
     // constant A of the correction MFMA: row 0 = offset + 8 of the pair parity, row 1 = ones
     uint32_t a_corr_even = 0, a_corr_odd = 0;
@@ -144,10 +158,8 @@ __device__ __forceinline__ void int4_mfma_body(
         }
 #pragma unroll
         for (int r = 0; r < MB; ++r)
-            if (row_live[r]) {  // columns m >= M keep the zeros they start with: no load, nothing stored
 #pragma unroll
-                for (int c = 0; c < 4; ++c) st.xv[r][c] = x_base[r][s * 16 + c];
-            }
+            for (int c = 0; c < 4; ++c) st.xv[r][c] = x_base[4 * r + c][s * 16];  // as loaded: rows 16 r + 4 c .. + 3
     };
 
     float yacc[NB][MB][4];
@@ -168,6 +180,16 @@ __device__ __forceinline__ void int4_mfma_body(
             aux[r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int b = 0; b < NB; ++b) d[b][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        // each block of 16 rows into the exchange area and this lane's four pieces out of it (LDS keeps a wavefront's
+        // accesses in order: the reads of the block before are served before these writes)
+        uint4 xq[MB][4];
+#pragma unroll
+        for (int r = 0; r < MB; ++r) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) *reinterpret_cast<uint4*>(xch_put + c * 4 * kXPitch) = st.xv[r][c];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) xq[r][c] = *reinterpret_cast<const uint4*>(xch_get + c * 16);
         }
         uint32_t v[NB][4][4];  // [block][word r][pair j] = codes at k = 2 r + 8 j, + 1 of the lane's k-tile
 #pragma unroll
@@ -218,7 +240,7 @@ __device__ __forceinline__ void int4_mfma_body(
             const uint32_t off = (u & 1) ? a_corr_odd : a_corr_even;
             word4_t xb[MB];
 #pragma unroll
-            for (int r = 0; r < MB; ++r) xb[r] = word4_t{st.xv[r][u].x, st.xv[r][u].y, st.xv[r][u].z, st.xv[r][u].w};
+            for (int r = 0; r < MB; ++r) xb[r] = word4_t{xq[r][u].x, xq[r][u].y, xq[r][u].z, xq[r][u].w};
             const word4_t ac = {off, off, off, off};
             if constexpr (!DEQ) {
 #pragma unroll
@@ -273,6 +295,7 @@ __device__ __forceinline__ void int4_mfma_body(
         if (s + 2 * WAVES < steps) compute(s0);
     }
 
+    __syncthreads();  // every wavefront is done with its exchange area
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
