@@ -237,10 +237,16 @@ __global__ __launch_bounds__(256) void int4_gemm_finish_kernel(const float* __re
     using L = Lane16<DT>;
     const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (e >= quads) return;
-    float4_t sum = reinterpret_cast<const float4_t*>(partial)[e];
-    for (int z = 1; z < slices; ++z) {
-        const float4_t more = reinterpret_cast<const float4_t*>(partial)[static_cast<int64_t>(z) * quads + e];
-        sum = float4_t{sum[0] + more[0], sum[1] + more[1], sum[2] + more[2], sum[3] + more[3]};
+    // four slices requested together (a loop of load and add would wait for memory once per slice), added in slice
+    // order; a batch past the last slice asks for the last one again and leaves it out of the sum
+    float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int z0 = 0; z0 < slices; z0 += 4) {
+        float4_t more[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) more[j] = reinterpret_cast<const float4_t*>(partial)[static_cast<int64_t>(z0 + j < slices ? z0 + j : slices - 1) * quads + e];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (z0 + j < slices) sum = float4_t{sum[0] + more[j][0], sum[1] + more[j][1], sum[2] + more[j][2], sum[3] + more[j][3]};
     }
     const uint32_t lo = L::out(sum[0]) | (static_cast<uint32_t>(L::out(sum[1])) << 16);
     const uint32_t hi = L::out(sum[2]) | (static_cast<uint32_t>(L::out(sum[3])) << 16);

@@ -129,9 +129,17 @@ __global__ __launch_bounds__(256) void int8_finish_kernel(const int32_t* __restr
                 const float4 b = has_bias ? *reinterpret_cast<const float4*>(bias + n) : make_float4(0, 0, 0, 0);
                 const float r = rs[m];
                 int4 v = make_int4(0, 0, 0, 0);
-                for (int z = 0; z < slices; ++z) {
-                    const uint4 p = nt_load(reinterpret_cast<const uint4*>(partial + z * total + idx));
-                    v.x += static_cast<int>(p.x); v.y += static_cast<int>(p.y); v.z += static_cast<int>(p.z); v.w += static_cast<int>(p.w);
+                // four slices requested together (a loop of load and add would wait for memory once per slice); a
+                // batch past the last slice asks for the last one again and leaves it out of the sum
+                for (int z0 = 0; z0 < slices; z0 += 4) {
+                    uint4 p[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) p[j] = nt_load(reinterpret_cast<const uint4*>(partial + (z0 + j < slices ? z0 + j : slices - 1) * total + idx));
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (z0 + j < slices) {
+                            v.x += static_cast<int>(p[j].x); v.y += static_cast<int>(p[j].y); v.z += static_cast<int>(p[j].z); v.w += static_cast<int>(p[j].w);
+                        }
                 }
                 const typename Elem<DT>::storage o[4] = {TileDequant<DT>::convert(v.x, r, c.x, b.x, has_bias), TileDequant<DT>::convert(v.y, r, c.y, b.y, has_bias),
                                                         TileDequant<DT>::convert(v.z, r, c.z, b.z, has_bias), TileDequant<DT>::convert(v.w, r, c.w, b.w, has_bias)};

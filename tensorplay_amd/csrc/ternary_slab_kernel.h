@@ -287,9 +287,15 @@ __global__ __launch_bounds__(256) void ternary_slab_finish_kernel(const int32_t*
     for (int e = 0; e < 4; ++e) bias_n[e] = ep.bias_of(e < count ? n + e : n);
     int v[4] = {0, 0, 0, 0};
     if (whole) {
-        for (int s = 0; s < splits; ++s) {
-            const int4 q = *reinterpret_cast<const int4*>(partial + s * total + idx);
-            v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
+        // four splits requested together (a loop of load and add would wait for memory once per split); a batch past
+        // the last split asks for the last one again and leaves it out of the sum
+        for (int s0 = 0; s0 < splits; s0 += 4) {
+            int4 q[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q[j] = *reinterpret_cast<const int4*>(partial + (s0 + j < splits ? s0 + j : splits - 1) * total + idx);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (s0 + j < splits) { v[0] += q[j].x; v[1] += q[j].y; v[2] += q[j].z; v[3] += q[j].w; }
         }
     } else {
         for (int s = 0; s < splits; ++s)
