@@ -65,6 +65,11 @@ int launch_tiled(const int8_t* a, const int8_t* w, int64_t M, int64_t N, int64_t
     const char* env = tuning_env("TPQ_INT8_FORM");
     if (slices > 1) {
         if (env && env[0] == 's') return launch_stagger(a, w, M, N, K, tile, s, slices);
+        // up to 128 rows the 256-row tiles of the lock-step kernel are half empty: the 128-row staggered tiles, cut the
+        // same way (us, 33 / 128 rows: 4096 x 4096 14.2 / 15.7 -> 12.2 / 14.5, 11008 -> 4096 21.3 / 23.6 -> 18.1 / 21.5,
+        // 8192 x 8192 26.2 / 29.5 -> 22.3 / 26.9)
+        if ((env && env[0] == 'h') || (!env && M <= 128 && K < (1 << 23)))
+            return launch_stagger_bytes<ArithI8, 2>(a, w, M, N, K, tile, s, slices, "int8 mfma gemm (staggered, 128 rows, slices)");
         return launch_dma(a, w, M, N, K, tile, s, slices);
     }
     if (K >= (1 << 23) || (env && env[0] == 'd')) return launch_dma(a, w, M, N, K, tile, s, 1);
