@@ -84,7 +84,11 @@ constexpr uint32_t kSignFlip = 0x80808080u;
 template <int BITS, bool LSB>
 constexpr int lowbit_x_pitch() { return Fields<BITS, LSB>::kStepK * 2 + 16; }
 
-template <int DT, int BITS, bool LSB, int WAVES, int XL>
+// NB blocks of 16 channels per workgroup share the activations of a step: every workgroup pulls all activation rows
+// through its compute unit, so with one block the activations outweigh a narrow packed weight many times over.
+// 4096 -> 11008 with three blocks against one (us, 1 / 2 / 4 bits): 2 rows 9.2 / 9.0 / 10.4 -> 8.2 / 8.6 / 9.3, 8 rows
+// 12.3 / 11.0 / 11.5 -> 9.9 / 10.5 / 11.1, 16 rows 12.8 / 12.4 / 13.4 -> 10.5 / 10.9 / 11.6.
+template <int DT, int BITS, bool LSB, int WAVES, int XL, int NB>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
     const float* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int group_shift) {
@@ -93,18 +97,23 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     constexpr int kRowsPerLoad = kWave / kPiecesPerRow;    // 4 or 8
     constexpr int kPitch = lowbit_x_pitch<BITS, LSB>();
     static_assert(XL * kRowsPerLoad <= 16, "at most 16 rows per launch");
-    __shared__ float red[WAVES][4][kWave];
+    __shared__ float red[WAVES][NB * 4][kWave];
     extern __shared__ __align__(16) unsigned char lowbit_xch[];  // [WAVES][16 rows][kPitch]
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const int steps = K / F::kStepK;
-    const int n0 = blockIdx.x * 16;
-    const int n_row = n0 + i < N ? n0 + i : N - 1;  // rows past N: a valid row, result dropped
-    const uint8_t* w_base = packed + static_cast<size_t>(n_row) * (K / F::kPerByte) + q * F::kBytes;
-    int n4 = n0 + 4 * q;  // this lane's four output channels
-    n4 = n4 + 4 <= N ? n4 : N - 4;
-    const float* sz_base = sz + static_cast<size_t>(n4) * 2;
+    const int n0 = blockIdx.x * (16 * NB);
+    const uint8_t* w_base[NB];
+    const float* sz_base[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int n_row = n0 + 16 * b + i < N ? n0 + 16 * b + i : N - 1;  // rows past N: a valid row, result dropped
+        w_base[b] = packed + static_cast<size_t>(n_row) * (K / F::kPerByte) + q * F::kBytes;
+        int n4 = n0 + 16 * b + 4 * q;  // this lane's four output channels of the block
+        n4 = n4 + 4 <= N ? n4 : N - 4;
+        sz_base[b] = sz + static_cast<size_t>(n4) * 2;
+    }
     const bool row_live = i < M;
     // load j of a step: row kRowsPerLoad j + lane / kPiecesPerRow, piece lane % kPiecesPerRow (rows past M: row 0, dropped)
     const uint4* x_base[XL];
@@ -130,26 +139,35 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     for (int t = 0; t < F::kMagics; ++t) asm volatile("v_mov_b32 %0, %1" : "=v"(magic[t]) : "s"(F::magic(t)));
 
     struct Step {
-        uint4 w;       // kBytes of it are used
-        uint4 p[2];    // (scale, zero) of four channels
-        uint4 xv[XL];  // as loaded: piece lane % kPiecesPerRow of row kRowsPerLoad j + lane / kPiecesPerRow
+        uint4 w[NB];     // kBytes of each are used
+        uint4 p[NB][2];  // (scale, zero) of four channels
+        uint4 xv[XL];    // as loaded: piece lane % kPiecesPerRow of row kRowsPerLoad j + lane / kPiecesPerRow
     };
     auto load = [&](int s, Step& st) {
-        const uint8_t* src = w_base + static_cast<size_t>(s) * (4 * F::kBytes);
-        if constexpr (F::kBytes == 16) st.w = nt_load(reinterpret_cast<const uint4*>(src));
-        if constexpr (F::kBytes == 8) { const uint2 t = nt_load(reinterpret_cast<const uint2*>(src)); st.w = make_uint4(t.x, t.y, 0, 0); }
-        if constexpr (F::kBytes == 4) st.w = make_uint4(nt_load(reinterpret_cast<const uint32_t*>(src)), 0, 0, 0);
-        if constexpr (BITS == 8) st.w = make_uint4(st.w.x ^ kSignFlip, st.w.y ^ kSignFlip, st.w.z ^ kSignFlip, st.w.w ^ kSignFlip);
-        const uint4* prm = reinterpret_cast<const uint4*>(sz_base + static_cast<size_t>(s >> group_shift) * N * 2);
-        st.p[0] = prm[0];
-        st.p[1] = prm[1];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint8_t* src = w_base[b] + static_cast<size_t>(s) * (4 * F::kBytes);
+            if constexpr (F::kBytes == 16) st.w[b] = nt_load(reinterpret_cast<const uint4*>(src));
+            if constexpr (F::kBytes == 8) { const uint2 t = nt_load(reinterpret_cast<const uint2*>(src)); st.w[b] = make_uint4(t.x, t.y, 0, 0); }
+            if constexpr (F::kBytes == 4) st.w[b] = make_uint4(nt_load(reinterpret_cast<const uint32_t*>(src)), 0, 0, 0);
+            if constexpr (BITS == 8) st.w[b] = make_uint4(st.w[b].x ^ kSignFlip, st.w[b].y ^ kSignFlip, st.w[b].z ^ kSignFlip, st.w[b].w ^ kSignFlip);
+            const uint4* prm = reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N * 2);
+            st.p[b][0] = prm[0];
+            st.p[b][1] = prm[1];
+        }
 #pragma unroll
         for (int j = 0; j < XL; ++j) st.xv[j] = x_base[j][static_cast<size_t>(s) * kPiecesPerRow];
     };
 
-    float yacc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float yacc[NB][4];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) yacc[b][v] = 0.0f;
     auto compute = [&](const Step& st) {
-        float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f}, d = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t aux = {0.0f, 0.0f, 0.0f, 0.0f}, d[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) d[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         // the step's activations into the exchange area and this lane's pieces out of it (LDS keeps a wavefront's
         // accesses in order: the reads of the step before are served before these writes)
 #pragma unroll
@@ -159,39 +177,42 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
         for (int c = 0; c < F::kCodes / 8; ++c) xb[c] = *reinterpret_cast<const uint4*>(xch_get + c * 16);
 #pragma unroll
         for (int u = 0; u < F::kCodes / 8; ++u) {  // MFMA u (16x16x32): codes 8u .. 8u+7 of the lane
-            uint32_t a[4];
-#pragma unroll
-            for (int h = 0; h < 4; ++h) {
-                const int t = 4 * u + h;
-                const uint32_t word = dword_at(st.w, F::byte_lo(t) >> 2);
-                if constexpr (DT == TPQ_DTYPE_F16) {
-                    const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
-                    a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
-                } else {
-                    const float lo = static_cast<float>((word >> (8 * (F::byte_lo(t) & 3) + F::pos_lo(t))) & F::kField);
-                    const float hi = static_cast<float>((word >> (8 * (F::byte_hi(t) & 3) + F::pos_hi(t))) & F::kField);
-                    a[h] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
-                }
-            }
-            const word4_t av = {a[0], a[1], a[2], a[3]}, cv = {a_corr[0], a_corr[1], a_corr[2], a_corr[3]};
+            const word4_t cv = {a_corr[0], a_corr[1], a_corr[2], a_corr[3]};
             const word4_t bv = {xb[u].x, xb[u].y, xb[u].z, xb[u].w};  // the same eight k of the activations
-            if constexpr (DT == TPQ_DTYPE_F16) {
-                aux = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, cv), __builtin_bit_cast(half8_t, bv), aux, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d, 0, 0, 0);
-            } else {
-                aux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, cv), __builtin_bit_cast(bf8_t, bv), aux, 0, 0, 0);
-                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), d, 0, 0, 0);
+            if constexpr (DT == TPQ_DTYPE_F16) aux = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, cv), __builtin_bit_cast(half8_t, bv), aux, 0, 0, 0);
+            else aux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, cv), __builtin_bit_cast(bf8_t, bv), aux, 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                uint32_t a[4];
+#pragma unroll
+                for (int h = 0; h < 4; ++h) {
+                    const int t = 4 * u + h;
+                    const uint32_t word = dword_at(st.w[b], F::byte_lo(t) >> 2);
+                    if constexpr (DT == TPQ_DTYPE_F16) {
+                        const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
+                        a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
+                    } else {
+                        const float lo = static_cast<float>((word >> (8 * (F::byte_lo(t) & 3) + F::pos_lo(t))) & F::kField);
+                        const float hi = static_cast<float>((word >> (8 * (F::byte_hi(t) & 3) + F::pos_hi(t))) & F::kField);
+                        a[h] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+                    }
+                }
+                const word4_t av = {a[0], a[1], a[2], a[3]};
+                if constexpr (DT == TPQ_DTYPE_F16) d[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d[b], 0, 0, 0);
+                else d[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), d[b], 0, 0, 0);
             }
         }
         // rows 0 and 1 of the offset product sit in lanes 0..15, registers 0 and 1
         const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const uint4& pv = st.p[v >> 1];
-            const float scale = __builtin_bit_cast(float, (v & 1) ? pv.z : pv.x);
-            const float zero = __builtin_bit_cast(float, (v & 1) ? pv.w : pv.y) + (BITS == 8 ? 128.0f : 0.0f);
-            yacc[v] = __builtin_fmaf(scale, (d[v] - corr) - zero * sx, yacc[v]);
-        }
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint4& pv = st.p[b][v >> 1];
+                const float scale = __builtin_bit_cast(float, (v & 1) ? pv.z : pv.x);
+                const float zero = __builtin_bit_cast(float, (v & 1) ? pv.w : pv.y) + (BITS == 8 ? 128.0f : 0.0f);
+                yacc[b][v] = __builtin_fmaf(scale, (d[b][v] - corr) - zero * sx, yacc[b][v]);
+            }
     };
 
     // this wavefront's steps: wave, wave + WAVES, ...; two in flight
@@ -213,22 +234,27 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     }
 
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][v][lane] = yacc[v];
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][4 * b + v][lane] = yacc[b][v];
     __syncthreads();
-    if (wave == 0) {  // lane (m, q): channels n0 + 4 q + v
-        const int n = n0 + 4 * q;
-        if (row_live && n < N) {  // N % 4 == 0: all four channels exist
-            float sum[4];
+    if (wave == 0 && row_live) {  // lane (m, q): channels n0 + 16 b + 4 q + v
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                sum[v] = 0.0f;
+        for (int b = 0; b < NB; ++b) {
+            const int n = n0 + 16 * b + 4 * q;
+            if (n < N) {  // N % 4 == 0: all four channels exist
+                float sum[4];
 #pragma unroll
-                for (int w = 0; w < WAVES; ++w) sum[v] += red[w][v][lane];
-                if (bias != nullptr) sum[v] += bias[n + v];
+                for (int v = 0; v < 4; ++v) {
+                    sum[v] = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) sum[v] += red[w][4 * b + v][lane];
+                    if (bias != nullptr) sum[v] += bias[n + v];
+                }
+                const uint32_t lo = Elem<DT>::store(sum[0]) | (static_cast<uint32_t>(Elem<DT>::store(sum[1])) << 16);
+                const uint32_t hi = Elem<DT>::store(sum[2]) | (static_cast<uint32_t>(Elem<DT>::store(sum[3])) << 16);
+                *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
             }
-            const uint32_t lo = Elem<DT>::store(sum[0]) | (static_cast<uint32_t>(Elem<DT>::store(sum[1])) << 16);
-            const uint32_t hi = Elem<DT>::store(sum[2]) | (static_cast<uint32_t>(Elem<DT>::store(sum[3])) << 16);
-            *reinterpret_cast<uint2*>(y + static_cast<size_t>(i) * N + n) = make_uint2(lo, hi);
         }
     }
 }
@@ -433,33 +459,32 @@ __global__ __launch_bounds__(256) void lowbit_unpack_kernel(const uint8_t* __res
 template <int DT, int BITS, bool LSB>
 int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const float* bias, void* out, int64_t M, int64_t N,
                 int64_t K, int group_shift, hipStream_t s) {
-    // wavefronts per 16-channel workgroup: each takes every WAVES-th step, two in flight
+    // wavefronts per workgroup: each takes every WAVES-th step, two in flight
     static const int forced = [] { const char* e = tuning_env("TPQ_LOWBIT_WAVES"); return e ? atoi(e) : 0; }();
+    static const int forced_nb = [] { const char* e = tuning_env("TPQ_LOWBIT_NB"); return e ? atoi(e) : 0; }();
     const int64_t steps = K / Fields<BITS, LSB>::kStepK;
     // measured at 4096 -> 11008, one row, 2 bits: 4 waves 11.1 us, 8 waves 10.4 - 11.0 us, 16 waves 14.3 us
-    const int waves = forced ? forced : steps >= 16 ? 8 : 4;
+    const int waves = forced == 4 || forced == 8 ? forced : steps >= 16 ? 8 : 4;
+    // blocks of 16 channels per workgroup (eight wavefronts only): as many as leave about one workgroup per compute unit
+    int nb = 1;
+    if (waves == 8) nb = forced_nb >= 1 && forced_nb <= 3 ? forced_nb : (N >= 10240 ? 3 : N > 4096 ? 2 : 1);
     constexpr int kRowsPerLoad = kWave / (Fields<BITS, LSB>::kStepK / 8);  // 4, or 8 at one code per byte
     constexpr int kFull = 16 / kRowsPerLoad;                               // loads of activations per step for 16 rows
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = static_cast<int>(M - m0 < 16 ? M - m0 : 16);
-        const dim3 grid(static_cast<unsigned>((N + 15) / 16));
+        const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
         const uint16_t* xs = static_cast<const uint16_t*>(x) + m0 * K;
         uint16_t* ys = static_cast<uint16_t*>(out) + m0 * N;
         const int n = static_cast<int>(N), k = static_cast<int>(K);
         const bool few = rows <= kRowsPerLoad;  // one load of activations per step
-        const size_t xch = static_cast<size_t>(waves >= 16 ? 16 : waves >= 8 ? 8 : 4) * 16 * lowbit_x_pitch<BITS, LSB>();
-#define TPQ_LB_MFMA(W, XLV)                                                                                                   \
-    do {                                                                                                                      \
-        auto kernel = lowbit_mfma_kernel<DT, BITS, LSB, W, XLV>;                                                              \
-        if (xch + sizeof(float) * W * 4 * kWave > 64 * 1024) {                                                                \
-            static std::atomic<uint64_t> configured{0};                                                                       \
-            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), xch, configured, "tpq_lowbit_mm (mfma)")) return rc; \
-        }                                                                                                                     \
-        kernel<<<grid, W * kWave, xch, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift);                               \
-    } while (0)
-        if (waves >= 16) { if (few) TPQ_LB_MFMA(16, 1); else TPQ_LB_MFMA(16, kFull); }
-        else if (waves >= 8) { if (few) TPQ_LB_MFMA(8, 1); else TPQ_LB_MFMA(8, kFull); }
-        else { if (few) TPQ_LB_MFMA(4, 1); else TPQ_LB_MFMA(4, kFull); }
+        const size_t xch = static_cast<size_t>(waves) * 16 * lowbit_x_pitch<BITS, LSB>();
+#define TPQ_LB_MFMA(W, XLV, NBV) lowbit_mfma_kernel<DT, BITS, LSB, W, XLV, NBV><<<grid, W * kWave, xch, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift)
+#define TPQ_LB_MFMA_X(W, NBV) do { if (few) TPQ_LB_MFMA(W, 1, NBV); else TPQ_LB_MFMA(W, kFull, NBV); } while (0)
+        if (waves == 4) TPQ_LB_MFMA_X(4, 1);
+        else if (nb == 3) TPQ_LB_MFMA_X(8, 3);
+        else if (nb == 2) TPQ_LB_MFMA_X(8, 2);
+        else TPQ_LB_MFMA_X(8, 1);
+#undef TPQ_LB_MFMA_X
 #undef TPQ_LB_MFMA
     }
     return check_launch("tpq_lowbit_mm (mfma)");

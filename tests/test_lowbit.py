@@ -187,6 +187,28 @@ def test_gpu_mm_decode_kernel(bits, lsb, N, K, group, M, tdt, tag, tol):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bits,lsb", [(1, True), (2, False), (3, False), (4, False), (8, False)])
+@pytest.mark.parametrize("N,K,group,M", [(4104, 2048, 128, 5), (10248, 2048, 128, 9), (10244, 4096, 128, 16), (4100, 2048, 64, 2), (8200, 2048, 256, 20)])
+@pytest.mark.parametrize("tdt,tag,tol", [(torch.float16, "f16", 1e-3), (torch.bfloat16, "bf16", 8e-3)])
+def test_gpu_mm_decode_kernel_wide_weights(bits, lsb, N, K, group, M, tdt, tag, tol):
+    """Wide weights with 16 steps of K and more: two and three blocks of 16 channels per workgroup share the activations
+    of a step; channel counts that leave the last workgroup with a partial block and with whole blocks missing, 2..20
+    rows (one and four loads of activations per step, a second slab of rows), with a bias."""
+    from tensorplay_amd import ops
+    rng = np.random.default_rng(bits * 17 + N + M)
+    codes, sz = make_case(rng, bits, N, K, group)
+    x16 = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(tdt)
+    bias = rng.standard_normal(N).astype(np.float32)
+    packed = oracle.lowbit_pack(codes, bits, lsb_first=lsb)
+    want = oracle.lowbit_mm(x16.view(torch.int16).numpy().view(np.uint16), tag, packed, bits, sz, K, group, bias=bias,
+                            lsb_first=lsb, want_f64=True)[1]
+    got = ops._lowbit_mm(x16.to(DEV), torch.from_numpy(packed).to(DEV), bits, K, torch.from_numpy(sz).to(DEV),
+                         torch.from_numpy(bias).to(DEV), lsb_first=lsb)
+    assert got.dtype == tdt and got.shape == (M, N)
+    assert rel_err(got.float().cpu().numpy(), want) < tol
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("bits,lsb", [(1, False), (1, True), (2, False), (2, True), (4, False), (4, True), (8, False)])
 @pytest.mark.parametrize("N,K,group", [(10, 4096, 128), (7, 8192, 64), (130, 4160, 32), (5, 20480, 1024), (1, 64, 64), (36, 11008, 128),
                                        # rows of 64 KB and 128 KB: the activation row in LDS beyond the default limit (1 and 2 bits)
