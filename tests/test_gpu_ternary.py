@@ -128,7 +128,7 @@ def test_ternary_slab_arbitrary_bytes(ops, M, K, N):
     np.testing.assert_array_equal(host(got_only), want)
 
 
-@pytest.mark.parametrize("K,N", [(64, 3), (64, 5), (192, 1000), (320, 77), (1024, 1), (2560, 6912), (6912, 2560), (4096, 4100),
+@pytest.mark.parametrize("K,N", [(64, 3), (64, 5), (64, 70001), (128, 262144), (192, 1000), (320, 77), (1024, 1), (2560, 6912), (6912, 2560), (4096, 4100),
                                  (8192, 4096), (5120, 5120), (2048, 259)])
 def test_ternary_one_row_kernel_arbitrary_bytes(ops, K, N):
     """One activation row on up to 8 MB of packed weights takes the flat dot-product kernel (one 16-byte chunk per
