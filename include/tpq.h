@@ -303,8 +303,8 @@ int tpq_packed_linear_float(const void* x, int x_unsigned, double x_scale, int64
  * gemm_impl(xf, wf.t(), out, 1.0, 0.0, nullptr) at :1339; likewise behind _weight_int8pack_mm and the low-bit linear):
  *   out[m][n] = T(sum_k float(x[m][k]) * float(w[n][k])),  float32 accumulation, one rounding to `dtype`.
  * x: [M, K], w: [N, K] (the dense weight that tpq_int4_dequantize / tpq_int8pack_dequantize / tpq_lowbit_dequantize
- * wrote), out: [M, N], all contiguous and of `dtype` = float16 or bfloat16; x and w 16-byte aligned.
- * TPQ_ERR_UNSUPPORTED for float32 or K not a multiple of 64 (nothing written).
+ * wrote), out: [M, N], all contiguous and of `dtype` = float16, bfloat16 or float32; x and w 16-byte aligned.
+ * TPQ_ERR_UNSUPPORTED for other types or K not a multiple of 64 (float32: of 32); nothing written then.
  */
 int tpq_dense_mm(const void* x, int dtype, int64_t M, int64_t K, const void* w, int64_t N, void* out, void* stream);
 

@@ -109,6 +109,16 @@ struct ArithBF16 {  // 64 k per stage, v_mfma_f32_16x16x32_bf16
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8_t, b), __builtin_bit_cast(b8_t, a), c, 0, 0, 0);
     }
 };
+struct ArithF32 {  // 32 k per stage, four v_mfma_f32_16x16x4_f32 per fragment: float t of every lane's four is k = 4 c + t
+    using acc_t = v4f;
+    static __device__ __forceinline__ acc_t mfma(const v4i& b, const v4i& a, const acc_t& c) {
+        const v4f bf = __builtin_bit_cast(v4f, b), af = __builtin_bit_cast(v4f, a);
+        acc_t d = __builtin_amdgcn_mfma_f32_16x16x4f32(bf.x, af.x, c, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(bf.y, af.y, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(bf.z, af.z, d, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(bf.w, af.w, d, 0, 0, 0);
+    }
+};
 
 // A, W: row-major [M][K], [N][K] with K contiguous; row_bytes = K * sizeof(element).
 // MB: blocks of 16 rows per wavefront: 4 (tile of 256 rows, what the description above and the numbers are about) or 2

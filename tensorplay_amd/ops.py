@@ -295,14 +295,21 @@ INT4_PREFILL_ROWS_BF16_VERY_WIDE = 768
 INT4_PREFILL_ROWS_F32 = 4
 
 
+DENSE_F32_ROWS = 768
+
+
 def _dense_mm(x: torch.Tensor, dense: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """``out = x @ dense.T`` behind the dequantise-then-multiply routes (QuantGemmKernels.cu:1339).
 
-    float16 / bfloat16 with K a multiple of 64 run the library's tile kernel; float32 activations and other K go to
-    the framework's GEMM."""
+    K a multiple of 64 (float32: 32) runs the library's tile kernel; other K go to the framework's GEMM, and so do
+    float32 activations below DENSE_F32_ROWS rows: the tile kernel takes 128 stages of four float32 MFMAs per fragment for
+    K = 4096 whatever the row count (4096 -> 11008, us, library / framework: 8 rows 227 / 32, 512 rows 457 / 376, 2048 rows
+    1362 / 1404 = 136 TFLOP/s of the 157 the matrix cores have for float32)."""
     m, k = x.shape
     n = dense.size(0)
-    if x.dtype != torch.float32 and k % 64 == 0 and k < (1 << 22) and x.data_ptr() % 16 == 0:
+    per_stage = 32 if x.dtype == torch.float32 else 64
+    if (k % per_stage == 0 and k * (128 // per_stage) < (1 << 23) and x.data_ptr() % 16 == 0 and dense.data_ptr() % 16 == 0
+            and (x.dtype != torch.float32 or m >= DENSE_F32_ROWS)):
         with torch.cuda.device(x.device):
             _check(_lib.load().tpq_dense_mm(_ptr(x), _DT[x.dtype], m, k, _ptr(dense), n, _ptr(out), _stream(x)))
         return out

@@ -79,7 +79,8 @@ def test_dense_mm_refuses_what_it_does_not_build(ops):
     out = torch.full((4, 8), 3.0, dtype=torch.float16, device=DEV)
     s = torch.cuda.current_stream().cuda_stream
     assert lib.tpq_dense_mm(x.data_ptr(), ops._DT[torch.float16], 4, 96, w.data_ptr(), 8, out.data_ptr(), s) == _lib.TPQ_ERR_UNSUPPORTED
-    assert lib.tpq_dense_mm(x.data_ptr(), ops._DT[torch.float32], 4, 64, w.data_ptr(), 8, out.data_ptr(), s) == _lib.TPQ_ERR_UNSUPPORTED
+    assert lib.tpq_dense_mm(x.data_ptr(), ops._DT[torch.float32], 4, 48, w.data_ptr(), 8, out.data_ptr(), s) == _lib.TPQ_ERR_UNSUPPORTED   # float32: multiples of 32
+    assert lib.tpq_dense_mm(x.data_ptr(), 7, 4, 64, w.data_ptr(), 8, out.data_ptr(), s) == _lib.TPQ_ERR_UNSUPPORTED
     assert lib.tpq_dense_mm(x.data_ptr(), ops._DT[torch.float16], 0, 64, w.data_ptr(), 8, out.data_ptr(), s) == 0
     torch.cuda.synchronize()
     assert bool((out == 3.0).all())
@@ -88,3 +89,34 @@ def test_dense_mm_refuses_what_it_does_not_build(ops):
     wr = torch.randn((8, 96), dtype=torch.float16, device=DEV)
     got = ops._dense_mm(xr, wr, torch.empty((4, 8), dtype=torch.float16, device=DEV))
     torch.testing.assert_close(got.float(), xr.float() @ wr.float().t(), rtol=2e-3, atol=2e-2)
+
+
+@pytest.mark.parametrize("shape", [(1, 8, 32), (7, 5, 96), (129, 136, 320), (300, 200, 192), (257, 137, 448), (513, 264, 4096),
+                                   (2048, 1000, 1024), (384, 11008, 256), (40, 72, 11008)])
+def test_dense_mm_float32(shape):
+    """float32 operands (a stage is 32 elements of k, four v_mfma_f32_16x16x4_f32 per fragment): against the exact
+    product in float64, every output within the drift of a float32 sum of K terms; small integers exact."""
+    from tensorplay_amd import _lib
+    lib = _lib.load()
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7919 + N * 31 + K + 1)
+    for ints in (False, True):
+        if ints:
+            x = rng.integers(-8, 9, (M, K)).astype(np.float32)
+            w = rng.integers(-8, 9, (N, K)).astype(np.float32)
+        else:
+            x = rng.normal(0, 1, (M, K)).astype(np.float32)
+            w = rng.normal(0, 0.05, (N, K)).astype(np.float32)
+        xd, wd = torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV)
+        out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+        rc = lib.tpq_dense_mm(xd.data_ptr(), _lib.F32, M, K, wd.data_ptr(), N, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, _lib.last_error()
+        got = out.cpu().numpy().astype(np.float64)
+        want = x.astype(np.float64) @ w.astype(np.float64).T
+        assert not np.isnan(got).any(), "an output was not written"
+        if ints:
+            np.testing.assert_array_equal(got, want)
+        else:
+            mass = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T
+            bad = np.abs(got - want) > (K + 2) * 2.0 ** -24 * mass + 1e-30
+            assert not bad.any(), f"{bad.sum()} of {bad.size} outside the bound; worst {np.abs(got - want).max():.3e}"

@@ -285,6 +285,29 @@ def test_mm_many_rows_takes_the_dense_route(ops, dtype):
     assert rel_err(got, y64) < {"f16": 2e-3, "bf16": 1e-2, "f32": 1e-4}[dtype]
 
 
+def test_mm_float32_many_rows_on_the_library_gemm(ops):
+    """float32 activations from DENSE_F32_ROWS rows on: dequantise, then the library's tile kernel with float32 MFMAs
+    (no framework GEMM); against the reference's formulation and the exact sums."""
+    M, N, K, group = ops.DENSE_F32_ROWS + 5, 264, 1024, 128
+    rng = np.random.default_rng(78)
+    codes, sz = asym_quant(rng.normal(0, 0.02, (N, K)).astype(np.float32), group)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xb, szb = cast_bits(x, "f32"), cast_bits(sz, "f32")
+    packed = oracle.int4_pack_tc(codes, 2)
+    calls = []
+    real = torch.matmul
+    torch.matmul = lambda *a, **k: calls.append(1) or real(*a, **k)
+    try:
+        got = ops._weight_int4pack_mm(dev(xb, "f32"), dev(packed), group, dev(szb, "f32")).float().cpu().numpy()
+    finally:
+        torch.matmul = real
+    assert not calls, "the many-row float32 route went through torch.matmul"
+    ref_dev = oracle.to_f32(oracle.int4_mm_tc(xb, "f32", packed, szb, group, round_w=True), "f32")
+    assert_close_norm(got, ref_dev, 1e-4, "vs reference formulation")
+    _, y64 = oracle.int4_mm_tc(xb, "f32", packed, szb, group, round_w=False, want_f64=True)
+    assert rel_err(got, y64) < 1e-5
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_mm_prefill_block_matches_cpu_formulation(ops, dtype):
     """2048 rows of 4096 -> 11008, the prefill block of the model the decode numbers are quoted on: dequantise, then
