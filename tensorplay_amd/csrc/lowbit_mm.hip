@@ -476,10 +476,15 @@ int launch_mfma(const void* x, const uint8_t* packed, const float* sz, const flo
         const uint16_t* xs = static_cast<const uint16_t*>(x) + m0 * K;
         uint16_t* ys = static_cast<uint16_t*>(out) + m0 * N;
         const int n = static_cast<int>(N), k = static_cast<int>(K);
-        const bool few = rows <= kRowsPerLoad;  // one load of activations per step
+        const int loads = (rows + kRowsPerLoad - 1) / kRowsPerLoad;  // loads of activations per step: 1, 2 or kFull
         const size_t xch = static_cast<size_t>(waves) * 16 * lowbit_x_pitch<BITS, LSB>();
 #define TPQ_LB_MFMA(W, XLV, NBV) lowbit_mfma_kernel<DT, BITS, LSB, W, XLV, NBV><<<grid, W * kWave, xch, s>>>(xs, packed, sz, bias, ys, rows, n, k, group_shift)
-#define TPQ_LB_MFMA_X(W, NBV) do { if (few) TPQ_LB_MFMA(W, 1, NBV); else TPQ_LB_MFMA(W, kFull, NBV); } while (0)
+#define TPQ_LB_MFMA_X(W, NBV)                                              \
+    do {                                                                   \
+        if (loads <= 1) TPQ_LB_MFMA(W, 1, NBV);                            \
+        else if (loads <= 2) TPQ_LB_MFMA(W, 2, NBV);                       \
+        else TPQ_LB_MFMA(W, kFull, NBV);                                   \
+    } while (0)
         if (waves == 4) TPQ_LB_MFMA_X(4, 1);
         else if (nb == 3) TPQ_LB_MFMA_X(8, 3);
         else if (nb == 2) TPQ_LB_MFMA_X(8, 2);
