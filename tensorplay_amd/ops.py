@@ -290,6 +290,33 @@ INT4_PREFILL_ROWS = 256
 INT4_PREFILL_ROWS_VERY_WIDE = 1024  # N >= 16384
 INT4_PREFILL_ROWS_BF16 = 112
 INT4_PREFILL_ROWS_BF16_VERY_WIDE = 768
+# Between INT4_PREFILL_ROWS_BF16 and INT4_PREFILL_ROWS rows bfloat16 takes the tiled kernel where its estimate (1.4 times
+# float16's, which is int4_gemm_plan of int4_gemm_kernel.h restated below: with a workspace that kernel deals K to
+# slices when its tiles are few) is below the dense route's: 0.55 us per million weights for the dequantize pass and one
+# round of tiles of the dense kernel.  Measured (us, dense / tiled, 128 and 255 rows): 4096 x 4096 38.4 / 23.0 and
+# 41.6 / 33.9; 11008 -> 4096 89.8 / 42.8 and 92.5 / 71.1; 8192 x 8192 80.9 / 55.7 and 90.1 / 96.9; 4096 -> 11008
+# 51.9 / 50.7 and 57.9 / 68.4.
+def _int4_tiled_estimate_us(m: int, n: int, k: int) -> float:
+    tiles = ((n + 63) // 64) * ((m + 127) // 128)
+
+    def estimate(slices: int) -> float:
+        per_unit = tiles * slices / 256.0
+        rounds = 1.0 if per_unit <= 1.0 else 1.7 * int((per_unit + 1.999) / 2.0)
+        return rounds * (5.0 + 7.2 * k / 1024.0 / slices) + (0.0 if slices == 1 else 1.6 + slices * m * n * 8.0 / 4e6)
+
+    if m > 256 or k < 1024:
+        return estimate(1)
+    return min(estimate(s) for s in range(1, max(1, min(k // 128 // 4, 16)) + 1))
+
+
+def _int4_dense_estimate_us(m: int, n: int, k: int) -> float:
+    stages = k / 64.0
+    short_rounds = -(-(((m + 127) // 128) * ((n + 127) // 128)) // 256)
+    tall_rounds = -(-(((m + 255) // 256) * ((n + 127) // 128)) // 256)
+    gemm = short_rounds * (stages * 690 + 8000) if short_rounds * 0.8 < tall_rounds else tall_rounds * (stages * 1080 + 9000)
+    return 1.6 + 0.55e-6 * n * k + gemm / 2000.0
+
+
 # float32 activations have no matrix-core decode kernel: the per-row kernel costs about 16 us a row at K = 4096,
 # N = 11008 (71 us at 4 rows, 253 us at 16), the dense float32 route (the framework's GEMM) 95 us at 16 rows and 134 us at 64.
 INT4_PREFILL_ROWS_F32 = 4
@@ -359,6 +386,8 @@ def _weight_int4pack_mm(self: torch.Tensor, mat2: torch.Tensor, qGroupSize: int,
         prefill_rows = INT4_PREFILL_ROWS_F32
     elif self.dtype == torch.bfloat16:
         prefill_rows = INT4_PREFILL_ROWS_BF16_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS_BF16
+        if prefill_rows < m <= INT4_PREFILL_ROWS and k % 128 == 0 and 1.4 * _int4_tiled_estimate_us(m, n, k) < _int4_dense_estimate_us(m, n, k):
+            prefill_rows = INT4_PREFILL_ROWS
     else:
         prefill_rows = INT4_PREFILL_ROWS_VERY_WIDE if n >= 16384 else INT4_PREFILL_ROWS
     if m > prefill_rows and inner == 2:
