@@ -591,6 +591,27 @@ def main() -> int:
         del dense, gp
         del packs[1:], szs[1:]
         torch.cuda.empty_cache()
+        # 64 and 128 rows on the down-projection shape (11008 -> 4096: 64 workgroups of the tiled kernel per 128 rows): with
+        # a workspace the steps of K go to slices whose fp32 sums a second launch adds
+        K2, N2 = 11008, 4096
+        packs2 = [ops._convert_weight_to_int4pack(torch.randint(0, 16, (N2, K2), dtype=torch.int32, device=dev), 2) for _ in range(12)]
+        sz2 = (torch.rand(K2 // GROUP, N2, 2, device=dev) * 0.01).half()
+        for mb in (64, 128):
+            xb = torch.from_numpy(rng.normal(0, 1, (mb, K2)).astype(np.float32)).to(dev).half()
+            yb = torch.empty((mb, N2), dtype=torch.float16, device=dev)
+            ws2 = torch.zeros(lib.tpq_int4_mm_rows_workspace_bytes(mb, N2, K2), dtype=torch.uint8, device=dev)
+
+            def mm2(i, xb=xb, yb=yb, mb=mb, ws2=ws2):
+                lib.tpq_int4_mm_ws(xb.data_ptr(), _lib.F16, mb, K2, packs2[i % 12].data_ptr(), 2, N2, GROUP, sz2.data_ptr(),
+                                   yb.data_ptr(), ws2.data_ptr(), ws2.numel(), cur())
+
+            g2 = graph_of(lambda: [mm2(i) for i in range(48)])
+            g2.replay(); sync()
+            ms = steady(g2.replay, sync) / 48
+            extras[f"int4_mm_M{mb}_11008x4096_us"] = ms * 1e3
+            extras[f"int4_mm_M{mb}_11008x4096_TFLOPs"] = 2.0 * mb * N2 * K2 / (ms * 1e-3) / 1e12
+        del packs2, g2
+        torch.cuda.empty_cache()
         # int8 weight-only decode (next-row op _weight_int8pack_mm): same shape, one byte per weight
         w8s = [torch.randint(-128, 128, (N, K), dtype=torch.int8, device=dev) for _ in range(14)]  # 631 MB
         s8 = torch.rand(N, device=dev) * 0.01
