@@ -82,6 +82,8 @@ __global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(cons
 //   1024 x 1024   2.03 / 2.61      2048 x 2048   2.41 / 3.15      2048 -> 4096  2.70 / 3.33      4096 x 4096  3.61 / 3.98
 //   5120 x 5120   4.43 / 5.46      4096 -> 11008 6.19 / 6.27      5120 -> 13824 9.47 / 8.10      8192 x 8192  8.57 / 7.70
 // (two chunks per thread were tried for the larger ones: 4096 -> 11008 5.94, 5120 -> 13824 7.83, 8192 x 8192 8.02)
+// More rows on the same kernel (the expanded fields shared, one v_dot4 and the LDS reads of the activations per row) cost
+// 1.4 us per row: 2560 -> 6912 at 2 / 3 / 4 rows 5.0 / 6.4 / 7.6 us against 4.2 / 4.3 / 4.3 on the matrix-core kernel.
 inline int ternary_row_rows_per_workgroup(int64_t M, int64_t N, int64_t K, int compute_units = 256) {
     if (M != 1 || K < 64 || K % 64 != 0 || K > kTernaryRowMaxK || N < 1 || N > 0x7FFFFFF0 || N * K > (int64_t{1} << 25)) return 0;
     const int64_t cpr = K / 64, most = kTernaryRowMaxThreads / cpr;
