@@ -68,7 +68,21 @@ __global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(cons
         for (int f = 0; f < 4; ++f)
             acc = __builtin_amdgcn_sdot4(static_cast<int>(fields[f]), static_cast<int>((words[d] << (2 * f)) & 0xC0C0C0C0u), acc, false);
     }
-    if (live) __hip_atomic_fetch_add(&sums[row], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    // Up to 128 lanes add to one channel's word, and LDS serves the lanes of one address one after the other: where four
+    // (eight) neighbouring chunks always belong to one channel, their lanes add up first and one of them goes to LDS.
+    if (!live) acc = 0;
+    if ((cpr & 3) == 0) {
+        acc += __builtin_amdgcn_mov_dpp(acc, 0xB1, 0xF, 0xF, true);  // quad_perm [1, 0, 3, 2]
+        acc += __builtin_amdgcn_mov_dpp(acc, 0x4E, 0xF, 0xF, true);  // quad_perm [2, 3, 0, 1]
+        if ((cpr & 7) == 0) {
+            acc += __builtin_amdgcn_mov_dpp(acc, 0x141, 0xF, 0xF, true);  // row_half_mirror: the other quad of the eight
+            if (live && (t & 7) == 0) __hip_atomic_fetch_add(&sums[row], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else if (live && (t & 3) == 0) {
+            __hip_atomic_fetch_add(&sums[row], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    } else if (live) {
+        __hip_atomic_fetch_add(&sums[row], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (t < rows_here) ep.store_scaled(n, sums[t] >> 6, row_scale, with_bias ? bias_raw : 0.0f);
 }
