@@ -7,7 +7,7 @@
 // weight is ever materialised (the reference unpacks to int8 on every call,
 // tensorplay/ao/quantization/bitnet.py:233).
 //
-// One row, K % 64 == 0, up to 8 MB of packed weights: the flat dot-product kernel of ternary_row_kernel.h.
+// One row, K % 64 == 0, K <= 8192: the flat dot-product kernel of ternary_row_kernel.h.
 // Up to 32 rows with K % 256 == 0: the matrix-core decode kernel of ternary_decode_mfma.h.
 //
 // Dot-product decode kernel (M <= 8, other K % 64 == 0): one wavefront per 4 weight rows, lane l owns the
@@ -136,7 +136,7 @@ int launch_ternary(const int8_t* x, const uint8_t* packed, int64_t M, int64_t N,
     // 5.2..29.6 us (the tile kernel 9.3..75 us for any row count up to 128; two slabs stay below it, three do not).
     static const int mfma_min = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_MIN"); return e ? std::atoi(e) : 1; }();
     static const int mfma_rows = [] { const char* e = tuning_env("TPQ_TERNARY_MFMA_ROWS"); return e ? std::atoi(e) : 32; }();
-    // One row over up to 8 MB of packed weights: the flat dot-product kernel (every wave-level load 1 KB of whole lines)
+    // One row, K up to 8192: the flat dot-product kernel (every wave-level load 1 KB of whole lines)
     if (forced_decode_rows < 0 && M == 1 && aligned(x, 16) && aligned(packed, 16) && !tuning_env("TPQ_TERNARY_NO_ROW")) {
         if (const int rows_wg = ternary_row_rows_per_workgroup(M, N, K)) return launch_ternary_row(x, packed, N, K, rows_wg, ep, s);
     }

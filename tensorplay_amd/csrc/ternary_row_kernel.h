@@ -87,25 +87,25 @@ __global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(cons
     if (t < rows_here) ep.store_scaled(n, sums[t] >> 6, row_scale, with_bias ? bias_raw : 0.0f);
 }
 
-// rows per workgroup (0: the kernel does not take the shape).  Whole rounds of workgroups over the compute units
-// where the channel count allows, at most 16 wavefronts and at least the K / 16 threads that park the activations.
-// One chunk per thread means one round of wavefronts up to 8 MB of packed weights (8192 wavefronts fit the chip at
-// once); beyond that the rounds queue and the matrix-core kernel, whose wavefronts loop, is ahead again.  Measured,
-// weights streamed from HBM (us, this kernel / ternary_decode_mfma.h):
-//   2560 -> 6912  3.50 / 4.33 (cache-resident 3.17 / 3.79)      6912 -> 2560  3.87 / 4.92 (3.42 / 4.22)
-//   1024 x 1024   2.03 / 2.61      2048 x 2048   2.41 / 3.15      2048 -> 4096  2.70 / 3.33      4096 x 4096  3.61 / 3.98
-//   5120 x 5120   4.43 / 5.46      4096 -> 11008 6.19 / 6.27      5120 -> 13824 9.47 / 8.10      8192 x 8192  8.57 / 7.70
-// (two chunks per thread were tried for the larger ones: 4096 -> 11008 5.94, 5120 -> 13824 7.83, 8192 x 8192 8.02)
-// More rows on the same kernel (the expanded fields shared, one v_dot4 and the LDS reads of the activations per row) cost
-// 1.4 us per row: 2560 -> 6912 at 2 / 3 / 4 rows 5.0 / 6.4 / 7.6 us against 4.2 / 4.3 / 4.3 on the matrix-core kernel.
+// rows per workgroup (0: the kernel does not take the shape).  Up to 8 MB of packed weights the wavefronts all fit the
+// chip at once (8192 of them): whole rounds of workgroups over the compute units where the channel count allows, at
+// most 16 wavefronts and at least the K / 16 threads that park the activations.  Larger weights: four rows, the
+// smallest workgroups, so that the rounds of wavefronts follow each other closely.  Measured, weights streamed from HBM
+// (us, this kernel / ternary_decode_mfma.h):
+//   2560 -> 6912  3.13 / 4.33 (cache-resident 2.60 / 3.79)      6912 -> 2560  3.29 / 4.92 (2.81 / 4.22)
+//   2048 x 2048   2.35 / 3.03      4096 x 4096   3.05 / 3.81      5120 x 5120   3.63 / 4.80      4096 -> 11008  4.41 / 5.80
+//   5120 -> 13824 6.10 / 7.27      8192 x 8192   5.80 / 7.79      8192 -> 16384 9.25 / 10.24     8192 -> 28672  14.6 / 15.9
+//   4096 -> 32000 8.55 / 10.4
+// (with every lane adding to the channel's LDS word by itself the kernel lost beyond 8 MB: 8192 x 8192 8.57)
 inline int ternary_row_rows_per_workgroup(int64_t M, int64_t N, int64_t K, int compute_units = 256) {
-    if (M != 1 || K < 64 || K % 64 != 0 || K > kTernaryRowMaxK || N < 1 || N > 0x7FFFFFF0 || N * K > (int64_t{1} << 25)) return 0;
+    if (M != 1 || K < 64 || K % 64 != 0 || K > kTernaryRowMaxK || N < 1 || N > 0x7FFFFFF0) return 0;
     const int64_t cpr = K / 64, most = kTernaryRowMaxThreads / cpr;
     if (most < 4) return 0;
     if (const char* e = tuning_env("TPQ_TERNARY_ROW_WG")) {
         const int64_t rows = std::atoll(e);
         return rows >= 4 && rows <= most ? static_cast<int>(rows) : 0;
     }
+    if (N * K > (int64_t{1} << 25)) return 4;
     for (int64_t rounds = 1; rounds <= 64; ++rounds) {
         const int64_t rows = (N + compute_units * rounds - 1) / (compute_units * rounds);
         if (rows <= most) return static_cast<int>(rows < 4 ? 4 : rows);

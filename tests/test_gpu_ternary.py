@@ -129,7 +129,7 @@ def test_ternary_slab_arbitrary_bytes(ops, M, K, N):
 
 
 @pytest.mark.parametrize("K,N", [(64, 3), (64, 5), (64, 70001), (128, 262144), (192, 1000), (320, 77), (1024, 1), (2560, 6912), (6912, 2560), (4096, 4100),
-                                 (8192, 4096), (5120, 5120), (2048, 259)])
+                                 (8192, 4096), (5120, 5120), (2048, 259), (8192, 28672), (4096, 32000)])
 def test_ternary_one_row_kernel_arbitrary_bytes(ops, K, N):
     """One activation row on up to 8 MB of packed weights takes the flat dot-product kernel (one 16-byte chunk per
     thread, the channel sums added up in LDS): any byte value in the packed weight (0b10 decodes to -2), activations
