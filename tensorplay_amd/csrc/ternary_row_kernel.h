@@ -26,13 +26,17 @@ namespace {
 
 constexpr int kTernaryRowMaxK = 8192;
 constexpr int kTernaryRowMaxThreads = 1024;
+__host__ __device__ constexpr int ternary_row_x_slots(int K) { return (K >> 4) + (K >> 8) + 1; }  // 16-byte slots of the parked activations
 
-// grid: ceil(N / rows_wg); block: 64 * ceil(rows_wg * K / 64 / 64) threads >= K / 16; LDS: K + 4 * rows_wg bytes
+// grid: ceil(N / rows_wg); block: 64 * ceil(rows_wg * K / 64 / 64) threads >= K / 16; LDS: 16 ternary_row_x_slots(K) + 4 rows_wg bytes
 template <class Epilogue>
 __global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(const int8_t* __restrict__ x, const uint8_t* __restrict__ packed, int N,
                                                                            int K, int rows_wg, float inv_chunks_per_row, Epilogue ep) {
-    extern __shared__ uint4 x_fields[];  // [K / 16], slot 4 c + ((d + c) & 3) holds the transposed piece d of chunk c
-    int* const sums = reinterpret_cast<int*>(x_fields + (K >> 4));
+    // [K / 16 + K / 256]: slot 4 c + d + c / 4 holds the transposed piece d of chunk c (one slot of padding per four
+    // chunks: the sixteen lanes a 16-byte read serves together, chunks c .. c + 15, then hit sixteen different groups of
+    // four banks; without it chunks four apart met in the same banks and most of the kernel's LDS cycles were conflicts)
+    extern __shared__ uint4 x_fields[];
+    int* const sums = reinterpret_cast<int*>(x_fields + ternary_row_x_slots(K));
     const int t = threadIdx.x;
     const int cpr = K >> 6;  // 16-byte chunks in a packed row
     const int row0 = blockIdx.x * rows_wg;
@@ -52,7 +56,7 @@ __global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(cons
     if (t < pieces) {
         const v4i f = transpose_4x4_bytes(xr);
         const int c = t >> 2, d = t & 3;
-        x_fields[4 * c + ((d + c) & 3)] = make_uint4(static_cast<uint32_t>(f[0]), static_cast<uint32_t>(f[1]), static_cast<uint32_t>(f[2]), static_cast<uint32_t>(f[3]));
+        x_fields[4 * c + d + (c >> 2)] = make_uint4(static_cast<uint32_t>(f[0]), static_cast<uint32_t>(f[1]), static_cast<uint32_t>(f[2]), static_cast<uint32_t>(f[3]));
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weights stay in flight
 
@@ -62,7 +66,7 @@ __global__ __launch_bounds__(kTernaryRowMaxThreads) void ternary_row_kernel(cons
     int acc = 0;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-        const uint4 xf = x_fields[4 * c + ((d + c) & 3)];
+        const uint4 xf = x_fields[4 * c + d + (c >> 2)];
         const uint32_t fields[4] = {xf.x, xf.y, xf.z, xf.w};
 #pragma unroll
         for (int f = 0; f < 4; ++f)
@@ -118,7 +122,7 @@ int launch_ternary_row(const int8_t* x, const uint8_t* packed, int64_t N, int64_
     const int64_t cpr = K / 64, threads = (rows_wg * cpr + 63) / 64 * 64;
     TPQ_REQUIRE(K % 64 == 0 && K <= kTernaryRowMaxK && rows_wg >= 4 && threads <= kTernaryRowMaxThreads && threads >= K / 16 && threads >= rows_wg,
                 TPQ_ERR_INVALID_VALUE, "ternary row kernel: workgroup shape");
-    const size_t smem = static_cast<size_t>(K) + 4 * static_cast<size_t>(rows_wg);
+    const size_t smem = 16 * static_cast<size_t>(ternary_row_x_slots(static_cast<int>(K))) + 4 * static_cast<size_t>(rows_wg);
     ternary_row_kernel<Epilogue><<<static_cast<unsigned>((N + rows_wg - 1) / rows_wg), static_cast<unsigned>(threads), smem, s>>>(
         x, packed, static_cast<int>(N), static_cast<int>(K), rows_wg, 1.0f / static_cast<float>(cpr), ep);
     return check_launch("tpq_ternary_mm (one row)");
