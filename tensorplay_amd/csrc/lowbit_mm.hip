@@ -651,18 +651,26 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
                     p[c][t].y += 128.0f;
                 }
             }
-        // Codes become 16-bit floats in place.  A field of BITS bits moved to the top of the mantissa of each half
-        // of the word (one shift), masked and given the exponent whose lowest field bit weighs one (one v_and_or_b32)
-        // is the pair (2^BITS + code, 2^BITS + code') of the two halves' codes at that position; one v_dot2 multiplies
-        // it with the matching pair of activations, and the constant is removed with the segment's sum of activations,
-        // which the zero point needs anyway:  y += scale (dot - (2^BITS + zero) sum x).
+        // Codes become 16-bit floats in place.  A field that lies at bit p of the mantissa of its 16-bit half, masked and
+        // given the exponent under which bit p weighs one (one v_and_or_b32), is the pair (2^(kMant - p) + code,
+        // 2^(kMant - p) + code') of the two halves' codes at that position; one v_dot2 multiplies it with the matching
+        // pair of activations.  The kMant / BITS field positions inside the mantissa need no shift; one shift of the
+        // word brings the next positions there.  The constants leave with the same pairs of activations multiplied by
+        // the bare exponents, once per lane for all its channels:  y += scale ((dot - offsets) - zero sum x).
+        // (One exponent for every position, each field shifted to the top of the mantissa first, was three
+        // instructions per pair of codes instead of two and a shift per group of positions: 4096 -> 11008 at 1 / 2 bits
+        // 6.6 / 6.8 -> 6.2 / 6.5 us, 8192 x 8192 8.0 / 8.5 -> 7.5 / 7.9, 8192 -> 28672 18.1 / 22.6 -> 16.3 / 20.2; 4 and 8 bits,
+        // where a shift serves two positions or one, are unchanged.)
         using L = Lane16<DT>;
         constexpr int kMant = DT == TPQ_DTYPE_F16 ? 10 : 7, kExpBias = DT == TPQ_DTYPE_F16 ? 15 : 127;
-        constexpr uint32_t kMagic = (static_cast<uint32_t>(kExpBias + BITS) << kMant) * 0x00010001u;
-        constexpr uint32_t kFieldMask = (((1u << BITS) - 1u) << (kMant - BITS)) * 0x00010001u;
         constexpr int kFieldsPerHalf = 16 / BITS;
-        uint32_t magic;  // kept in a VGPR behind an opaque move: v_and_or_b32 takes one literal only
-        asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(kMagic));
+        constexpr int kSpan = kMant / BITS < kFieldsPerHalf ? kMant / BITS : kFieldsPerHalf;  // positions served by one shift
+        static_assert(kSpan >= 1, "a field fits the mantissa");
+        constexpr int kShiftGroups = (kFieldsPerHalf + kSpan - 1) / kSpan;
+        uint32_t magic[kSpan];  // kept in VGPRs behind an opaque move: v_and_or_b32 takes one literal only
+#pragma unroll
+        for (int i = 0; i < kSpan; ++i)
+            asm volatile("v_mov_b32 %0, %1" : "=v"(magic[i]) : "s"((static_cast<uint32_t>(kExpBias + kMant - i * BITS) << kMant) * 0x00010001u));
 #pragma unroll
         for (int t = 0; t < kTurns; ++t) {
             // activations: the natural pairs (k, k + 1) for the sum, and for every (word, position) the pair that
@@ -672,7 +680,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
                 const uint32_t pair = ((e >> 1) & 3) == 0 ? xq.x : ((e >> 1) & 3) == 1 ? xq.y : ((e >> 1) & 3) == 2 ? xq.z : xq.w;
                 return (e & 1) ? pair >> 16 : pair & 0xFFFFu;
             };
-            float sx = 0.0f;
+            float sx = 0.0f, off = 0.0f;
 #pragma unroll
             for (int e = 0; e < kCpl; e += 2) sx = L::dot(half_of(e) | (half_of(e + 1) << 16), L::kOnes, sx);
             float s[kLbRowChannels];
@@ -681,22 +689,26 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_
 #pragma unroll
             for (int w = 0; w < kWords; ++w)
 #pragma unroll
-                for (int fp = 0; fp < kFieldsPerHalf; ++fp) {  // field position inside a 16-bit half, from its low end
-                    const int byte = 4 * w + fp / kPerByte, pos = fp % kPerByte;
-                    const int e = byte * kPerByte + (LSB ? pos : kPerByte - 1 - pos);
-                    const uint32_t xpair = half_of(e) | (half_of(e + 2 * kPerByte) << 16);
-                    constexpr int kTop = kMant - BITS;
-                    const int shift = kTop - fp * BITS;  // to the top of the mantissa
+                for (int sg = 0; sg < kShiftGroups; ++sg) {
+                    uint32_t moved[kLbRowChannels];
 #pragma unroll
-                    for (int c = 0; c < kLbRowChannels; ++c) {
-                        const uint32_t word = wv[c][t][w];
-                        const uint32_t moved = shift >= 0 ? word << shift : word >> -shift;
-                        s[c] = L::dot(xpair, (moved & kFieldMask) | magic, s[c]);
+                    for (int c = 0; c < kLbRowChannels; ++c) moved[c] = sg == 0 ? wv[c][t][w] : wv[c][t][w] >> (sg * kSpan * BITS);
+#pragma unroll
+                    for (int i = 0; i < kSpan; ++i) {
+                        const int fp = sg * kSpan + i;  // field position inside a 16-bit half, from its low end
+                        if (fp >= kFieldsPerHalf) continue;
+                        const int byte = 4 * w + fp / kPerByte, pos = fp % kPerByte;
+                        const int e = byte * kPerByte + (LSB ? pos : kPerByte - 1 - pos);
+                        const uint32_t xpair = half_of(e) | (half_of(e + 2 * kPerByte) << 16);
+                        const uint32_t mask = (((1u << BITS) - 1u) << (i * BITS)) * 0x00010001u;
+                        off = L::dot(xpair, magic[i], off);
+#pragma unroll
+                        for (int c = 0; c < kLbRowChannels; ++c) s[c] = L::dot(xpair, (moved[c] & mask) | magic[i], s[c]);
                     }
                 }
 #pragma unroll
             for (int c = 0; c < kLbRowChannels; ++c)
-                acc[c] = __builtin_fmaf(p[c][t].x, s[c] - (static_cast<float>(1 << BITS) + p[c][t].y) * sx, acc[c]);
+                acc[c] = __builtin_fmaf(p[c][t].x, (s[c] - off) - p[c][t].y * sx, acc[c]);
         }
 #pragma unroll
         for (int c = 0; c < kLbRowChannels; ++c) acc[c] = wave_sum(acc[c]);
