@@ -9,7 +9,7 @@
 // dequantizes to a dense float weight and calls a float GEMM (_intx_mm, intx_weight_only.py:127-133).
 //
 // Decode kernel (fp16 / bf16 activations, 1..16 rows): v_mfma_f32_16x16x32 with the weights as A (fp16 below;
-// bf16 converts each code to float and keeps the upper half).  Lane
+// bf16 the same with seven mantissa bits, see Fields).  Lane
 // (i, q) owns weight row n0 + i and, per step, 32 consecutive codes of it (16 when a code has a byte
 // to itself): 4 to 16 bytes, one load.  A code becomes an fp16 number without leaving its bits: the
 // byte is copied into both halves of a dword (v_perm_b32), a mask keeps one field per half and an
@@ -56,6 +56,17 @@ struct Fields {
     static constexpr uint32_t mask(int t) { return (kField << pos_lo(t)) | (kField << (pos_hi(t) + 16)); }
     static constexpr uint32_t magic(int t) { return base_bits(pos_lo(t)) | (base_bits(pos_hi(t)) << 16); }
     static constexpr int kMagics = kPerByte >= 2 ? kPerByte / 2 : 1;  // magic(t) repeats with this period
+    // bfloat16 (BITS < 8): seven mantissa bits, so the top field of a byte reaches into the exponent.  It is taken from
+    // the word shifted right by one (its byte then holds the field one bit lower; the bit that comes in from the next
+    // byte is masked away): v_perm_b32 picks each half's byte from the word or from the shifted word.
+    static constexpr bool top(int p) { return p + BITS > 7; }
+    static constexpr int pos_bf(int p) { return top(p) ? p - 1 : p; }
+    static constexpr uint32_t base_bits_bf(int p) { return static_cast<uint32_t>(127 + 7 - p) << 7; }  // bf16 bits of 2^(7 - p)
+    static constexpr uint32_t select_bf(int t) {
+        return 0x0C000C00u | ((byte_lo(t) & 3) + (top(pos_lo(t)) ? 4 : 0)) | (((byte_hi(t) & 3) + (top(pos_hi(t)) ? 4 : 0)) << 16);
+    }
+    static constexpr uint32_t mask_bf(int t) { return (kField << pos_bf(pos_lo(t))) | (kField << (pos_bf(pos_hi(t)) + 16)); }
+    static constexpr uint32_t magic_bf(int t) { return base_bits_bf(pos_bf(pos_lo(t))) | (base_bits_bf(pos_bf(pos_hi(t))) << 16); }
 };
 
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
@@ -68,9 +79,10 @@ constexpr uint32_t kSignFlip = 0x80808080u;
 
 // x: [M][K] fp16 or bf16; packed: [N][K / per_byte]; sz: [K / group][N][2] fp32; steps = K / kStepK; a group
 // is kStepK << group_shift k.  N % 4 == 0.
-// bf16 has seven mantissa bits, too few for the exponent trick: there a code is cut out of its dword,
-// converted to float (exact) and the upper halves of two floats are packed; no offsets to take out, the
-// constant-A MFMA only sums x.
+// bf16 has seven mantissa bits: the same exponent trick with the top field of every byte taken from the word shifted
+// right by one bit (Fields::select_bf); only at 8 bits, where a byte does not fit, a code is cut out of its dword,
+// converted to float (exact) and the upper halves of two floats are packed, with no offsets to take out (the
+// constant-A MFMA then only sums x).
 //
 // The activations of a step are kStepK * 2 bytes of every row.  Asked for in the MFMA's order (lane (m, q): its 16-byte
 // pieces of row m) every load touches two or three lines of every row, and the vector memory path charges a load by the
@@ -88,6 +100,8 @@ constexpr int lowbit_x_pitch() { return Fields<BITS, LSB>::kStepK * 2 + 16; }
 // through its compute unit, so with one block the activations outweigh a narrow packed weight many times over.
 // 4096 -> 11008 with three blocks against one (us, 1 / 2 / 4 bits): 2 rows 9.2 / 9.0 / 10.4 -> 8.2 / 8.6 / 9.3, 8 rows
 // 12.3 / 11.0 / 11.5 -> 9.9 / 10.5 / 11.1, 16 rows 12.8 / 12.4 / 13.4 -> 10.5 / 10.9 / 11.6.
+// bfloat16 with the fields expanded in place instead of converted one by one (2 / 8 rows, us): 1 bit 9.7 / 10.3 -> 8.4 / 9.1,
+// 2 bits 10.0 / 10.7 -> 9.3 / 10.0, 4 bits 10.5 / 10.9 -> 9.5 / 10.5.
 template <int DT, int BITS, bool LSB, int WAVES, int XL, int NB>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed, const float* __restrict__ sz,
@@ -97,6 +111,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     constexpr int kRowsPerLoad = kWave / kPiecesPerRow;    // 4 or 8
     constexpr int kPitch = lowbit_x_pitch<BITS, LSB>();
     static_assert(XL * kRowsPerLoad <= 16, "at most 16 rows per launch");
+    constexpr bool kFieldsInPlace = DT == TPQ_DTYPE_F16 || BITS < 8;  // codes become 16-bit floats without leaving their bits
     __shared__ float red[WAVES][NB * 4][kWave];
     extern __shared__ __align__(16) unsigned char lowbit_xch[];  // [WAVES][16 rows][kPitch]
     const int lane = threadIdx.x & (kWave - 1);
@@ -132,11 +147,11 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
         if constexpr (DT == TPQ_DTYPE_F16) a_corr[h] = i == 0 ? F::magic(h) : i == 1 ? 0x3C003C00u : 0u;
-        else a_corr[h] = i == 1 ? 0x3F803F80u : 0u;
+        else a_corr[h] = (i == 0 && kFieldsInPlace) ? F::magic_bf(h) : i == 1 ? 0x3F803F80u : 0u;
     }
     uint32_t magic[F::kMagics];  // kept in VGPRs behind opaque moves: v_and_or_b32 takes one scalar operand
 #pragma unroll
-    for (int t = 0; t < F::kMagics; ++t) asm volatile("v_mov_b32 %0, %1" : "=v"(magic[t]) : "s"(F::magic(t)));
+    for (int t = 0; t < F::kMagics; ++t) asm volatile("v_mov_b32 %0, %1" : "=v"(magic[t]) : "s"(DT == TPQ_DTYPE_F16 ? F::magic(t) : F::magic_bf(t)));
 
     struct Step {
         uint4 w[NB];     // kBytes of each are used
@@ -191,6 +206,9 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
                     if constexpr (DT == TPQ_DTYPE_F16) {
                         const uint32_t both = __builtin_amdgcn_perm(0u, word, F::select(t));
                         a[h] = (both & F::mask(t)) | magic[t % F::kMagics];
+                    } else if constexpr (kFieldsInPlace) {
+                        const uint32_t both = __builtin_amdgcn_perm(word >> 1, word, F::select_bf(t));
+                        a[h] = (both & F::mask_bf(t)) | magic[t % F::kMagics];
                     } else {
                         const float lo = static_cast<float>((word >> (8 * (F::byte_lo(t) & 3) + F::pos_lo(t))) & F::kField);
                         const float hi = static_cast<float>((word >> (8 * (F::byte_hi(t) & 3) + F::pos_hi(t))) & F::kField);
@@ -201,6 +219,11 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
                 if constexpr (DT == TPQ_DTYPE_F16) d[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), __builtin_bit_cast(half8_t, bv), d[b], 0, 0, 0);
                 else d[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), d[b], 0, 0, 0);
             }
+            // Without this the compiler expands the codes of all MFMAs of a step ahead of the first one; bfloat16 then
+            // runs out of registers at three blocks of channels (scratch traffic).  fp16 stays within them, and the
+            // fence helps it only with two activation loads per step (4096 -> 11008 at 8 rows, 1 / 2 / 4 bits:
+            // 9.6 / 9.9 / 10.6 -> 9.0 / 9.7 / 10.2 us; at 2 and 4 rows it costs 0.2 - 0.4).
+            if constexpr (kFieldsInPlace && (DT != TPQ_DTYPE_F16 || XL == 2)) __builtin_amdgcn_sched_barrier(0);
         }
         // rows 0 and 1 of the offset product sit in lanes 0..15, registers 0 and 1
         const float corr = __shfl(aux[0], i, kWave), sx = __shfl(aux[1], i, kWave);
