@@ -555,6 +555,8 @@ int launch_generic(const void* x, const uint8_t* packed, const float* sz, const 
 // 8 bits: 6.4 / 6.7 / 7.8 / 11.5 -> 6.9 / 7.6 / 8.5 / 12.6 us): at these sizes every wavefront's loads arrive together and
 // the 450 vector instructions of the three wavefronts a SIMD holds run one after the other behind the arrival, so the
 // kernel is bound by that arithmetic and anything that sits between arrival and arithmetic adds to it.
+// Fetching the pairs of two neighbouring channels with one 16-byte load (half the load instructions, the same lines)
+// changed nothing either.
 template <int DT, int BITS, bool LSB, int WAVES, int CH>
 __global__ __launch_bounds__(WAVES * kWave) void lowbit_row_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ packed,
                                                                   const float* __restrict__ sz, const float* __restrict__ bias,
