@@ -240,7 +240,8 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
 
     // this wavefront's steps: wave, wave + WAVES, ...; two in flight (three or four, as many as 180 registers hold,
     // so that K = 4096 would be one trip to memory per wavefront, were measured and lost at every width and row count:
-    // 4096 -> 11008, 1 bit, 2 / 8 / 16 rows 8.2 / 9.6 / 10.5 -> 9.4 / 10.2 / 12.7 us)
+    // 4096 -> 11008, 1 bit, 2 / 8 / 16 rows 8.2 / 9.6 / 10.5 -> 9.4 / 10.2 / 12.7 us; at 8 bits, where a step is 64 k, four in
+    // flight leave registers for two blocks of channels only, a second round of workgroups: 8 rows 16.0 -> 22.7 us)
     Step s0 = {}, s1 = {};
     int s = wave;
     if (s < steps) load(s, s0);
