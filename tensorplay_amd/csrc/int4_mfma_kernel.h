@@ -153,7 +153,8 @@ __device__ __forceinline__ void int4_mfma_body(
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             st.w[b] = nt_load(w_base[b] + static_cast<size_t>(s) * 32);             // four k-tiles further per step
-            if constexpr (DEQ) st.p[b].x = sz_base[b][static_cast<size_t>((4 * s + q) / GKT) * N];  // group of k-tile 4 s + q
+            // (the whole vector is assigned: writing one member left the steps in scratch memory)
+            if constexpr (DEQ) st.p[b] = make_uint4(sz_base[b][static_cast<size_t>((4 * s + q) / GKT) * N], 0u, 0u, 0u);  // group of k-tile 4 s + q
             else st.p[b] = *reinterpret_cast<const uint4*>(sz_base[b] + static_cast<size_t>(s >> group_shift) * N);
         }
 #pragma unroll
