@@ -278,7 +278,8 @@ __device__ __forceinline__ void int4_mfma_body(
         }
     };
 
-    // this wavefront's steps: wave, wave + WAVES, ...; two in flight
+    // this wavefront's steps: wave, wave + WAVES, ...; two in flight (waiting for the prologue's loads in front of the loop,
+    // which makes the waits inside it exact, changed nothing here: 4096 x 4096, groups of 64, 8 rows 5.5 -> 5.7 us)
     Step s0 = {}, s1 = {};
     int s = wave;
     if (s < steps) load(s, s0);

@@ -246,6 +246,7 @@ __global__ __launch_bounds__(WAVES * kWave) void lowbit_mfma_kernel(
     int s = wave;
     if (s < steps) load(s, s0);
     if (s + WAVES < steps) load(s + WAVES, s1);
+    drain_vector_loads();  // exact waits inside the loop (4096 -> 11008 at 8 rows, 1 / 2 / 4 bits: 9.0 / 9.7 / 10.2 -> 8.5 / 9.3 / 9.8 us)
     for (; s + 3 * WAVES < steps; s += 2 * WAVES) {  // steady state: no branches in the body
         compute(s0);
         load(s + 2 * WAVES, s0);
