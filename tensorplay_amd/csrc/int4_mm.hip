@@ -648,14 +648,14 @@ bool launch_row(const void* x, const int32_t* packed, const void* sz, void* y, i
     const char* force = tuning_env("TPQ_INT4_KERNEL");  // "row" pins it, any other value excludes it (sweeps)
     const int pinned = route_override_int4_row();
     if ((force && force[0] != 'r') || pinned == 0) return false;
-    if (K % 256 != 0 || K > 12288 || N % 8 != 0) return false;  // three 1 KB blocks per wavefront and tile at most (registers)
+    if (K % 256 != 0 || K > 16384 || N % 8 != 0) return false;  // four 1 KB blocks per wavefront and tile at most (registers)
     int cus = compute_units() / 32 * 32;
     if (cus < 32) cus = 32;
     const int n_tiles = N / 8;
     const int blocks = K / 256;
     const int seg = (blocks + kRowWaves - 1) / kRowWaves;
     const int waves = (blocks + seg - 1) / seg;  // <= 16; the last one may own a segment past K (zero activations)
-    const int rounds = seg == 1 ? 6 : seg == 2 ? 3 : 2;
+    const int rounds = seg == 1 ? 6 : seg == 2 ? 3 : seg == 3 ? 2 : 1;
     // Where it wins (measured, one row, fp16, us: this kernel / matrix-core kernel / column-per-lane kernel):
     // 11008 -> 4096: 7.0 / 8.7 / 12.1;  5120 x 5120: 5.9 / 6.8 / 7.1.  Not for K <= 4096 (4096 -> 11008: 7.2 / 8.1 / 6.8;
     // 4096 x 4096: 6.0 / 4.7 / 5.8), not when the tiles need a second batch of rounds (4096 -> 14336: 10.1 / 8.6 / 7.7;
@@ -670,7 +670,10 @@ bool launch_row(const void* x, const int32_t* packed, const void* sz, void* y, i
     const int column_groups = (N + kWave - 1) / kWave, last_round = column_groups % compute_units();
     const bool short_last_round = column_groups > compute_units() && last_round > 0 && last_round * 10 <= compute_units() * 6;
     const bool wide = K > 4096 && (short_last_round || (K >= 7680 && K < 10240 && N >= 10240) || (K >= 12288 && N >= 8192));
-    const bool wins = K > 4096 && ((n_tiles >= 2 * cus && n_tiles <= rounds * cus) || wide);
+    // 12288 < K <= 16384 (four blocks per wavefront, one round in flight): ahead of the looped column-per-lane kernel or
+    // level with it (us, this kernel / default): 13824 -> 5120 12.1 / 14.5, 16384 -> 4096 9.9 / 14.4, 14336 -> 4096 9.3 / 9.5,
+    // 16384 -> 8192 17.0 / 16.7.
+    const bool wins = K > 4096 && ((n_tiles >= 2 * cus && n_tiles <= rounds * cus) || wide || seg == 4);
     if (!(force || pinned == 1) && !wins) return false;
     const int shift = group == 32 ? 0 : group == 64 ? 1 : group == 128 ? 2 : 3;
     const dim3 grid(cus), block(waves * kWave);
@@ -681,7 +684,8 @@ bool launch_row(const void* x, const int32_t* packed, const void* sz, void* y, i
     switch (seg) {
         case 1: int4_row_kernel<DT, 1, 1, 6><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
         case 2: int4_row_kernel<DT, 1, 2, 3><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
-        default: int4_row_kernel<DT, 1, 3, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
+        case 3: int4_row_kernel<DT, 1, 3, 2><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;
+        default: int4_row_kernel<DT, 1, 4, 1><<<grid, block, 0, s>>>(xp, pp, sp, yp, N, K, n_tiles, shift); break;  // (two rounds do not fit the registers)
     }
     *rc = check_launch("tpq_int4_mm (row)");
     return true;

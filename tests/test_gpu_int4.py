@@ -723,6 +723,8 @@ def test_decoder_layer_linears_batch8_against_oracle(ops):
     (4104, 5120, 64),      # two blocks per wavefront (ten wavefronts)
     (2048, 11008, 128),    # three blocks per wavefront, 15 wavefronts, the last with a block past K
     (520, 8192, 128),      # fewer tiles than workgroups: most workgroups idle
+    (5120, 13824, 128),    # four blocks per wavefront (14 wavefronts, the last with two blocks past K), several batches of one round
+    (1032, 16384, 64),     # four blocks for each of 16 wavefronts, groups of 64
 ])
 def test_mm_one_row_tile_streaming_kernel(ops, kernel_override, dtype, N, K, group):
     """kernel_override("int4_row", 1) pins the one-row kernel for every shape it can take (its default shapes are few and
