@@ -203,14 +203,22 @@ __global__ __launch_bounds__(WPB* kWave) void int4_decode_kernel(
     Chunk<MROWS, kGroups> ring[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) issue(ring[u], first + u * stride);
-    for (int c = first; c < n_chunks; c += kRing * stride) {
+    // Steady state without a branch in the body: a condition around a request makes every later wait a wait for all
+    // outstanding loads, the chunk just asked for included.  Then the chunks that are left, at most 2 kRing - 1.
+    int c = first;
+    for (; c + (2 * kRing - 1) * stride < n_chunks; c += kRing * stride) {
 #pragma unroll
         for (int u = 0; u < kRing; ++u) {
-            const int cu = c + u * stride;
-            if (cu < n_chunks) {
-                consume(ring[u], cu);
-                if (cu + kRing * stride < n_chunks) issue(ring[u], cu + kRing * stride);
-            }
+            consume(ring[u], c + u * stride);
+            issue(ring[u], c + (kRing + u) * stride);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 2 * kRing - 1; ++r) {
+        const int cu = c + r * stride;
+        if (cu < n_chunks) {
+            consume(ring[r % kRing], cu);
+            if (cu + kRing * stride < n_chunks) issue(ring[r % kRing], cu + kRing * stride);
         }
     }
     }
