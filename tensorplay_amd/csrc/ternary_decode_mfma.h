@@ -198,7 +198,10 @@ int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M
     //   N < 16384: 16 x 4 (4096 -> 11008, 2 rows: 6.7 us; 8 wavefronts 7.6, 32 channels 7.9)
     //   above: 32 x 4 (8192 -> 28672, 8 rows: 24.3 us; 16 channels 28.2, 8 wavefronts 29.4)
     const int nb = forced_nb ? forced_nb : ((N >= 8192 && N < 10240) || N >= 16384 ? 2 : 1);
-    const int waves = forced_waves ? forced_waves : (N < 10240 ? 8 : 4);
+    //   at most 256 workgroups of 16 channels and 24 steps of K or more: 16 wavefronts, two steps each instead of four
+    //   (6912 -> 2560 at 8 rows 5.4 -> 5.1 us in the sweep's harness; 2560 -> 6912, 432 workgroups: 4.7 -> 6.5, stays at 8)
+    const bool long_and_narrow = nb == 1 && N <= 16 * 256 && K >= 24 * 256;
+    const int waves = forced_waves ? forced_waves : (long_and_narrow ? 16 : N < 10240 ? 8 : 4);
     const dim3 grid(static_cast<unsigned>((N + 16 * nb - 1) / (16 * nb)));
     const int n = static_cast<int>(N), k = static_cast<int>(K);
     for (int64_t m0 = 0; m0 < M;) {
@@ -226,7 +229,7 @@ int launch_ternary_decode_mfma(const int8_t* x, const uint8_t* packed, int64_t M
         else TPQ_TDEC(NBV, 1, 1, WV);                            \
     } while (0)
         if (nb == 2) { if (waves == 8) TPQ_TDEC_X(2, 8); else TPQ_TDEC_X(2, 4); }
-        else { if (waves == 8) TPQ_TDEC_X(1, 8); else TPQ_TDEC_X(1, 4); }
+        else { if (waves == 16) TPQ_TDEC_X(1, 16); else if (waves == 8) TPQ_TDEC_X(1, 8); else TPQ_TDEC_X(1, 4); }
 #undef TPQ_TDEC_X
 #undef TPQ_TDEC
         m0 += rows;

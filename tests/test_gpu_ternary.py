@@ -51,6 +51,8 @@ CASES = [(1, 2560, 6912), (1, 6912, 2560), (4, 2560, 256), (8, 128, 67), (5, 64,
          # matrix-core decode kernel: each workgroup shape (by N), ragged N, one and two slabs of rows
          (1, 4096, 4100), (2, 2560, 8200), (16, 512, 8192), (3, 1024, 11010), (15, 256, 16390), (17, 768, 50),
          (32, 512, 8208), (31, 6912, 2560), (12, 256, 1), (1, 256, 17), (64, 512, 100), (49, 256, 8200), (63, 768, 16400),
+         # long K against at most 256 blocks of 16 channels: 16 wavefronts per workgroup (1, 2, 4 activation loads, two slabs)
+         (3, 6144, 4096), (8, 6912, 2560), (16, 8192, 1048), (23, 7168, 520),
          # slab kernel (33 rows and more, K % 128 == 0): one unit, ragged rows and channels, 21 units = two splits,
          # 40 units = two full splits, three splits with a short last one
          (33, 128, 8), (40, 384, 136), (129, 2688, 200), (128, 5120, 264), (70, 5248, 130),
